@@ -1,0 +1,41 @@
+"""The oracle the reference's own tests use: PyTorch's grouped conv on the CPU.
+
+test/test_forward.py:14 compares against ``F.conv2d(x, k, stride, padding,
+groups=C)``; test/test_grad.py:23-39 checks the gradients in fp64.  Here both
+are done in fp64 on the CPU.  TEST INFRASTRUCTURE ONLY.
+"""
+import time
+
+import torch
+from torch.nn import functional as F
+
+
+def torch_reference(x, w, gy=None, stride=1, padding=0):
+    """fp64 CPU forward (and, given gy, both gradients). Returns (y, gx, gw)."""
+    xd = x.detach().to("cpu", torch.float64).requires_grad_(gy is not None)
+    wd = w.detach().to("cpu", torch.float64).requires_grad_(gy is not None)
+    y = F.conv2d(xd, wd, stride=stride, padding=padding, groups=xd.shape[1])
+    if gy is None:
+        return y.detach(), None, None
+    gx, gw = torch.autograd.grad(y, (xd, wd), gy.detach().to("cpu", torch.float64))
+    return y.detach(), gx, gw
+
+
+def torch_cpu_fp32_step(x, w, gy, stride, padding, iters=3, threads=None):
+    """Time fp32 ``F.conv2d(groups=C)`` forward + both gradients on the host cores.
+
+    Baseline only (never the correctness oracle).  Returns (median seconds, threads).
+    """
+    if threads:
+        torch.set_num_threads(threads)
+    x = x.detach().to("cpu", torch.float32).requires_grad_(True)
+    w = w.detach().to("cpu", torch.float32).requires_grad_(True)
+    gy = gy.detach().to("cpu", torch.float32)
+    times = []
+    for _ in range(iters + 1):
+        t0 = time.perf_counter()
+        y = F.conv2d(x, w, stride=stride, padding=padding, groups=x.shape[1])
+        torch.autograd.grad(y, (x, w), gy)
+        times.append(time.perf_counter() - t0)
+    times = sorted(times[1:])
+    return times[len(times) // 2], torch.get_num_threads()
