@@ -1,0 +1,295 @@
+// extern "C" surface of libdwconv_hip (declared in include/dwconv_hip.h):
+// argument checks, kernel-family selection, error strings.
+#include "dwconv_common.hpp"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+namespace dwconv {
+
+namespace {
+thread_local char g_error[512] = "";
+thread_local char g_variant[128] = "";
+
+// DWCONV_FORCE_GENERIC=1 routes every call to the generic kernels (used by the
+// tests to cover that path at fp32 as well).
+bool force_generic()
+{
+    const char *e = std::getenv("DWCONV_FORCE_GENERIC");
+    return e != nullptr && e[0] != '\0' && e[0] != '0';
+}
+}  // namespace
+
+int fail(dwconv_status code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    std::vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+void note_variant(const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    std::vsnprintf(g_variant, sizeof(g_variant), fmt, ap);
+    va_end(ap);
+}
+
+int check_launch(const char *what)
+{
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess)
+        return fail(DWCONV_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return DWCONV_OK;
+}
+
+namespace {
+
+constexpr int kMaxSmallKernel = 15;
+
+int make_geometry(Geometry &g, const void *in, const void *taps, const void *out, int batch,
+                  int channel, int in_h, int in_w, int kernel_h, int kernel_w, int up_h, int up_w,
+                  int down_h, int down_w, int pad_h0, int pad_h1, int pad_w0, int pad_w1, int forward)
+{
+    if (batch < 0 || channel < 0 || in_h < 0 || in_w < 0)
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "negative tensor extent (%d,%d,%d,%d)", batch, channel,
+                    in_h, in_w);
+    if (kernel_h < 1 || kernel_w < 1)
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "kernel extent must be >= 1, got %dx%d", kernel_h,
+                    kernel_w);
+    if (up_h < 1 || up_w < 1 || down_h < 1 || down_w < 1)
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "up/down factors must be >= 1, got up %dx%d down %dx%d",
+                    up_h, up_w, down_h, down_w);
+    g = Geometry{batch, channel, in_h, in_w, kernel_h, kernel_w, up_h, up_w, down_h, down_w,
+                 pad_h0, pad_h1, pad_w0, pad_w1, 0, 0, forward ? 1 : 0};
+    g.out_h = dwconv_out_size(in_h, up_h, down_h, pad_h0, pad_h1, kernel_h);
+    g.out_w = dwconv_out_size(in_w, up_w, down_w, pad_w0, pad_w1, kernel_w);
+    if (g.out_h < 0) g.out_h = 0;
+    if (g.out_w < 0) g.out_w = 0;
+    const long long in_elems = 1ll * batch * channel * in_h * in_w;
+    const long long out_elems = 1ll * batch * channel * g.out_h * g.out_w;
+    if (in_elems >= (1ll << 40) || out_elems >= (1ll << 40))
+        return fail(DWCONV_ERR_UNSUPPORTED, "tensor too large");
+    if (out_elems > 0 && (taps == nullptr || out == nullptr || (in_elems > 0 && in == nullptr)))
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");
+    return DWCONV_OK;
+}
+
+template <typename T>
+int run_fir(const T *in, const T *taps, T *out, const Geometry &g, hipStream_t stream)
+{
+    if (g.planes() * g.out_h * g.out_w == 0) {
+        note_variant("empty");
+        return DWCONV_OK;
+    }
+    if constexpr (sizeof(T) == 4) {
+        if (!force_generic()) {
+            const int rc = try_launch_fir_tiled(in, taps, out, g, stream);
+            if (rc >= 0) return rc;
+        }
+    }
+    return launch_fir_direct<T>(in, taps, out, g, stream);
+}
+
+template <typename T>
+int dwconv2d_any(const T *in, const T *taps, T *out, int batch, int channel, int in_h, int in_w,
+                 int kernel_h, int kernel_w, int up_h, int up_w, int down_h, int down_w, int pad_h0,
+                 int pad_h1, int pad_w0, int pad_w1, int forward, void *stream)
+{
+    Geometry g;
+    const int rc = make_geometry(g, in, taps, out, batch, channel, in_h, in_w, kernel_h, kernel_w,
+                                 up_h, up_w, down_h, down_w, pad_h0, pad_h1, pad_w0, pad_w1, forward);
+    if (rc != DWCONV_OK) return rc;
+    return run_fir<T>(in, taps, out, g, static_cast<hipStream_t>(stream));
+}
+
+template <typename T>
+int dwconv2d_small_any(const T *in, const T *taps, T *out, int batch, int channel, int in_h,
+                       int in_w, int kernel_h, int kernel_w, int up_h, int up_w, int down_h,
+                       int down_w, int pad_h, int pad_w, int forward, void *stream)
+{
+    if (up_h != 1 || up_w != 1 || down_h != 1 || down_w != 1)
+        return fail(DWCONV_ERR_UNSUPPORTED,
+                    "dwconv2d_small handles stride-1 same-size convolutions only (up %dx%d, down %dx%d)",
+                    up_h, up_w, down_h, down_w);
+    if (in_h > 32 || in_w > 32)
+        return fail(DWCONV_ERR_UNSUPPORTED, "dwconv2d_small handles planes up to 32x32, got %dx%d",
+                    in_h, in_w);
+    if (kernel_h < 1 || kernel_w < 1 || kernel_h > kMaxSmallKernel || kernel_w > kMaxSmallKernel)
+        return fail(DWCONV_ERR_UNSUPPORTED, "dwconv2d_small handles kernels from 1x1 to %dx%d, got %dx%d",
+                    kMaxSmallKernel, kMaxSmallKernel, kernel_h, kernel_w);
+    if (pad_h < 0 || pad_h >= kernel_h || pad_w < 0 || pad_w >= kernel_w)
+        return fail(DWCONV_ERR_UNSUPPORTED, "dwconv2d_small needs 0 <= pad < kernel, got pad %dx%d kernel %dx%d",
+                    pad_h, pad_w, kernel_h, kernel_w);
+    // Same-size output: trailing pad = kernel - 1 - leading pad.
+    return dwconv2d_any<T>(in, taps, out, batch, channel, in_h, in_w, kernel_h, kernel_w, 1, 1, 1, 1,
+                           pad_h, kernel_h - 1 - pad_h, pad_w, kernel_w - 1 - pad_w, forward, stream);
+}
+
+int make_wgrad_geometry(WgradGeometry &g, const void *in, const void *gy, const void *gw, int batch,
+                        int channel, int in_h, int in_w, int out_h, int out_w, int kernel_h,
+                        int kernel_w, int up_h, int up_w, int down_h, int down_w, int pad_h, int pad_w)
+{
+    if (batch < 0 || channel < 0 || in_h < 0 || in_w < 0 || out_h < 0 || out_w < 0)
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "negative tensor extent");
+    if (kernel_h < 1 || kernel_w < 1)
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "kernel extent must be >= 1, got %dx%d", kernel_h,
+                    kernel_w);
+    if (up_h != 1 || up_w != 1)
+        return fail(DWCONV_ERR_UNSUPPORTED, "grad-weight is defined for up == 1 only, got %dx%d", up_h,
+                    up_w);
+    if (down_h < 1 || down_w < 1)
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "down factors must be >= 1");
+    if (1ll * batch * channel * in_h * in_w >= (1ll << 40) ||
+        1ll * batch * channel * out_h * out_w >= (1ll << 40))
+        return fail(DWCONV_ERR_UNSUPPORTED, "tensor too large");
+    if (channel > 0 && gw == nullptr)
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "null kernel_grad pointer");
+    const bool has_work = 1ll * batch * channel * out_h * out_w > 0 && in_h > 0 && in_w > 0;
+    if (has_work && (in == nullptr || gy == nullptr))
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");
+    g = WgradGeometry{batch, channel, in_h, in_w, out_h, out_w, kernel_h, kernel_w, down_h, down_w,
+                      pad_h, pad_w};
+    return DWCONV_OK;
+}
+
+template <typename T>
+size_t wgrad_workspace(const WgradGeometry &g)
+{
+    size_t need = wgrad_direct_workspace<T>(g);
+    if constexpr (sizeof(T) == 4) {
+        const size_t t = wgrad_tiled_workspace(g);
+        if (t > need) need = t;
+    }
+    return need;
+}
+
+template <typename T>
+int wgrad_any(const T *in, const T *gy, T *gw, void *ws, size_t ws_bytes, int batch, int channel,
+              int in_h, int in_w, int out_h, int out_w, int kernel_h, int kernel_w, int up_h, int up_w,
+              int down_h, int down_w, int pad_h, int pad_w, void *stream_)
+{
+    WgradGeometry g;
+    const int rc = make_wgrad_geometry(g, in, gy, gw, batch, channel, in_h, in_w, out_h, out_w, kernel_h,
+                                       kernel_w, up_h, up_w, down_h, down_w, pad_h, pad_w);
+    if (rc != DWCONV_OK) return rc;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const long taps = static_cast<long>(channel) * kernel_h * kernel_w;
+    if (taps == 0) {
+        note_variant("empty");
+        return DWCONV_OK;
+    }
+    if (1ll * batch * out_h * out_w == 0 || in_h == 0 || in_w == 0) {
+        // nothing to sum: the gradient is zero (a fill kernel, not a memset node,
+        // so that the call may be captured into a graph)
+        note_variant("zero");
+        return launch_fill_zero(gw, static_cast<size_t>(taps) * sizeof(T), stream);
+    }
+    if constexpr (sizeof(T) == 4) {
+        if (!force_generic() && wgrad_tiled_workspace(g) > 0) {
+            const int r = try_launch_wgrad_tiled(in, gy, gw, ws, ws_bytes, g, stream);
+            if (r >= 0) return r;
+        }
+    }
+    return launch_wgrad_direct<T>(in, gy, gw, ws, ws_bytes, g, stream);
+}
+
+}  // namespace
+}  // namespace dwconv
+
+using namespace dwconv;
+
+extern "C" {
+
+const char *dwconv_last_error(void) { return g_error; }
+const char *dwconv_last_variant(void) { return g_variant; }
+const char *dwconv_version(void) { return "dwconv_hip 0.1 gfx950"; }
+
+int dwconv_out_size(int in, int up, int down, int pad0, int pad1, int k)
+{
+    if (down < 1) return 0;
+    return (in * up + pad0 + pad1 - k + down) / down;
+}
+
+int dwconv_use_dwconv2d_small(int in_h, int in_w, int kernel_h, int kernel_w, int up_h, int up_w,
+                              int down_h, int down_w, int pad_h, int pad_w)
+{
+    if (down_h != 1 || down_w != 1) return 0;
+    if (in_h > 32 || in_w > 32) return 0;
+    if (pad_h < 0 || pad_h >= kernel_h || pad_w < 0 || pad_w >= kernel_w) return 0;
+    const int out_h = dwconv_out_size(in_h, up_h, 1, pad_h, pad_h, kernel_h);
+    const int out_w = dwconv_out_size(in_w, up_w, 1, pad_w, pad_w, kernel_w);
+    if (out_h != in_h || out_w != in_w) return 0;
+    // the reference's lane budget: one lane per two rows must cover the taps
+    return kernel_h * kernel_w <= (in_h + 1) / 2 * in_w ? 1 : 0;
+}
+
+int dwconv2d_f32(const float *input, const float *kernel, float *out, int batch, int channel,
+                 int in_h, int in_w, int kernel_h, int kernel_w, int up_h, int up_w, int down_h,
+                 int down_w, int pad_h0, int pad_h1, int pad_w0, int pad_w1, int forward, void *stream)
+{
+    return dwconv2d_any<float>(input, kernel, out, batch, channel, in_h, in_w, kernel_h, kernel_w, up_h,
+                               up_w, down_h, down_w, pad_h0, pad_h1, pad_w0, pad_w1, forward, stream);
+}
+
+int dwconv2d_f64(const double *input, const double *kernel, double *out, int batch, int channel,
+                 int in_h, int in_w, int kernel_h, int kernel_w, int up_h, int up_w, int down_h,
+                 int down_w, int pad_h0, int pad_h1, int pad_w0, int pad_w1, int forward, void *stream)
+{
+    return dwconv2d_any<double>(input, kernel, out, batch, channel, in_h, in_w, kernel_h, kernel_w, up_h,
+                                up_w, down_h, down_w, pad_h0, pad_h1, pad_w0, pad_w1, forward, stream);
+}
+
+int dwconv2d_small_f32(const float *input, const float *kernel, float *out, int batch, int channel,
+                       int in_h, int in_w, int kernel_h, int kernel_w, int up_h, int up_w, int down_h,
+                       int down_w, int pad_h, int pad_w, int forward, void *stream)
+{
+    return dwconv2d_small_any<float>(input, kernel, out, batch, channel, in_h, in_w, kernel_h, kernel_w,
+                                     up_h, up_w, down_h, down_w, pad_h, pad_w, forward, stream);
+}
+
+int dwconv2d_small_f64(const double *input, const double *kernel, double *out, int batch, int channel,
+                       int in_h, int in_w, int kernel_h, int kernel_w, int up_h, int up_w, int down_h,
+                       int down_w, int pad_h, int pad_w, int forward, void *stream)
+{
+    return dwconv2d_small_any<double>(input, kernel, out, batch, channel, in_h, in_w, kernel_h, kernel_w,
+                                      up_h, up_w, down_h, down_w, pad_h, pad_w, forward, stream);
+}
+
+size_t dwconv2d_backward_kernel_workspace_bytes(int batch, int channel, int in_h, int in_w, int out_h,
+                                                int out_w, int kernel_h, int kernel_w, int down_h,
+                                                int down_w, int pad_h, int pad_w, int elem_size)
+{
+    if (batch <= 0 || channel <= 0 || kernel_h < 1 || kernel_w < 1 || down_h < 1 || down_w < 1) return 0;
+    const WgradGeometry g{batch, channel, in_h, in_w, out_h, out_w, kernel_h, kernel_w,
+                          down_h, down_w, pad_h, pad_w};
+    return elem_size == 8 ? wgrad_workspace<double>(g) : wgrad_workspace<float>(g);
+}
+
+int dwconv2d_backward_kernel_f32(const float *input, const float *out_grad, float *kernel_grad,
+                                 void *workspace, size_t workspace_bytes, int batch, int channel,
+                                 int in_h, int in_w, int out_h, int out_w, int kernel_h, int kernel_w,
+                                 int up_h, int up_w, int down_h, int down_w, int pad_h, int pad_w,
+                                 void *stream)
+{
+    return wgrad_any<float>(input, out_grad, kernel_grad, workspace, workspace_bytes, batch, channel,
+                            in_h, in_w, out_h, out_w, kernel_h, kernel_w, up_h, up_w, down_h, down_w,
+                            pad_h, pad_w, stream);
+}
+
+int dwconv2d_backward_kernel_f64(const double *input, const double *out_grad, double *kernel_grad,
+                                 void *workspace, size_t workspace_bytes, int batch, int channel,
+                                 int in_h, int in_w, int out_h, int out_w, int kernel_h, int kernel_w,
+                                 int up_h, int up_w, int down_h, int down_w, int pad_h, int pad_w,
+                                 void *stream)
+{
+    return wgrad_any<double>(input, out_grad, kernel_grad, workspace, workspace_bytes, batch, channel,
+                             in_h, in_w, out_h, out_w, kernel_h, kernel_w, up_h, up_w, down_h, down_w,
+                             pad_h, pad_w, stream);
+}
+
+}  // extern "C"

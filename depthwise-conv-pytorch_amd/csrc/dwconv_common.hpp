@@ -1,0 +1,75 @@
+// Shared declarations of libdwconv_hip: geometry, error reporting and the
+// launch functions each translation unit provides.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+#include "dwconv_hip.h"
+
+namespace dwconv {
+
+// Geometry of one up/FIR/down call on dense NCHW planes.  The same fields as the
+// reference's DWConv2dKernelParams (torch_dwconv/dwconv_kernel.cu:42-67), with the
+// batch and channel extents folded into `planes` where a kernel does not need them.
+struct Geometry {
+    int batch, channel;
+    int in_h, in_w;
+    int kernel_h, kernel_w;
+    int up_h, up_w;
+    int down_h, down_w;
+    int pad_h0, pad_h1, pad_w0, pad_w1;
+    int out_h, out_w;
+    int forward;
+    long planes() const { return static_cast<long>(batch) * channel; }
+};
+
+// Geometry of a grad-weight call.
+struct WgradGeometry {
+    int batch, channel;
+    int in_h, in_w;
+    int out_h, out_w;
+    int kernel_h, kernel_w;
+    int down_h, down_w;
+    int pad_h, pad_w;
+};
+
+// Thread-local error/variant strings behind dwconv_last_error()/dwconv_last_variant().
+int fail(dwconv_status code, const char *fmt, ...);
+void note_variant(const char *fmt, ...);
+int check_launch(const char *what);
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+inline int round_up(int a, int b) { return ceil_div(a, b) * b; }
+
+// Reciprocal m with n / d == (n * m) >> 32 for 0 <= n < 65536 and 2 <= d < 65536;
+// d == 1 is encoded as m == 0 (the kernels test for it).
+inline unsigned magic_u16(unsigned d) { return d <= 1 ? 0u : static_cast<unsigned>((0x100000000ull + d - 1) / d); }
+
+// ---- generic kernels (any geometry, float or double): dwconv_generic.hip ----
+template <typename T>
+int launch_fir_direct(const T *in, const T *taps, T *out, const Geometry &g, hipStream_t stream);
+// Zero-fills `bytes` (a multiple of 4) with a kernel rather than a memset node.
+int launch_fill_zero(void *p, size_t bytes, hipStream_t stream);
+template <typename T>
+size_t wgrad_direct_workspace(const WgradGeometry &g);
+template <typename T>
+int launch_wgrad_direct(const T *in, const T *gy, T *gw, void *ws, size_t ws_bytes,
+                        const WgradGeometry &g, hipStream_t stream);
+
+// ---- LDS-tiled fp32 kernels: dwconv_tile.hip ----
+// Return DWCONV_OK after launching, a negative value (-1) when the geometry is
+// outside what the tiled kernels cover (the caller then uses the generic kernel),
+// or a positive dwconv_status on a launch error.
+int try_launch_fir_tiled(const float *in, const float *taps, float *out, const Geometry &g,
+                         hipStream_t stream);
+
+// ---- fp32 grad-weight with LDS tiles and a fixed-order two-pass reduction: dwconv_wgrad.hip ----
+size_t wgrad_tiled_workspace(const WgradGeometry &g);  // 0 when the tiled kernel does not cover g
+int try_launch_wgrad_tiled(const float *in, const float *gy, float *gw, void *ws, size_t ws_bytes,
+                           const WgradGeometry &g, hipStream_t stream);
+
+}  // namespace dwconv

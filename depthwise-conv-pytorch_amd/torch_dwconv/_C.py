@@ -1,0 +1,174 @@
+"""Binding of libdwconv_hip.so that stands where the reference's pybind11
+module ``torch_dwconv._C`` stands (torch_dwconv/dwconv.cpp:60-67).
+
+The four functions keep the reference's names, argument order and error
+behaviour (a non-GPU tensor raises ``RuntimeError('... must be a CUDA
+tensor')``, torch_dwconv/dwconv.cpp:24-25).  They allocate the result with
+torch, pass raw device pointers plus the current HIP stream through the C ABI
+declared in include/dwconv_hip.h, and return immediately (no synchronisation).
+
+There is no CPU implementation behind this module: if the shared library is
+missing, importing it raises ImportError.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIBRARY_PATH = os.path.join(_HERE, "libdwconv_hip.so")
+
+if not os.path.exists(LIBRARY_PATH):
+    raise ImportError(
+        f"{LIBRARY_PATH} is missing: build it with `make -C depthwise-conv-pytorch_amd/csrc` "
+        "(hipcc, --offload-arch=gfx950). torch_dwconv has no fallback implementation."
+    )
+
+_lib = ctypes.CDLL(LIBRARY_PATH)
+
+_i, _p, _z = ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
+_lib.dwconv_last_error.restype = ctypes.c_char_p
+_lib.dwconv_last_variant.restype = ctypes.c_char_p
+_lib.dwconv_version.restype = ctypes.c_char_p
+_lib.dwconv_out_size.restype = _i
+_lib.dwconv_out_size.argtypes = [_i] * 6
+_lib.dwconv_use_dwconv2d_small.restype = _i
+_lib.dwconv_use_dwconv2d_small.argtypes = [_i] * 10
+for _name in ("dwconv2d_f32", "dwconv2d_f64"):
+    getattr(_lib, _name).restype = _i
+    getattr(_lib, _name).argtypes = [_p, _p, _p] + [_i] * 15 + [_p]
+for _name in ("dwconv2d_small_f32", "dwconv2d_small_f64"):
+    getattr(_lib, _name).restype = _i
+    getattr(_lib, _name).argtypes = [_p, _p, _p] + [_i] * 13 + [_p]
+_lib.dwconv2d_backward_kernel_workspace_bytes.restype = _z
+_lib.dwconv2d_backward_kernel_workspace_bytes.argtypes = [_i] * 13
+for _name in ("dwconv2d_backward_kernel_f32", "dwconv2d_backward_kernel_f64"):
+    getattr(_lib, _name).restype = _i
+    getattr(_lib, _name).argtypes = [_p, _p, _p, _p, _z] + [_i] * 14 + [_p]
+
+_SUFFIX = {torch.float32: "f32", torch.float64: "f64"}
+
+
+def version():
+    return _lib.dwconv_version().decode()
+
+
+def last_variant():
+    """Name of the kernel variant the last call on this thread launched."""
+    return _lib.dwconv_last_variant().decode()
+
+
+def _check_cuda(t, name):
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+
+
+def _suffix(*tensors):
+    dtype = tensors[0].dtype
+    if dtype not in _SUFFIX:
+        raise RuntimeError(f"torch_dwconv supports float32 and float64 tensors, got {dtype}")
+    for t in tensors[1:]:
+        if t.dtype != dtype:
+            raise RuntimeError(f"torch_dwconv needs tensors of one dtype, got {dtype} and {t.dtype}")
+        if t.device != tensors[0].device:
+            raise RuntimeError(f"torch_dwconv needs tensors on one device, got {tensors[0].device} and {t.device}")
+    return _SUFFIX[dtype]
+
+
+def _check_shapes(input, kernel):
+    if input.dim() != 4 or kernel.dim() != 4:
+        raise RuntimeError("torch_dwconv expects a 4-D input (N,C,H,W) and a 4-D kernel (C,1,KH,KW)")
+    if kernel.shape[0] != input.shape[1] or kernel.shape[1] != 1:
+        raise RuntimeError(
+            f"kernel of shape {tuple(kernel.shape)} does not match an input with {input.shape[1]} channels: "
+            "expected (C,1,KH,KW)"
+        )
+
+
+def _raise(status):
+    raise RuntimeError(f"libdwconv_hip error {status}: {_lib.dwconv_last_error().decode()}")
+
+
+def _stream(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def use_dwconv2d_small(input, kernel, up_h, up_w, down_h, down_w, pad_h, pad_w):
+    """torch_dwconv/dwconv_kernel.cu:652-662; pure geometry, no device work."""
+    return bool(
+        _lib.dwconv_use_dwconv2d_small(
+            input.shape[2], input.shape[3], kernel.shape[2], kernel.shape[3],
+            up_h, up_w, down_h, down_w, pad_h, pad_w,
+        )
+    )
+
+
+def dwconv2d(input, kernel, up_h, up_w, down_h, down_w, pad_h0, pad_h1, pad_w0, pad_w1, forward):
+    """torch_dwconv/dwconv.cpp:27-35: up-sample / filter / down-sample of every plane."""
+    _check_cuda(input, "input")
+    _check_cuda(kernel, "kernel")
+    _check_shapes(input, kernel)
+    sfx = _suffix(input, kernel)
+    x, k = input.contiguous(), kernel.contiguous()
+    n, c, h, w = x.shape
+    kh, kw = k.shape[2], k.shape[3]
+    oh = max(_lib.dwconv_out_size(h, up_h, down_h, pad_h0, pad_h1, kh), 0)
+    ow = max(_lib.dwconv_out_size(w, up_w, down_w, pad_w0, pad_w1, kw), 0)
+    out = torch.empty((n, c, oh, ow), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = getattr(_lib, "dwconv2d_" + sfx)(
+            x.data_ptr(), k.data_ptr(), out.data_ptr(), n, c, h, w, kh, kw,
+            up_h, up_w, down_h, down_w, pad_h0, pad_h1, pad_w0, pad_w1, int(bool(forward)), _stream(x),
+        )
+    if rc != 0:
+        _raise(rc)
+    return out
+
+
+def dwconv2d_small(input, kernel, up_h, up_w, down_h, down_w, pad_h, pad_w, forward):
+    """torch_dwconv/dwconv.cpp:37-46: whole-plane stride-1 same-size convolution."""
+    _check_cuda(input, "input")
+    _check_cuda(kernel, "kernel")
+    _check_shapes(input, kernel)
+    sfx = _suffix(input, kernel)
+    x, k = input.contiguous(), kernel.contiguous()
+    n, c, h, w = x.shape
+    out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        rc = getattr(_lib, "dwconv2d_small_" + sfx)(
+            x.data_ptr(), k.data_ptr(), out.data_ptr(), n, c, h, w, k.shape[2], k.shape[3],
+            up_h, up_w, down_h, down_w, pad_h, pad_w, int(bool(forward)), _stream(x),
+        )
+    if rc != 0:
+        _raise(rc)
+    return out
+
+
+def dwconv2d_backward_kernel(input, out_grad, kernel, up_h, up_w, down_h, down_w, pad_h, pad_w):
+    """torch_dwconv/dwconv.cpp:48-58: gradient of the filter; `kernel` only lends its shape."""
+    _check_cuda(input, "input")
+    _check_cuda(out_grad, "out_grad")
+    if input.dim() != 4 or out_grad.dim() != 4 or kernel.dim() != 4:
+        raise RuntimeError("torch_dwconv expects 4-D tensors")
+    if out_grad.shape[:2] != input.shape[:2] or kernel.shape[0] != input.shape[1]:
+        raise RuntimeError(
+            f"shapes do not belong to one depthwise conv: input {tuple(input.shape)}, "
+            f"out_grad {tuple(out_grad.shape)}, kernel {tuple(kernel.shape)}"
+        )
+    sfx = _suffix(input, out_grad)
+    x, gy = input.contiguous(), out_grad.contiguous()
+    n, c, h, w = x.shape
+    oh, ow = gy.shape[2], gy.shape[3]
+    kh, kw = kernel.shape[2], kernel.shape[3]
+    gw = torch.empty((c, 1, kh, kw), dtype=x.dtype, device=x.device)
+    geom = (n, c, h, w, oh, ow, kh, kw)
+    ws_bytes = _lib.dwconv2d_backward_kernel_workspace_bytes(*geom, down_h, down_w, pad_h, pad_w, x.element_size())
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = getattr(_lib, "dwconv2d_backward_kernel_" + sfx)(
+            x.data_ptr(), gy.data_ptr(), gw.data_ptr(), ws.data_ptr(), ws_bytes, *geom,
+            up_h, up_w, down_h, down_w, pad_h, pad_w, _stream(x),
+        )
+    if rc != 0:
+        _raise(rc)
+    return gw

@@ -1,0 +1,5 @@
+"""Depthwise conv2d for AMD MI355X behind the ``torch_dwconv`` API.
+
+Public surface of the reference package (torch_dwconv/__init__.py:1).
+"""
+from .dwconv import depthwise_conv2d, DepthwiseConv2d  # noqa: F401

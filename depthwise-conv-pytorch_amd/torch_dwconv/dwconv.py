@@ -1,0 +1,146 @@
+"""Python surface of the depthwise conv2d op: same names, argument order and
+errors as the reference's torch_dwconv/dwconv.py, on top of the HIP library.
+
+``depthwise_conv2d(input, weight, bias=None, stride=1, padding=0, dilation=1,
+groups=None)`` computes what ``F.conv2d(input, weight, stride=stride,
+padding=padding, groups=C)`` computes, for GPU tensors in float32 or float64.
+
+One deliberate difference: the reference hands planes of at most 32x32 that its
+small kernel cannot take (stride 2, or a filter too large for the plane) to
+``F.conv2d`` (torch_dwconv/dwconv.py:125-128).  Here those go through the HIP
+library as well, so nothing inside ``custom=True`` ever leaves it; the values
+are the same function either way.
+"""
+import torch
+from torch import nn
+from torch.autograd import Function
+from torch.nn import functional as F
+
+from . import _C
+
+
+def make_tuple(value, n_value):
+    """Reference: torch_dwconv/dwconv.py:76-91.
+
+    A scalar becomes ``n_value`` copies; a list/tuple that is longer raises
+    ``ValueError``; one of exactly that length is returned unchanged; a shorter
+    one is repeated ``n_value`` times.
+    """
+    if isinstance(value, (list, tuple)):
+        have = len(value)
+        if have > n_value:
+            raise ValueError(
+                f'Number items does not match with requirements: {have}, expected: {n_value}'
+            )
+        return value if have == n_value else value * n_value
+    return (value,) * n_value
+
+
+_UNSUPPORTED = (
+    # (predicate over the normalised options, message) in the reference's order,
+    # torch_dwconv/dwconv.py:99-112
+    (lambda o: o['dilation'][0] > 1 or o['dilation'][1] > 1,
+     'DepthwiseConv2d does not support dilations > 1'),
+    (lambda o: o['groups'] is not None and o['groups'] != o['in_channels'],
+     'DepthwiseConv2d does not support groups != in_channels'),
+    (lambda o: o['in_channels'] != o['out_channels'],
+     'DepthwiseConv2d does not support in_channels != out_channels'),
+    (lambda o: bool(o['bias']),
+     'DepthwiseConv2d does not support bias'),
+    (lambda o: o['padding_mode'] != 'zeros',
+     'DepthwiseConv2d does not non-zero paddings'),
+)
+
+
+def check_options(in_channels, out_channels, dilation, groups, bias, padding_mode='zeros'):
+    """Reference: torch_dwconv/dwconv.py:94-112. Raises ``ValueError`` on the first unsupported option."""
+    options = dict(
+        in_channels=in_channels, out_channels=out_channels, dilation=make_tuple(dilation, 2),
+        groups=groups, bias=bias, padding_mode=padding_mode,
+    )
+    for rejected, message in _UNSUPPORTED:
+        if rejected(options):
+            raise ValueError(message)
+
+
+def use_dwconv2d_small(input, weight, up, stride, padding):
+    """Reference: torch_dwconv/dwconv.py:9-12."""
+    return _C.use_dwconv2d_small(input, weight, up[0], up[1], stride[0], stride[1], padding[0], padding[1])
+
+
+class DepthwiseConv2dFunction(Function):
+    """Reference: torch_dwconv/dwconv.py:15-70 (same arguments, same six-value backward)."""
+
+    @staticmethod
+    def forward(ctx, input, kernel, stride, pad, small):
+        ctx.save_for_backward(input, kernel)
+        ctx.stride, ctx.pad, ctx.use_small = stride, pad, small
+        if small:
+            out = _C.dwconv2d_small(input, kernel, 1, 1, stride[0], stride[1], pad[0], pad[1], True)
+        else:
+            out = _C.dwconv2d(input, kernel, 1, 1, stride[0], stride[1], pad[0], pad[0], pad[1], pad[1], True)
+        # Padding of the transposed problem (reference :39-44): leading k-1-p zeros, and trailing
+        # whatever makes the gradient come out with the input's extent (this also covers the rows
+        # and columns a stride leaves unused).
+        ctx.g_pad = tuple(
+            v
+            for axis in (0, 1)
+            for v in (
+                kernel.shape[2 + axis] - pad[axis] - 1,
+                input.shape[2 + axis] - out.shape[2 + axis] * stride[axis] + pad[axis],
+            )
+        )
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, kernel = ctx.saved_tensors
+        stride, pad, g_pad = ctx.stride, ctx.pad, ctx.g_pad
+        # The reference always computes both gradients (:48-70).
+        if ctx.use_small:
+            grad_input = _C.dwconv2d_small(
+                grad_output, kernel, stride[0], stride[1], 1, 1, g_pad[0], g_pad[2], False
+            )
+        else:
+            grad_input = _C.dwconv2d(grad_output, kernel, stride[0], stride[1], 1, 1, *g_pad, False)
+        grad_kernel = _C.dwconv2d_backward_kernel(
+            input, grad_output, kernel, 1, 1, stride[0], stride[1], pad[0], pad[1]
+        )
+        return grad_input, grad_kernel, None, None, None, None
+
+
+depthwise_conv2d_fn = DepthwiseConv2dFunction.apply
+
+
+def depthwise_conv2d(input, weight, bias=None, stride=1, padding=0, dilation=1, groups=None):
+    """Reference: torch_dwconv/dwconv.py:115-130."""
+    stride = make_tuple(stride, 2)
+    padding = make_tuple(padding, 2)
+    check_options(input.shape[1], weight.shape[0], dilation, groups, bias)
+    small = use_dwconv2d_small(input, weight, (1, 1), stride, padding)
+    return depthwise_conv2d_fn(input, weight, stride, padding, small)
+
+
+class DepthwiseConv2d(nn.Module):
+    """Reference: torch_dwconv/dwconv.py:133-175.
+
+    ``weight`` has the shape and ``state_dict`` key of ``nn.Conv2d(C, C, k, groups=C, bias=False)``;
+    ``custom=False`` runs PyTorch's own grouped convolution instead of this library.
+    """
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
+                 groups=None, bias=False, padding_mode='zeros', custom=True):
+        super().__init__()
+        check_options(in_channels, out_channels, dilation, groups, bias, padding_mode)
+        self.in_channel = in_channels
+        self.kernel_size = kernel_size
+        self.stride = stride
+        self.padding = padding
+        self.custom = custom
+        self.weight = nn.Parameter(torch.randn(out_channels, 1, kernel_size, kernel_size))
+
+    def forward(self, input):
+        if not self.custom:
+            return F.conv2d(input, self.weight, stride=self.stride, padding=self.padding,
+                            groups=input.shape[1])
+        return depthwise_conv2d(input, self.weight, None, self.stride, self.padding)

@@ -1,0 +1,142 @@
+/*
+ * libdwconv_hip -- depthwise conv2d (forward, grad-input, grad-weight) for
+ * AMD MI355X (gfx950), plain C ABI.
+ *
+ * These entry points are what a binding of the reference's extension module
+ * `torch_dwconv._C` (torch_dwconv/dwconv.cpp:60-67) needs: one C function per
+ * bound function, taking raw device pointers and integer geometry instead of
+ * torch::Tensor.  Tensors are dense NCHW, `kernel` is (C,1,KH,KW).  All
+ * pointers are device pointers valid on the device that is current when the
+ * call is made; `stream` is a hipStream_t (NULL = the null stream).  Calls
+ * only enqueue work and return; nothing is synchronised and nothing is kept
+ * after the call returns.  The library allocates no device memory.
+ *
+ * Return value: DWCONV_OK (0) or a dwconv_status error code.  After an error
+ * dwconv_last_error() returns a message for the calling thread.
+ *
+ * Geometry common to all entry points (the reference's DWConv2dKernelParams,
+ * torch_dwconv/dwconv_kernel.cu:42-67):
+ *   up_*   zero-stuffing factor applied to the input before filtering
+ *   down_* decimation applied after filtering (the conv stride)
+ *   pad_*  zeros added before (pad_*0) and after (pad_*1) the stuffed input
+ *   forward != 0: taps used as stored (cross-correlation);
+ *   forward == 0: taps rotated by 180 degrees (the grad-input direction).
+ */
+#ifndef DWCONV_HIP_H
+#define DWCONV_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum dwconv_status {
+    DWCONV_OK = 0,
+    DWCONV_ERR_INVALID_ARGUMENT = 1, /* null pointer, non-positive extent, ... */
+    DWCONV_ERR_UNSUPPORTED = 2,      /* geometry outside what the entry point accepts */
+    DWCONV_ERR_WORKSPACE = 3,        /* workspace missing or too small */
+    DWCONV_ERR_LAUNCH = 4            /* HIP reported an error at launch */
+} dwconv_status;
+
+/* Message describing the last error returned to this thread ("" if none). */
+const char *dwconv_last_error(void);
+
+/* Library version string, e.g. "dwconv_hip 0.1 gfx950". */
+const char *dwconv_version(void);
+
+/* Output extent along one axis: (in*up + pad0 + pad1 - k + down) / down.
+ * Replaces the arithmetic of make_conv2d_params,
+ * torch_dwconv/dwconv_kernel.cu:612-615. */
+int dwconv_out_size(int in, int up, int down, int pad0, int pad1, int k);
+
+/* Replaces `_C.use_dwconv2d_small` (torch_dwconv/dwconv.cpp:60,
+ * torch_dwconv/dwconv_kernel.cu:652-662): 1 when the geometry is a stride-1,
+ * same-size convolution of a plane no larger than 32x32 that the whole-plane
+ * entry point dwconv2d_small_* accepts, else 0. */
+int dwconv_use_dwconv2d_small(int in_h, int in_w, int kernel_h, int kernel_w,
+                              int up_h, int up_w, int down_h, int down_w,
+                              int pad_h, int pad_w);
+
+/* Replaces `_C.dwconv2d` (torch_dwconv/dwconv.cpp:27-35 ->
+ * dwconv2d_op, torch_dwconv/dwconv_kernel.cu:847-869).
+ *   out[n,c,oy,ox] = sum_{ty,tx} U[oy*down_h - pad_h0 + ty, ox*down_w - pad_w0 + tx] * f[c,ty,tx]
+ * U = input with up-1 zeros stuffed after every sample, zero outside.
+ * `out` holds batch*channel*out_h*out_w elements, out_* = dwconv_out_size(...).
+ * Accepts every up>=1, down>=1, kernel extent >=1 and pad >= -(extent) (the
+ * reference supports nine hard-coded combinations and is undefined elsewhere,
+ * dwconv_kernel.cu:808-845).  Forward convolution: up=1, down=stride,
+ * pad0=pad1=padding.  Grad-input: input=grad_output, up=stride, down=1,
+ * pads = g_pad of torch_dwconv/dwconv.py:39-44, forward=0. */
+int dwconv2d_f32(const float *input, const float *kernel, float *out,
+                 int batch, int channel, int in_h, int in_w,
+                 int kernel_h, int kernel_w, int up_h, int up_w,
+                 int down_h, int down_w, int pad_h0, int pad_h1,
+                 int pad_w0, int pad_w1, int forward, void *stream);
+int dwconv2d_f64(const double *input, const double *kernel, double *out,
+                 int batch, int channel, int in_h, int in_w,
+                 int kernel_h, int kernel_w, int up_h, int up_w,
+                 int down_h, int down_w, int pad_h0, int pad_h1,
+                 int pad_w0, int pad_w1, int forward, void *stream);
+
+/* Replaces `_C.dwconv2d_small` (torch_dwconv/dwconv.cpp:37-46 ->
+ * dwconv2d_small_op, torch_dwconv/dwconv_kernel.cu:734-771): stride-1
+ * convolution whose output has the input's extent; `pad_h`,`pad_w` zeros lead
+ * each axis and kernel-1-pad trail it.  up_* and down_* must be 1 and the plane
+ * at most 32x32 (DWCONV_ERR_UNSUPPORTED otherwise); unlike the reference the
+ * kernel may be any size up to 15x15. */
+int dwconv2d_small_f32(const float *input, const float *kernel, float *out,
+                       int batch, int channel, int in_h, int in_w,
+                       int kernel_h, int kernel_w, int up_h, int up_w,
+                       int down_h, int down_w, int pad_h, int pad_w,
+                       int forward, void *stream);
+int dwconv2d_small_f64(const double *input, const double *kernel, double *out,
+                       int batch, int channel, int in_h, int in_w,
+                       int kernel_h, int kernel_w, int up_h, int up_w,
+                       int down_h, int down_w, int pad_h, int pad_w,
+                       int forward, void *stream);
+
+/* Bytes of device scratch that dwconv2d_backward_kernel_* needs for this
+ * geometry (0 is possible).  The reference allocates its own zero-filled
+ * result and accumulates into it with atomics (dwconv_kernel.cu:1026, :304,
+ * :583); here the caller lends a workspace for per-workgroup partial sums that
+ * a second kernel adds up in a fixed order.  `elem_size` is 4 or 8. */
+size_t dwconv2d_backward_kernel_workspace_bytes(int batch, int channel,
+                                                int in_h, int in_w,
+                                                int out_h, int out_w,
+                                                int kernel_h, int kernel_w,
+                                                int down_h, int down_w,
+                                                int pad_h, int pad_w,
+                                                int elem_size);
+
+/* Replaces `_C.dwconv2d_backward_kernel` (torch_dwconv/dwconv.cpp:48-58 ->
+ * dwconv2d_backward_kernel_op, torch_dwconv/dwconv_kernel.cu:1015-1036).
+ *   kernel_grad[c,i,j] = sum_{n,oy,ox} out_grad[n,c,oy,ox] *
+ *                        input[n,c, oy*down_h - pad_h + i, ox*down_w - pad_w + j]
+ * (taps falling outside `input` contribute nothing).  kernel_grad (C*KH*KW
+ * elements) is overwritten; it need not be zeroed.  The result is bit-identical
+ * from run to run.  up_* must be 1 (the reference ignores it). */
+int dwconv2d_backward_kernel_f32(const float *input, const float *out_grad,
+                                 float *kernel_grad, void *workspace,
+                                 size_t workspace_bytes, int batch, int channel,
+                                 int in_h, int in_w, int out_h, int out_w,
+                                 int kernel_h, int kernel_w, int up_h, int up_w,
+                                 int down_h, int down_w, int pad_h, int pad_w,
+                                 void *stream);
+int dwconv2d_backward_kernel_f64(const double *input, const double *out_grad,
+                                 double *kernel_grad, void *workspace,
+                                 size_t workspace_bytes, int batch, int channel,
+                                 int in_h, int in_w, int out_h, int out_w,
+                                 int kernel_h, int kernel_w, int up_h, int up_w,
+                                 int down_h, int down_w, int pad_h, int pad_w,
+                                 void *stream);
+
+/* Tuning/diagnostic hook: name of the kernel variant the last successful call
+ * on this thread launched (e.g. "tile_f32<k3,s1,v4>"), for benchmarks and tests. */
+const char *dwconv_last_variant(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* DWCONV_HIP_H */

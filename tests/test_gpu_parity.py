@@ -1,0 +1,319 @@
+"""GPU parity: the HIP library (through its C ABI, via torch_dwconv._C) against the CPU oracle.
+
+Tolerances (fp32): forward and grad-input rtol = atol = 1e-5 against the fp64
+oracle; grad-weight rtol 1e-4 with atol = 1e-4 * max|gw_ref| (its entries are
+sums of up to N*Ho*Wo products, so a bare relative bound fails on entries that
+happen to land near zero whatever the summation order), and bit-identical from
+run to run.  fp64 kernels: 1e-11.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from shapes import (CFG1, CFG2, CFG4, CONVNEXT_T, REF_FORWARD, REF_GRAD, STRESS, effnet_layers,
+                    make_inputs, out_hw, shape_id)
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "dwconv_golden.npz")
+
+
+@pytest.fixture(scope="module")
+def dw(gpu):
+    import torch_dwconv.dwconv as m
+
+    return m
+
+
+def _np(t):
+    return t.detach().cpu().numpy()
+
+
+def _announce(*what):
+    print("[case]", *what, flush=True)
+
+
+def run_three_passes(dw, x, w, gy, stride, padding):
+    """forward, grad-input, grad-weight through the autograd Function."""
+    from torch_dwconv import _C
+
+    xg = x.detach().clone().requires_grad_(True)
+    wg = w.detach().clone().requires_grad_(True)
+    y = dw.depthwise_conv2d(xg, wg, stride=stride, padding=padding)
+    v_fwd = _C.last_variant()
+    gx, gw = torch.autograd.grad(y, (xg, wg), gy)
+    return y.detach(), gx, gw, v_fwd
+
+
+def assert_parity(y, gx, gw, y_ref, gx_ref, gw_ref, dtype):
+    if dtype == torch.float32:
+        tol = dict(rtol=1e-5, atol=1e-5)
+        gw_rtol = 1e-4
+    else:
+        tol = dict(rtol=1e-11, atol=1e-11)
+        gw_rtol = 1e-11
+    np.testing.assert_allclose(_np(y).astype(np.float64), y_ref, **tol)
+    np.testing.assert_allclose(_np(gx).astype(np.float64), gx_ref, **tol)
+    gw_atol = gw_rtol * max(float(np.abs(gw_ref).max()), 1e-30)
+    np.testing.assert_allclose(_np(gw).astype(np.float64), gw_ref, rtol=gw_rtol, atol=gw_atol)
+
+
+def check_against_c_oracle(dw, gpu, shape, dtype=torch.float32, seed=0):
+    n, c, h, w, k, s, p = shape
+    x, wt, gy = make_inputs(shape, seed=seed, dtype=dtype)
+    y, gx, gw, variant = run_three_passes(dw, x.to(gpu), wt.to(gpu), gy.to(gpu), s, p)
+    _announce(shape_id(shape), str(dtype), variant)
+    assert y.shape == gy.shape and gx.shape == x.shape and gw.shape == wt.shape
+    y_ref = oracle.forward(_np(x), _np(wt), s, p)
+    gx_ref = oracle.grad_input(_np(gy), _np(wt), (h, w), s, p)
+    gw_ref = oracle.grad_weight(_np(x), _np(gy), wt.shape, s, p)
+    assert_parity(y, gx, gw, y_ref, gx_ref, gw_ref, dtype)
+    return variant
+
+
+# Small and awkward shapes: every kernel family, ragged edges, odd extents.
+SMALL = [
+    (2, 3, 6, 7, 3, 1, 1), (2, 3, 6, 7, 3, 2, 1), (2, 3, 9, 8, 5, 1, 2), (2, 3, 9, 8, 5, 2, 2),
+    (1, 2, 7, 7, 7, 1, 3), (3, 5, 7, 7, 5, 1, 2), (3, 5, 7, 7, 3, 1, 1), (1, 2, 12, 11, 7, 2, 3),
+    (2, 2, 11, 13, 3, 2, 0), (2, 2, 11, 13, 5, 1, 0), (1, 3, 10, 10, 4, 2, 1), (1, 3, 13, 10, 2, 3, 0),
+    (1, 2, 5, 5, 1, 1, 0), (1, 2, 9, 9, 3, 3, 1), (2, 7, 14, 14, 3, 1, 1), (2, 7, 14, 14, 5, 1, 2),
+    (2, 7, 14, 14, 5, 2, 2), (2, 7, 14, 14, 7, 1, 3), (2, 5, 28, 28, 5, 1, 2), (2, 5, 28, 28, 3, 2, 1),
+    (2, 5, 28, 28, 7, 1, 3), (3, 4, 56, 56, 3, 1, 1), (3, 4, 56, 56, 5, 2, 2), (3, 4, 56, 56, 7, 1, 3),
+    (2, 3, 112, 112, 3, 1, 1), (2, 3, 112, 112, 3, 2, 1), (1, 2, 128, 96, 5, 2, 2), (1, 2, 256, 256, 5, 1, 2),
+    (1, 1, 1, 1, 3, 1, 1), (1, 1, 3, 300, 3, 1, 1), (1, 1, 300, 3, 5, 2, 2), (1, 2, 40, 1000, 7, 2, 3),
+    (2, 3, 57, 59, 7, 2, 3), (2, 3, 58, 60, 5, 2, 1), (2, 3, 61, 64, 3, 2, 0), (1, 3, 64, 64, 7, 1, 0),
+]
+
+
+@pytest.mark.parametrize("shape", SMALL, ids=shape_id)
+def test_small_and_awkward_shapes_fp32(dw, gpu, shape):
+    check_against_c_oracle(dw, gpu, shape)
+
+
+@pytest.mark.parametrize("shape", SMALL[::3], ids=shape_id)
+def test_small_and_awkward_shapes_fp64(dw, gpu, shape):
+    check_against_c_oracle(dw, gpu, shape, dtype=torch.float64)
+
+
+@pytest.mark.parametrize("shape", SMALL[::2], ids=shape_id)
+def test_generic_kernels_fp32(dw, gpu, shape, monkeypatch):
+    monkeypatch.setenv("DWCONV_FORCE_GENERIC", "1")
+    variant = check_against_c_oracle(dw, gpu, shape)
+    assert variant.startswith("direct")
+
+
+@pytest.mark.parametrize("shape", REF_FORWARD, ids=shape_id)
+def test_reference_forward_matrix(dw, gpu, shape):
+    # test/test_forward.py:20-73, same shapes (N=32), all three passes instead of forward only
+    check_against_c_oracle(dw, gpu, shape)
+
+
+@pytest.mark.parametrize("shape", REF_GRAD, ids=shape_id)
+def test_reference_grad_matrix_fp64_values(dw, gpu, shape):
+    # test/test_grad.py:44-153 shapes in fp64; values against the oracle with a random upstream gradient
+    check_against_c_oracle(dw, gpu, shape, dtype=torch.float64)
+
+
+@pytest.mark.parametrize("shape", [(2, 2) + s[2:] for s in REF_GRAD[::3]], ids=shape_id)
+def test_reference_gradcheck_fp64(dw, gpu, shape):
+    # the reference's own probe: numerical Jacobian of depthwise_conv2d(...).sum()
+    n, c, h, w, k, s, p = shape
+    h, w = min(h, 12), min(w, 13)
+    g = torch.Generator("cpu").manual_seed(1)
+    x = torch.randn(n, c, h, w, generator=g, dtype=torch.float64).to(gpu).requires_grad_(True)
+    wt = torch.randn(c, 1, k, k, generator=g, dtype=torch.float64).to(gpu).requires_grad_(True)
+    assert torch.autograd.gradcheck(lambda a: dw.depthwise_conv2d(a, wt.detach(), stride=s, padding=p).sum(), x)
+    assert torch.autograd.gradcheck(lambda b: dw.depthwise_conv2d(x.detach(), b, stride=s, padding=p).sum(), wt)
+
+
+def test_golden_vectors(dw, gpu):
+    z = np.load(GOLDEN)
+    ncases = len([k for k in z.files if k.endswith("_geom")])
+    for dtype in (torch.float32, torch.float64):
+        for i in range(ncases):
+            n, c, h, w, kh, kw, sh, sw, ph, pw = (int(v) for v in z[f"c{i}_geom"])
+            _announce("golden", i, dtype)
+            x, wt, gy = (torch.from_numpy(z[f"c{i}_{k}"]).to(dtype).to(gpu) for k in ("x", "w", "gy"))
+            y, gx, gw, _ = run_three_passes(dw, x, wt, gy, (sh, sw), (ph, pw))
+            if dtype == torch.float64:
+                assert_parity(y, gx, gw, z[f"c{i}_y"], z[f"c{i}_gx"], z[f"c{i}_gw"], dtype)
+            else:
+                # inputs were rounded to fp32: compare against the oracle on the rounded inputs
+                xr, wr, gr = _np(x), _np(wt), _np(gy)
+                assert_parity(y, gx, gw, oracle.forward(xr, wr, (sh, sw), (ph, pw)),
+                              oracle.grad_input(gr, wr, (h, w), (sh, sw), (ph, pw)),
+                              oracle.grad_weight(xr, gr, wt.shape, (sh, sw), (ph, pw)), dtype)
+
+
+# ---- benchmark configurations at full size ---------------------------------------------
+def check_full_size(dw, gpu, shape, seed=0, n_planes=6, n_channels=3):
+    """Full-size run; values checked on sampled planes/channels (planes are independent),
+    plus the adjoint identities over the whole tensors."""
+    n, c, h, w, k, s, p = shape
+    x, wt, gy = make_inputs(shape, seed=seed)
+    xg, wg, gg = x.to(gpu), wt.to(gpu), gy.to(gpu)
+    y, gx, gw, variant = run_three_passes(dw, xg, wg, gg, s, p)
+    _announce(shape_id(shape), variant)
+    rng = np.random.default_rng(seed + 1)
+    yc, gxc = y.cpu(), gx.cpu()
+    for _ in range(n_planes):
+        b, ch = int(rng.integers(n)), int(rng.integers(c))
+        xs, ws, gs = _np(x[b:b + 1, ch:ch + 1]), _np(wt[ch:ch + 1]), _np(gy[b:b + 1, ch:ch + 1])
+        np.testing.assert_allclose(_np(yc[b, ch]).astype(np.float64), oracle.forward(xs, ws, s, p)[0, 0], rtol=1e-5, atol=1e-5)
+        np.testing.assert_allclose(_np(gxc[b, ch]).astype(np.float64), oracle.grad_input(gs, ws, (h, w), s, p)[0, 0], rtol=1e-5, atol=1e-5)
+    chans = sorted(set(int(v) for v in rng.integers(c, size=n_channels)) | {0, c - 1})
+    gw_ref = oracle.grad_weight(_np(x[:, chans]), _np(gy[:, chans]), (len(chans), 1, k, k), s, p)
+    atol = 1e-4 * float(np.abs(gw_ref).max())
+    np.testing.assert_allclose(_np(gw[chans]).astype(np.float64), gw_ref, rtol=1e-4, atol=atol)
+    # size-independent property: <y, gy> == <x, gx> == <w, gw>, accumulated in fp64 on the device
+    lhs = (y.double() * gg.double()).sum().item()
+    mid = (xg.double() * gx.double()).sum().item()
+    rhs = (wg.double() * gw.double()).sum().item()
+    scale = (y.double().abs() * gg.double().abs()).sum().item()
+    assert abs(lhs - mid) <= 1e-6 * scale and abs(lhs - rhs) <= 1e-6 * scale
+    # bit-identical grad-weight on a second run
+    _, _, gw2, _ = run_three_passes(dw, xg, wg, gg, s, p)
+    assert torch.equal(gw, gw2)
+
+
+def test_cfg1_whole_tensor(dw, gpu):
+    check_against_c_oracle(dw, gpu, CFG1)
+
+
+def test_cfg2_large_map(dw, gpu):
+    check_full_size(dw, gpu, CFG2)
+
+
+@pytest.mark.parametrize("shape", effnet_layers(), ids=shape_id)
+def test_efficientnet_b0_layers_full_batch(dw, gpu, shape):
+    check_full_size(dw, gpu, shape)
+
+
+@pytest.mark.parametrize("shape", CFG4 + CONVNEXT_T, ids=shape_id)
+def test_large_kernel_small_map_layers(dw, gpu, shape):
+    check_full_size(dw, gpu, shape)
+
+
+def test_stress_grad_weight_determinism(dw, gpu):
+    n, c, h, w, k, s, p = STRESS
+    check_full_size(dw, gpu, STRESS, n_planes=3, n_channels=2)
+    from torch_dwconv import _C
+
+    x, wt, gy = make_inputs(STRESS, seed=4)
+    xg, gg, wg = x.to(gpu), gy.to(gpu), wt.to(gpu)
+    runs = [_C.dwconv2d_backward_kernel(xg, gg, wg, 1, 1, s, s, p, p) for _ in range(5)]
+    torch.cuda.synchronize()
+    for r in runs[1:]:
+        assert torch.equal(runs[0], r)
+
+
+# ---- closed forms on the device ----------------------------------------------------------
+def test_delta_filter_is_identity_bitwise(dw, gpu):
+    x = torch.randn(3, 5, 56, 56, device=gpu)
+    for k in (3, 5, 7):
+        w = torch.zeros(5, 1, k, k, device=gpu)
+        w[:, 0, k // 2, k // 2] = 1.0
+        assert torch.equal(dw.depthwise_conv2d(x, w, padding=k // 2), x)
+
+
+def test_linearity_on_device(dw, gpu):
+    x1, x2 = torch.randn(2, 4, 30, 33, device=gpu), torch.randn(2, 4, 30, 33, device=gpu)
+    w = torch.randn(4, 1, 5, 5, device=gpu) / 5
+    a = dw.depthwise_conv2d(x1 + x2, w, stride=2, padding=2)
+    b = dw.depthwise_conv2d(x1, w, stride=2, padding=2) + dw.depthwise_conv2d(x2, w, stride=2, padding=2)
+    torch.testing.assert_close(a, b, rtol=1e-5, atol=1e-5)
+
+
+# ---- boundary behaviour ---------------------------------------------------------------------
+def test_empty_and_degenerate_inputs(dw, gpu):
+    w = torch.randn(4, 1, 3, 3, device=gpu)
+    y = dw.depthwise_conv2d(torch.empty(0, 4, 8, 8, device=gpu), w, padding=1)
+    assert y.shape == (0, 4, 8, 8)
+    # plane smaller than the filter and no padding: empty output
+    x = torch.randn(1, 4, 2, 2, device=gpu, requires_grad=True)
+    wp = w.clone().requires_grad_(True)
+    y = dw.depthwise_conv2d(x, wp)
+    assert y.shape == (1, 4, 0, 0)
+    gx, gw = torch.autograd.grad(y, (x, wp), torch.empty_like(y))
+    assert torch.count_nonzero(gx) == 0 and torch.count_nonzero(gw) == 0
+
+
+def test_unaligned_and_noncontiguous_inputs(dw, gpu):
+    shape = (2, 3, 20, 24, 3, 1, 1)
+    x, wt, gy = make_inputs(shape, seed=8)
+    y_ref = oracle.forward(_np(x), _np(wt), 1, 1)
+    # contiguous but only 4-byte aligned: a view one element into a flat buffer
+    flat = torch.empty(x.numel() + 1, device=gpu)
+    flat[1:] = x.to(gpu).flatten()
+    xv = flat[1:].view_as(x)
+    assert xv.data_ptr() % 16 != 0 and xv.is_contiguous()
+    np.testing.assert_allclose(_np(dw.depthwise_conv2d(xv, wt.to(gpu), padding=1)), y_ref, rtol=1e-5, atol=1e-5)
+    # non-contiguous (channels-last memory): made contiguous by the binding, like the reference (:855-856)
+    xc = x.to(gpu).contiguous(memory_format=torch.channels_last)
+    np.testing.assert_allclose(_np(dw.depthwise_conv2d(xc, wt.to(gpu), padding=1)), y_ref, rtol=1e-5, atol=1e-5)
+
+
+def test_rectangular_filter_stride_and_padding(dw, gpu):
+    g = torch.Generator("cpu").manual_seed(11)
+    x = torch.randn(2, 3, 12, 10, generator=g)
+    wt = torch.randn(3, 1, 5, 2, generator=g)
+    s, p = (2, 1), (1, 0)
+    oh, ow = (12 + 2 - 5) // 2 + 1, (10 - 2) // 1 + 1
+    gy = torch.randn(2, 3, oh, ow, generator=g)
+    y, gx, gw, _ = run_three_passes(dw, x.to(gpu), wt.to(gpu), gy.to(gpu), s, p)
+    assert_parity(y, gx, gw, oracle.forward(_np(x), _np(wt), s, p), oracle.grad_input(_np(gy), _np(wt), (12, 10), s, p),
+                  oracle.grad_weight(_np(x), _np(gy), wt.shape, s, p), torch.float32)
+
+
+def test_c_entry_points_directly(dw, gpu):
+    """The generic operator with asymmetric pads / up and down together, and the small entry point."""
+    from torch_dwconv import _C
+
+    g = torch.Generator("cpu").manual_seed(5)
+    x = torch.randn(2, 3, 9, 11, generator=g)
+    for (kh, kw, up, down, pads, fwd) in [(3, 3, 2, 1, (1, 2, 0, 3), False), (5, 5, 2, 2, (2, 1, 3, 0), True),
+                                           (4, 3, 3, 2, (0, 0, 1, 1), False), (3, 3, 1, 1, (2, 0, 0, 2), True)]:
+        wt = torch.randn(3, 1, kh, kw, generator=g)
+        got = _C.dwconv2d(x.to(gpu), wt.to(gpu), up, up, down, down, *pads, fwd)
+        ref = oracle.dwconv2d(_np(x), _np(wt), up, up, down, down, *pads, fwd)
+        np.testing.assert_allclose(_np(got), ref, rtol=1e-5, atol=1e-5)
+    for (kh, kw, ph, pw, fwd) in [(3, 3, 1, 1, True), (5, 5, 2, 2, False), (5, 3, 0, 2, True), (7, 7, 3, 3, False)]:
+        wt = torch.randn(3, 1, kh, kw, generator=g)
+        got = _C.dwconv2d_small(x.to(gpu), wt.to(gpu), 1, 1, 1, 1, ph, pw, fwd)
+        ref = oracle.dwconv2d_small(_np(x), _np(wt), ph, pw, fwd)
+        np.testing.assert_allclose(_np(got), ref, rtol=1e-5, atol=1e-5)
+    with pytest.raises(RuntimeError, match="stride-1"):
+        _C.dwconv2d_small(x.to(gpu), torch.randn(3, 1, 3, 3, device=gpu), 1, 1, 2, 2, 1, 1, True)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        _C.dwconv2d(x, torch.randn(3, 1, 3, 3, device=gpu), 1, 1, 1, 1, 1, 1, 1, 1, True)
+
+
+def test_module_matches_plain_conv(dw, gpu):
+    m = dw.DepthwiseConv2d(16, 16, 3, stride=1, padding=1).to(gpu)
+    x = torch.randn(4, 16, 40, 40, device=gpu, requires_grad=True)
+    y = m(x)
+    y.square().mean().backward()
+    gx, gw = x.grad.clone(), m.weight.grad.clone()
+    x.grad = None
+    m.weight.grad = None
+    m.custom = False
+    y2 = m(x)
+    y2.square().mean().backward()
+    torch.testing.assert_close(y, y2, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(gx, x.grad, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(gw, m.weight.grad, rtol=1e-4, atol=1e-5)
+
+
+def test_runs_on_the_current_stream(dw, gpu):
+    x = torch.randn(4, 8, 64, 64, device=gpu)
+    w = torch.randn(8, 1, 3, 3, device=gpu)
+    ref = dw.depthwise_conv2d(x, w, padding=1)
+    side = torch.cuda.Stream(device=gpu)
+    side.wait_stream(torch.cuda.current_stream(gpu))
+    with torch.cuda.stream(side):
+        out = dw.depthwise_conv2d(x, w, padding=1)
+    side.synchronize()
+    assert torch.equal(out, ref)
