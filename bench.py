@@ -1,0 +1,275 @@
+#!/usr/bin/env python3
+"""Benchmark of the depthwise conv2d hot path on one MI355X.
+
+Workload (BASELINE.json, configs[2]): the 12 depthwise layers of EfficientNet-B0,
+fp32 NCHW, batch 128, padding k//2.  One "step" = forward of layers 1..12, then
+grad-input and grad-weight of layers 12..1 (training order): 36 calls into the
+C ABI of libdwconv_hip, all tensors resident in HBM before the clock starts.
+
+Prints one JSON line.  `value` is achieved HBM GB/s = algorithmic bytes of the
+step (every tensor of every pass touched exactly once: 12(|x|+|y|+|w|) bytes per
+layer) / step time; `ms_per_step` carries the fwd+bwd time itself.
+"""
+import argparse
+import ctypes
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "depthwise-conv-pytorch_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+
+# (C, H_in, k, stride), batch 128, padding k//2
+EFFNET_B0 = [
+    (32, 112, 3, 1), (96, 112, 3, 2), (144, 56, 3, 1), (144, 56, 5, 2),
+    (240, 28, 5, 1), (240, 28, 3, 2), (480, 14, 3, 1), (480, 14, 5, 1),
+    (672, 14, 5, 1), (672, 14, 5, 2), (1152, 7, 5, 1), (1152, 7, 3, 1),
+]
+WORKLOADS = {
+    "effnet_b0": lambda batch: [(batch, c, h, h, k, s, k // 2) for (c, h, k, s) in EFFNET_B0],
+    "cfg1": lambda batch: [(8, 32, 56, 56, 3, 1, 1)],
+    "cfg2": lambda batch: [(16, 64, 256, 256, 5, 1, 2)],
+    "cfg4": lambda batch: [(256, 1024, 7, 7, 7, 1, 3), (128, 512, 14, 14, 7, 1, 3)],
+    "convnext_t": lambda batch: [(64, 96, 56, 56, 7, 1, 3), (64, 192, 28, 28, 7, 1, 3),
+                                 (64, 384, 14, 14, 7, 1, 3), (64, 768, 7, 7, 7, 1, 3)],
+    "stress": lambda batch: [(64, 256, 128, 96, 5, 2, 2)],
+}
+
+
+class Layer:
+    """Device tensors and the three C-ABI calls of one depthwise layer."""
+
+    def __init__(self, shape, lib, torch, dev, gen):
+        n, c, h, w, k, s, p = shape
+        self.shape = shape
+        self.lib = lib
+        oh, ow = (h + 2 * p - k) // s + 1, (w + 2 * p - k) // s + 1
+        self.geom = (n, c, h, w, oh, ow, k, s, p)
+        self.x = torch.randn(n, c, h, w, generator=gen).to(dev)
+        self.w = (torch.randn(c, 1, k, k, generator=gen) / k).to(dev)
+        self.gy = torch.randn(n, c, oh, ow, generator=gen).to(dev)
+        self.y = torch.empty(n, c, oh, ow, device=dev)
+        self.gx = torch.empty_like(self.x)
+        self.gw = torch.empty_like(self.w)
+        self.ws_bytes = lib.dwconv2d_backward_kernel_workspace_bytes(n, c, h, w, oh, ow, k, k, s, s, p, p, 4)
+        self.ws = torch.empty(max(self.ws_bytes, 16), dtype=torch.uint8, device=dev)
+        nx, ny, nw = n * c * h * w, n * c * oh * ow, c * k * k
+        self.bytes = {"fwd": 4 * (nx + ny + nw), "gx": 4 * (ny + nx + nw), "gw": 4 * (nx + ny + nw)}
+        self.flops = 2 * ny * k * k
+        # transposed-problem padding, torch_dwconv/dwconv.py:39-44
+        self.g_pad = (k - p - 1, h - oh * s + p, k - p - 1, w - ow * s + p)
+        self.name = f"C{c}_{h}x{w}_k{k}s{s}"
+
+    def _check(self, rc):
+        if rc != 0:
+            raise RuntimeError(self.lib.dwconv_last_error().decode())
+
+    def fwd(self, stream):
+        n, c, h, w, oh, ow, k, s, p = self.geom
+        self._check(self.lib.dwconv2d_f32(self.x.data_ptr(), self.w.data_ptr(), self.y.data_ptr(), n, c, h, w, k, k,
+                                          1, 1, s, s, p, p, p, p, 1, stream))
+
+    def bwd_input(self, stream):
+        n, c, h, w, oh, ow, k, s, p = self.geom
+        g = self.g_pad
+        self._check(self.lib.dwconv2d_f32(self.gy.data_ptr(), self.w.data_ptr(), self.gx.data_ptr(), n, c, oh, ow, k, k,
+                                          s, s, 1, 1, g[0], g[1], g[2], g[3], 0, stream))
+
+    def bwd_filter(self, stream):
+        n, c, h, w, oh, ow, k, s, p = self.geom
+        self._check(self.lib.dwconv2d_backward_kernel_f32(
+            self.x.data_ptr(), self.gy.data_ptr(), self.gw.data_ptr(), self.ws.data_ptr(), self.ws_bytes,
+            n, c, h, w, oh, ow, k, k, 1, 1, s, s, p, p, stream))
+
+
+def schedule(layers):
+    """Training order: all forwards, then the backward passes last layer first."""
+    calls = [(l, "fwd", l.fwd) for l in layers]
+    for l in reversed(layers):
+        calls.append((l, "gx", l.bwd_input))
+        calls.append((l, "gw", l.bwd_filter))
+    return calls
+
+
+def cpu_baseline(layers_shapes, torch, budget_s=20.0):
+    """fp32 F.conv2d(groups=C) forward + both gradients on the host cores, on a batch
+    slice of every layer of the workload; scaled to the full batch."""
+    from oracle import torch_cpu_fp32_step
+
+    cores = os.cpu_count() or 1
+    threads = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    full_batch = layers_shapes[0][0]
+    sample_batch = max(1, min(full_batch, 8))
+    g = torch.Generator("cpu").manual_seed(0)
+    t_total, bytes_total = 0.0, 0
+    t_start = time.perf_counter()
+    done = 0
+    for (n, c, h, w, k, s, p) in layers_shapes:
+        nb = max(1, min(n, sample_batch))
+        oh, ow = (h + 2 * p - k) // s + 1, (w + 2 * p - k) // s + 1
+        x = torch.randn(nb, c, h, w, generator=g)
+        wt = torch.randn(c, 1, k, k, generator=g) / k
+        gy = torch.randn(nb, c, oh, ow, generator=g)
+        t, threads = torch_cpu_fp32_step(x, wt, gy, s, p, iters=3, threads=threads)
+        t_total += t * (n / nb)
+        bytes_total += 12 * (n * c * h * w + n * c * oh * ow + c * k * k)
+        done += 1
+        if time.perf_counter() - t_start > budget_s:
+            break
+    sample = (f"torch {torch.__version__} F.conv2d(groups=C) fp32 fwd + autograd.grad(x,w), median of 3, "
+              f"batch slice {sample_batch} of {full_batch} on {done} of {len(layers_shapes)} layers, time scaled to the full batch")
+    return {"value": round(bytes_total / t_total / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": sample, "ms_per_step_scaled": round(t_total * 1e3, 1)}
+
+
+def miopen_native(layers, torch, iters=3):
+    """The same layers through F.conv2d(groups=C) on the GPU (MIOpen's depthwise)."""
+    import torch.nn.functional as F
+
+    per_layer = []
+    for l in layers:
+        n, c, h, w, oh, ow, k, s, p = l.geom
+        x = l.x.detach().requires_grad_(True)
+        wt = l.w.detach().requires_grad_(True)
+        ts = []
+        for i in range(iters + 2):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            y = F.conv2d(x, wt, stride=s, padding=p, groups=c)
+            torch.autograd.grad(y, (x, wt), l.gy)
+            e1.record()
+            torch.cuda.synchronize()
+            if i >= 2:
+                ts.append(e0.elapsed_time(e1))
+        per_layer.append(statistics.median(ts))
+    return per_layer
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="effnet_b0", choices=sorted(WORKLOADS))
+    ap.add_argument("--batch", type=int, default=128)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-miopen", action="store_true")
+    ap.add_argument("--table", action="store_true", help="print a per-layer, per-pass table to stderr")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: depthwise conv2d is a single-GPU kernel path; run with --gpus 1")
+
+    import torch
+    from torch_dwconv import _C
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU (no HIP device visible)")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib = _C._lib
+    shapes = WORKLOADS[args.workload](args.batch)
+    gen = torch.Generator("cpu").manual_seed(0)
+    layers = [Layer(s, lib, torch, dev, gen) for s in shapes]
+    calls = schedule(layers)
+    stream_obj = torch.cuda.current_stream(dev)
+    stream = ctypes.c_void_p(stream_obj.cuda_stream)
+    step_bytes = sum(sum(l.bytes.values()) for l in layers)
+
+    def step():
+        for _, _, fn in calls:
+            fn(stream)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(stream_obj)
+    for _ in range(args.steps):
+        step()
+    e1.record(stream_obj)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+
+    # Per-launch durations, same order and cache state, events on the launch stream.
+    variants, durs = [], [[] for _ in calls]
+    for it in range(max(3, min(args.steps, 20))):
+        evs = []
+        for i, (l, kind, fn) in enumerate(calls):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(stream_obj)
+            fn(stream)
+            b.record(stream_obj)
+            if it == 0:
+                variants.append(lib.dwconv_last_variant().decode())
+            evs.append((a, b))
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(evs):
+            durs[i].append(a.elapsed_time(b))
+    rows = []
+    for i, (l, kind, fn) in enumerate(calls):
+        ms = statistics.mean(durs[i])
+        rows.append({"layer": l.name, "pass": kind, "variant": variants[i], "us": round(ms * 1e3, 1),
+                     "GBs": round(l.bytes[kind] / ms / 1e6, 1), "bytes": l.bytes[kind]})
+    # dominant kernel = the kernel function (template instance) with the largest share of the step
+    by_kernel = {}
+    for r in rows:
+        key = r["variant"].split(">")[0] + (">" if ">" in r["variant"] else "")
+        agg = by_kernel.setdefault(key, {"ms": 0.0, "bytes": 0, "launches": 0})
+        agg["ms"] += r["us"] / 1e3
+        agg["bytes"] += r["bytes"]
+        agg["launches"] += 1
+    dom_name, dom = max(by_kernel.items(), key=lambda kv: kv[1]["ms"])
+    achieved = dom["bytes"] / dom["ms"] / 1e6
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": dom_name,
+                "launches_per_step": dom["launches"], "avg_launch_us": round(dom["ms"] * 1e3 / dom["launches"], 1),
+                "bytes_per_launch": dom["bytes"] // dom["launches"]}
+
+    result = {
+        "metric": "fwd+bwd achieved HBM GB/s, EfficientNet-B0 dw stack, 1 GPU" if args.workload == "effnet_b0"
+        else f"fwd+bwd achieved HBM GB/s, {args.workload}, 1 GPU",
+        "value": round(step_bytes / ms_per_step / 1e6, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {len(layers)} depthwise layers, fp32 NCHW, batch {shapes[0][0]}, "
+                               "fwd + grad-input + grad-weight per layer, training order",
+                   "layers": [l.name for l in layers], "algorithmic_bytes_per_step": step_bytes},
+        "frac_of_hbm_roofline": round(step_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, 4),
+        "host_wall_ms_per_step": round(wall_ms, 4),
+        "sum_of_launch_us": round(sum(r["us"] for r in rows), 1),
+        "roofline": roofline,
+    }
+    if args.table:
+        for r in rows:
+            print(f"{r['layer']:>18} {r['pass']:>3} {r['us']:9.1f} us {r['GBs']:8.1f} GB/s  {r['variant']}", file=sys.stderr)
+    result["per_pass_us"] = {k: round(sum(r["us"] for r in rows if r["pass"] == k), 1) for k in ("fwd", "gx", "gw")}
+    if not args.no_miopen:
+        try:
+            per_layer = miopen_native(layers, torch)
+            result["miopen_native_ms_per_step"] = round(sum(per_layer), 3)
+            result["speedup_vs_miopen_native"] = round(sum(per_layer) / ms_per_step, 2)
+        except Exception as e:  # the comparison is informative only
+            result["miopen_native_ms_per_step"] = f"failed: {type(e).__name__}"
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(shapes, torch)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
