@@ -21,62 +21,32 @@
 //                    stride-2 layers, computed as four interleaved stride-1
 //                    correlations (one per output parity) without ever
 //                    forming the zero-stuffed intermediate.
-#include "dwconv_common.hpp"
-
-#include <cstdlib>
+#include "dwconv_tile_common.hpp"
 
 namespace dwconv {
 
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kSlack = 4;            // spare floats on both sides of every LDS row
-constexpr int kLdsBudget = 48 * 1024;  // bytes of LDS one tile may take
-constexpr int kXcds = 8;
-
 struct TilePlan {
+    StageLayout st;
     const float *in;
     const float *taps;
     float *out;
     long planes;
     int channel;
-    int in_h, in_w, out_h, out_w;
-    int in_plane, out_plane;   // elements per plane
-    int row_shift, col_shift;  // LDS row r / column c hold input row iy0 + r / column c - col_shift
+    int out_h, out_w, out_plane;
+    int row_shift;             // LDS row r of a tile holds input row (first row of the tile) - row_shift + r
     int rows_per_tile;         // output rows (down) or half-resolution rows (up) per tile
     int row_tiles;             // tiles per plane
     int planes_per_tile;
     int n_tiles;
-    int lds_rows;              // rows of one plane image
-    unsigned lds_rows_magic;
-    int g_lo;                  // first (possibly negative) float4 column fetched per row
-    int spr;                   // float4 slots per row
-    unsigned spr_magic;
-    int pitch;                 // floats per LDS row, slack included
-    int plane_pitch;           // floats per plane image
     int ncb;                   // column blocks per row band
     unsigned ncb_magic;
     int items_per_plane;
     unsigned ipp_magic;
     int tap_base;              // float offset of the tap table in LDS
-    int vec_in, vec_out;       // 128-bit global accesses are legal
+    int vec_out;               // 128-bit global stores are legal
 };
-
-// n / d through the reciprocal made by magic_u16(d); a zero reciprocal stands for d == 1.
-__device__ __forceinline__ int fast_div(int n, unsigned magic)
-{
-    return magic ? static_cast<int>(__umulhi(static_cast<unsigned>(n), magic)) : n;
-}
-
-// Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
-// Give every XCD a contiguous run of tiles so that the row bands of one plane,
-// which share halo rows, meet in the same L2.
-__device__ __forceinline__ int xcd_contiguous_tile(int bid, int n_tiles)
-{
-    const int per = n_tiles / kXcds, rem = n_tiles - per * kXcds;
-    const int xcd = bid % kXcds, k = bid / kXcds;
-    return xcd * per + min(xcd, rem) + k;
-}
 
 // Copies the tap tables of the tile's planes into LDS, rotated by 180 degrees if FLIP.
 template <int KK, bool FLIP>
@@ -86,37 +56,6 @@ __device__ __forceinline__ void stage_taps(const TilePlan &p, float *lds, long p
         const int pl = i / KK, t = i - pl * KK;
         const int c = static_cast<int>((plane0 + pl) % p.channel);
         lds[p.tap_base + i] = p.taps[c * KK + (FLIP ? KK - 1 - t : t)];
-    }
-}
-
-// Fills the LDS image of the tile: every float4 slot of every row is written,
-// with zeros where the row or the columns fall outside the plane.
-__device__ __forceinline__ void stage_tile(const TilePlan &p, float *lds, long plane0, int nplanes, int iy0)
-{
-    const int total = nplanes * p.lds_rows * p.spr;
-    for (int slot = threadIdx.x; slot < total; slot += kThreads) {
-        const int rowidx = fast_div(slot, p.spr_magic);
-        const int sc = slot - rowidx * p.spr;
-        const int pl = fast_div(rowidx, p.lds_rows_magic);
-        const int r = rowidx - pl * p.lds_rows;
-        const int ix = 4 * (p.g_lo + sc);
-        const int iy = iy0 + r;
-        const bool row_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
-        const float *src = p.in + (plane0 + pl) * p.in_plane + static_cast<long>(iy) * p.in_w + ix;
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (p.vec_in) {
-            if (row_ok && ix >= 0 && ix < p.in_w) v = *reinterpret_cast<const float4 *>(src);
-        } else if (row_ok) {
-            if (static_cast<unsigned>(ix + 0) < static_cast<unsigned>(p.in_w)) v.x = src[0];
-            if (static_cast<unsigned>(ix + 1) < static_cast<unsigned>(p.in_w)) v.y = src[1];
-            if (static_cast<unsigned>(ix + 2) < static_cast<unsigned>(p.in_w)) v.z = src[2];
-            if (static_cast<unsigned>(ix + 3) < static_cast<unsigned>(p.in_w)) v.w = src[3];
-        }
-        float *dst = lds + pl * p.plane_pitch + r * p.pitch + kSlack + ix + p.col_shift;
-        dst[0] = v.x;
-        dst[1] = v.y;
-        dst[2] = v.z;
-        dst[3] = v.w;
     }
 }
 
@@ -137,7 +76,7 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
     const int oy0 = rt * p.rows_per_tile;
 
     stage_taps<KK, FLIP>(p, lds, plane0, nplanes);
-    stage_tile(p, lds, plane0, nplanes, oy0 * S - p.row_shift);
+    stage_tile(p.st, p.in, lds, plane0, nplanes, oy0 * S - p.row_shift);
     __syncthreads();
 
     const int n_items = nplanes * p.items_per_plane;
@@ -151,7 +90,7 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
 #pragma unroll
         for (int t = 0; t < KK; ++t) tapv[t] = lds[p.tap_base + pl * KK + t];
 
-        const float *base = lds + pl * p.plane_pitch + (rb * BH * S) * p.pitch + kSlack + 4 * cb * S;
+        const float *base = lds + pl * p.st.plane_pitch + (rb * BH * S) * p.st.pitch + kSlack + 4 * cb * S;
         float acc[BH][4];
 #pragma unroll
         for (int b = 0; b < BH; ++b)
@@ -163,7 +102,7 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
             float win[4 * NV];
 #pragma unroll
             for (int v = 0; v < NV; ++v) {
-                const float4 q = *reinterpret_cast<const float4 *>(base + wr * p.pitch + 4 * v);
+                const float4 q = *reinterpret_cast<const float4 *>(base + wr * p.st.pitch + 4 * v);
                 win[4 * v + 0] = q.x;
                 win[4 * v + 1] = q.y;
                 win[4 * v + 2] = q.z;
@@ -220,7 +159,7 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
     const int qy0 = rt * p.rows_per_tile;
 
     stage_taps<KK, true>(p, lds, plane0, nplanes);
-    stage_tile(p, lds, plane0, nplanes, qy0 - p.row_shift);
+    stage_tile(p.st, p.in, lds, plane0, nplanes, qy0 - p.row_shift);
     __syncthreads();
 
     const int n_items = nplanes * p.items_per_plane;
@@ -234,7 +173,7 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
 #pragma unroll
         for (int t = 0; t < KK; ++t) tapv[t] = lds[p.tap_base + pl * KK + t];
 
-        const float *base = lds + pl * p.plane_pitch + (rb * BQ) * p.pitch + kSlack + 4 * cb;
+        const float *base = lds + pl * p.st.plane_pitch + (rb * BQ) * p.st.pitch + kSlack + 4 * cb;
         float acc[2 * BQ][8];
 #pragma unroll
         for (int b = 0; b < 2 * BQ; ++b)
@@ -245,8 +184,8 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
         for (int wr = 0; wr < WIN_ROWS; ++wr) {
             float win[8];
             {
-                const float4 q0 = *reinterpret_cast<const float4 *>(base + wr * p.pitch);
-                const float4 q1 = *reinterpret_cast<const float4 *>(base + wr * p.pitch + 4);
+                const float4 q0 = *reinterpret_cast<const float4 *>(base + wr * p.st.pitch);
+                const float4 q1 = *reinterpret_cast<const float4 *>(base + wr * p.st.pitch + 4);
                 win[0] = q0.x; win[1] = q0.y; win[2] = q0.z; win[3] = q0.w;
                 win[4] = q1.x; win[5] = q1.y; win[6] = q1.z; win[7] = q1.w;
             }
@@ -293,20 +232,6 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
     }
 }
 
-int floor_div(int a, int b)
-{
-    int q = a / b;
-    if ((a % b != 0) && ((a < 0) != (b < 0))) --q;
-    return q;
-}
-
-int env_int(const char *name, int dflt)
-{
-    const char *e = std::getenv(name);
-    if (e == nullptr || e[0] == '\0') return dflt;
-    return std::atoi(e);
-}
-
 // Fills in the tiling of `p` for a plane whose output is split into `row_units`
 // units of rows (BH output rows or BQ half-resolution rows each) and `ncb` column
 // blocks.  `rows_for(units)` gives the LDS rows a band of that many units needs.
@@ -315,12 +240,10 @@ template <typename RowsFor>
 bool plan_tiles(TilePlan &p, int row_units, int unit_rows, int used_cols, int taps_per_plane, RowsFor rows_for)
 {
     const int target_items = env_int("DWCONV_TILE_ITEMS", 2 * kThreads);
-    p.pitch = kSlack + round_up(used_cols, 4) + kSlack;
-    p.g_lo = floor_div(-p.col_shift, 4);
-    p.spr = ceil_div(used_cols - p.col_shift, 4) - p.g_lo;
+    layout_columns(p.st, used_cols);
 
     auto bytes = [&](int units, int planes) {
-        return static_cast<long>(planes) * (static_cast<long>(rows_for(units)) * p.pitch + taps_per_plane) * 4;
+        return static_cast<long>(planes) * (static_cast<long>(rows_for(units)) * p.st.pitch + taps_per_plane) * 4;
     };
 
     const int ipp_full = row_units * p.ncb;
@@ -349,18 +272,15 @@ bool plan_tiles(TilePlan &p, int row_units, int unit_rows, int used_cols, int ta
     p.planes_per_tile = planes_per_tile;
     p.rows_per_tile = units_per_tile * unit_rows;
     p.row_tiles = ceil_div(row_units, units_per_tile);
-    p.lds_rows = rows_for(units_per_tile);
-    p.plane_pitch = p.lds_rows * p.pitch;
+    if (!layout_rows(p.st, rows_for(units_per_tile), planes_per_tile)) return false;
     p.items_per_plane = units_per_tile * p.ncb;
-    p.tap_base = planes_per_tile * p.plane_pitch;
+    p.tap_base = planes_per_tile * p.st.plane_pitch;
     const long groups = (p.planes + planes_per_tile - 1) / planes_per_tile;
     const long tiles = groups * p.row_tiles;
     if (tiles > 0x7fffffffL) return false;
     p.n_tiles = static_cast<int>(tiles);
     // the in-kernel divisions use a 16-bit reciprocal
-    if (planes_per_tile * p.lds_rows * p.spr >= 65536 || planes_per_tile * p.items_per_plane >= 65536) return false;
-    p.lds_rows_magic = magic_u16(p.lds_rows);
-    p.spr_magic = magic_u16(p.spr);
+    if (planes_per_tile * p.items_per_plane >= 65536) return false;
     p.ncb_magic = magic_u16(p.ncb);
     p.ipp_magic = magic_u16(p.items_per_plane);
     return true;
@@ -368,7 +288,7 @@ bool plan_tiles(TilePlan &p, int row_units, int unit_rows, int used_cols, int ta
 
 size_t lds_bytes(const TilePlan &p, int taps_per_plane)
 {
-    return static_cast<size_t>(p.planes_per_tile) * (p.plane_pitch + taps_per_plane) * 4;
+    return static_cast<size_t>(p.planes_per_tile) * (p.st.plane_pitch + taps_per_plane) * 4;
 }
 
 template <int K, int S, bool FLIP, int BH>
@@ -382,7 +302,7 @@ int launch_down(TilePlan &p, hipStream_t stream)
     hipLaunchKernelGGL((fir_down_kernel<K, S, FLIP, BH>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K),
                        stream, p);
     note_variant("tile_down<k%d,s%d,%s,bh%d> P%d rows%d vin%d vout%d", K, S, FLIP ? "rot" : "fwd", BH,
-                 p.planes_per_tile, p.rows_per_tile, p.vec_in, p.vec_out);
+                 p.planes_per_tile, p.rows_per_tile, p.st.vec_in, p.vec_out);
     return check_launch("fir_down_kernel");
 }
 
@@ -406,7 +326,7 @@ int launch_up2(TilePlan &p, hipStream_t stream)
     hipLaunchKernelGGL((fir_up2_kernel<K, EY, EX, BQ>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K), stream,
                        p);
     note_variant("tile_up2<k%d,e%d%d,bq%d> P%d rows%d vin%d vout%d", K, EY, EX, BQ, p.planes_per_tile,
-                 p.rows_per_tile, p.vec_in, p.vec_out);
+                 p.rows_per_tile, p.st.vec_in, p.vec_out);
     return check_launch("fir_up2_kernel");
 }
 
@@ -437,18 +357,18 @@ int try_launch_fir_tiled(const float *in, const float *taps, float *out, const G
     p.out = out;
     p.planes = g.planes();
     p.channel = g.channel;
-    p.in_h = g.in_h;
-    p.in_w = g.in_w;
+    p.st.in_h = g.in_h;
+    p.st.in_w = g.in_w;
     p.out_h = g.out_h;
     p.out_w = g.out_w;
-    p.in_plane = g.in_h * g.in_w;
+    p.st.in_plane = g.in_h * g.in_w;
     p.out_plane = g.out_h * g.out_w;
-    p.vec_in = (g.in_w % 4 == 0) && aligned16(in);
+    p.st.vec_in = (g.in_w % 4 == 0) && aligned16(in);
     p.vec_out = (g.out_w % 4 == 0) && aligned16(out);
 
     if (g.up_h == 1 && g.up_w == 1 && g.down_h == g.down_w && (g.down_h == 1 || g.down_h == 2)) {
         p.row_shift = g.pad_h0;
-        p.col_shift = g.pad_w0;
+        p.st.col_shift = g.pad_w0;
         const bool rot = !g.forward;
         if (g.down_h == 1) {
             if (K == 3) return rot ? launch_down_bh<3, 1, true>(p, stream) : launch_down_bh<3, 1, false>(p, stream);
@@ -463,7 +383,7 @@ int try_launch_fir_tiled(const float *in, const float *taps, float *out, const G
     if (g.up_h == 2 && g.up_w == 2 && g.down_h == 1 && g.down_w == 1 && !g.forward) {
         const int ey = g.pad_h0 & 1, ex = g.pad_w0 & 1;
         p.row_shift = (g.pad_h0 + ey) / 2;
-        p.col_shift = (g.pad_w0 + ex) / 2;
+        p.st.col_shift = (g.pad_w0 + ex) / 2;
         if (K == 3) return launch_up2_parity<3>(p, ey, ex, stream);
         if (K == 5) return launch_up2_parity<5>(p, ey, ex, stream);
         return launch_up2_parity<7>(p, ey, ex, stream);

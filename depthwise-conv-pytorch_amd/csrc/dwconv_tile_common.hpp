@@ -1,0 +1,114 @@
+// Device and host helpers shared by the LDS-tiled kernels (forward/grad-input
+// and grad-weight): the LDS image of a band of input rows and how it is filled.
+#pragma once
+
+#include "dwconv_common.hpp"
+
+#include <cstdlib>
+
+namespace dwconv {
+
+constexpr int kThreads = 256;           // lanes per workgroup (4 wavefronts)
+constexpr int kSlack = 4;               // spare floats on both sides of every LDS row
+constexpr int kLdsBudget = 48 * 1024;   // bytes of LDS one tile may take
+constexpr int kXcds = 8;
+
+// The LDS image of a tile: `planes` images of `lds_rows` rows of `pitch` floats.
+// Row r, column c (after the slack) of an image holds input row iy0 + r, column c - col_shift,
+// or zero where that falls outside the plane.
+struct StageLayout {
+    int in_h, in_w, in_plane;
+    int col_shift;
+    int lds_rows;
+    unsigned lds_rows_magic;
+    int g_lo;   // first (possibly negative) float4 column fetched per row
+    int spr;    // float4 slots per row
+    unsigned spr_magic;
+    int pitch;        // floats per LDS row, slack included
+    int plane_pitch;  // floats per plane image
+    int vec_in;       // 128-bit global loads are legal (in_w % 4 == 0, 16-byte aligned base)
+};
+
+// n / d through the reciprocal made by magic_u16(d); a zero reciprocal stands for d == 1.
+__device__ __forceinline__ int fast_div(int n, unsigned magic)
+{
+    return magic ? static_cast<int>(__umulhi(static_cast<unsigned>(n), magic)) : n;
+}
+
+// Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
+// Give every XCD a contiguous run of tiles so that the row bands of one plane,
+// which share halo rows, meet in the same L2.
+__device__ __forceinline__ int xcd_contiguous_tile(int bid, int n_tiles)
+{
+    const int per = n_tiles / kXcds, rem = n_tiles - per * kXcds;
+    const int xcd = bid % kXcds, k = bid / kXcds;
+    return xcd * per + min(xcd, rem) + k;
+}
+
+// Fills the LDS image of the tile: every float4 slot of every row is written,
+// with zeros where the row or the columns fall outside the plane.
+__device__ __forceinline__ void stage_tile(const StageLayout &s, const float *__restrict__ in, float *lds,
+                                           long plane0, int nplanes, int iy0)
+{
+    const int total = nplanes * s.lds_rows * s.spr;
+    for (int slot = threadIdx.x; slot < total; slot += kThreads) {
+        const int rowidx = fast_div(slot, s.spr_magic);
+        const int sc = slot - rowidx * s.spr;
+        const int pl = fast_div(rowidx, s.lds_rows_magic);
+        const int r = rowidx - pl * s.lds_rows;
+        const int ix = 4 * (s.g_lo + sc);
+        const int iy = iy0 + r;
+        const bool row_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(s.in_h);
+        const float *src = in + (plane0 + pl) * s.in_plane + static_cast<long>(iy) * s.in_w + ix;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (s.vec_in) {
+            if (row_ok && ix >= 0 && ix < s.in_w) v = *reinterpret_cast<const float4 *>(src);
+        } else if (row_ok) {
+            if (static_cast<unsigned>(ix + 0) < static_cast<unsigned>(s.in_w)) v.x = src[0];
+            if (static_cast<unsigned>(ix + 1) < static_cast<unsigned>(s.in_w)) v.y = src[1];
+            if (static_cast<unsigned>(ix + 2) < static_cast<unsigned>(s.in_w)) v.z = src[2];
+            if (static_cast<unsigned>(ix + 3) < static_cast<unsigned>(s.in_w)) v.w = src[3];
+        }
+        float *dst = lds + pl * s.plane_pitch + r * s.pitch + kSlack + ix + s.col_shift;
+        dst[0] = v.x;
+        dst[1] = v.y;
+        dst[2] = v.z;
+        dst[3] = v.w;
+    }
+}
+
+inline int floor_div(int a, int b)
+{
+    int q = a / b;
+    if ((a % b != 0) && ((a < 0) != (b < 0))) --q;
+    return q;
+}
+
+inline int env_int(const char *name, int dflt)
+{
+    const char *e = std::getenv(name);
+    if (e == nullptr || e[0] == '\0') return dflt;
+    return std::atoi(e);
+}
+
+// Row pitch and float4 slots of an image `used_cols` floats wide (col_shift must be set).
+inline void layout_columns(StageLayout &s, int used_cols)
+{
+    s.pitch = kSlack + round_up(used_cols, 4) + kSlack;
+    s.g_lo = floor_div(-s.col_shift, 4);
+    s.spr = ceil_div(used_cols - s.col_shift, 4) - s.g_lo;
+}
+
+// Finishes the layout once the rows per image are known.  False if the 16-bit
+// reciprocals the kernels divide with would not be exact.
+inline bool layout_rows(StageLayout &s, int lds_rows, int planes_per_tile)
+{
+    s.lds_rows = lds_rows;
+    s.plane_pitch = lds_rows * s.pitch;
+    if (static_cast<long>(planes_per_tile) * lds_rows * s.spr >= 65536) return false;
+    s.lds_rows_magic = magic_u16(lds_rows);
+    s.spr_magic = magic_u16(s.spr);
+    return true;
+}
+
+}  // namespace dwconv

@@ -1,14 +1,369 @@
-// fp32 grad-weight with LDS tiles (placeholder until the tiled kernel lands).
-#include "dwconv_common.hpp"
+// fp32 grad-weight with LDS tiles and a fixed-order two-pass reduction.
+//
+//   gw[c,i,j] = sum_{n,oy,ox} gy[n,c,oy,ox] * x[n,c, oy*S - pad_h + i, ox*S - pad_w + j]
+//
+// Pass 1: workgroup (channel group g, chunk k) walks the tiles (image n, band of
+// rows) of its chunk.  Per tile the band of x (with halo) is staged in LDS exactly
+// as in the forward kernel; each lane owns a BH x 4 block of gy, read straight
+// from global memory, and accumulates all K*K taps in registers from one pass
+// over the LDS window.  So x and gy are read once, not K*K times as in the
+// reference's one-block-per-tap kernel (torch_dwconv/dwconv_kernel.cu:260-306),
+// and nothing is accumulated with atomics.  At the end the lanes' K*K sums are
+// reduced in a fixed order (DPP within a wavefront, LDS across wavefronts) and
+// stored as partial[c][k][tap].
+// Pass 2: one lane per (c, tap) adds the chunk partials front to back in double.
+//
+// Large maps use one channel per workgroup (all 256 lanes reduce into one tap
+// table); small maps put P channels of one image side by side, each lane staying
+// with its channel for the whole chunk.
+#include "dwconv_tile_common.hpp"
 
 namespace dwconv {
 
-size_t wgrad_tiled_workspace(const WgradGeometry &) { return 0; }
+namespace {
 
-int try_launch_wgrad_tiled(const float *, const float *, float *, void *, size_t, const WgradGeometry &,
-                           hipStream_t)
+struct WgradPlan {
+    StageLayout st;
+    const float *x;
+    const float *gy;
+    float *partial;
+    int batch, channel;
+    int out_h, out_w, out_plane;
+    int pad_h;
+    int rows_per_tile, row_tiles;
+    int planes_per_tile;   // channels a workgroup carries
+    int groups;            // channel groups = ceil(C / planes_per_tile)
+    int chunks;            // chunks per channel group
+    int tiles_per_group;   // batch * row_tiles
+    int tiles_per_chunk;
+    int ncb;
+    unsigned ncb_magic;
+    int items_per_plane;
+    unsigned ipp_magic;
+    int vec_gy;
+};
+
+template <int CTRL, int ROW_MASK, int BANK_MASK>
+__device__ __forceinline__ float dpp_add(float v)
 {
-    return -1;
+    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, BANK_MASK, true);
+    return v + __int_as_float(moved);
+}
+
+// Sum of the 64 lanes, delivered in lane 63; fixed association order.
+__device__ __forceinline__ float wave_sum_to_last_lane(float v)
+{
+    v = dpp_add<0x111, 0xf, 0xf>(v);  // row_shr:1
+    v = dpp_add<0x112, 0xf, 0xf>(v);  // row_shr:2
+    v = dpp_add<0x114, 0xf, 0xf>(v);  // row_shr:4
+    v = dpp_add<0x118, 0xf, 0xf>(v);  // row_shr:8  -> lane 15 of each row of 16 holds the row sum
+    v = dpp_add<0x142, 0xa, 0xf>(v);  // row_bcast:15 into rows 1 and 3
+    v = dpp_add<0x143, 0xc, 0xf>(v);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+constexpr int kRedPitch = kThreads + 1;  // odd pitch: lanes of one wave reading one column spread over the banks
+
+template <int K, int S, int BH>
+__global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
+{
+    extern __shared__ float4 lds_raw[];
+    float *lds = reinterpret_cast<float *>(lds_raw);
+    constexpr int KK = K * K;
+    constexpr int WIN_ROWS = (BH - 1) * S + K;
+    constexpr int NV = (3 * S + K + 3) / 4;
+
+    const int group = blockIdx.x / p.chunks;
+    const int chunk = blockIdx.x - group * p.chunks;
+    const int c0 = group * p.planes_per_tile;
+    const int nplanes = min(p.planes_per_tile, p.channel - c0);
+    const int t_begin = chunk * p.tiles_per_chunk;
+    const int t_end = min(p.tiles_per_group, t_begin + p.tiles_per_chunk);
+    const int n_items = nplanes * p.items_per_plane;
+
+    float acc[KK];
+#pragma unroll
+    for (int t = 0; t < KK; ++t) acc[t] = 0.f;
+
+    for (int tile = t_begin; tile < t_end; ++tile) {
+        const int n = tile / p.row_tiles, rt = tile - n * p.row_tiles;
+        const long plane0 = static_cast<long>(n) * p.channel + c0;
+        const int oy0 = rt * p.rows_per_tile;
+
+        if (tile != t_begin) __syncthreads();  // the previous tile's window reads are done
+        stage_tile(p.st, p.x, lds, plane0, nplanes, oy0 * S - p.pad_h);
+        __syncthreads();
+
+        for (int item = threadIdx.x; item < n_items; item += kThreads) {
+            const int pl = fast_div(item, p.ipp_magic);
+            const int rem = item - pl * p.items_per_plane;
+            const int rb = fast_div(rem, p.ncb_magic);
+            const int cb = rem - rb * p.ncb;
+
+            // this lane's block of gy (zero where it hangs over the edge of the plane)
+            float g[BH][4];
+            const int ox = 4 * cb;
+            const float *gsrc = p.gy + (plane0 + pl) * p.out_plane + ox;
+#pragma unroll
+            for (int b = 0; b < BH; ++b) {
+                const int oy = oy0 + rb * BH + b;
+                const float *row = gsrc + static_cast<long>(oy) * p.out_w;
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (oy < p.out_h) {
+                    if (p.vec_gy) {
+                        v = *reinterpret_cast<const float4 *>(row);
+                    } else {
+                        if (ox + 0 < p.out_w) v.x = row[0];
+                        if (ox + 1 < p.out_w) v.y = row[1];
+                        if (ox + 2 < p.out_w) v.z = row[2];
+                        if (ox + 3 < p.out_w) v.w = row[3];
+                    }
+                }
+                g[b][0] = v.x;
+                g[b][1] = v.y;
+                g[b][2] = v.z;
+                g[b][3] = v.w;
+            }
+
+            const float *base = lds + pl * p.st.plane_pitch + (rb * BH * S) * p.st.pitch + kSlack + 4 * cb * S;
+#pragma unroll
+            for (int wr = 0; wr < WIN_ROWS; ++wr) {
+                float win[4 * NV];
+#pragma unroll
+                for (int v = 0; v < NV; ++v) {
+                    const float4 q = *reinterpret_cast<const float4 *>(base + wr * p.st.pitch + 4 * v);
+                    win[4 * v + 0] = q.x;
+                    win[4 * v + 1] = q.y;
+                    win[4 * v + 2] = q.z;
+                    win[4 * v + 3] = q.w;
+                }
+#pragma unroll
+                for (int b = 0; b < BH; ++b) {
+                    const int ty = wr - b * S;
+                    if (ty < 0 || ty >= K) continue;
+#pragma unroll
+                    for (int tx = 0; tx < K; ++tx)
+#pragma unroll
+                        for (int o = 0; o < 4; ++o)
+                            acc[ty * K + tx] = fmaf(g[b][o], win[o * S + tx], acc[ty * K + tx]);
+                }
+            }
+        }
+    }
+
+    __syncthreads();  // the tile image is dead; its LDS is reused for the reduction
+    float *out = p.partial + (static_cast<long>(c0) * p.chunks + chunk) * KK;
+    if (p.planes_per_tile == 1) {
+        // every lane worked on the same channel: wavefront sums, then the four wavefronts in order
+#pragma unroll
+        for (int t = 0; t < KK; ++t) {
+            const float s = wave_sum_to_last_lane(acc[t]);
+            if ((threadIdx.x & 63) == 63) lds[(threadIdx.x >> 6) * KK + t] = s;
+        }
+        __syncthreads();
+        if (threadIdx.x < KK) {
+            float s = lds[threadIdx.x];
+#pragma unroll
+            for (int w = 1; w < kThreads / 64; ++w) s += lds[w * KK + threadIdx.x];
+            out[threadIdx.x] = s;
+        }
+    } else {
+        // lanes [pl*ipp, (pl+1)*ipp) hold channel c0+pl: transpose through LDS, then add each run front to back
+#pragma unroll
+        for (int t = 0; t < KK; ++t) lds[t * kRedPitch + threadIdx.x] = acc[t];
+        __syncthreads();
+        for (int e = threadIdx.x; e < nplanes * KK; e += kThreads) {
+            const int pl = e / KK, t = e - pl * KK;
+            const float *col = lds + t * kRedPitch + pl * p.items_per_plane;
+            float s = 0.f;
+            for (int i = 0; i < p.items_per_plane; ++i) s += col[i];
+            out[static_cast<long>(pl) * p.chunks * KK + t] = s;
+        }
+    }
+}
+
+// Pass 2: gw[c,tap] = sum over chunks of partial[c][chunk][tap], front to back, in double.
+__global__ void wgrad_tile_final_kernel(const float *__restrict__ partial, float *__restrict__ gw,
+                                        const int channel_taps, const int taps, const int chunks)
+{
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= channel_taps) return;
+    const int c = e / taps, t = e - c * taps;
+    const float *p = partial + static_cast<long>(c) * chunks * taps + t;
+    double s = 0.0;
+    for (int k = 0; k < chunks; ++k) s += static_cast<double>(p[static_cast<long>(k) * taps]);
+    gw[e] = static_cast<float>(s);
+}
+
+template <int K, int S, int BH>
+bool make_plan(WgradPlan &p, const WgradGeometry &g)
+{
+    constexpr int NV = (3 * S + K + 3) / 4;
+    constexpr int KK = K * K;
+    const int target_wgs = env_int("DWCONV_WGRAD_WGS", 2048);
+    p.batch = g.batch;
+    p.channel = g.channel;
+    p.out_h = g.out_h;
+    p.out_w = g.out_w;
+    p.out_plane = g.out_h * g.out_w;
+    p.pad_h = g.pad_h;
+    p.st.in_h = g.in_h;
+    p.st.in_w = g.in_w;
+    p.st.in_plane = g.in_h * g.in_w;
+    p.st.col_shift = g.pad_w;
+    p.ncb = ceil_div(g.out_w, 4);
+    const int used_cols = 4 * (p.ncb - 1) * S + 4 * NV;
+    layout_columns(p.st, used_cols);
+    auto rows_for = [](int units) { return (units * BH - 1) * S + K; };
+    auto tile_bytes = [&](int units, int planes) {
+        return static_cast<long>(planes) * rows_for(units) * p.st.pitch * 4;
+    };
+    const int row_units = ceil_div(g.out_h, BH);
+    const int ipp_full = row_units * p.ncb;
+    int units_per_tile, planes_per_tile;
+    if (2 * ipp_full <= kThreads && g.channel > 1) {
+        // whole planes, P channels side by side, one item per lane
+        units_per_tile = row_units;
+        planes_per_tile = kThreads / ipp_full;
+        if (planes_per_tile > g.channel) planes_per_tile = g.channel;
+        while (planes_per_tile > 1 && tile_bytes(units_per_tile, planes_per_tile) > kLdsBudget) --planes_per_tile;
+        if (tile_bytes(units_per_tile, planes_per_tile) > kLdsBudget) return false;
+    } else {
+        planes_per_tile = 1;
+        units_per_tile = 2 * kThreads / p.ncb;
+        if (units_per_tile < 1) units_per_tile = 1;
+        if (units_per_tile > row_units) units_per_tile = row_units;
+        while (units_per_tile > 1 && tile_bytes(units_per_tile, 1) > kLdsBudget) --units_per_tile;
+        if (tile_bytes(units_per_tile, 1) > kLdsBudget) return false;
+        const int bands = ceil_div(row_units, units_per_tile);
+        units_per_tile = ceil_div(row_units, bands);
+    }
+    p.planes_per_tile = planes_per_tile;
+    p.rows_per_tile = units_per_tile * BH;
+    p.row_tiles = ceil_div(row_units, units_per_tile);
+    if (!layout_rows(p.st, rows_for(units_per_tile), planes_per_tile)) return false;
+    p.items_per_plane = units_per_tile * p.ncb;
+    if (planes_per_tile * p.items_per_plane >= 65536) return false;
+    p.ncb_magic = magic_u16(p.ncb);
+    p.ipp_magic = magic_u16(p.items_per_plane);
+    p.groups = ceil_div(g.channel, planes_per_tile);
+    const long tiles_per_group = static_cast<long>(g.batch) * p.row_tiles;
+    if (tiles_per_group > 0x7fffffffL) return false;
+    p.tiles_per_group = static_cast<int>(tiles_per_group);
+    int chunks = ceil_div(target_wgs, p.groups);
+    if (chunks > p.tiles_per_group) chunks = p.tiles_per_group;
+    if (chunks < 1) chunks = 1;
+    p.tiles_per_chunk = ceil_div(p.tiles_per_group, chunks);
+    p.chunks = ceil_div(p.tiles_per_group, p.tiles_per_chunk);
+    if (static_cast<long>(p.groups) * p.chunks > 0x7fffffffL) return false;
+    (void)KK;
+    return true;
+}
+
+template <int K, int S, int BH>
+size_t lds_bytes(const WgradPlan &p)
+{
+    const size_t tile = static_cast<size_t>(p.planes_per_tile) * p.st.plane_pitch * 4;
+    const size_t red = p.planes_per_tile == 1 ? static_cast<size_t>(kThreads / 64) * K * K * 4
+                                              : static_cast<size_t>(K) * K * kRedPitch * 4;
+    return tile > red ? tile : red;
+}
+
+// Calls fn.template operator()<K,S,BH>() for the instance that covers g; false if none does.
+template <typename Fn>
+bool dispatch(const WgradGeometry &g, Fn &&fn)
+{
+    const int K = g.kernel_h, S = g.down_h;
+    if (g.kernel_w != K || g.down_w != S) return false;
+    if (g.pad_h < 0 || g.pad_w < 0 || g.pad_h > 7 || g.pad_w > 7) return false;
+    if (g.in_h < 1 || g.in_w < 1 || g.out_h < 1 || g.out_w < 1) return false;
+    if (static_cast<long>(g.in_h) * g.in_w >= (1l << 30) || static_cast<long>(g.out_h) * g.out_w >= (1l << 30))
+        return false;
+    // every gy element must map inside the padded plane the LDS image covers
+    if ((g.out_h - 1) * S - g.pad_h + K - 1 > g.in_h - 1 + 7 || (g.out_w - 1) * S - g.pad_w + K - 1 > g.in_w - 1 + 7)
+        return false;
+    const int forced = env_int("DWCONV_TILE_BH", 0);
+    const bool seven = forced ? forced == 7 : (g.out_h % 7 == 0 || g.out_h > 64) && g.out_h % 4 != 0;
+#define DWCONV_WGRAD_CASE(KV, SV)                                                   \
+    if (K == KV && S == SV) {                                                       \
+        if (seven) fn.template operator()<KV, SV, 7>();                            \
+        else fn.template operator()<KV, SV, 4>();                                  \
+        return true;                                                                \
+    }
+    DWCONV_WGRAD_CASE(3, 1)
+    DWCONV_WGRAD_CASE(5, 1)
+    DWCONV_WGRAD_CASE(7, 1)
+    DWCONV_WGRAD_CASE(3, 2)
+    DWCONV_WGRAD_CASE(5, 2)
+    DWCONV_WGRAD_CASE(7, 2)
+#undef DWCONV_WGRAD_CASE
+    return false;
+}
+
+struct WorkspaceQuery {
+    const WgradGeometry &g;
+    size_t bytes = 0;
+    template <int K, int S, int BH>
+    void operator()()
+    {
+        WgradPlan p{};
+        if (make_plan<K, S, BH>(p, g))
+            bytes = static_cast<size_t>(p.groups) * p.planes_per_tile * p.chunks * K * K * sizeof(float);
+    }
+};
+
+struct Launcher {
+    const float *x;
+    const float *gy;
+    float *gw;
+    void *ws;
+    size_t ws_bytes;
+    const WgradGeometry &g;
+    hipStream_t stream;
+    int rc = -1;
+    template <int K, int S, int BH>
+    void operator()()
+    {
+        WgradPlan p{};
+        if (!make_plan<K, S, BH>(p, g)) return;
+        const size_t need = static_cast<size_t>(p.groups) * p.planes_per_tile * p.chunks * K * K * sizeof(float);
+        if (ws == nullptr || ws_bytes < need) {
+            rc = fail(DWCONV_ERR_WORKSPACE, "grad-weight needs a workspace of %zu bytes, got %zu", need, ws_bytes);
+            return;
+        }
+        p.x = x;
+        p.gy = gy;
+        p.partial = static_cast<float *>(ws);
+        p.st.vec_in = (g.in_w % 4 == 0) && aligned16(x);
+        p.vec_gy = (g.out_w % 4 == 0) && aligned16(gy);
+        const size_t shmem = lds_bytes<K, S, BH>(p);
+        hipLaunchKernelGGL((wgrad_tile_kernel<K, S, BH>), dim3(p.groups * p.chunks), dim3(kThreads), shmem, stream, p);
+        rc = check_launch("wgrad_tile_kernel");
+        if (rc != DWCONV_OK) return;
+        const int total = g.channel * K * K;
+        hipLaunchKernelGGL(wgrad_tile_final_kernel, dim3(ceil_div(total, 256)), dim3(256), 0, stream,
+                           static_cast<const float *>(ws), gw, total, K * K, p.chunks);
+        note_variant("wgrad_tile<k%d,s%d,bh%d> P%d rows%d chunks%d vin%d vgy%d", K, S, BH, p.planes_per_tile,
+                     p.rows_per_tile, p.chunks, p.st.vec_in, p.vec_gy);
+        rc = check_launch("wgrad_tile_final_kernel");
+    }
+};
+
+}  // namespace
+
+size_t wgrad_tiled_workspace(const WgradGeometry &g)
+{
+    WorkspaceQuery q{g};
+    dispatch(g, q);
+    return q.bytes;
+}
+
+int try_launch_wgrad_tiled(const float *in, const float *gy, float *gw, void *ws, size_t ws_bytes,
+                           const WgradGeometry &g, hipStream_t stream)
+{
+    Launcher l{in, gy, gw, ws, ws_bytes, g, stream};
+    if (!dispatch(g, l)) return -1;
+    return l.rc;
 }
 
 }  // namespace dwconv
