@@ -161,6 +161,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-miopen", action="store_true")
     ap.add_argument("--table", action="store_true", help="print a per-layer, per-pass table to stderr")
+    ap.add_argument("--calibration-copy-mib", type=int, default=0,
+                    help="also run one plain device copy of this many MiB first (a kernel of known traffic, "
+                         "to scale rocprofv3 FETCH_SIZE/WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: depthwise conv2d is a single-GPU kernel path; run with --gpus 1")
@@ -185,6 +188,13 @@ def main():
         for _, _, fn in calls:
             fn(stream)
 
+    if args.calibration_copy_mib:
+        src = torch.ones(args.calibration_copy_mib * 1024 * 1024 // 4, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

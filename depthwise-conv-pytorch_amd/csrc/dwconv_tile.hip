@@ -52,7 +52,7 @@ struct TilePlan {
 template <int KK, bool FLIP>
 __device__ __forceinline__ void stage_taps(const TilePlan &p, float *lds, long plane0, int nplanes)
 {
-    for (int i = threadIdx.x; i < nplanes * KK; i += kThreads) {
+    for (int i = threadIdx.x; i < nplanes * KK; i += blockDim.x) {
         const int pl = i / KK, t = i - pl * KK;
         const int c = static_cast<int>((plane0 + pl) % p.channel);
         lds[p.tap_base + i] = p.taps[c * KK + (FLIP ? KK - 1 - t : t)];
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
     __syncthreads();
 
     const int n_items = nplanes * p.items_per_plane;
-    for (int item = threadIdx.x; item < n_items; item += kThreads) {
+    for (int item = threadIdx.x; item < n_items; item += blockDim.x) {
         const int pl = fast_div(item, p.ipp_magic);
         const int rem = item - pl * p.items_per_plane;
         const int rb = fast_div(rem, p.ncb_magic);
@@ -163,7 +163,7 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
     __syncthreads();
 
     const int n_items = nplanes * p.items_per_plane;
-    for (int item = threadIdx.x; item < n_items; item += kThreads) {
+    for (int item = threadIdx.x; item < n_items; item += blockDim.x) {
         const int pl = fast_div(item, p.ipp_magic);
         const int rem = item - pl * p.items_per_plane;
         const int rb = fast_div(rem, p.ncb_magic);
@@ -239,7 +239,8 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
 template <typename RowsFor>
 bool plan_tiles(TilePlan &p, int row_units, int unit_rows, int used_cols, int taps_per_plane, RowsFor rows_for)
 {
-    const int target_items = env_int("DWCONV_TILE_ITEMS", 2 * kThreads);
+    const int threads = env_int("DWCONV_TILE_THREADS", kThreads);
+    const int target_items = env_int("DWCONV_TILE_ITEMS", threads);
     layout_columns(p.st, used_cols);
 
     auto bytes = [&](int units, int planes) {
@@ -248,7 +249,7 @@ bool plan_tiles(TilePlan &p, int row_units, int unit_rows, int used_cols, int ta
 
     const int ipp_full = row_units * p.ncb;
     int units_per_tile, planes_per_tile;
-    if (ipp_full <= target_items / 2) {
+    if (2 * ipp_full <= target_items) {
         // whole planes, several per tile
         units_per_tile = row_units;
         planes_per_tile = target_items / ipp_full;
@@ -299,7 +300,7 @@ int launch_down(TilePlan &p, hipStream_t stream)
     const int used_cols = 4 * (p.ncb - 1) * S + 4 * NV;
     auto rows_for = [](int units) { return (units * BH - 1) * S + K; };
     if (!plan_tiles(p, ceil_div(p.out_h, BH), BH, used_cols, K * K, rows_for)) return -1;
-    hipLaunchKernelGGL((fir_down_kernel<K, S, FLIP, BH>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K),
+    hipLaunchKernelGGL((fir_down_kernel<K, S, FLIP, BH>), dim3(p.n_tiles), dim3(env_int("DWCONV_TILE_THREADS", kThreads)), lds_bytes(p, K * K),
                        stream, p);
     note_variant("tile_down<k%d,s%d,%s,bh%d> P%d rows%d vin%d vout%d", K, S, FLIP ? "rot" : "fwd", BH,
                  p.planes_per_tile, p.rows_per_tile, p.st.vec_in, p.vec_out);
@@ -323,7 +324,7 @@ int launch_up2(TilePlan &p, hipStream_t stream)
     const int used_cols = 4 * (p.ncb - 1) + 8;
     auto rows_for = [](int units) { return units * BQ + KAY; };
     if (!plan_tiles(p, ceil_div(ceil_div(p.out_h, 2), BQ), BQ, used_cols, K * K, rows_for)) return -1;
-    hipLaunchKernelGGL((fir_up2_kernel<K, EY, EX, BQ>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K), stream,
+    hipLaunchKernelGGL((fir_up2_kernel<K, EY, EX, BQ>), dim3(p.n_tiles), dim3(env_int("DWCONV_TILE_THREADS", kThreads)), lds_bytes(p, K * K), stream,
                        p);
     note_variant("tile_up2<k%d,e%d%d,bq%d> P%d rows%d vin%d vout%d", K, EY, EX, BQ, p.planes_per_tile,
                  p.rows_per_tile, p.st.vec_in, p.vec_out);

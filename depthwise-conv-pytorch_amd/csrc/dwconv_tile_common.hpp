@@ -51,7 +51,7 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const float *__
                                            long plane0, int nplanes, int iy0)
 {
     const int total = nplanes * s.lds_rows * s.spr;
-    for (int slot = threadIdx.x; slot < total; slot += kThreads) {
+    for (int slot = threadIdx.x; slot < total; slot += blockDim.x) {
         const int rowidx = fast_div(slot, s.spr_magic);
         const int sc = slot - rowidx * s.spr;
         const int pl = fast_div(rowidx, s.lds_rows_magic);

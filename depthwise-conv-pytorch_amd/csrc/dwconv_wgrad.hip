@@ -94,7 +94,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
         stage_tile(p.st, p.x, lds, plane0, nplanes, oy0 * S - p.pad_h);
         __syncthreads();
 
-        for (int item = threadIdx.x; item < n_items; item += kThreads) {
+        for (int item = threadIdx.x; item < n_items; item += blockDim.x) {
             const int pl = fast_div(item, p.ipp_magic);
             const int rem = item - pl * p.items_per_plane;
             const int rb = fast_div(rem, p.ncb_magic);
@@ -172,7 +172,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
 #pragma unroll
         for (int t = 0; t < KK; ++t) lds[t * kRedPitch + threadIdx.x] = acc[t];
         __syncthreads();
-        for (int e = threadIdx.x; e < nplanes * KK; e += kThreads) {
+        for (int e = threadIdx.x; e < nplanes * KK; e += blockDim.x) {
             const int pl = e / KK, t = e - pl * KK;
             const float *col = lds + t * kRedPitch + pl * p.items_per_plane;
             float s = 0.f;
