@@ -88,7 +88,9 @@ int run_fir(const T *in, const T *taps, T *out, const Geometry &g, hipStream_t s
     }
     if constexpr (sizeof(T) == 4) {
         if (!force_generic()) {
-            const int rc = try_launch_fir_tiled(in, taps, out, g, stream);
+            int rc = try_launch_fir_small(in, taps, out, g, stream);
+            if (rc >= 0) return rc;
+            rc = try_launch_fir_tiled(in, taps, out, g, stream);
             if (rc >= 0) return rc;
         }
     }

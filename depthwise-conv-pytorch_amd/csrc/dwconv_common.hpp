@@ -67,6 +67,10 @@ int launch_wgrad_direct(const T *in, const T *gy, T *gw, void *ws, size_t ws_byt
 int try_launch_fir_tiled(const float *in, const float *taps, float *out, const Geometry &g,
                          hipStream_t stream);
 
+// ---- whole-plane fp32 kernels for maps 7, 14 or 28 wide: dwconv_small.hip (same return convention) ----
+int try_launch_fir_small(const float *in, const float *taps, float *out, const Geometry &g,
+                         hipStream_t stream);
+
 // ---- fp32 grad-weight with LDS tiles and a fixed-order two-pass reduction: dwconv_wgrad.hip ----
 size_t wgrad_tiled_workspace(const WgradGeometry &g);  // 0 when the tiled kernel does not cover g
 int try_launch_wgrad_tiled(const float *in, const float *gy, float *gw, void *ws, size_t ws_bytes,

@@ -1,0 +1,369 @@
+// Whole-plane fp32 kernels for small feature maps (width 7, 14 or 28, "same" padding).
+//
+// Planes of a small map are tiny (196 B to 3 KiB) and sit back to back in memory,
+// so the only way to move them at HBM speed is to treat a run of P planes as one
+// flat stream: 128-bit loads of the run into LDS (same layout as in memory, no
+// index arithmetic), arithmetic out of LDS, results back into LDS in their
+// memory layout, 128-bit stores of the run.  One wavefront (a 64-lane workgroup,
+// so no cross-wave barrier exists) owns a run; a CU holds about ten such
+// wavefronts, each with several loads in flight.
+//
+// A lane owns BH full-width output rows of one plane.  Because it holds whole
+// rows, which taps fall off the left/right edge is known at compile time (they
+// are simply not emitted); rows above/below the plane are replaced by zeros
+// with a select.  The reference's counterpart (torch_dwconv/dwconv_kernel.cu:308-442,
+// :444-588) keeps a zero-filled padded tile in shared memory and re-reads every
+// tap for every output.
+//
+//   small_down_kernel : up = 1, decimation S; forward, and grad-input of stride-1 layers (FLIP)
+//   small_up2_kernel  : up = 2, taps rotated; grad-input of stride-2 layers
+//   small_wgrad_kernel: grad-weight pass 1 (lane keeps its channel across the images of a chunk)
+#include "dwconv_tile_common.hpp"
+
+namespace dwconv {
+
+namespace {
+
+constexpr int kWave = 64;
+
+struct SmallPlan {
+    const float *in;
+    const float *taps;
+    float *out;
+    long planes;
+    int channel;
+    int in_h, out_h;
+    int pad_h;             // leading zero rows (down) or m = (pad0 + E) / 2 (up2)
+    int planes_per_run;    // P
+    int lanes_per_plane;   // LPP
+    unsigned lpp_magic;
+};
+
+// ---- LDS rows -----------------------------------------------------------------------------
+template <int N>
+__device__ __forceinline__ void lds_load_row(const float *p, float (&r)[N])
+{
+    if constexpr (N % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < N / 4; ++i) {
+            const float4 v = reinterpret_cast<const float4 *>(p)[i];
+            r[4 * i] = v.x; r[4 * i + 1] = v.y; r[4 * i + 2] = v.z; r[4 * i + 3] = v.w;
+        }
+    } else if constexpr (N % 2 == 0) {
+#pragma unroll
+        for (int i = 0; i < N / 2; ++i) {
+            const float2 v = reinterpret_cast<const float2 *>(p)[i];
+            r[2 * i] = v.x; r[2 * i + 1] = v.y;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) r[i] = p[i];
+    }
+}
+
+template <int N>
+__device__ __forceinline__ void lds_store_row(float *p, const float *r)
+{
+    if constexpr (N % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < N / 4; ++i)
+            reinterpret_cast<float4 *>(p)[i] = make_float4(r[4 * i], r[4 * i + 1], r[4 * i + 2], r[4 * i + 3]);
+    } else if constexpr (N % 2 == 0) {
+#pragma unroll
+        for (int i = 0; i < N / 2; ++i) reinterpret_cast<float2 *>(p)[i] = make_float2(r[2 * i], r[2 * i + 1]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) p[i] = r[i];
+    }
+}
+
+// ---- flat runs between global memory and LDS ---------------------------------------------------
+// `g` is 16-byte aligned; n floats; the last partial float4 (only at the very end of a tensor) goes scalar.
+__device__ __forceinline__ void run_to_lds(const float *__restrict__ g, float *lds, int n)
+{
+    const int n4 = n >> 2;
+    for (int i = threadIdx.x; i < n4; i += kWave)
+        reinterpret_cast<float4 *>(lds)[i] = reinterpret_cast<const float4 *>(g)[i];
+    const int tail = n4 * 4 + threadIdx.x;
+    if (tail < n) lds[tail] = g[tail];
+}
+
+__device__ __forceinline__ void lds_to_run(float *__restrict__ g, const float *lds, int n)
+{
+    const int n4 = n >> 2;
+    for (int i = threadIdx.x; i < n4; i += kWave)
+        reinterpret_cast<float4 *>(g)[i] = reinterpret_cast<const float4 *>(lds)[i];
+    const int tail = n4 * 4 + threadIdx.x;
+    if (tail < n) g[tail] = lds[tail];
+}
+
+// This lane's K*K taps straight from global memory (the lanes of one plane read the same addresses).
+template <int KK, bool FLIP>
+__device__ __forceinline__ void load_taps(const float *__restrict__ taps, int c, float (&t)[KK])
+{
+#pragma unroll
+    for (int i = 0; i < KK; ++i) t[i] = taps[c * KK + (FLIP ? KK - 1 - i : i)];
+}
+
+// out[oy,ox] = sum_{ty,tx} in[oy*S - pad_h + ty, ox*S - K/2 + tx] * f[ty,tx], planes W wide.
+template <int W, int K, int S, bool FLIP, int BH>
+__global__ __launch_bounds__(kWave) void small_down_kernel(const SmallPlan p)
+{
+    extern __shared__ float4 lds_raw[];
+    float *lds = reinterpret_cast<float *>(lds_raw);
+    constexpr int OW = (W - 1) / S + 1;
+    constexpr int PW = K / 2;
+    constexpr int WIN_ROWS = (BH - 1) * S + K;
+
+    const long plane0 = static_cast<long>(blockIdx.x) * p.planes_per_run;
+    const int nplanes = static_cast<int>(min(static_cast<long>(p.planes_per_run), p.planes - plane0));
+    const int in_plane = p.in_h * W, out_plane = p.out_h * OW;
+
+    const int pl_raw = fast_div(threadIdx.x, p.lpp_magic);
+    const int rb = threadIdx.x - pl_raw * p.lanes_per_plane;
+    const bool active = pl_raw < nplanes;
+    const int pl = active ? pl_raw : 0;
+
+    float tapv[K * K];
+    load_taps<K * K, FLIP>(p.taps, static_cast<int>((plane0 + pl) % p.channel), tapv);
+    run_to_lds(p.in + plane0 * in_plane, lds, nplanes * in_plane);
+    __syncthreads();
+
+    float acc[BH][OW];
+#pragma unroll
+    for (int b = 0; b < BH; ++b)
+#pragma unroll
+        for (int o = 0; o < OW; ++o) acc[b][o] = 0.f;
+
+    const int oy0 = rb * BH;
+    const float *plane = lds + pl * in_plane;
+#pragma unroll
+    for (int wr = 0; wr < WIN_ROWS; ++wr) {
+        const int iy = oy0 * S - p.pad_h + wr;
+        const bool ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
+        float row[W];
+        lds_load_row<W>(plane + (ok ? iy : 0) * W, row);
+#pragma unroll
+        for (int i = 0; i < W; ++i) row[i] = ok ? row[i] : 0.f;
+#pragma unroll
+        for (int b = 0; b < BH; ++b) {
+            const int ty = wr - b * S;
+            if (ty < 0 || ty >= K) continue;
+#pragma unroll
+            for (int tx = 0; tx < K; ++tx)
+#pragma unroll
+                for (int o = 0; o < OW; ++o) {
+                    const int ix = o * S - PW + tx;
+                    if (ix < 0 || ix >= W) continue;
+                    acc[b][o] = fmaf(row[ix], tapv[ty * K + tx], acc[b][o]);
+                }
+        }
+    }
+    __syncthreads();  // every lane has read its input rows: the run can be overwritten in place
+
+    if (active) {
+        float *dst = lds + pl * out_plane;
+#pragma unroll
+        for (int b = 0; b < BH; ++b)
+            if (oy0 + b < p.out_h) lds_store_row<OW>(dst + (oy0 + b) * OW, acc[b]);
+    }
+    __syncthreads();
+    lds_to_run(p.out + plane0 * out_plane, lds, nplanes * out_plane);
+}
+
+// up = 2, taps rotated, "same" padding of the forward conv (leading pad of the transposed problem = K/2):
+//   out[2q + r] = sum_a in[q - m + r + a] * g'[r + 2a],  g'[t] = g[t - E],  E = (K/2) & 1,  m = (K/2 + E) / 2.
+// Input planes are W wide, output planes 2W wide; a lane owns output rows 2q, 2q+1.
+template <int W, int K>
+__global__ __launch_bounds__(kWave) void small_up2_kernel(const SmallPlan p)
+{
+    extern __shared__ float4 lds_raw[];
+    float *lds = reinterpret_cast<float *>(lds_raw);
+    constexpr int OW = 2 * W;
+    constexpr int E = (K / 2) & 1;
+    constexpr int M = (K / 2 + E) / 2;
+    constexpr int KA = (K + E + 1) / 2;
+    constexpr int WIN_ROWS = KA + 1;
+
+    const long plane0 = static_cast<long>(blockIdx.x) * p.planes_per_run;
+    const int nplanes = static_cast<int>(min(static_cast<long>(p.planes_per_run), p.planes - plane0));
+    const int in_plane = p.in_h * W, out_plane = p.out_h * OW;
+
+    const int pl_raw = fast_div(threadIdx.x, p.lpp_magic);
+    const int q = threadIdx.x - pl_raw * p.lanes_per_plane;
+    const bool active = pl_raw < nplanes;
+    const int pl = active ? pl_raw : 0;
+
+    float tapv[K * K];
+    load_taps<K * K, true>(p.taps, static_cast<int>((plane0 + pl) % p.channel), tapv);
+    run_to_lds(p.in + plane0 * in_plane, lds, nplanes * in_plane);
+    __syncthreads();
+
+    float acc[2][OW];
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int o = 0; o < OW; ++o) acc[r][o] = 0.f;
+
+    const float *plane = lds + pl * in_plane;
+#pragma unroll
+    for (int wr = 0; wr < WIN_ROWS; ++wr) {
+        const int iy = q - p.pad_h + wr;
+        const bool ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
+        float row[W];
+        lds_load_row<W>(plane + (ok ? iy : 0) * W, row);
+#pragma unroll
+        for (int i = 0; i < W; ++i) row[i] = ok ? row[i] : 0.f;
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const int a = wr - r;
+            if (a < 0 || a >= KA) continue;
+            const int fy = r + 2 * a - E;
+            if (fy < 0 || fy >= K) continue;
+#pragma unroll
+            for (int o = 0; o < OW; ++o) {
+                const int xq = o / 2, rx = o % 2;
+#pragma unroll
+                for (int ax = 0; ax < KA; ++ax) {
+                    const int fx = rx + 2 * ax - E;
+                    const int ix = xq - M + rx + ax;
+                    if (fx < 0 || fx >= K || ix < 0 || ix >= W) continue;
+                    acc[r][o] = fmaf(row[ix], tapv[fy * K + fx], acc[r][o]);
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    if (active) {
+        float *dst = lds + pl * out_plane;
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+            if (2 * q + r < p.out_h) lds_store_row<OW>(dst + (2 * q + r) * OW, acc[r]);
+    }
+    __syncthreads();
+    lds_to_run(p.out + plane0 * out_plane, lds, nplanes * out_plane);
+}
+
+size_t small_lds_bytes(int planes, int in_plane, int out_plane)
+{
+    return static_cast<size_t>(planes) * (in_plane > out_plane ? in_plane : out_plane) * 4;
+}
+
+// Planes per wavefront: as many as there are lane slots, a multiple of 4 when a plane is not a
+// multiple of 4 floats (so that every run starts on a 16-byte boundary), within the LDS budget.
+int planes_per_run(int lanes_per_plane, int in_plane, int out_plane, long planes)
+{
+    int P = kWave / lanes_per_plane;
+    while (P > 0 && small_lds_bytes(P, in_plane, out_plane) > 16 * 1024) --P;
+    if (in_plane % 4 != 0 || out_plane % 4 != 0) P -= P % 4;
+    if (static_cast<long>(P) > planes && in_plane % 4 == 0 && out_plane % 4 == 0) P = static_cast<int>(planes);
+    return P;
+}
+
+template <int W, int K, int S, bool FLIP, int BH>
+int launch_small_down(SmallPlan &p, hipStream_t stream)
+{
+    constexpr int OW = (W - 1) / S + 1;
+    p.lanes_per_plane = ceil_div(p.out_h, BH);
+    if (p.lanes_per_plane > kWave) return -1;
+    const int in_plane = p.in_h * W, out_plane = p.out_h * OW;
+    p.planes_per_run = planes_per_run(p.lanes_per_plane, in_plane, out_plane, p.planes);
+    if (p.planes_per_run < 1) return -1;
+    p.lpp_magic = magic_u16(p.lanes_per_plane);
+    const long runs = (p.planes + p.planes_per_run - 1) / p.planes_per_run;
+    if (runs > 0x7fffffffL) return -1;
+    const size_t shmem = small_lds_bytes(p.planes_per_run, in_plane, out_plane);
+    hipLaunchKernelGGL((small_down_kernel<W, K, S, FLIP, BH>), dim3(static_cast<unsigned>(runs)), dim3(kWave), shmem,
+                       stream, p);
+    note_variant("small_down<w%d,k%d,s%d,%s,bh%d> P%d", W, K, S, FLIP ? "rot" : "fwd", BH, p.planes_per_run);
+    return check_launch("small_down_kernel");
+}
+
+template <int W, int K>
+int launch_small_up2(SmallPlan &p, hipStream_t stream)
+{
+    p.lanes_per_plane = ceil_div(p.out_h, 2);
+    if (p.lanes_per_plane > kWave) return -1;
+    const int in_plane = p.in_h * W, out_plane = p.out_h * 2 * W;
+    p.planes_per_run = planes_per_run(p.lanes_per_plane, in_plane, out_plane, p.planes);
+    if (p.planes_per_run < 1) return -1;
+    p.lpp_magic = magic_u16(p.lanes_per_plane);
+    const long runs = (p.planes + p.planes_per_run - 1) / p.planes_per_run;
+    if (runs > 0x7fffffffL) return -1;
+    const size_t shmem = small_lds_bytes(p.planes_per_run, in_plane, out_plane);
+    hipLaunchKernelGGL((small_up2_kernel<W, K>), dim3(static_cast<unsigned>(runs)), dim3(kWave), shmem, stream, p);
+    note_variant("small_up2<w%d,k%d> P%d", W, K, p.planes_per_run);
+    return check_launch("small_up2_kernel");
+}
+
+template <int W, int K>
+int launch_small_down_any(SmallPlan &p, int S, bool rot, hipStream_t stream)
+{
+    constexpr int BH1 = W == 7 ? 7 : 2;
+    if (S == 1) return rot ? launch_small_down<W, K, 1, true, BH1>(p, stream) : launch_small_down<W, K, 1, false, BH1>(p, stream);
+    if constexpr (W % 2 == 0) {
+        if (S == 2 && !rot) return launch_small_down<W, K, 2, false, 1>(p, stream);
+    }
+    return -1;
+}
+
+template <int W>
+int launch_small_down_k(SmallPlan &p, int K, int S, bool rot, hipStream_t stream)
+{
+    if (K == 3) return launch_small_down_any<W, 3>(p, S, rot, stream);
+    if (K == 5) return launch_small_down_any<W, 5>(p, S, rot, stream);
+    if (K == 7) return launch_small_down_any<W, 7>(p, S, rot, stream);
+    return -1;
+}
+
+template <int W>
+int launch_small_up2_k(SmallPlan &p, int K, hipStream_t stream)
+{
+    if (K == 3) return launch_small_up2<W, 3>(p, stream);
+    if (K == 5) return launch_small_up2<W, 5>(p, stream);
+    if (K == 7) return launch_small_up2<W, 7>(p, stream);
+    return -1;
+}
+
+}  // namespace
+
+int try_launch_fir_small(const float *in, const float *taps, float *out, const Geometry &g, hipStream_t stream)
+{
+    if (env_int("DWCONV_NO_SMALL", 0)) return -1;
+    const int K = g.kernel_h;
+    if (g.kernel_w != K || (K != 3 && K != 5 && K != 7)) return -1;
+    if (!aligned16(in) || !aligned16(out)) return -1;
+    if (g.in_h < 1 || g.in_h > 64 || g.out_h < 1 || g.out_h > 128) return -1;
+    SmallPlan p{};
+    p.in = in;
+    p.taps = taps;
+    p.out = out;
+    p.planes = g.planes();
+    p.channel = g.channel;
+    p.in_h = g.in_h;
+    p.out_h = g.out_h;
+    const int W = g.in_w;
+    if (g.up_h == 1 && g.up_w == 1 && g.down_h == g.down_w && (g.down_h == 1 || g.down_h == 2)) {
+        const int S = g.down_h;
+        // full-width rows with the column padding of a "same" convolution
+        if (g.pad_w0 != K / 2 || g.out_w != (W - 1) / S + 1) return -1;
+        if (g.pad_h0 < 0 || g.pad_h0 > 7) return -1;
+        p.pad_h = g.pad_h0;
+        if (W == 7) return launch_small_down_k<7>(p, K, S, !g.forward, stream);
+        if (W == 14) return launch_small_down_k<14>(p, K, S, !g.forward, stream);
+        if (W == 28) return launch_small_down_k<28>(p, K, S, !g.forward, stream);
+        return -1;
+    }
+    if (g.up_h == 2 && g.up_w == 2 && g.down_h == 1 && g.down_w == 1 && !g.forward) {
+        if (g.pad_w0 != K / 2 || g.pad_h0 != K / 2 || g.out_w != 2 * W) return -1;
+        const int E = (K / 2) & 1;
+        p.pad_h = (K / 2 + E) / 2;
+        if (W == 7) return launch_small_up2_k<7>(p, K, stream);
+        if (W == 14) return launch_small_up2_k<14>(p, K, stream);
+        return -1;
+    }
+    return -1;
+}
+
+}  // namespace dwconv
