@@ -166,6 +166,8 @@ size_t wgrad_workspace(const WgradGeometry &g)
     if constexpr (sizeof(T) == 4) {
         const size_t t = wgrad_tiled_workspace(g);
         if (t > need) need = t;
+        const size_t sm = wgrad_small_workspace(g);
+        if (sm > need) need = sm;
     }
     return need;
 }
@@ -192,9 +194,15 @@ int wgrad_any(const T *in, const T *gy, T *gw, void *ws, size_t ws_bytes, int ba
         return launch_fill_zero(gw, static_cast<size_t>(taps) * sizeof(T), stream);
     }
     if constexpr (sizeof(T) == 4) {
-        if (!force_generic() && wgrad_tiled_workspace(g) > 0) {
-            const int r = try_launch_wgrad_tiled(in, gy, gw, ws, ws_bytes, g, stream);
-            if (r >= 0) return r;
+        if (!force_generic()) {
+            if (wgrad_small_workspace(g) > 0) {
+                const int r = try_launch_wgrad_small(in, gy, gw, ws, ws_bytes, g, stream);
+                if (r >= 0) return r;
+            }
+            if (wgrad_tiled_workspace(g) > 0) {
+                const int r = try_launch_wgrad_tiled(in, gy, gw, ws, ws_bytes, g, stream);
+                if (r >= 0) return r;
+            }
         }
     }
     return launch_wgrad_direct<T>(in, gy, gw, ws, ws_bytes, g, stream);

@@ -71,6 +71,12 @@ int try_launch_fir_tiled(const float *in, const float *taps, float *out, const G
 int try_launch_fir_small(const float *in, const float *taps, float *out, const Geometry &g,
                          hipStream_t stream);
 
+size_t wgrad_small_workspace(const WgradGeometry &g);  // 0 when the whole-plane kernel does not cover g
+int try_launch_wgrad_small(const float *in, const float *gy, float *gw, void *ws, size_t ws_bytes,
+                           const WgradGeometry &g, hipStream_t stream);
+// Pass 2 shared by the fp32 grad-weight kernels: gw[c][tap] = sum over chunks of partial[c][chunk][tap].
+int launch_wgrad_final(const float *partial, float *gw, int channel, int taps, int chunks, hipStream_t stream);
+
 // ---- fp32 grad-weight with LDS tiles and a fixed-order two-pass reduction: dwconv_wgrad.hip ----
 size_t wgrad_tiled_workspace(const WgradGeometry &g);  // 0 when the tiled kernel does not cover g
 int try_launch_wgrad_tiled(const float *in, const float *gy, float *gw, void *ws, size_t ws_bytes,

@@ -183,6 +183,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
 }
 
 // Pass 2: gw[c,tap] = sum over chunks of partial[c][chunk][tap], front to back, in double.
+// Loads are issued eight at a time so that their latencies overlap; the additions keep their order.
 __global__ void wgrad_tile_final_kernel(const float *__restrict__ partial, float *__restrict__ gw,
                                         const int channel_taps, const int taps, const int chunks)
 {
@@ -191,7 +192,15 @@ __global__ void wgrad_tile_final_kernel(const float *__restrict__ partial, float
     const int c = e / taps, t = e - c * taps;
     const float *p = partial + static_cast<long>(c) * chunks * taps + t;
     double s = 0.0;
-    for (int k = 0; k < chunks; ++k) s += static_cast<double>(p[static_cast<long>(k) * taps]);
+    int k = 0;
+    for (; k + 8 <= chunks; k += 8) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = p[static_cast<long>(k + j) * taps];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s += static_cast<double>(v[j]);
+    }
+    for (; k < chunks; ++k) s += static_cast<double>(p[static_cast<long>(k) * taps]);
     gw[e] = static_cast<float>(s);
 }
 
@@ -340,16 +349,21 @@ struct Launcher {
         hipLaunchKernelGGL((wgrad_tile_kernel<K, S, BH>), dim3(p.groups * p.chunks), dim3(kThreads), shmem, stream, p);
         rc = check_launch("wgrad_tile_kernel");
         if (rc != DWCONV_OK) return;
-        const int total = g.channel * K * K;
-        hipLaunchKernelGGL(wgrad_tile_final_kernel, dim3(ceil_div(total, 256)), dim3(256), 0, stream,
-                           static_cast<const float *>(ws), gw, total, K * K, p.chunks);
         note_variant("wgrad_tile<k%d,s%d,bh%d> P%d rows%d chunks%d vin%d vgy%d", K, S, BH, p.planes_per_tile,
                      p.rows_per_tile, p.chunks, p.st.vec_in, p.vec_gy);
-        rc = check_launch("wgrad_tile_final_kernel");
+        rc = launch_wgrad_final(static_cast<const float *>(ws), gw, g.channel, K * K, p.chunks, stream);
     }
 };
 
 }  // namespace
+
+int launch_wgrad_final(const float *partial, float *gw, int channel, int taps, int chunks, hipStream_t stream)
+{
+    const int total = channel * taps;
+    hipLaunchKernelGGL(wgrad_tile_final_kernel, dim3(ceil_div(total, 64)), dim3(64), 0, stream, partial, gw, total,
+                       taps, chunks);
+    return check_launch("wgrad_tile_final_kernel");
+}
 
 size_t wgrad_tiled_workspace(const WgradGeometry &g)
 {
