@@ -79,20 +79,63 @@ __device__ __forceinline__ void lds_store_row(float *p, const float *r)
 
 // ---- flat runs between global memory and LDS ---------------------------------------------------
 // `g` is 16-byte aligned; n floats; the last partial float4 (only at the very end of a tensor) goes scalar.
+// Loads are issued kRunBatch at a time before any of them is consumed, so their latencies overlap.
+constexpr int kRunBatch = 8;
+
 __device__ __forceinline__ void run_to_lds(const float *__restrict__ g, float *lds, int n)
 {
     const int n4 = n >> 2;
-    for (int i = threadIdx.x; i < n4; i += kWave)
-        reinterpret_cast<float4 *>(lds)[i] = reinterpret_cast<const float4 *>(g)[i];
+    for (int base = threadIdx.x; base < n4; base += kWave * kRunBatch) {
+        float4 v[kRunBatch];
+        // out-of-range slots re-read the last float4 of the run (always a valid address) and are not stored
+#pragma unroll
+        for (int u = 0; u < kRunBatch; ++u)
+            v[u] = reinterpret_cast<const float4 *>(g)[min(base + u * kWave, n4 - 1)];
+#pragma unroll
+        for (int u = 0; u < kRunBatch; ++u)
+            if (base + u * kWave < n4) reinterpret_cast<float4 *>(lds)[base + u * kWave] = v[u];
+    }
     const int tail = n4 * 4 + threadIdx.x;
     if (tail < n) lds[tail] = g[tail];
+}
+
+// Two runs at once (grad-weight: x and gy of the same planes): all loads of a batch of both runs fly together.
+__device__ __forceinline__ void runs_to_lds(const float *__restrict__ ga, float *la, int na,
+                                            const float *__restrict__ gb, float *lb, int nb)
+{
+    const int na4 = na >> 2, nb4 = nb >> 2;
+    const int nmax = na4 > nb4 ? na4 : nb4;
+    constexpr int U = kRunBatch / 2;
+    for (int base = threadIdx.x; base < nmax; base += kWave * U) {
+        float4 va[U], vb[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            va[u] = reinterpret_cast<const float4 *>(ga)[min(base + u * kWave, na4 - 1)];
+            vb[u] = reinterpret_cast<const float4 *>(gb)[min(base + u * kWave, nb4 - 1)];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (base + u * kWave < na4) reinterpret_cast<float4 *>(la)[base + u * kWave] = va[u];
+            if (base + u * kWave < nb4) reinterpret_cast<float4 *>(lb)[base + u * kWave] = vb[u];
+        }
+    }
+    const int ta = na4 * 4 + threadIdx.x, tb = nb4 * 4 + threadIdx.x;
+    if (ta < na) la[ta] = ga[ta];
+    if (tb < nb) lb[tb] = gb[tb];
 }
 
 __device__ __forceinline__ void lds_to_run(float *__restrict__ g, const float *lds, int n)
 {
     const int n4 = n >> 2;
-    for (int i = threadIdx.x; i < n4; i += kWave)
-        reinterpret_cast<float4 *>(g)[i] = reinterpret_cast<const float4 *>(lds)[i];
+    constexpr int U = 4;
+    for (int base = threadIdx.x; base < n4; base += kWave * U) {
+        float4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = reinterpret_cast<const float4 *>(lds)[min(base + u * kWave, n4 - 1)];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (base + u * kWave < n4) reinterpret_cast<float4 *>(g)[base + u * kWave] = v[u];
+    }
     const int tail = n4 * 4 + threadIdx.x;
     if (tail < n) g[tail] = lds[tail];
 }
@@ -380,8 +423,8 @@ __global__ __launch_bounds__(kWave) void small_wgrad_kernel(const SmallWgradPlan
     for (int n = n0; n < n1; ++n) {
         const long plane0 = static_cast<long>(n) * p.channel + c0;
         if (n != n0) __syncthreads();
-        run_to_lds(p.x + plane0 * in_plane, lds_x, nplanes * in_plane);
-        run_to_lds(p.gy + plane0 * out_plane, lds_g, nplanes * out_plane);
+        runs_to_lds(p.x + plane0 * in_plane, lds_x, nplanes * in_plane, p.gy + plane0 * out_plane, lds_g,
+                    nplanes * out_plane);
         __syncthreads();
 
         float g[BH][OW];

@@ -46,34 +46,53 @@ __device__ __forceinline__ int xcd_contiguous_tile(int bid, int n_tiles)
 }
 
 // Fills the LDS image of the tile: every float4 slot of every row is written,
-// with zeros where the row or the columns fall outside the plane.
+// with zeros where the row or the columns fall outside the plane.  A lane issues
+// the global loads of kStageBatch slots before it consumes any of them, so that
+// their latencies overlap instead of adding up.
+constexpr int kStageBatch = 4;
+
 __device__ __forceinline__ void stage_tile(const StageLayout &s, const float *__restrict__ in, float *lds,
                                            long plane0, int nplanes, int iy0)
 {
     const int total = nplanes * s.lds_rows * s.spr;
-    for (int slot = threadIdx.x; slot < total; slot += blockDim.x) {
-        const int rowidx = fast_div(slot, s.spr_magic);
-        const int sc = slot - rowidx * s.spr;
-        const int pl = fast_div(rowidx, s.lds_rows_magic);
-        const int r = rowidx - pl * s.lds_rows;
-        const int ix = 4 * (s.g_lo + sc);
-        const int iy = iy0 + r;
-        const bool row_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(s.in_h);
-        const float *src = in + (plane0 + pl) * s.in_plane + static_cast<long>(iy) * s.in_w + ix;
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (s.vec_in) {
-            if (row_ok && ix >= 0 && ix < s.in_w) v = *reinterpret_cast<const float4 *>(src);
-        } else if (row_ok) {
-            if (static_cast<unsigned>(ix + 0) < static_cast<unsigned>(s.in_w)) v.x = src[0];
-            if (static_cast<unsigned>(ix + 1) < static_cast<unsigned>(s.in_w)) v.y = src[1];
-            if (static_cast<unsigned>(ix + 2) < static_cast<unsigned>(s.in_w)) v.z = src[2];
-            if (static_cast<unsigned>(ix + 3) < static_cast<unsigned>(s.in_w)) v.w = src[3];
+    for (int base = threadIdx.x; base < total; base += blockDim.x * kStageBatch) {
+        float4 v[kStageBatch];
+        int dst[kStageBatch];
+#pragma unroll
+        for (int u = 0; u < kStageBatch; ++u) {
+            const int slot = base + u * blockDim.x;
+            v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+            dst[u] = -1;
+            if (slot < total) {
+                const int rowidx = fast_div(slot, s.spr_magic);
+                const int sc = slot - rowidx * s.spr;
+                const int pl = fast_div(rowidx, s.lds_rows_magic);
+                const int r = rowidx - pl * s.lds_rows;
+                const int ix = 4 * (s.g_lo + sc);
+                const int iy = iy0 + r;
+                const bool row_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(s.in_h);
+                const float *src = in + (plane0 + pl) * s.in_plane + static_cast<long>(iy) * s.in_w + ix;
+                if (s.vec_in) {
+                    if (row_ok && ix >= 0 && ix < s.in_w) v[u] = *reinterpret_cast<const float4 *>(src);
+                } else if (row_ok) {
+                    if (static_cast<unsigned>(ix + 0) < static_cast<unsigned>(s.in_w)) v[u].x = src[0];
+                    if (static_cast<unsigned>(ix + 1) < static_cast<unsigned>(s.in_w)) v[u].y = src[1];
+                    if (static_cast<unsigned>(ix + 2) < static_cast<unsigned>(s.in_w)) v[u].z = src[2];
+                    if (static_cast<unsigned>(ix + 3) < static_cast<unsigned>(s.in_w)) v[u].w = src[3];
+                }
+                dst[u] = pl * s.plane_pitch + r * s.pitch + kSlack + ix + s.col_shift;
+            }
         }
-        float *dst = lds + pl * s.plane_pitch + r * s.pitch + kSlack + ix + s.col_shift;
-        dst[0] = v.x;
-        dst[1] = v.y;
-        dst[2] = v.z;
-        dst[3] = v.w;
+#pragma unroll
+        for (int u = 0; u < kStageBatch; ++u) {
+            if (dst[u] >= 0) {
+                float *d = lds + dst[u];
+                d[0] = v[u].x;
+                d[1] = v[u].y;
+                d[2] = v[u].z;
+                d[3] = v[u].w;
+            }
+        }
     }
 }
 
