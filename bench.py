@@ -61,6 +61,8 @@ class Layer:
         self.ws = torch.empty(max(self.ws_bytes, 16), dtype=torch.uint8, device=dev)
         nx, ny, nw = n * c * h * w, n * c * oh * ow, c * k * k
         self.bytes = {"fwd": 4 * (nx + ny + nw), "gx": 4 * (ny + nx + nw), "gw": 4 * (nx + ny + nw)}
+        # the combined backward call is credited with the bytes of the two passes it replaces
+        self.bytes["bwd"] = self.bytes["gx"] + self.bytes["gw"]
         self.flops = 2 * ny * k * k
         # transposed-problem padding, torch_dwconv/dwconv.py:39-44
         self.g_pad = (k - p - 1, h - oh * s + p, k - p - 1, w - ow * s + p)
@@ -88,12 +90,22 @@ class Layer:
             n, c, h, w, oh, ow, k, k, 1, 1, s, s, p, p, stream))
 
 
-def schedule(layers):
+    def bwd(self, stream):
+        n, c, h, w, oh, ow, k, s, p = self.geom
+        self._check(self.lib.dwconv2d_backward_f32(
+            self.x.data_ptr(), self.gy.data_ptr(), self.w.data_ptr(), self.gx.data_ptr(), self.gw.data_ptr(),
+            self.ws.data_ptr(), self.ws_bytes, n, c, h, w, oh, ow, k, k, s, s, p, p, stream))
+
+
+def schedule(layers, separate_backward):
     """Training order: all forwards, then the backward passes last layer first."""
     calls = [(l, "fwd", l.fwd) for l in layers]
     for l in reversed(layers):
-        calls.append((l, "gx", l.bwd_input))
-        calls.append((l, "gw", l.bwd_filter))
+        if separate_backward:
+            calls.append((l, "gx", l.bwd_input))
+            calls.append((l, "gw", l.bwd_filter))
+        else:
+            calls.append((l, "bwd", l.bwd))
     return calls
 
 
@@ -160,6 +172,9 @@ def main():
     ap.add_argument("--batch", type=int, default=128)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-miopen", action="store_true")
+    ap.add_argument("--separate-backward", action="store_true",
+                    help="call grad-input and grad-weight as two entry points (36 calls per step) instead of the "
+                         "combined backward entry point (24 calls)")
     ap.add_argument("--table", action="store_true", help="print a per-layer, per-pass table to stderr")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB first (a kernel of known traffic, "
@@ -179,10 +194,10 @@ def main():
     shapes = WORKLOADS[args.workload](args.batch)
     gen = torch.Generator("cpu").manual_seed(0)
     layers = [Layer(s, lib, torch, dev, gen) for s in shapes]
-    calls = schedule(layers)
+    calls = schedule(layers, args.separate_backward)
     stream_obj = torch.cuda.current_stream(dev)
     stream = ctypes.c_void_p(stream_obj.cuda_stream)
-    step_bytes = sum(sum(l.bytes.values()) for l in layers)
+    step_bytes = sum(l.bytes["fwd"] + l.bytes["gx"] + l.bytes["gw"] for l in layers)
 
     def step():
         for _, _, fn in calls:
@@ -258,7 +273,8 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: {len(layers)} depthwise layers, fp32 NCHW, batch {shapes[0][0]}, "
-                               "fwd + grad-input + grad-weight per layer, training order",
+                               "fwd + grad-input + grad-weight per layer, training order, "
+                               f"{len(calls)} C-ABI calls per step",
                    "layers": [l.name for l in layers], "algorithmic_bytes_per_step": step_bytes},
         "frac_of_hbm_roofline": round(step_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, 4),
         "host_wall_ms_per_step": round(wall_ms, 4),
@@ -268,7 +284,8 @@ def main():
     if args.table:
         for r in rows:
             print(f"{r['layer']:>18} {r['pass']:>3} {r['us']:9.1f} us {r['GBs']:8.1f} GB/s  {r['variant']}", file=sys.stderr)
-    result["per_pass_us"] = {k: round(sum(r["us"] for r in rows if r["pass"] == k), 1) for k in ("fwd", "gx", "gw")}
+    result["per_pass_us"] = {k: round(sum(r["us"] for r in rows if r["pass"] == k), 1)
+                             for k in ("fwd", "gx", "gw", "bwd") if any(r["pass"] == k for r in rows)}
     if not args.no_miopen:
         try:
             per_layer = miopen_native(layers, torch)

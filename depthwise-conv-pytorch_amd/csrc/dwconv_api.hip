@@ -208,6 +208,43 @@ int wgrad_any(const T *in, const T *gy, T *gw, void *ws, size_t ws_bytes, int ba
     return launch_wgrad_direct<T>(in, gy, gw, ws, ws_bytes, g, stream);
 }
 
+// Both gradients of one layer.  Fused kernels where they exist; otherwise the two separate passes.
+int backward_f32(const float *in, const float *gy, const float *taps, float *gx, float *gw, void *ws,
+                 size_t ws_bytes, int batch, int channel, int in_h, int in_w, int out_h, int out_w, int kernel_h,
+                 int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w, void *stream_)
+{
+    WgradGeometry g;
+    int rc = make_wgrad_geometry(g, in, gy, gw, batch, channel, in_h, in_w, out_h, out_w, kernel_h, kernel_w, 1, 1,
+                                 stride_h, stride_w, pad_h, pad_w);
+    if (rc != DWCONV_OK) return rc;
+    if (dwconv_out_size(in_h, 1, stride_h, pad_h, pad_h, kernel_h) != out_h ||
+        dwconv_out_size(in_w, 1, stride_w, pad_w, pad_w, kernel_w) != out_w)
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "out_grad extent %dx%d does not match the convolution geometry",
+                    out_h, out_w);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const bool has_work = 1ll * batch * channel * out_h * out_w > 0 && in_h > 0 && in_w > 0;
+    if (has_work && !force_generic()) {
+        if (taps == nullptr || gx == nullptr) return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");
+        rc = try_launch_bwd_small(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+        if (rc >= 0) return rc;
+    }
+    // grad-input as the transposed problem (torch_dwconv/dwconv.py:39-44, :61-64), then grad-weight
+    rc = dwconv2d_any<float>(gy, taps, gx, batch, channel, out_h, out_w, kernel_h, kernel_w, stride_h, stride_w, 1, 1,
+                             kernel_h - pad_h - 1, in_h - out_h * stride_h + pad_h, kernel_w - pad_w - 1,
+                             in_w - out_w * stride_w + pad_w, 0, stream_);
+    if (rc != DWCONV_OK) return rc;
+    char first[sizeof(g_variant)];
+    std::snprintf(first, sizeof(first), "%s", g_variant);
+    rc = wgrad_any<float>(in, gy, gw, ws, ws_bytes, batch, channel, in_h, in_w, out_h, out_w, kernel_h, kernel_w, 1, 1,
+                          stride_h, stride_w, pad_h, pad_w, stream_);
+    if (rc == DWCONV_OK) {
+        char second[sizeof(g_variant)];
+        std::snprintf(second, sizeof(second), "%s", g_variant);
+        note_variant("%.60s + %.60s", first, second);
+    }
+    return rc;
+}
+
 }  // namespace
 }  // namespace dwconv
 
@@ -300,6 +337,15 @@ int dwconv2d_backward_kernel_f64(const double *input, const double *out_grad, do
     return wgrad_any<double>(input, out_grad, kernel_grad, workspace, workspace_bytes, batch, channel,
                              in_h, in_w, out_h, out_w, kernel_h, kernel_w, up_h, up_w, down_h, down_w,
                              pad_h, pad_w, stream);
+}
+
+int dwconv2d_backward_f32(const float *input, const float *out_grad, const float *kernel, float *in_grad,
+                          float *kernel_grad, void *workspace, size_t workspace_bytes, int batch, int channel,
+                          int in_h, int in_w, int out_h, int out_w, int kernel_h, int kernel_w, int stride_h,
+                          int stride_w, int pad_h, int pad_w, void *stream)
+{
+    return backward_f32(input, out_grad, kernel, in_grad, kernel_grad, workspace, workspace_bytes, batch, channel,
+                        in_h, in_w, out_h, out_w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, stream);
 }
 
 }  // extern "C"

@@ -74,6 +74,9 @@ int try_launch_fir_small(const float *in, const float *taps, float *out, const G
 size_t wgrad_small_workspace(const WgradGeometry &g);  // 0 when the whole-plane kernel does not cover g
 int try_launch_wgrad_small(const float *in, const float *gy, float *gw, void *ws, size_t ws_bytes,
                            const WgradGeometry &g, hipStream_t stream);
+// Fused grad-weight + grad-input for the same maps (gy read once); same return convention.
+int try_launch_bwd_small(const float *in, const float *gy, const float *taps, float *gx, float *gw, void *ws,
+                         size_t ws_bytes, const WgradGeometry &g, hipStream_t stream);
 // Pass 2 shared by the fp32 grad-weight kernels: gw[c][tap] = sum over chunks of partial[c][chunk][tap].
 int launch_wgrad_final(const float *partial, float *gw, int channel, int taps, int chunks, hipStream_t stream);
 

@@ -1,0 +1,120 @@
+// Helpers shared by the whole-plane kernels for small feature maps: LDS rows of a
+// compile-time width and flat runs of planes between global memory and LDS.
+#pragma once
+
+#include "dwconv_tile_common.hpp"
+
+namespace dwconv {
+
+constexpr int kWave = 64;
+
+// ---- LDS rows -----------------------------------------------------------------------------
+template <int N>
+__device__ __forceinline__ void lds_load_row(const float *p, float (&r)[N])
+{
+    if constexpr (N % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < N / 4; ++i) {
+            const float4 v = reinterpret_cast<const float4 *>(p)[i];
+            r[4 * i] = v.x; r[4 * i + 1] = v.y; r[4 * i + 2] = v.z; r[4 * i + 3] = v.w;
+        }
+    } else if constexpr (N % 2 == 0) {
+#pragma unroll
+        for (int i = 0; i < N / 2; ++i) {
+            const float2 v = reinterpret_cast<const float2 *>(p)[i];
+            r[2 * i] = v.x; r[2 * i + 1] = v.y;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) r[i] = p[i];
+    }
+}
+
+template <int N>
+__device__ __forceinline__ void lds_store_row(float *p, const float *r)
+{
+    if constexpr (N % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < N / 4; ++i)
+            reinterpret_cast<float4 *>(p)[i] = make_float4(r[4 * i], r[4 * i + 1], r[4 * i + 2], r[4 * i + 3]);
+    } else if constexpr (N % 2 == 0) {
+#pragma unroll
+        for (int i = 0; i < N / 2; ++i) reinterpret_cast<float2 *>(p)[i] = make_float2(r[2 * i], r[2 * i + 1]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) p[i] = r[i];
+    }
+}
+
+// ---- flat runs between global memory and LDS ---------------------------------------------------
+// `g` is 16-byte aligned; n floats; the last partial float4 (only at the very end of a tensor) goes scalar.
+// Loads are issued kRunBatch at a time before any of them is consumed, so their latencies overlap.
+constexpr int kRunBatch = 8;
+
+__device__ __forceinline__ void run_to_lds(const float *__restrict__ g, float *lds, int n)
+{
+    const int n4 = n >> 2;
+    for (int base = threadIdx.x; base < n4; base += kWave * kRunBatch) {
+        float4 v[kRunBatch];
+        // out-of-range slots re-read the last float4 of the run (always a valid address) and are not stored
+#pragma unroll
+        for (int u = 0; u < kRunBatch; ++u)
+            v[u] = reinterpret_cast<const float4 *>(g)[min(base + u * kWave, n4 - 1)];
+#pragma unroll
+        for (int u = 0; u < kRunBatch; ++u)
+            if (base + u * kWave < n4) reinterpret_cast<float4 *>(lds)[base + u * kWave] = v[u];
+    }
+    const int tail = n4 * 4 + threadIdx.x;
+    if (tail < n) lds[tail] = g[tail];
+}
+
+// Two runs at once (grad-weight: x and gy of the same planes): all loads of a batch of both runs fly together.
+__device__ __forceinline__ void runs_to_lds(const float *__restrict__ ga, float *la, int na,
+                                            const float *__restrict__ gb, float *lb, int nb)
+{
+    const int na4 = na >> 2, nb4 = nb >> 2;
+    const int nmax = na4 > nb4 ? na4 : nb4;
+    constexpr int U = kRunBatch / 2;
+    for (int base = threadIdx.x; base < nmax; base += kWave * U) {
+        float4 va[U], vb[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            va[u] = reinterpret_cast<const float4 *>(ga)[min(base + u * kWave, na4 - 1)];
+            vb[u] = reinterpret_cast<const float4 *>(gb)[min(base + u * kWave, nb4 - 1)];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (base + u * kWave < na4) reinterpret_cast<float4 *>(la)[base + u * kWave] = va[u];
+            if (base + u * kWave < nb4) reinterpret_cast<float4 *>(lb)[base + u * kWave] = vb[u];
+        }
+    }
+    const int ta = na4 * 4 + threadIdx.x, tb = nb4 * 4 + threadIdx.x;
+    if (ta < na) la[ta] = ga[ta];
+    if (tb < nb) lb[tb] = gb[tb];
+}
+
+__device__ __forceinline__ void lds_to_run(float *__restrict__ g, const float *lds, int n)
+{
+    const int n4 = n >> 2;
+    constexpr int U = 4;
+    for (int base = threadIdx.x; base < n4; base += kWave * U) {
+        float4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = reinterpret_cast<const float4 *>(lds)[min(base + u * kWave, n4 - 1)];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (base + u * kWave < n4) reinterpret_cast<float4 *>(g)[base + u * kWave] = v[u];
+    }
+    const int tail = n4 * 4 + threadIdx.x;
+    if (tail < n) g[tail] = lds[tail];
+}
+
+// This lane's K*K taps straight from global memory (the lanes of one plane read the same addresses).
+template <int KK, bool FLIP>
+__device__ __forceinline__ void load_taps(const float *__restrict__ taps, int c, float (&t)[KK])
+{
+#pragma unroll
+    for (int i = 0; i < KK; ++i) t[i] = taps[c * KK + (FLIP ? KK - 1 - i : i)];
+}
+
+}  // namespace dwconv

@@ -142,6 +142,8 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
 // rotated filter g shifted by E (g'[t] = g[t-E]):
 //   out[2q + r] = sum_a in[q - m + r + a] * g'[r + 2a]      along each axis,
 // i.e. a stride-1 correlation per output parity r with every other tap.
+// A lane owns 2*BQ output rows x 4 output columns (BQ x 2 half-resolution positions), so that the
+// 128-bit stores of consecutive lanes are contiguous in memory.
 template <int K, int EY, int EX, int BQ>
 __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
 {
@@ -150,7 +152,7 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
     constexpr int KK = K * K;
     constexpr int KAY = (K + EY + 1) / 2, KAX = (K + EX + 1) / 2;
     constexpr int WIN_ROWS = BQ + KAY;
-    static_assert(KAX + 3 < 8, "column window must fit two float4s");
+    constexpr int NW = 2 * ((KAX + 2 + 1) / 2);  // floats of a row two half-resolution positions touch, as float2s
 
     const int tile = xcd_contiguous_tile(blockIdx.x, p.n_tiles);
     const int pg = tile / p.row_tiles, rt = tile - pg * p.row_tiles;
@@ -173,21 +175,21 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
 #pragma unroll
         for (int t = 0; t < KK; ++t) tapv[t] = lds[p.tap_base + pl * KK + t];
 
-        const float *base = lds + pl * p.st.plane_pitch + (rb * BQ) * p.st.pitch + kSlack + 4 * cb;
-        float acc[2 * BQ][8];
+        const float *base = lds + pl * p.st.plane_pitch + (rb * BQ) * p.st.pitch + kSlack + 2 * cb;
+        float acc[2 * BQ][4];
 #pragma unroll
         for (int b = 0; b < 2 * BQ; ++b)
 #pragma unroll
-            for (int o = 0; o < 8; ++o) acc[b][o] = 0.f;
+            for (int o = 0; o < 4; ++o) acc[b][o] = 0.f;
 
 #pragma unroll
         for (int wr = 0; wr < WIN_ROWS; ++wr) {
-            float win[8];
-            {
-                const float4 q0 = *reinterpret_cast<const float4 *>(base + wr * p.st.pitch);
-                const float4 q1 = *reinterpret_cast<const float4 *>(base + wr * p.st.pitch + 4);
-                win[0] = q0.x; win[1] = q0.y; win[2] = q0.z; win[3] = q0.w;
-                win[4] = q1.x; win[5] = q1.y; win[6] = q1.z; win[7] = q1.w;
+            float win[NW];
+#pragma unroll
+            for (int v = 0; v < NW / 2; ++v) {
+                const float2 q = *reinterpret_cast<const float2 *>(base + wr * p.st.pitch + 2 * v);
+                win[2 * v] = q.x;
+                win[2 * v + 1] = q.y;
             }
 #pragma unroll
             for (int bq = 0; bq < BQ; ++bq)
@@ -198,7 +200,7 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
                     const int fy = r + 2 * a - EY;
                     if (fy < 0 || fy >= K) continue;
 #pragma unroll
-                    for (int xq = 0; xq < 4; ++xq)
+                    for (int xq = 0; xq < 2; ++xq)
 #pragma unroll
                         for (int rx = 0; rx < 2; ++rx)
 #pragma unroll
@@ -211,7 +213,7 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
                 }
         }
 
-        const int ox = 8 * cb;
+        const int ox = 4 * cb;
         float *dst = p.out + (plane0 + pl) * p.out_plane + ox;
 #pragma unroll
         for (int b = 0; b < 2 * BQ; ++b) {
@@ -219,13 +221,10 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
             if (oy >= p.out_h) continue;
             float *row = dst + static_cast<long>(oy) * p.out_w;
             if (p.vec_out) {
-                if (ox < p.out_w)
-                    *reinterpret_cast<float4 *>(row) = make_float4(acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
-                if (ox + 4 < p.out_w)
-                    *reinterpret_cast<float4 *>(row + 4) = make_float4(acc[b][4], acc[b][5], acc[b][6], acc[b][7]);
+                *reinterpret_cast<float4 *>(row) = make_float4(acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
             } else {
 #pragma unroll
-                for (int o = 0; o < 8; ++o)
+                for (int o = 0; o < 4; ++o)
                     if (ox + o < p.out_w) row[o] = acc[b][o];
             }
         }
@@ -318,10 +317,11 @@ int launch_down_bh(TilePlan &p, hipStream_t stream)
 template <int K, int EY, int EX>
 int launch_up2(TilePlan &p, hipStream_t stream)
 {
-    constexpr int BQ = 2;
-    constexpr int KAY = (K + EY + 1) / 2;
-    p.ncb = ceil_div(p.out_w, 8);
-    const int used_cols = 4 * (p.ncb - 1) + 8;
+    constexpr int BQ = 4;
+    constexpr int KAY = (K + EY + 1) / 2, KAX = (K + EX + 1) / 2;
+    constexpr int NW = 2 * ((KAX + 2 + 1) / 2);
+    p.ncb = ceil_div(p.out_w, 4);
+    const int used_cols = 2 * (p.ncb - 1) + NW;
     auto rows_for = [](int units) { return units * BQ + KAY; };
     if (!plan_tiles(p, ceil_div(ceil_div(p.out_h, 2), BQ), BQ, used_cols, K * K, rows_for)) return -1;
     hipLaunchKernelGGL((fir_up2_kernel<K, EY, EX, BQ>), dim3(p.n_tiles), dim3(env_int("DWCONV_TILE_THREADS", kThreads)), lds_bytes(p, K * K), stream,

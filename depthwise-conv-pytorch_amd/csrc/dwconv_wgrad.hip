@@ -41,6 +41,7 @@ struct WgradPlan {
     int items_per_plane;
     unsigned ipp_magic;
     int vec_gy;
+    int strided;           // chunk k takes tiles k, k+chunks, ... instead of a contiguous range
 };
 
 template <int CTRL, int ROW_MASK, int BANK_MASK>
@@ -77,76 +78,81 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
     const int chunk = blockIdx.x - group * p.chunks;
     const int c0 = group * p.planes_per_tile;
     const int nplanes = min(p.planes_per_tile, p.channel - c0);
-    const int t_begin = chunk * p.tiles_per_chunk;
-    const int t_end = min(p.tiles_per_group, t_begin + p.tiles_per_chunk);
+    // Chunk k takes tiles k, k + chunks, k + 2*chunks, ...: at any moment the workgroups of the grid
+    // work on a narrow window of images, which keeps the DRAM pages they stream from open.
+    const int t_begin = p.strided ? chunk : chunk * p.tiles_per_chunk;
+    const int t_end = p.strided ? p.tiles_per_group : min(p.tiles_per_group, t_begin + p.tiles_per_chunk);
+    const int t_step = p.strided ? p.chunks : 1;
     const int n_items = nplanes * p.items_per_plane;
 
     float acc[KK];
 #pragma unroll
     for (int t = 0; t < KK; ++t) acc[t] = 0.f;
 
-    for (int tile = t_begin; tile < t_end; ++tile) {
+    // One item per lane (the planner guarantees n_items <= blockDim.x): its place in the tile is fixed.
+    const bool has_item = static_cast<int>(threadIdx.x) < n_items;
+    const int item = has_item ? threadIdx.x : 0;
+    const int pl = fast_div(item, p.ipp_magic);
+    const int rem = item - pl * p.items_per_plane;
+    const int rb = fast_div(rem, p.ncb_magic);
+    const int cb = rem - rb * p.ncb;
+    const int ox = 4 * cb;
+    const float *base = lds + pl * p.st.plane_pitch + (rb * BH * S) * p.st.pitch + kSlack + 4 * cb * S;
+
+    for (int tile = t_begin; tile < t_end; tile += t_step) {
         const int n = tile / p.row_tiles, rt = tile - n * p.row_tiles;
         const long plane0 = static_cast<long>(n) * p.channel + c0;
         const int oy0 = rt * p.rows_per_tile;
+
+        // this lane's block of gy (zero where it hangs over the edge of the plane); issued before the
+        // x band is staged so that both sets of loads are in flight together
+        float g[BH][4];
+        const float *gsrc = p.gy + (plane0 + pl) * p.out_plane + ox;
+#pragma unroll
+        for (int b = 0; b < BH; ++b) {
+            const int oy = oy0 + rb * BH + b;
+            const float *row = gsrc + static_cast<long>(oy) * p.out_w;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (has_item && oy < p.out_h) {
+                if (p.vec_gy) {
+                    v = *reinterpret_cast<const float4 *>(row);
+                } else {
+                    if (ox + 0 < p.out_w) v.x = row[0];
+                    if (ox + 1 < p.out_w) v.y = row[1];
+                    if (ox + 2 < p.out_w) v.z = row[2];
+                    if (ox + 3 < p.out_w) v.w = row[3];
+                }
+            }
+            g[b][0] = v.x;
+            g[b][1] = v.y;
+            g[b][2] = v.z;
+            g[b][3] = v.w;
+        }
 
         if (tile != t_begin) __syncthreads();  // the previous tile's window reads are done
         stage_tile(p.st, p.x, lds, plane0, nplanes, oy0 * S - p.pad_h);
         __syncthreads();
 
-        for (int item = threadIdx.x; item < n_items; item += blockDim.x) {
-            const int pl = fast_div(item, p.ipp_magic);
-            const int rem = item - pl * p.items_per_plane;
-            const int rb = fast_div(rem, p.ncb_magic);
-            const int cb = rem - rb * p.ncb;
-
-            // this lane's block of gy (zero where it hangs over the edge of the plane)
-            float g[BH][4];
-            const int ox = 4 * cb;
-            const float *gsrc = p.gy + (plane0 + pl) * p.out_plane + ox;
+#pragma unroll
+        for (int wr = 0; wr < WIN_ROWS; ++wr) {
+            float win[4 * NV];
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                const float4 q = *reinterpret_cast<const float4 *>(base + wr * p.st.pitch + 4 * v);
+                win[4 * v + 0] = q.x;
+                win[4 * v + 1] = q.y;
+                win[4 * v + 2] = q.z;
+                win[4 * v + 3] = q.w;
+            }
 #pragma unroll
             for (int b = 0; b < BH; ++b) {
-                const int oy = oy0 + rb * BH + b;
-                const float *row = gsrc + static_cast<long>(oy) * p.out_w;
-                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (oy < p.out_h) {
-                    if (p.vec_gy) {
-                        v = *reinterpret_cast<const float4 *>(row);
-                    } else {
-                        if (ox + 0 < p.out_w) v.x = row[0];
-                        if (ox + 1 < p.out_w) v.y = row[1];
-                        if (ox + 2 < p.out_w) v.z = row[2];
-                        if (ox + 3 < p.out_w) v.w = row[3];
-                    }
-                }
-                g[b][0] = v.x;
-                g[b][1] = v.y;
-                g[b][2] = v.z;
-                g[b][3] = v.w;
-            }
-
-            const float *base = lds + pl * p.st.plane_pitch + (rb * BH * S) * p.st.pitch + kSlack + 4 * cb * S;
+                const int ty = wr - b * S;
+                if (ty < 0 || ty >= K) continue;
 #pragma unroll
-            for (int wr = 0; wr < WIN_ROWS; ++wr) {
-                float win[4 * NV];
+                for (int tx = 0; tx < K; ++tx)
 #pragma unroll
-                for (int v = 0; v < NV; ++v) {
-                    const float4 q = *reinterpret_cast<const float4 *>(base + wr * p.st.pitch + 4 * v);
-                    win[4 * v + 0] = q.x;
-                    win[4 * v + 1] = q.y;
-                    win[4 * v + 2] = q.z;
-                    win[4 * v + 3] = q.w;
-                }
-#pragma unroll
-                for (int b = 0; b < BH; ++b) {
-                    const int ty = wr - b * S;
-                    if (ty < 0 || ty >= K) continue;
-#pragma unroll
-                    for (int tx = 0; tx < K; ++tx)
-#pragma unroll
-                        for (int o = 0; o < 4; ++o)
-                            acc[ty * K + tx] = fmaf(g[b][o], win[o * S + tx], acc[ty * K + tx]);
-                }
+                    for (int o = 0; o < 4; ++o)
+                        acc[ty * K + tx] = fmaf(g[b][o], win[o * S + tx], acc[ty * K + tx]);
             }
         }
     }
@@ -239,7 +245,7 @@ bool make_plan(WgradPlan &p, const WgradGeometry &g)
         if (tile_bytes(units_per_tile, planes_per_tile) > kLdsBudget) return false;
     } else {
         planes_per_tile = 1;
-        units_per_tile = 2 * kThreads / p.ncb;
+        units_per_tile = kThreads / p.ncb;
         if (units_per_tile < 1) units_per_tile = 1;
         if (units_per_tile > row_units) units_per_tile = row_units;
         while (units_per_tile > 1 && tile_bytes(units_per_tile, 1) > kLdsBudget) --units_per_tile;
@@ -252,7 +258,7 @@ bool make_plan(WgradPlan &p, const WgradGeometry &g)
     p.row_tiles = ceil_div(row_units, units_per_tile);
     if (!layout_rows(p.st, rows_for(units_per_tile), planes_per_tile)) return false;
     p.items_per_plane = units_per_tile * p.ncb;
-    if (planes_per_tile * p.items_per_plane >= 65536) return false;
+    if (planes_per_tile * p.items_per_plane > kThreads) return false;  // one item per lane
     p.ncb_magic = magic_u16(p.ncb);
     p.ipp_magic = magic_u16(p.items_per_plane);
     p.groups = ceil_div(g.channel, planes_per_tile);
@@ -345,6 +351,7 @@ struct Launcher {
         p.partial = static_cast<float *>(ws);
         p.st.vec_in = (g.in_w % 4 == 0) && aligned16(x);
         p.vec_gy = (g.out_w % 4 == 0) && aligned16(gy);
+        p.strided = env_int("DWCONV_WGRAD_STRIDED", 1);
         const size_t shmem = lds_bytes<K, S, BH>(p);
         hipLaunchKernelGGL((wgrad_tile_kernel<K, S, BH>), dim3(p.groups * p.chunks), dim3(kThreads), shmem, stream, p);
         rc = check_launch("wgrad_tile_kernel");

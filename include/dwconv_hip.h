@@ -131,6 +131,20 @@ int dwconv2d_backward_kernel_f64(const double *input, const double *out_grad,
                                  int down_h, int down_w, int pad_h, int pad_w,
                                  void *stream);
 
+/* Both gradients of one layer in one call: in_grad (batch*channel*in_h*in_w) and kernel_grad
+ * (channel*kernel_h*kernel_w), from the forward input, the output gradient and the taps.
+ * Stands for the two calls the reference's autograd Function makes in a row in its backward
+ * (torch_dwconv/dwconv.py:56-68: `_C.dwconv2d` in the backward direction with g_pad, then
+ * `_C.dwconv2d_backward_kernel`); the reference has no single function for it.  Results are
+ * the same as those two calls give; where a fused kernel covers the geometry out_grad is read
+ * from memory once instead of twice.  out_h/out_w must be the forward output extent for
+ * (stride, pad).  Workspace as for dwconv2d_backward_kernel_f32. */
+int dwconv2d_backward_f32(const float *input, const float *out_grad, const float *kernel,
+                          float *in_grad, float *kernel_grad, void *workspace,
+                          size_t workspace_bytes, int batch, int channel, int in_h, int in_w,
+                          int out_h, int out_w, int kernel_h, int kernel_w, int stride_h,
+                          int stride_w, int pad_h, int pad_w, void *stream);
+
 /* Tuning/diagnostic hook: name of the kernel variant the last successful call
  * on this thread launched (e.g. "tile_f32<k3,s1,v4>"), for benchmarks and tests. */
 const char *dwconv_last_variant(void);

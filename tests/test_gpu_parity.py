@@ -48,6 +48,20 @@ def run_three_passes(dw, x, w, gy, stride, padding):
     return y.detach(), gx, gw, v_fwd
 
 
+def run_separate_backward(x, w, gy, stride, padding):
+    """grad-input and grad-weight through the two entry points the reference's backward calls
+    (torch_dwconv/dwconv.py:56-68), not through the combined one."""
+    from torch_dwconv import _C
+    from torch_dwconv.dwconv import make_tuple
+
+    s, p = make_tuple(stride, 2), make_tuple(padding, 2)
+    kh, kw = w.shape[2:]
+    g_pad = (kh - p[0] - 1, x.shape[2] - gy.shape[2] * s[0] + p[0], kw - p[1] - 1, x.shape[3] - gy.shape[3] * s[1] + p[1])
+    gx = _C.dwconv2d(gy, w, s[0], s[1], 1, 1, *g_pad, False)
+    gw = _C.dwconv2d_backward_kernel(x, gy, w, 1, 1, s[0], s[1], p[0], p[1])
+    return gx, gw
+
+
 def assert_parity(y, gx, gw, y_ref, gx_ref, gw_ref, dtype):
     if dtype == torch.float32:
         tol = dict(rtol=1e-5, atol=1e-5)
@@ -71,6 +85,8 @@ def check_against_c_oracle(dw, gpu, shape, dtype=torch.float32, seed=0):
     gx_ref = oracle.grad_input(_np(gy), _np(wt), (h, w), s, p)
     gw_ref = oracle.grad_weight(_np(x), _np(gy), wt.shape, s, p)
     assert_parity(y, gx, gw, y_ref, gx_ref, gw_ref, dtype)
+    gx2, gw2 = run_separate_backward(x.to(gpu), wt.to(gpu), gy.to(gpu), s, p)
+    assert_parity(y, gx2, gw2, y_ref, gx_ref, gw_ref, dtype)
     return variant
 
 
@@ -85,6 +101,10 @@ SMALL = [
     (2, 3, 112, 112, 3, 1, 1), (2, 3, 112, 112, 3, 2, 1), (1, 2, 128, 96, 5, 2, 2), (1, 2, 256, 256, 5, 1, 2),
     (1, 1, 1, 1, 3, 1, 1), (1, 1, 3, 300, 3, 1, 1), (1, 1, 300, 3, 5, 2, 2), (1, 2, 40, 1000, 7, 2, 3),
     (2, 3, 57, 59, 7, 2, 3), (2, 3, 58, 60, 5, 2, 1), (2, 3, 61, 64, 3, 2, 0), (1, 3, 64, 64, 7, 1, 0),
+    # whole-plane kernels with ragged channel groups, several images per chunk, odd plane sizes
+    (3, 12, 7, 7, 5, 1, 2), (5, 20, 7, 7, 3, 1, 1), (3, 8, 7, 7, 7, 1, 3), (2, 13, 14, 14, 3, 1, 1),
+    (3, 10, 14, 14, 5, 2, 2), (5, 11, 28, 28, 3, 2, 1), (3, 6, 28, 28, 5, 1, 2), (2, 4, 28, 28, 7, 2, 3),
+    (2, 70, 14, 14, 7, 1, 3), (2, 68, 7, 7, 5, 1, 2), (2, 3, 20, 14, 3, 1, 1), (2, 4, 10, 7, 5, 1, 2),
 ]
 
 
@@ -159,8 +179,8 @@ def check_full_size(dw, gpu, shape, seed=0, n_planes=6, n_channels=3):
     _announce(shape_id(shape), variant)
     rng = np.random.default_rng(seed + 1)
     yc, gxc = y.cpu(), gx.cpu()
-    for _ in range(n_planes):
-        b, ch = int(rng.integers(n)), int(rng.integers(c))
+    sampled = [(int(rng.integers(n)), int(rng.integers(c))) for _ in range(n_planes)]
+    for b, ch in sampled:
         xs, ws, gs = _np(x[b:b + 1, ch:ch + 1]), _np(wt[ch:ch + 1]), _np(gy[b:b + 1, ch:ch + 1])
         np.testing.assert_allclose(_np(yc[b, ch]).astype(np.float64), oracle.forward(xs, ws, s, p)[0, 0], rtol=1e-5, atol=1e-5)
         np.testing.assert_allclose(_np(gxc[b, ch]).astype(np.float64), oracle.grad_input(gs, ws, (h, w), s, p)[0, 0], rtol=1e-5, atol=1e-5)
@@ -177,6 +197,15 @@ def check_full_size(dw, gpu, shape, seed=0, n_planes=6, n_channels=3):
     # bit-identical grad-weight on a second run
     _, _, gw2, _ = run_three_passes(dw, xg, wg, gg, s, p)
     assert torch.equal(gw, gw2)
+    # the two separate backward entry points agree with the oracle as well, and are deterministic too
+    gx3, gw3 = run_separate_backward(xg, wg, gg, s, p)
+    gx3c = gx3.cpu()
+    for b, ch in sampled:
+        gs, ws = _np(gy[b:b + 1, ch:ch + 1]), _np(wt[ch:ch + 1])
+        np.testing.assert_allclose(_np(gx3c[b, ch]).astype(np.float64), oracle.grad_input(gs, ws, (h, w), s, p)[0, 0], rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(_np(gw3[chans]).astype(np.float64), gw_ref, rtol=1e-4, atol=atol)
+    _, gw4 = run_separate_backward(xg, wg, gg, s, p)
+    assert torch.equal(gw3, gw4)
 
 
 def test_cfg1_whole_tensor(dw, gpu):
