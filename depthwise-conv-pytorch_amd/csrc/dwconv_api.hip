@@ -227,6 +227,8 @@ int backward_f32(const float *in, const float *gy, const float *taps, float *gx,
         if (taps == nullptr || gx == nullptr) return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");
         rc = try_launch_bwd_small(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
         if (rc >= 0) return rc;
+        rc = try_launch_bwd_tiled(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+        if (rc >= 0) return rc;
     }
     // grad-input as the transposed problem (torch_dwconv/dwconv.py:39-44, :61-64), then grad-weight
     rc = dwconv2d_any<float>(gy, taps, gx, batch, channel, out_h, out_w, kernel_h, kernel_w, stride_h, stride_w, 1, 1,

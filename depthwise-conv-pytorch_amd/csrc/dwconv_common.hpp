@@ -85,4 +85,8 @@ size_t wgrad_tiled_workspace(const WgradGeometry &g);  // 0 when the tiled kerne
 int try_launch_wgrad_tiled(const float *in, const float *gy, float *gw, void *ws, size_t ws_bytes,
                            const WgradGeometry &g, hipStream_t stream);
 
+// Fused grad-weight + grad-input with LDS tiles (stride 1, "same" padding); same return convention.
+int try_launch_bwd_tiled(const float *in, const float *gy, const float *taps, float *gx, float *gw, void *ws,
+                         size_t ws_bytes, const WgradGeometry &g, hipStream_t stream);
+
 }  // namespace dwconv

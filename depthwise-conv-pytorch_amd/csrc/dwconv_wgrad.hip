@@ -41,6 +41,11 @@ struct WgradPlan {
     int items_per_plane;
     unsigned ipp_magic;
     int vec_gy;
+    // fused grad-input (stride 1, "same" padding): taps, destination, and where the gy image sits in LDS
+    const float *taps;
+    float *gx;
+    int g_base;            // float offset of the gy image (same layout as the x image)
+    int vec_gx;
     int strided;           // chunk k takes tiles k, k+chunks, ... instead of a contiguous range
 };
 
@@ -65,7 +70,11 @@ __device__ __forceinline__ float wave_sum_to_last_lane(float v)
 
 constexpr int kRedPitch = kThreads + 1;  // odd pitch: lanes of one wave reading one column spread over the banks
 
-template <int K, int S, int BH>
+// GX (stride 1, pad = K/2 only): the band of gy is staged in LDS next to the band of x, with the same
+// layout.  The lane first walks its gy window: that gives its block of grad-input (gy against the
+// rotated taps, stored straight to memory) and, from the window's centre, its block of gy for the
+// grad-weight sums.  gy is read from HBM once for both gradients.
+template <int K, int S, int BH, bool GX>
 __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -73,6 +82,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
     constexpr int KK = K * K;
     constexpr int WIN_ROWS = (BH - 1) * S + K;
     constexpr int NV = (3 * S + K + 3) / 4;
+    static_assert(!GX || S == 1, "the fused variant is the stride-1 one");
 
     const int group = blockIdx.x / p.chunks;
     const int chunk = blockIdx.x - group * p.chunks;
@@ -99,6 +109,12 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
     const int ox = 4 * cb;
     const float *base = lds + pl * p.st.plane_pitch + (rb * BH * S) * p.st.pitch + kSlack + 4 * cb * S;
 
+    float rot[GX ? KK : 1];
+    if constexpr (GX) {
+#pragma unroll
+        for (int t = 0; t < KK; ++t) rot[t] = p.taps[(c0 + pl) * KK + KK - 1 - t];
+    }
+
     for (int tile = t_begin; tile < t_end; tile += t_step) {
         const int n = tile / p.row_tiles, rt = tile - n * p.row_tiles;
         const long plane0 = static_cast<long>(n) * p.channel + c0;
@@ -110,6 +126,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
         const float *gsrc = p.gy + (plane0 + pl) * p.out_plane + ox;
 #pragma unroll
         for (int b = 0; b < BH; ++b) {
+            if constexpr (GX) break;
             const int oy = oy0 + rb * BH + b;
             const float *row = gsrc + static_cast<long>(oy) * p.out_w;
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -131,7 +148,59 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
 
         if (tile != t_begin) __syncthreads();  // the previous tile's window reads are done
         stage_tile(p.st, p.x, lds, plane0, nplanes, oy0 * S - p.pad_h);
+        if constexpr (GX) stage_tile(p.st, p.gy, lds + p.g_base, plane0, nplanes, oy0 - p.pad_h);
         __syncthreads();
+
+        if constexpr (GX) {
+            constexpr int PC = K / 2;  // the lane's own gy block sits PC rows and columns into its window
+            float xacc[BH][4];
+#pragma unroll
+            for (int b = 0; b < BH; ++b)
+#pragma unroll
+                for (int o = 0; o < 4; ++o) xacc[b][o] = 0.f;
+#pragma unroll
+            for (int wr = 0; wr < WIN_ROWS; ++wr) {
+                float win[4 * NV];
+#pragma unroll
+                for (int v = 0; v < NV; ++v) {
+                    const float4 q = *reinterpret_cast<const float4 *>(base + p.g_base + wr * p.st.pitch + 4 * v);
+                    win[4 * v + 0] = q.x;
+                    win[4 * v + 1] = q.y;
+                    win[4 * v + 2] = q.z;
+                    win[4 * v + 3] = q.w;
+                }
+                const int gb = wr - PC;
+                if (gb >= 0 && gb < BH) {
+#pragma unroll
+                    for (int o = 0; o < 4; ++o) g[gb >= 0 && gb < BH ? gb : 0][o] = has_item ? win[o + PC] : 0.f;
+                }
+#pragma unroll
+                for (int b = 0; b < BH; ++b) {
+                    const int ty = wr - b;
+                    if (ty < 0 || ty >= K) continue;
+#pragma unroll
+                    for (int tx = 0; tx < K; ++tx)
+#pragma unroll
+                        for (int o = 0; o < 4; ++o) xacc[b][o] = fmaf(win[o + tx], rot[ty * K + tx], xacc[b][o]);
+                }
+            }
+            if (has_item) {
+                float *dst = p.gx + (plane0 + pl) * p.st.in_plane + ox;
+#pragma unroll
+                for (int b = 0; b < BH; ++b) {
+                    const int oy = oy0 + rb * BH + b;
+                    if (oy >= p.st.in_h) continue;
+                    float *row = dst + static_cast<long>(oy) * p.st.in_w;
+                    if (p.vec_gx) {
+                        *reinterpret_cast<float4 *>(row) = make_float4(xacc[b][0], xacc[b][1], xacc[b][2], xacc[b][3]);
+                    } else {
+#pragma unroll
+                        for (int o = 0; o < 4; ++o)
+                            if (ox + o < p.st.in_w) row[o] = xacc[b][o];
+                    }
+                }
+            }
+        }
 
 #pragma unroll
         for (int wr = 0; wr < WIN_ROWS; ++wr) {
@@ -211,7 +280,7 @@ __global__ void wgrad_tile_final_kernel(const float *__restrict__ partial, float
 }
 
 template <int K, int S, int BH>
-bool make_plan(WgradPlan &p, const WgradGeometry &g)
+bool make_plan(WgradPlan &p, const WgradGeometry &g, bool fused)
 {
     constexpr int NV = (3 * S + K + 3) / 4;
     constexpr int KK = K * K;
@@ -231,7 +300,7 @@ bool make_plan(WgradPlan &p, const WgradGeometry &g)
     layout_columns(p.st, used_cols);
     auto rows_for = [](int units) { return (units * BH - 1) * S + K; };
     auto tile_bytes = [&](int units, int planes) {
-        return static_cast<long>(planes) * rows_for(units) * p.st.pitch * 4;
+        return static_cast<long>(planes) * rows_for(units) * p.st.pitch * 4 * (fused ? 2 : 1);
     };
     const int row_units = ceil_div(g.out_h, BH);
     const int ipp_full = row_units * p.ncb;
@@ -257,6 +326,7 @@ bool make_plan(WgradPlan &p, const WgradGeometry &g)
     p.rows_per_tile = units_per_tile * BH;
     p.row_tiles = ceil_div(row_units, units_per_tile);
     if (!layout_rows(p.st, rows_for(units_per_tile), planes_per_tile)) return false;
+    p.g_base = planes_per_tile * p.st.plane_pitch;
     p.items_per_plane = units_per_tile * p.ncb;
     if (planes_per_tile * p.items_per_plane > kThreads) return false;  // one item per lane
     p.ncb_magic = magic_u16(p.ncb);
@@ -276,9 +346,9 @@ bool make_plan(WgradPlan &p, const WgradGeometry &g)
 }
 
 template <int K, int S, int BH>
-size_t lds_bytes(const WgradPlan &p)
+size_t lds_bytes(const WgradPlan &p, bool fused)
 {
-    const size_t tile = static_cast<size_t>(p.planes_per_tile) * p.st.plane_pitch * 4;
+    const size_t tile = static_cast<size_t>(p.planes_per_tile) * p.st.plane_pitch * 4 * (fused ? 2 : 1);
     const size_t red = p.planes_per_tile == 1 ? static_cast<size_t>(kThreads / 64) * K * K * 4
                                               : static_cast<size_t>(K) * K * kRedPitch * 4;
     return tile > red ? tile : red;
@@ -321,9 +391,12 @@ struct WorkspaceQuery {
     template <int K, int S, int BH>
     void operator()()
     {
-        WgradPlan p{};
-        if (make_plan<K, S, BH>(p, g))
-            bytes = static_cast<size_t>(p.groups) * p.planes_per_tile * p.chunks * K * K * sizeof(float);
+        for (int fused = 0; fused < 2; ++fused) {
+            WgradPlan p{};
+            if (!make_plan<K, S, BH>(p, g, fused != 0)) continue;
+            const size_t need = static_cast<size_t>(p.groups) * p.planes_per_tile * p.chunks * K * K * sizeof(float);
+            if (need > bytes) bytes = need;
+        }
     }
 };
 
@@ -335,12 +408,16 @@ struct Launcher {
     size_t ws_bytes;
     const WgradGeometry &g;
     hipStream_t stream;
+    const float *taps = nullptr;  // with gx: also produce grad-input (stride 1, "same" padding)
+    float *gx = nullptr;
     int rc = -1;
     template <int K, int S, int BH>
     void operator()()
     {
+        const bool fused = gx != nullptr;
+        if (fused && S != 1) return;
         WgradPlan p{};
-        if (!make_plan<K, S, BH>(p, g)) return;
+        if (!make_plan<K, S, BH>(p, g, fused)) return;
         const size_t need = static_cast<size_t>(p.groups) * p.planes_per_tile * p.chunks * K * K * sizeof(float);
         if (ws == nullptr || ws_bytes < need) {
             rc = fail(DWCONV_ERR_WORKSPACE, "grad-weight needs a workspace of %zu bytes, got %zu", need, ws_bytes);
@@ -352,12 +429,25 @@ struct Launcher {
         p.st.vec_in = (g.in_w % 4 == 0) && aligned16(x);
         p.vec_gy = (g.out_w % 4 == 0) && aligned16(gy);
         p.strided = env_int("DWCONV_WGRAD_STRIDED", 1);
-        const size_t shmem = lds_bytes<K, S, BH>(p);
-        hipLaunchKernelGGL((wgrad_tile_kernel<K, S, BH>), dim3(p.groups * p.chunks), dim3(kThreads), shmem, stream, p);
+        p.taps = taps;
+        p.gx = gx;
+        p.vec_gx = (g.in_w % 4 == 0) && aligned16(gx);
+        const size_t shmem = lds_bytes<K, S, BH>(p, fused);
+        if constexpr (S == 1) {
+            if (fused) {
+                // the gy image is staged with the x image's layout: it needs the same 128-bit rule
+                p.st.vec_in = p.st.vec_in && aligned16(gy);
+                hipLaunchKernelGGL((wgrad_tile_kernel<K, S, BH, true>), dim3(p.groups * p.chunks), dim3(kThreads), shmem,
+                                   stream, p);
+            }
+        }
+        if (!fused)
+            hipLaunchKernelGGL((wgrad_tile_kernel<K, S, BH, false>), dim3(p.groups * p.chunks), dim3(kThreads), shmem,
+                               stream, p);
         rc = check_launch("wgrad_tile_kernel");
         if (rc != DWCONV_OK) return;
-        note_variant("wgrad_tile<k%d,s%d,bh%d> P%d rows%d chunks%d vin%d vgy%d", K, S, BH, p.planes_per_tile,
-                     p.rows_per_tile, p.chunks, p.st.vec_in, p.vec_gy);
+        note_variant("%s<k%d,s%d,bh%d> P%d rows%d chunks%d vin%d vgy%d", fused ? "bwd_tile" : "wgrad_tile", K, S, BH,
+                     p.planes_per_tile, p.rows_per_tile, p.chunks, p.st.vec_in, p.vec_gy);
         rc = launch_wgrad_final(static_cast<const float *>(ws), gw, g.channel, K * K, p.chunks, stream);
     }
 };
@@ -383,6 +473,20 @@ int try_launch_wgrad_tiled(const float *in, const float *gy, float *gw, void *ws
                            const WgradGeometry &g, hipStream_t stream)
 {
     Launcher l{in, gy, gw, ws, ws_bytes, g, stream};
+    if (!dispatch(g, l)) return -1;
+    return l.rc;
+}
+
+int try_launch_bwd_tiled(const float *in, const float *gy, const float *taps, float *gx, float *gw, void *ws,
+                         size_t ws_bytes, const WgradGeometry &g, hipStream_t stream)
+{
+    if (env_int("DWCONV_NO_FUSED_TILE", 0)) return -1;
+    const int K = g.kernel_h;
+    // stride 1 and "same" padding: the gradient planes have the input's extent and the gy band can share
+    // the x band's LDS layout
+    if (g.down_h != 1 || g.down_w != 1 || g.kernel_w != K || g.pad_h != K / 2 || g.pad_w != K / 2) return -1;
+    if (g.out_h != g.in_h || g.out_w != g.in_w) return -1;
+    Launcher l{in, gy, gw, ws, ws_bytes, g, stream, taps, gx};
     if (!dispatch(g, l)) return -1;
     return l.rc;
 }
