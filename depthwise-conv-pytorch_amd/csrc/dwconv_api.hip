@@ -168,6 +168,8 @@ size_t wgrad_workspace(const WgradGeometry &g)
         if (t > need) need = t;
         const size_t sm = wgrad_small_workspace(g);
         if (sm > need) need = sm;
+        const size_t s2 = bwd_s2_workspace(g);
+        if (s2 > need) need = s2;
     }
     return need;
 }
@@ -228,6 +230,8 @@ int backward_f32(const float *in, const float *gy, const float *taps, float *gx,
         rc = try_launch_bwd_small(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
         if (rc >= 0) return rc;
         rc = try_launch_bwd_tiled(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+        if (rc >= 0) return rc;
+        rc = try_launch_bwd_s2(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
         if (rc >= 0) return rc;
     }
     // grad-input as the transposed problem (torch_dwconv/dwconv.py:39-44, :61-64), then grad-weight

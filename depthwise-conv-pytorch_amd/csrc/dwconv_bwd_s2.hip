@@ -1,0 +1,329 @@
+// Fused backward pass (grad-weight + grad-input) for stride-2 layers on large maps, fp32.
+//
+// Workgroup (channel c, chunk k) walks tiles (image n, band of rows).  Per tile two images are staged
+// in LDS: the band of x the grad-weight sums need, and the (four times smaller) band of gy.  A lane
+// owns BQ x 2 elements of gy:
+//   grad-input : out[2q + r] = sum_a gy[q - m + r + a] * rot'[r + 2a] along each axis (the zero-stuffed
+//                gradient never exists); the lane's 2*BQ x 4 block of gx goes straight to memory
+//                with 128-bit stores that are contiguous across lanes;
+//   grad-weight: its gy elements (the centre of the window it just walked) against the x window
+//                they touch, accumulated in K*K registers for the whole chunk, then reduced in a fixed
+//                order exactly like the stride-1 kernel (DPP within a wavefront, LDS across
+//                wavefronts) into partial[c][k][tap].
+// gy is read from HBM once for both gradients; the reference reads it twice
+// (torch_dwconv/dwconv.py:56-68) and x K*K times (torch_dwconv/dwconv_kernel.cu:260-306).
+#include "dwconv_tile_common.hpp"
+
+namespace dwconv {
+
+namespace {
+
+constexpr int kBq = 4;                        // half-resolution rows per lane
+constexpr int kFusedLdsBudget = 36 * 1024;    // both images of a tile
+
+struct BwdS2Plan {
+    StageLayout sx;   // x image: row r holds x row 2*q0 - pad + r, column c holds x column c - pad
+    StageLayout sg;   // gy image: row r holds gy row q0 - m + r, column c holds gy column c - m
+    const float *x;
+    const float *gy;
+    const float *taps;
+    float *gx;
+    float *partial;
+    int channel;
+    int pad;          // forward padding (both axes)
+    int m;            // (K - 1 - pad + E) / 2
+    int g_base;       // float offset of the gy image in LDS
+    int rows_per_tile;  // half-resolution rows per tile
+    int row_tiles;
+    int tiles_per_group, chunks;
+    int ncb;
+    unsigned ncb_magic;
+    int n_items;
+    int vec_gx;
+};
+
+template <int CTRL, int ROW_MASK, int BANK_MASK>
+__device__ __forceinline__ float dpp_add(float v)
+{
+    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, BANK_MASK, true);
+    return v + __int_as_float(moved);
+}
+
+// Sum of the 64 lanes, delivered in lane 63; fixed association order.
+__device__ __forceinline__ float wave_sum_to_last_lane(float v)
+{
+    v = dpp_add<0x111, 0xf, 0xf>(v);  // row_shr:1
+    v = dpp_add<0x112, 0xf, 0xf>(v);  // row_shr:2
+    v = dpp_add<0x114, 0xf, 0xf>(v);  // row_shr:4
+    v = dpp_add<0x118, 0xf, 0xf>(v);  // row_shr:8
+    v = dpp_add<0x142, 0xa, 0xf>(v);  // row_bcast:15 into rows 1 and 3
+    v = dpp_add<0x143, 0xc, 0xf>(v);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+// E = parity of the transposed problem's leading pad K - 1 - pad (the same on both axes).
+template <int K, int E>
+__global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
+{
+    extern __shared__ float4 lds_raw[];
+    float *lds = reinterpret_cast<float *>(lds_raw);
+    constexpr int KK = K * K;
+    constexpr int BQ = kBq;
+    constexpr int KA = (K + E + 1) / 2;
+    constexpr int GW_ROWS = BQ + KA;                  // gy window rows
+    constexpr int NWG = 2 * ((KA + 2 + 1) / 2);       // gy window columns, as float2s
+    constexpr int XW_ROWS = (BQ - 1) * 2 + K;         // x window rows
+    constexpr int NVX = (K + 2 + 3) / 4;              // x window columns, as float4s
+
+    const int c = blockIdx.x / p.chunks;
+    const int chunk = blockIdx.x - c * p.chunks;
+
+    const bool has_item = static_cast<int>(threadIdx.x) < p.n_items;
+    const int item = has_item ? threadIdx.x : 0;
+    const int rb = fast_div(item, p.ncb_magic);
+    const int cb = item - rb * p.ncb;
+    const float *base_x = lds + (rb * BQ * 2) * p.sx.pitch + kSlack + 4 * cb;
+    const float *base_g = lds + p.g_base + (rb * BQ) * p.sg.pitch + kSlack + 2 * cb;
+
+    float rot[KK];
+#pragma unroll
+    for (int t = 0; t < KK; ++t) rot[t] = p.taps[c * KK + KK - 1 - t];
+    float wacc[KK];
+#pragma unroll
+    for (int t = 0; t < KK; ++t) wacc[t] = 0.f;
+
+    for (int tile = chunk; tile < p.tiles_per_group; tile += p.chunks) {
+        const int n = tile / p.row_tiles, rt = tile - n * p.row_tiles;
+        const long plane0 = static_cast<long>(n) * p.channel + c;
+        const int q0 = rt * p.rows_per_tile;
+
+        if (tile != chunk) __syncthreads();  // the previous tile's window reads are done
+        stage_tile(p.sx, p.x, lds, plane0, 1, 2 * q0 - p.pad);
+        stage_tile(p.sg, p.gy, lds + p.g_base, plane0, 1, q0 - p.m);
+        __syncthreads();
+
+        // ---- gy window: grad-input block, and this lane's gy elements from the window's centre
+        float g[BQ][2];
+        float xacc[2 * BQ][4];
+#pragma unroll
+        for (int b = 0; b < 2 * BQ; ++b)
+#pragma unroll
+            for (int o = 0; o < 4; ++o) xacc[b][o] = 0.f;
+#pragma unroll
+        for (int wr = 0; wr < GW_ROWS; ++wr) {
+            float win[NWG];
+#pragma unroll
+            for (int v = 0; v < NWG / 2; ++v) {
+                const float2 q = *reinterpret_cast<const float2 *>(base_g + wr * p.sg.pitch + 2 * v);
+                win[2 * v] = q.x;
+                win[2 * v + 1] = q.y;
+            }
+            if (wr >= p.m && wr - p.m < BQ) {
+                // the centre row index depends on m (1 or 2 for the kernels served here): select at run time
+#pragma unroll
+                for (int bq = 0; bq < BQ; ++bq)
+                    if (wr - p.m == bq) {
+                        g[bq][0] = has_item ? (p.m == 1 ? win[1] : (p.m == 2 ? win[2] : win[0])) : 0.f;
+                        g[bq][1] = has_item ? (p.m == 1 ? win[2] : (p.m == 2 ? win[3] : win[1])) : 0.f;
+                    }
+            }
+#pragma unroll
+            for (int bq = 0; bq < BQ; ++bq)
+#pragma unroll
+                for (int r = 0; r < 2; ++r) {
+                    const int a = wr - bq - r;
+                    if (a < 0 || a >= KA) continue;
+                    const int fy = r + 2 * a - E;
+                    if (fy < 0 || fy >= K) continue;
+#pragma unroll
+                    for (int xq = 0; xq < 2; ++xq)
+#pragma unroll
+                        for (int rx = 0; rx < 2; ++rx)
+#pragma unroll
+                            for (int ax = 0; ax < KA; ++ax) {
+                                const int fx = rx + 2 * ax - E;
+                                if (fx < 0 || fx >= K) continue;
+                                xacc[2 * bq + r][2 * xq + rx] =
+                                    fmaf(win[xq + rx + ax], rot[fy * K + fx], xacc[2 * bq + r][2 * xq + rx]);
+                            }
+                }
+        }
+        if (has_item) {
+            const int ox = 4 * cb;
+            float *dst = p.gx + plane0 * p.sx.in_plane + ox;
+#pragma unroll
+            for (int b = 0; b < 2 * BQ; ++b) {
+                const int oy = 2 * (q0 + rb * BQ) + b;
+                if (oy >= p.sx.in_h) continue;
+                float *row = dst + static_cast<long>(oy) * p.sx.in_w;
+                if (p.vec_gx) {
+                    if (ox < p.sx.in_w)
+                        *reinterpret_cast<float4 *>(row) = make_float4(xacc[b][0], xacc[b][1], xacc[b][2], xacc[b][3]);
+                } else {
+#pragma unroll
+                    for (int o = 0; o < 4; ++o)
+                        if (ox + o < p.sx.in_w) row[o] = xacc[b][o];
+                }
+            }
+        }
+
+        // ---- x window: grad-weight sums
+#pragma unroll
+        for (int wr = 0; wr < XW_ROWS; ++wr) {
+            float win[4 * NVX];
+#pragma unroll
+            for (int v = 0; v < NVX; ++v) {
+                const float4 q = *reinterpret_cast<const float4 *>(base_x + wr * p.sx.pitch + 4 * v);
+                win[4 * v + 0] = q.x;
+                win[4 * v + 1] = q.y;
+                win[4 * v + 2] = q.z;
+                win[4 * v + 3] = q.w;
+            }
+#pragma unroll
+            for (int bq = 0; bq < BQ; ++bq) {
+                const int ty = wr - 2 * bq;
+                if (ty < 0 || ty >= K) continue;
+#pragma unroll
+                for (int tx = 0; tx < K; ++tx)
+#pragma unroll
+                    for (int o = 0; o < 2; ++o) wacc[ty * K + tx] = fmaf(g[bq][o], win[2 * o + tx], wacc[ty * K + tx]);
+            }
+        }
+    }
+
+    __syncthreads();  // the images are dead; their LDS is reused for the reduction
+#pragma unroll
+    for (int t = 0; t < KK; ++t) {
+        const float s = wave_sum_to_last_lane(wacc[t]);
+        if ((threadIdx.x & 63) == 63) lds[(threadIdx.x >> 6) * KK + t] = s;
+    }
+    __syncthreads();
+    if (threadIdx.x < KK) {
+        float s = lds[threadIdx.x];
+#pragma unroll
+        for (int w = 1; w < kThreads / 64; ++w) s += lds[w * KK + threadIdx.x];
+        p.partial[(static_cast<long>(c) * p.chunks + chunk) * KK + threadIdx.x] = s;
+    }
+}
+
+template <int K>
+bool plan_bwd_s2(BwdS2Plan &p, const WgradGeometry &g)
+{
+    const int pad0 = K - 1 - g.pad_h;  // leading pad of the transposed problem
+    const int E = pad0 & 1;
+    const int KA = (K + E + 1) / 2;
+    const int NWG = 2 * ((KA + 2 + 1) / 2);
+    const int NVX = (K + 2 + 3) / 4;
+    p.channel = g.channel;
+    p.pad = g.pad_h;
+    p.m = (pad0 + E) / 2;
+    if (p.m > 2) return false;
+    p.ncb = ceil_div(std::max((g.in_w + 1) / 2, g.out_w), 2);
+    if (p.ncb > kThreads) return false;
+
+    p.sx.in_h = g.in_h;
+    p.sx.in_w = g.in_w;
+    p.sx.in_plane = g.in_h * g.in_w;
+    p.sx.col_shift = g.pad_w;
+    layout_columns(p.sx, 4 * (p.ncb - 1) + 4 * NVX);
+    p.sg.in_h = g.out_h;
+    p.sg.in_w = g.out_w;
+    p.sg.in_plane = g.out_h * g.out_w;
+    p.sg.col_shift = p.m;
+    layout_columns(p.sg, 2 * (p.ncb - 1) + NWG);
+
+    const int qrows = std::max((g.in_h + 1) / 2, g.out_h);
+    const int row_units = ceil_div(qrows, kBq);
+    auto rows_x = [](int units) { return (units * kBq - 1) * 2 + K; };
+    auto rows_g = [&](int units) { return units * kBq + KA; };
+    auto bytes = [&](int units) {
+        return (static_cast<long>(rows_x(units)) * p.sx.pitch + static_cast<long>(rows_g(units)) * p.sg.pitch) * 4;
+    };
+    int units = kThreads / p.ncb;
+    if (units < 1) units = 1;
+    if (units > row_units) units = row_units;
+    const int budget = env_int("DWCONV_FUSED_LDS", kFusedLdsBudget);
+    while (units > 1 && bytes(units) > budget) --units;
+    if (bytes(units) > 60 * 1024) return false;
+    const int bands = ceil_div(row_units, units);
+    units = ceil_div(row_units, bands);
+    p.rows_per_tile = units * kBq;
+    p.row_tiles = bands;
+    if (!layout_rows(p.sx, rows_x(units), 1) || !layout_rows(p.sg, rows_g(units), 1)) return false;
+    p.g_base = p.sx.plane_pitch;
+    p.n_items = units * p.ncb;
+    p.ncb_magic = magic_u16(p.ncb);
+    const long tiles = static_cast<long>(g.batch) * bands;
+    if (tiles > 0x7fffffffL) return false;
+    p.tiles_per_group = static_cast<int>(tiles);
+    int chunks = ceil_div(env_int("DWCONV_WGRAD_WGS", 2048), g.channel);
+    if (chunks > p.tiles_per_group) chunks = p.tiles_per_group;
+    if (chunks < 1) chunks = 1;
+    p.chunks = chunks;
+    if (static_cast<long>(g.channel) * chunks > 0x7fffffffL) return false;
+    return true;
+}
+
+template <int K>
+long bwd_s2_case(int mode, const float *x, const float *gy, const float *taps, float *gx, float *gw, void *ws,
+                 size_t ws_bytes, const WgradGeometry &g, hipStream_t stream)
+{
+    BwdS2Plan p{};
+    if (!plan_bwd_s2<K>(p, g)) return -1;
+    const size_t need = static_cast<size_t>(g.channel) * p.chunks * K * K * sizeof(float);
+    if (mode == 0) return static_cast<long>(need);
+    if (ws == nullptr || ws_bytes < need)
+        return fail(DWCONV_ERR_WORKSPACE, "backward needs a workspace of %zu bytes, got %zu", need, ws_bytes);
+    p.x = x;
+    p.gy = gy;
+    p.taps = taps;
+    p.gx = gx;
+    p.partial = static_cast<float *>(ws);
+    p.sx.vec_in = (g.in_w % 4 == 0) && aligned16(x);
+    p.sg.vec_in = (g.out_w % 4 == 0) && aligned16(gy);
+    p.vec_gx = (g.in_w % 4 == 0) && aligned16(gx);
+    const size_t images = static_cast<size_t>(p.sx.plane_pitch + p.sg.plane_pitch) * 4;
+    const size_t red = static_cast<size_t>(kThreads / 64) * K * K * 4;
+    const size_t shmem = images > red ? images : red;
+    const int E = (K - 1 - g.pad_h) & 1;
+    if (E)
+        hipLaunchKernelGGL((bwd_s2_kernel<K, 1>), dim3(g.channel * p.chunks), dim3(kThreads), shmem, stream, p);
+    else
+        hipLaunchKernelGGL((bwd_s2_kernel<K, 0>), dim3(g.channel * p.chunks), dim3(kThreads), shmem, stream, p);
+    const int rc = check_launch("bwd_s2_kernel");
+    if (rc != DWCONV_OK) return rc;
+    note_variant("bwd_tile_s2<k%d,e%d> rows%d chunks%d vin%d vgy%d vgx%d", K, E, p.rows_per_tile, p.chunks, p.sx.vec_in,
+                 p.sg.vec_in, p.vec_gx);
+    return launch_wgrad_final(p.partial, gw, g.channel, K * K, p.chunks, stream);
+}
+
+long bwd_s2_any(int mode, const float *x, const float *gy, const float *taps, float *gx, float *gw, void *ws,
+                size_t ws_bytes, const WgradGeometry &g, hipStream_t stream)
+{
+    if (env_int("DWCONV_NO_FUSED_TILE", 0)) return -1;
+    const int K = g.kernel_h;
+    if (g.kernel_w != K || g.down_h != 2 || g.down_w != 2) return -1;
+    if (g.pad_h != g.pad_w || g.pad_h < 0 || g.pad_h > K - 1) return -1;
+    if (g.in_h < 1 || g.in_w < 1 || g.out_h < 1 || g.out_w < 1) return -1;
+    if (static_cast<long>(g.in_h) * g.in_w >= (1l << 30)) return -1;
+    if (K == 3) return bwd_s2_case<3>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+    if (K == 5) return bwd_s2_case<5>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+    if (K == 7) return bwd_s2_case<7>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+    return -1;
+}
+
+}  // namespace
+
+size_t bwd_s2_workspace(const WgradGeometry &g)
+{
+    const long n = bwd_s2_any(0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, g, nullptr);
+    return n > 0 ? static_cast<size_t>(n) : 0;
+}
+
+int try_launch_bwd_s2(const float *in, const float *gy, const float *taps, float *gx, float *gw, void *ws,
+                      size_t ws_bytes, const WgradGeometry &g, hipStream_t stream)
+{
+    return static_cast<int>(bwd_s2_any(1, in, gy, taps, gx, gw, ws, ws_bytes, g, stream));
+}
+
+}  // namespace dwconv

@@ -89,4 +89,9 @@ int try_launch_wgrad_tiled(const float *in, const float *gy, float *gw, void *ws
 int try_launch_bwd_tiled(const float *in, const float *gy, const float *taps, float *gx, float *gw, void *ws,
                          size_t ws_bytes, const WgradGeometry &g, hipStream_t stream);
 
+// The same for stride-2 layers: dwconv_bwd_s2.hip.
+size_t bwd_s2_workspace(const WgradGeometry &g);  // 0 when that kernel does not cover g
+int try_launch_bwd_s2(const float *in, const float *gy, const float *taps, float *gx, float *gw, void *ws,
+                      size_t ws_bytes, const WgradGeometry &g, hipStream_t stream);
+
 }  // namespace dwconv
