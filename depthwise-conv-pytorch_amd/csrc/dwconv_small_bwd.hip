@@ -121,14 +121,24 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
                 for (int o = 0; o < OW; ++o) g[b][o] = ok ? g[b][o] : 0.f;
             }
             const float *plane = lds_x + pl * in_plane;
+            // rows are read one ahead of their use and the sums pinned after every row (see pin_registers)
+            float nxt[W];
+            bool nxt_ok;
+            {
+                const int iy = oy0 * S - p.pad_h;
+                nxt_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
+                lds_load_row<W>(plane + (nxt_ok ? iy : 0) * W, nxt);
+            }
 #pragma unroll
             for (int wr = 0; wr < WIN_ROWS; ++wr) {
-                const int iy = oy0 * S - p.pad_h + wr;
-                const bool ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
                 float row[W];
-                lds_load_row<W>(plane + (ok ? iy : 0) * W, row);
 #pragma unroll
-                for (int i = 0; i < W; ++i) row[i] = ok ? row[i] : 0.f;
+                for (int i = 0; i < W; ++i) row[i] = nxt_ok ? nxt[i] : 0.f;
+                if (wr + 1 < WIN_ROWS) {
+                    const int iy = oy0 * S - p.pad_h + wr + 1;
+                    nxt_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
+                    lds_load_row<W>(plane + (nxt_ok ? iy : 0) * W, nxt);
+                }
 #pragma unroll
                 for (int b = 0; b < BH; ++b) {
                     const int ty = wr - b * S;
@@ -142,6 +152,7 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
                             wacc[ty * K + tx] = fmaf(g[b][o], row[ix], wacc[ty * K + tx]);
                         }
                 }
+                pin_registers(wacc);
             }
         }
 
@@ -156,14 +167,23 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
             const float *gplane = lds_g + pl * out_plane;
             if constexpr (S == 1) {
                 // gx[iy,ix] = sum_{ty,tx} gy[iy - PW + ty, ix - PW + tx] * rot[ty,tx]   (out extent == in extent)
+                float nxt[OW];
+                bool nxt_ok;
+                {
+                    const int gyr = oy0 - PW;
+                    nxt_ok = static_cast<unsigned>(gyr) < static_cast<unsigned>(p.out_h);
+                    lds_load_row<OW>(gplane + (nxt_ok ? gyr : 0) * OW, nxt);
+                }
 #pragma unroll
                 for (int wr = 0; wr < BH - 1 + K; ++wr) {
-                    const int gyr = oy0 - PW + wr;
-                    const bool ok = static_cast<unsigned>(gyr) < static_cast<unsigned>(p.out_h);
                     float row[OW];
-                    lds_load_row<OW>(gplane + (ok ? gyr : 0) * OW, row);
 #pragma unroll
-                    for (int i = 0; i < OW; ++i) row[i] = ok ? row[i] : 0.f;
+                    for (int i = 0; i < OW; ++i) row[i] = nxt_ok ? nxt[i] : 0.f;
+                    if (wr + 1 < BH - 1 + K) {
+                        const int gyr = oy0 - PW + wr + 1;
+                        nxt_ok = static_cast<unsigned>(gyr) < static_cast<unsigned>(p.out_h);
+                        lds_load_row<OW>(gplane + (nxt_ok ? gyr : 0) * OW, nxt);
+                    }
 #pragma unroll
                     for (int b = 0; b < BH; ++b) {
                         const int ty = wr - b;
@@ -177,20 +197,30 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
                                 xacc[b][o] = fmaf(row[ix], tapv[ty * K + tx], xacc[b][o]);
                             }
                     }
+                    pin_registers(xacc);
                 }
             } else {
                 // gx[2q + r] = sum_a gy[q - M + r + a] * rot'[r + 2a], rot'[t] = rot[t - E]  (see small_up2_kernel)
                 constexpr int E = PW & 1;
                 constexpr int M = (PW + E) / 2;
                 constexpr int KA = (K + E + 1) / 2;
+                float nxt[OW];
+                bool nxt_ok;
+                {
+                    const int gyr = rb - M;
+                    nxt_ok = static_cast<unsigned>(gyr) < static_cast<unsigned>(p.out_h);
+                    lds_load_row<OW>(gplane + (nxt_ok ? gyr : 0) * OW, nxt);
+                }
 #pragma unroll
                 for (int wr = 0; wr < KA + 1; ++wr) {
-                    const int gyr = rb - M + wr;
-                    const bool ok = static_cast<unsigned>(gyr) < static_cast<unsigned>(p.out_h);
                     float row[OW];
-                    lds_load_row<OW>(gplane + (ok ? gyr : 0) * OW, row);
 #pragma unroll
-                    for (int i = 0; i < OW; ++i) row[i] = ok ? row[i] : 0.f;
+                    for (int i = 0; i < OW; ++i) row[i] = nxt_ok ? nxt[i] : 0.f;
+                    if (wr + 1 < KA + 1) {
+                        const int gyr = rb - M + wr + 1;
+                        nxt_ok = static_cast<unsigned>(gyr) < static_cast<unsigned>(p.out_h);
+                        lds_load_row<OW>(gplane + (nxt_ok ? gyr : 0) * OW, nxt);
+                    }
 #pragma unroll
                     for (int r = 0; r < 2; ++r) {
                         const int a = wr - r;
@@ -209,6 +239,7 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
                             }
                         }
                     }
+                    pin_registers(xacc);
                 }
             }
             __syncthreads();  // every lane is done with the x run: overwrite it with the gx run

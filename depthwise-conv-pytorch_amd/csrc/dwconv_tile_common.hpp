@@ -96,6 +96,27 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const float *__
     }
 }
 
+// Pins an accumulator array at this point of a fully unrolled loop nest.  The empty asm makes every
+// element an input and an output, so all FMAs feeding it must be issued before, and its memory clobber
+// keeps later LDS reads after it.  Without such pins the compiler sinks every FMA of a window below
+// the LDS reads of all its rows and keeps the whole window in registers (several hundred VGPRs).
+// It emits no instruction.
+template <int N>
+__device__ __forceinline__ void pin_registers(float (&a)[N])
+{
+#pragma unroll
+    for (int i = 0; i < N; ++i) asm volatile("" : "+v"(a[i]) : : "memory");
+}
+
+template <int R, int C>
+__device__ __forceinline__ void pin_registers(float (&a)[R][C])
+{
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int c = 0; c < C; ++c) asm volatile("" : "+v"(a[r][c]) : : "memory");
+}
+
 inline int floor_div(int a, int b)
 {
     int q = a / b;
