@@ -69,14 +69,24 @@ __global__ __launch_bounds__(kWave) void small_down_kernel(const SmallPlan p)
 
     const int oy0 = rb * BH;
     const float *plane = lds + pl * in_plane;
+    // rows are read one ahead of their use and the sums pinned after every row (see pin_registers)
+    float nxt[W];
+    bool nxt_ok;
+    {
+        const int iy = oy0 * S - p.pad_h;
+        nxt_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
+        lds_load_row<W>(plane + (nxt_ok ? iy : 0) * W, nxt);
+    }
 #pragma unroll
     for (int wr = 0; wr < WIN_ROWS; ++wr) {
-        const int iy = oy0 * S - p.pad_h + wr;
-        const bool ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
         float row[W];
-        lds_load_row<W>(plane + (ok ? iy : 0) * W, row);
 #pragma unroll
-        for (int i = 0; i < W; ++i) row[i] = ok ? row[i] : 0.f;
+        for (int i = 0; i < W; ++i) row[i] = nxt_ok ? nxt[i] : 0.f;
+        if (wr + 1 < WIN_ROWS) {
+            const int iy = oy0 * S - p.pad_h + wr + 1;
+            nxt_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
+            lds_load_row<W>(plane + (nxt_ok ? iy : 0) * W, nxt);
+        }
 #pragma unroll
         for (int b = 0; b < BH; ++b) {
             const int ty = wr - b * S;
@@ -90,6 +100,7 @@ __global__ __launch_bounds__(kWave) void small_down_kernel(const SmallPlan p)
                     acc[b][o] = fmaf(row[ix], tapv[ty * K + tx], acc[b][o]);
                 }
         }
+        pin_registers(acc);
     }
     __syncthreads();  // every lane has read its input rows: the run can be overwritten in place
 
@@ -138,14 +149,23 @@ __global__ __launch_bounds__(kWave) void small_up2_kernel(const SmallPlan p)
         for (int o = 0; o < OW; ++o) acc[r][o] = 0.f;
 
     const float *plane = lds + pl * in_plane;
+    float nxt[W];
+    bool nxt_ok;
+    {
+        const int iy = q - p.pad_h;
+        nxt_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
+        lds_load_row<W>(plane + (nxt_ok ? iy : 0) * W, nxt);
+    }
 #pragma unroll
     for (int wr = 0; wr < WIN_ROWS; ++wr) {
-        const int iy = q - p.pad_h + wr;
-        const bool ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
         float row[W];
-        lds_load_row<W>(plane + (ok ? iy : 0) * W, row);
 #pragma unroll
-        for (int i = 0; i < W; ++i) row[i] = ok ? row[i] : 0.f;
+        for (int i = 0; i < W; ++i) row[i] = nxt_ok ? nxt[i] : 0.f;
+        if (wr + 1 < WIN_ROWS) {
+            const int iy = q - p.pad_h + wr + 1;
+            nxt_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
+            lds_load_row<W>(plane + (nxt_ok ? iy : 0) * W, nxt);
+        }
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
             const int a = wr - r;
@@ -164,6 +184,7 @@ __global__ __launch_bounds__(kWave) void small_up2_kernel(const SmallPlan p)
                 }
             }
         }
+        pin_registers(acc);
     }
     __syncthreads();
 
