@@ -20,6 +20,7 @@ namespace {
 
 constexpr int kBq = 4;                        // half-resolution rows per lane
 constexpr int kFusedLdsBudget = 36 * 1024;    // both images of a tile
+constexpr int kUx = 8, kUg = 2;               // float4 slots per lane that hold the next tile's x / gy band
 
 struct BwdS2Plan {
     StageLayout sx;   // x image: row r holds x row 2*q0 - pad + r, column c holds x column c - pad
@@ -40,6 +41,7 @@ struct BwdS2Plan {
     unsigned ncb_magic;
     int n_items;
     int vec_gx;
+    int prefetch;     // the images of a tile fit the prefetch registers
 };
 
 template <int CTRL, int ROW_MASK, int BANK_MASK>
@@ -62,7 +64,9 @@ __device__ __forceinline__ float wave_sum_to_last_lane(float v)
 }
 
 // E = parity of the transposed problem's leading pad K - 1 - pad (the same on both axes).
-template <int K, int E>
+// PF: keep the next tile's bands in flight in registers (worth its ~50 registers for the 3x3 kernel only;
+// with more taps the lower occupancy costs more than the overlap brings).
+template <int K, int E, bool PF>
 __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -92,15 +96,41 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
 #pragma unroll
     for (int t = 0; t < KK; ++t) wacc[t] = 0.f;
 
+    StagedTile<PF ? kUx : 1> tx;
+    StagedTile<PF ? kUg : 1> tg;
+    if constexpr (PF) {
+        if (chunk < p.tiles_per_group) {
+        const int n = chunk / p.row_tiles, rt = chunk - n * p.row_tiles;
+        const long plane0 = static_cast<long>(n) * p.channel + c;
+        stage_fetch(p.sx, p.x, plane0, 1, 2 * rt * p.rows_per_tile - p.pad, tx);
+        stage_fetch(p.sg, p.gy, plane0, 1, rt * p.rows_per_tile - p.m, tg);
+        }
+    }
+
     for (int tile = chunk; tile < p.tiles_per_group; tile += p.chunks) {
         const int n = tile / p.row_tiles, rt = tile - n * p.row_tiles;
         const long plane0 = static_cast<long>(n) * p.channel + c;
         const int q0 = rt * p.rows_per_tile;
 
         if (tile != chunk) __syncthreads();  // the previous tile's window reads are done
-        stage_tile(p.sx, p.x, lds, plane0, 1, 2 * q0 - p.pad);
-        stage_tile(p.sg, p.gy, lds + p.g_base, plane0, 1, q0 - p.m);
+        if constexpr (PF) {
+            stage_commit(p.sx, lds, 1, tx);
+            stage_commit(p.sg, lds + p.g_base, 1, tg);
+        } else {
+            stage_tile(p.sx, p.x, lds, plane0, 1, 2 * q0 - p.pad);
+            stage_tile(p.sg, p.gy, lds + p.g_base, plane0, 1, q0 - p.m);
+        }
         __syncthreads();
+        if constexpr (PF) {
+          if (tile + p.chunks < p.tiles_per_group) {
+            // the next tile's bands travel while this one is computed
+            const int t1 = tile + p.chunks;
+            const int n1 = t1 / p.row_tiles, rt1 = t1 - n1 * p.row_tiles;
+            const long plane1 = static_cast<long>(n1) * p.channel + c;
+            stage_fetch(p.sx, p.x, plane1, 1, 2 * rt1 * p.rows_per_tile - p.pad, tx);
+            stage_fetch(p.sg, p.gy, plane1, 1, rt1 * p.rows_per_tile - p.m, tg);
+          }
+        }
 
         // ---- gy window: grad-input block, and this lane's gy elements from the window's centre
         float g[BQ][2];
@@ -200,8 +230,7 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
     __syncthreads();
     if (threadIdx.x < KK) {
         float s = lds[threadIdx.x];
-#pragma unroll
-        for (int w = 1; w < kThreads / 64; ++w) s += lds[w * KK + threadIdx.x];
+        for (int w = 1; w < static_cast<int>(blockDim.x) / 64; ++w) s += lds[w * KK + threadIdx.x];
         p.partial[(static_cast<long>(c) * p.chunks + chunk) * KK + threadIdx.x] = s;
     }
 }
@@ -282,18 +311,23 @@ long bwd_s2_case(int mode, const float *x, const float *gy, const float *taps, f
     p.sx.vec_in = (g.in_w % 4 == 0) && aligned16(x);
     p.sg.vec_in = (g.out_w % 4 == 0) && aligned16(gy);
     p.vec_gx = (g.in_w % 4 == 0) && aligned16(gx);
+    // all 256 lanes stage the images even when the tile has fewer items than that
+    const int threads = kThreads;
+    p.prefetch = K == 3 && env_int("DWCONV_PREFETCH", 1) && p.sx.lds_rows * p.sx.spr <= kUx * threads &&
+                 p.sg.lds_rows * p.sg.spr <= kUg * threads;
     const size_t images = static_cast<size_t>(p.sx.plane_pitch + p.sg.plane_pitch) * 4;
     const size_t red = static_cast<size_t>(kThreads / 64) * K * K * 4;
     const size_t shmem = images > red ? images : red;
     const int E = (K - 1 - g.pad_h) & 1;
-    if (E)
-        hipLaunchKernelGGL((bwd_s2_kernel<K, 1>), dim3(g.channel * p.chunks), dim3(kThreads), shmem, stream, p);
-    else
-        hipLaunchKernelGGL((bwd_s2_kernel<K, 0>), dim3(g.channel * p.chunks), dim3(kThreads), shmem, stream, p);
+    const dim3 grid(g.channel * p.chunks), block(threads);
+    if (E && p.prefetch) hipLaunchKernelGGL((bwd_s2_kernel<K, 1, true>), grid, block, shmem, stream, p);
+    else if (E) hipLaunchKernelGGL((bwd_s2_kernel<K, 1, false>), grid, block, shmem, stream, p);
+    else if (p.prefetch) hipLaunchKernelGGL((bwd_s2_kernel<K, 0, true>), grid, block, shmem, stream, p);
+    else hipLaunchKernelGGL((bwd_s2_kernel<K, 0, false>), grid, block, shmem, stream, p);
     const int rc = check_launch("bwd_s2_kernel");
     if (rc != DWCONV_OK) return rc;
-    note_variant("bwd_tile_s2<k%d,e%d> rows%d chunks%d vin%d vgy%d vgx%d", K, E, p.rows_per_tile, p.chunks, p.sx.vec_in,
-                 p.sg.vec_in, p.vec_gx);
+    note_variant("bwd_tile_s2<k%d,e%d> rows%d chunks%d vin%d vgy%d vgx%d pf%d", K, E, p.rows_per_tile, p.chunks, p.sx.vec_in,
+                 p.sg.vec_in, p.vec_gx, p.prefetch);
     return launch_wgrad_final(p.partial, gw, g.channel, K * K, p.chunks, stream);
 }
 

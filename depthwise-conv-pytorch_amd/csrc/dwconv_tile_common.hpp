@@ -96,6 +96,74 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const float *__
     }
 }
 
+// The same staging in two halves, for kernels that walk several tiles: `stage_fetch` issues the global
+// loads of a tile into registers (U float4 slots per lane; the planner guarantees the tile has no more
+// than U * blockDim.x slots), `stage_commit` writes them to LDS.  Fetching tile t+1 right after
+// committing tile t keeps its loads in flight while tile t is being computed.
+template <int U>
+struct StagedTile {
+    float4 v[U];
+};
+
+// LDS offset (floats) of slot `slot` of the image, or -1 past its end; tile-independent.
+__device__ __forceinline__ int stage_slot_offset(const StageLayout &s, int slot, int nplanes)
+{
+    if (slot >= nplanes * s.lds_rows * s.spr) return -1;
+    const int rowidx = fast_div(slot, s.spr_magic);
+    const int sc = slot - rowidx * s.spr;
+    const int pl = fast_div(rowidx, s.lds_rows_magic);
+    const int r = rowidx - pl * s.lds_rows;
+    return pl * s.plane_pitch + r * s.pitch + kSlack + 4 * (s.g_lo + sc) + s.col_shift;
+}
+
+template <int U>
+__device__ __forceinline__ void stage_fetch(const StageLayout &s, const float *__restrict__ in, long plane0,
+                                            int nplanes, int iy0, StagedTile<U> &t)
+{
+    const int total = nplanes * s.lds_rows * s.spr;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int slot = threadIdx.x + u * blockDim.x;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (slot < total) {
+            const int rowidx = fast_div(slot, s.spr_magic);
+            const int sc = slot - rowidx * s.spr;
+            const int pl = fast_div(rowidx, s.lds_rows_magic);
+            const int r = rowidx - pl * s.lds_rows;
+            const int ix = 4 * (s.g_lo + sc);
+            const int iy = iy0 + r;
+            const bool row_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(s.in_h);
+            const float *src = in + (plane0 + pl) * s.in_plane + static_cast<long>(iy) * s.in_w + ix;
+            if (s.vec_in) {
+                if (row_ok && ix >= 0 && ix < s.in_w) v = *reinterpret_cast<const float4 *>(src);
+            } else if (row_ok) {
+                if (static_cast<unsigned>(ix + 0) < static_cast<unsigned>(s.in_w)) v.x = src[0];
+                if (static_cast<unsigned>(ix + 1) < static_cast<unsigned>(s.in_w)) v.y = src[1];
+                if (static_cast<unsigned>(ix + 2) < static_cast<unsigned>(s.in_w)) v.z = src[2];
+                if (static_cast<unsigned>(ix + 3) < static_cast<unsigned>(s.in_w)) v.w = src[3];
+            }
+        }
+        t.v[u] = v;
+    }
+}
+
+template <int U>
+__device__ __forceinline__ void stage_commit(const StageLayout &s, float *lds, int nplanes, const StagedTile<U> &t)
+{
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const float4 v = t.v[u];
+        const int d = stage_slot_offset(s, threadIdx.x + u * blockDim.x, nplanes);
+        if (d >= 0) {
+            float *dst = lds + d;
+            dst[0] = v.x;
+            dst[1] = v.y;
+            dst[2] = v.z;
+            dst[3] = v.w;
+        }
+    }
+}
+
 // Pins an accumulator array at this point of a fully unrolled loop nest.  The empty asm makes every
 // element an input and an output, so all FMAs feeding it must be issued before, and its memory clobber
 // keeps later LDS reads after it.  Without such pins the compiler sinks every FMA of a window below
