@@ -18,7 +18,6 @@ namespace dwconv {
 
 namespace {
 
-constexpr int kBq = 4;                        // half-resolution rows per lane
 constexpr int kFusedLdsBudget = 36 * 1024;    // both images of a tile
 constexpr int kUx = 8, kUg = 2;               // float4 slots per lane that hold the next tile's x / gy band
 
@@ -40,6 +39,7 @@ struct BwdS2Plan {
     int ncb;
     unsigned ncb_magic;
     int n_items;
+    int bq;
     int vec_gx;
     int prefetch;     // the images of a tile fit the prefetch registers
 };
@@ -66,13 +66,13 @@ __device__ __forceinline__ float wave_sum_to_last_lane(float v)
 // E = parity of the transposed problem's leading pad K - 1 - pad (the same on both axes).
 // PF: keep the next tile's bands in flight in registers (worth its ~50 registers for the 3x3 kernel only;
 // with more taps the lower occupancy costs more than the overlap brings).
-template <int K, int E, bool PF>
+// BQ: half-resolution rows per lane (4; 2 for planes too low to give every lane a block of 4).
+template <int K, int E, bool PF, int BQ>
 __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
 {
     extern __shared__ float4 lds_raw[];
     float *lds = reinterpret_cast<float *>(lds_raw);
     constexpr int KK = K * K;
-    constexpr int BQ = kBq;
     constexpr int KA = (K + E + 1) / 2;
     constexpr int GW_ROWS = BQ + KA;                  // gy window rows
     constexpr int NWG = 2 * ((KA + 2 + 1) / 2);       // gy window columns, as float2s
@@ -236,7 +236,7 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
 }
 
 template <int K>
-bool plan_bwd_s2(BwdS2Plan &p, const WgradGeometry &g)
+bool plan_bwd_s2(BwdS2Plan &p, const WgradGeometry &g, int kBq)
 {
     const int pad0 = K - 1 - g.pad_h;  // leading pad of the transposed problem
     const int E = pad0 & 1;
@@ -244,6 +244,7 @@ bool plan_bwd_s2(BwdS2Plan &p, const WgradGeometry &g)
     const int NWG = 2 * ((KA + 2 + 1) / 2);
     const int NVX = (K + 2 + 3) / 4;
     p.channel = g.channel;
+    p.bq = kBq;
     p.pad = g.pad_h;
     p.m = (pad0 + E) / 2;
     if (p.m > 2) return false;
@@ -263,7 +264,7 @@ bool plan_bwd_s2(BwdS2Plan &p, const WgradGeometry &g)
 
     const int qrows = std::max((g.in_h + 1) / 2, g.out_h);
     const int row_units = ceil_div(qrows, kBq);
-    auto rows_x = [](int units) { return (units * kBq - 1) * 2 + K; };
+    auto rows_x = [&](int units) { return (units * kBq - 1) * 2 + K; };
     auto rows_g = [&](int units) { return units * kBq + KA; };
     auto bytes = [&](int units) {
         return (static_cast<long>(rows_x(units)) * p.sx.pitch + static_cast<long>(rows_g(units)) * p.sg.pitch) * 4;
@@ -297,8 +298,11 @@ template <int K>
 long bwd_s2_case(int mode, const float *x, const float *gy, const float *taps, float *gx, float *gw, void *ws,
                  size_t ws_bytes, const WgradGeometry &g, hipStream_t stream)
 {
+    // blocks of 4 half-resolution rows, or of 2 when that is what it takes to give most lanes an item
+    const int qrows = std::max((g.in_h + 1) / 2, g.out_h), pairs = ceil_div(std::max((g.in_w + 1) / 2, g.out_w), 2);
+    const int bq = ceil_div(qrows, 4) * pairs * 2 <= kThreads ? 2 : 4;
     BwdS2Plan p{};
-    if (!plan_bwd_s2<K>(p, g)) return -1;
+    if (!plan_bwd_s2<K>(p, g, bq)) return -1;
     const size_t need = static_cast<size_t>(g.channel) * p.chunks * K * K * sizeof(float);
     if (mode == 0) return static_cast<long>(need);
     if (ws == nullptr || ws_bytes < need)
@@ -313,20 +317,23 @@ long bwd_s2_case(int mode, const float *x, const float *gy, const float *taps, f
     p.vec_gx = (g.in_w % 4 == 0) && aligned16(gx);
     // all 256 lanes stage the images even when the tile has fewer items than that
     const int threads = kThreads;
-    p.prefetch = K == 3 && env_int("DWCONV_PREFETCH", 1) && p.sx.lds_rows * p.sx.spr <= kUx * threads &&
+    p.prefetch = bq == 4 && K == 3 && env_int("DWCONV_PREFETCH", 1) && p.sx.lds_rows * p.sx.spr <= kUx * threads &&
                  p.sg.lds_rows * p.sg.spr <= kUg * threads;
     const size_t images = static_cast<size_t>(p.sx.plane_pitch + p.sg.plane_pitch) * 4;
     const size_t red = static_cast<size_t>(kThreads / 64) * K * K * 4;
     const size_t shmem = images > red ? images : red;
     const int E = (K - 1 - g.pad_h) & 1;
     const dim3 grid(g.channel * p.chunks), block(threads);
-    if (E && p.prefetch) hipLaunchKernelGGL((bwd_s2_kernel<K, 1, true>), grid, block, shmem, stream, p);
-    else if (E) hipLaunchKernelGGL((bwd_s2_kernel<K, 1, false>), grid, block, shmem, stream, p);
-    else if (p.prefetch) hipLaunchKernelGGL((bwd_s2_kernel<K, 0, true>), grid, block, shmem, stream, p);
-    else hipLaunchKernelGGL((bwd_s2_kernel<K, 0, false>), grid, block, shmem, stream, p);
+    if (bq == 2) {
+        if (E) hipLaunchKernelGGL((bwd_s2_kernel<K, 1, false, 2>), grid, block, shmem, stream, p);
+        else hipLaunchKernelGGL((bwd_s2_kernel<K, 0, false, 2>), grid, block, shmem, stream, p);
+    } else if (E && p.prefetch) hipLaunchKernelGGL((bwd_s2_kernel<K, 1, true, 4>), grid, block, shmem, stream, p);
+    else if (E) hipLaunchKernelGGL((bwd_s2_kernel<K, 1, false, 4>), grid, block, shmem, stream, p);
+    else if (p.prefetch) hipLaunchKernelGGL((bwd_s2_kernel<K, 0, true, 4>), grid, block, shmem, stream, p);
+    else hipLaunchKernelGGL((bwd_s2_kernel<K, 0, false, 4>), grid, block, shmem, stream, p);
     const int rc = check_launch("bwd_s2_kernel");
     if (rc != DWCONV_OK) return rc;
-    note_variant("bwd_tile_s2<k%d,e%d> rows%d chunks%d vin%d vgy%d vgx%d pf%d", K, E, p.rows_per_tile, p.chunks, p.sx.vec_in,
+    note_variant("bwd_tile_s2<k%d,e%d,bq%d> rows%d chunks%d vin%d vgy%d vgx%d pf%d", K, E, bq, p.rows_per_tile, p.chunks, p.sx.vec_in,
                  p.sg.vec_in, p.vec_gx, p.prefetch);
     return launch_wgrad_final(p.partial, gw, g.channel, K * K, p.chunks, stream);
 }

@@ -284,26 +284,37 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
     }
 }
 
-// Pass 2: gw[c,tap] = sum over chunks of partial[c][chunk][tap], front to back, in double.
-// Loads are issued eight at a time so that their latencies overlap; the additions keep their order.
-__global__ void wgrad_tile_final_kernel(const float *__restrict__ partial, float *__restrict__ gw,
-                                        const int channel_taps, const int taps, const int chunks)
+// Pass 2: gw[c,tap] = sum over chunks of partial[c][chunk][tap], in double and in a fixed order.
+// Eight lanes share one output: each adds a contiguous eighth of the chunks front to back (all its loads
+// are independent, so the kernel costs one memory latency instead of one per chunk), then the eight
+// sums are combined by a fixed butterfly.
+constexpr int kFinalLanes = 8;
+
+__global__ __launch_bounds__(256) void wgrad_tile_final_kernel(const float *__restrict__ partial,
+                                                               float *__restrict__ gw, const int channel_taps,
+                                                               const int taps, const int chunks)
 {
-    const int e = blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= channel_taps) return;
-    const int c = e / taps, t = e - c * taps;
+    const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+    const int e = gid / kFinalLanes, part = gid - e * kFinalLanes;
+    const bool live = e < channel_taps;
+    const int ee = live ? e : 0;
+    const int c = ee / taps, t = ee - c * taps;
     const float *p = partial + static_cast<long>(c) * chunks * taps + t;
+    const int per = (chunks + kFinalLanes - 1) / kFinalLanes;
+    const int k0 = part * per, k1 = min(chunks, k0 + per);
     double s = 0.0;
-    int k = 0;
-    for (; k + 8 <= chunks; k += 8) {
+    int k = k0;
+    for (; k + 8 <= k1; k += 8) {
         float v[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] = p[static_cast<long>(k + j) * taps];
 #pragma unroll
         for (int j = 0; j < 8; ++j) s += static_cast<double>(v[j]);
     }
-    for (; k < chunks; ++k) s += static_cast<double>(p[static_cast<long>(k) * taps]);
-    gw[e] = static_cast<float>(s);
+    for (; k < k1; ++k) s += static_cast<double>(p[static_cast<long>(k) * taps]);
+#pragma unroll
+    for (int off = 1; off < kFinalLanes; off <<= 1) s += __shfl_xor(s, off, 64);
+    if (live && part == 0) gw[e] = static_cast<float>(s);
 }
 
 template <int K, int S, int BH>
@@ -494,8 +505,8 @@ struct Launcher {
 int launch_wgrad_final(const float *partial, float *gw, int channel, int taps, int chunks, hipStream_t stream)
 {
     const int total = channel * taps;
-    hipLaunchKernelGGL(wgrad_tile_final_kernel, dim3(ceil_div(total, 64)), dim3(64), 0, stream, partial, gw, total,
-                       taps, chunks);
+    hipLaunchKernelGGL(wgrad_tile_final_kernel, dim3(ceil_div(total * kFinalLanes, 256)), dim3(256), 0, stream, partial,
+                       gw, total, taps, chunks);
     return check_launch("wgrad_tile_final_kernel");
 }
 
