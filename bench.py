@@ -3,8 +3,9 @@
 
 Workload (BASELINE.json, configs[2]): the 12 depthwise layers of EfficientNet-B0,
 fp32 NCHW, batch 128, padding k//2.  One "step" = forward of layers 1..12, then
-grad-input and grad-weight of layers 12..1 (training order): 36 calls into the
-C ABI of libdwconv_hip, all tensors resident in HBM before the clock starts.
+grad-input and grad-weight of layers 12..1 (training order): 24 calls into the
+C ABI of libdwconv_hip (12 forward, 12 combined backward; --separate-backward
+makes it 36), all tensors resident in HBM before the clock starts.
 
 Prints one JSON line.  `value` is achieved HBM GB/s = algorithmic bytes of the
 step (every tensor of every pass touched exactly once: 12(|x|+|y|+|w|) bytes per
@@ -253,8 +254,16 @@ def main():
         agg["launches"] += 1
     dom_name, dom = max(by_kernel.items(), key=lambda kv: kv[1]["ms"])
     achieved = dom["bytes"] / dom["ms"] / 1e6
+    # measured HBM bytes per launch of that kernel, from the committed rocprofv3 --pmc summary (null if the
+    # summary does not cover this variant)
+    traffic = None
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            traffic = json.load(f)["bytes_per_launch"].get(dom_name)
+    except (OSError, ValueError, KeyError):
+        traffic = None
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": dom_name,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": dom_name,
                 "launches_per_step": dom["launches"], "avg_launch_us": round(dom["ms"] * 1e3 / dom["launches"], 1),
                 "bytes_per_launch": dom["bytes"] // dom["launches"]}
 

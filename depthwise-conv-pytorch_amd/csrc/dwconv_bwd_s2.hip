@@ -286,7 +286,7 @@ bool plan_bwd_s2(BwdS2Plan &p, const WgradGeometry &g, int kBq)
     const long tiles = static_cast<long>(g.batch) * bands;
     if (tiles > 0x7fffffffL) return false;
     p.tiles_per_group = static_cast<int>(tiles);
-    int chunks = ceil_div(env_int("DWCONV_WGRAD_WGS", 2048), g.channel);
+    int chunks = ceil_div(env_int("DWCONV_WGRAD_WGS", 3072), g.channel);
     if (chunks > p.tiles_per_group) chunks = p.tiles_per_group;
     if (chunks < 1) chunks = 1;
     p.chunks = chunks;

@@ -291,7 +291,7 @@ bool plan_small_bwd(SmallBwdPlan &p, const WgradGeometry &g)
     p.planes_per_run = P;
     p.lpp_magic = magic_u16(p.lanes_per_plane);
     const int groups = ceil_div(g.channel, P);
-    int chunks = ceil_div(env_int("DWCONV_SMALL_WGRAD_WAVES", 4096), groups);
+    int chunks = ceil_div(env_int("DWCONV_SMALL_WGRAD_WAVES", 2048), groups);
     if (chunks > g.batch) chunks = g.batch;
     if (chunks < 1) chunks = 1;
     p.images_per_chunk = ceil_div(g.batch, chunks);

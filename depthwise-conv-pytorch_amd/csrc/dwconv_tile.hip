@@ -240,6 +240,7 @@ bool plan_tiles(TilePlan &p, int row_units, int unit_rows, int used_cols, int ta
 {
     const int threads = env_int("DWCONV_TILE_THREADS", kThreads);
     const int target_items = env_int("DWCONV_TILE_ITEMS", threads);
+    const int kLdsBudget = env_int("DWCONV_TILE_LDS", dwconv::kLdsBudget);
     layout_columns(p.st, used_cols);
 
     auto bytes = [&](int units, int planes) {

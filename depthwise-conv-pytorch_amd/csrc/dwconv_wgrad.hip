@@ -322,7 +322,7 @@ bool make_plan(WgradPlan &p, const WgradGeometry &g, bool fused)
 {
     constexpr int NV = (3 * S + K + 3) / 4;
     constexpr int KK = K * K;
-    const int target_wgs = env_int("DWCONV_WGRAD_WGS", 2048);
+    const int target_wgs = env_int("DWCONV_WGRAD_WGS", 3072);
     p.batch = g.batch;
     p.channel = g.channel;
     p.out_h = g.out_h;

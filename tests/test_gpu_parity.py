@@ -320,6 +320,37 @@ def test_c_entry_points_directly(dw, gpu):
         _C.dwconv2d(x, torch.randn(3, 1, 3, 3, device=gpu), 1, 1, 1, 1, 1, 1, 1, 1, True)
 
 
+def test_combined_backward_entry_point(dw, gpu):
+    """dwconv2d_backward: fused kernels where they exist, the two separate passes otherwise; errors as status codes."""
+    from torch_dwconv import _C
+
+    cases = [(2, 6, 14, 14, 3, 1, 1), (2, 6, 30, 33, 5, 2, 2), (2, 3, 40, 44, 3, 1, 0), (1, 4, 64, 64, 5, 1, 2),
+             (2, 4, 64, 48, 3, 2, 1), (1, 2, 20, 20, 4, 2, 1), (2, 3, 31, 29, 7, 2, 3), (2, 3, 48, 52, 5, 2, 0)]
+    seen = set()
+    for shape in cases:
+        n, c, h, w, k, s, p = shape
+        x, wt, gy = make_inputs(shape, seed=13)
+        gx, gw = _C.dwconv2d_backward(x.to(gpu), gy.to(gpu), wt.to(gpu), s, s, p, p)
+        seen.add(_C.last_variant().split("<")[0])
+        _announce(shape_id(shape), _C.last_variant())
+        gx_ref = oracle.grad_input(_np(gy), _np(wt), (h, w), s, p)
+        gw_ref = oracle.grad_weight(_np(x), _np(gy), wt.shape, s, p)
+        np.testing.assert_allclose(_np(gx).astype(np.float64), gx_ref, rtol=1e-5, atol=1e-5)
+        np.testing.assert_allclose(_np(gw).astype(np.float64), gw_ref, rtol=1e-4, atol=1e-4 * np.abs(gw_ref).max())
+    assert {"small_bwd", "bwd_tile", "bwd_tile_s2"} <= seen, seen
+    # an out_grad whose extent does not belong to the geometry is refused
+    x, wt, gy = make_inputs((1, 2, 16, 16, 3, 1, 1), seed=1)
+    with pytest.raises(RuntimeError, match="does not match the convolution geometry"):
+        _C.dwconv2d_backward(x.to(gpu), gy[:, :, :15].contiguous().to(gpu), wt.to(gpu), 1, 1, 1, 1)
+    # a workspace that is too small comes back as DWCONV_ERR_WORKSPACE, not as a fault
+    xg, gg, wg = x.to(gpu), gy.to(gpu), wt.to(gpu)
+    gxo, gwo = torch.empty_like(xg), torch.empty_like(wg)
+    tiny = torch.empty(4, dtype=torch.uint8, device=gpu)
+    rc = _C._lib.dwconv2d_backward_f32(xg.data_ptr(), gg.data_ptr(), wg.data_ptr(), gxo.data_ptr(), gwo.data_ptr(),
+                                       tiny.data_ptr(), 4, 1, 2, 16, 16, 16, 16, 3, 3, 1, 1, 1, 1, None)
+    assert rc == 3 and b"workspace" in _C._lib.dwconv_last_error()
+
+
 def test_module_matches_plain_conv(dw, gpu):
     m = dw.DepthwiseConv2d(16, 16, 3, stride=1, padding=1).to(gpu)
     x = torch.randn(4, 16, 40, 40, device=gpu, requires_grad=True)
