@@ -139,15 +139,14 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
         for (int b = 0; b < 2 * BQ; ++b)
 #pragma unroll
             for (int o = 0; o < 4; ++o) xacc[b][o] = 0.f;
+        float nxg[NWG];
+        load_window_row2<NWG / 2>(base_g, nxg);
 #pragma unroll
         for (int wr = 0; wr < GW_ROWS; ++wr) {
             float win[NWG];
 #pragma unroll
-            for (int v = 0; v < NWG / 2; ++v) {
-                const float2 q = *reinterpret_cast<const float2 *>(base_g + wr * p.sg.pitch + 2 * v);
-                win[2 * v] = q.x;
-                win[2 * v + 1] = q.y;
-            }
+            for (int i = 0; i < NWG; ++i) win[i] = nxg[i];
+            if (wr + 1 < GW_ROWS) load_window_row2<NWG / 2>(base_g + (wr + 1) * p.sg.pitch, nxg);
             if (wr >= p.m && wr - p.m < BQ) {
                 // the centre row index depends on m (1 or 2 for the kernels served here): select at run time
 #pragma unroll
@@ -177,6 +176,7 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
                                     fmaf(win[xq + rx + ax], rot[fy * K + fx], xacc[2 * bq + r][2 * xq + rx]);
                             }
                 }
+            pin_registers(xacc);
         }
         if (has_item) {
             const int ox = 4 * cb;
@@ -198,17 +198,14 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
         }
 
         // ---- x window: grad-weight sums
+        float nxx[4 * NVX];
+        load_window_row<NVX>(base_x, nxx);
 #pragma unroll
         for (int wr = 0; wr < XW_ROWS; ++wr) {
             float win[4 * NVX];
 #pragma unroll
-            for (int v = 0; v < NVX; ++v) {
-                const float4 q = *reinterpret_cast<const float4 *>(base_x + wr * p.sx.pitch + 4 * v);
-                win[4 * v + 0] = q.x;
-                win[4 * v + 1] = q.y;
-                win[4 * v + 2] = q.z;
-                win[4 * v + 3] = q.w;
-            }
+            for (int i = 0; i < 4 * NVX; ++i) win[i] = nxx[i];
+            if (wr + 1 < XW_ROWS) load_window_row<NVX>(base_x + (wr + 1) * p.sx.pitch, nxx);
 #pragma unroll
             for (int bq = 0; bq < BQ; ++bq) {
                 const int ty = wr - 2 * bq;
@@ -218,6 +215,7 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
 #pragma unroll
                     for (int o = 0; o < 2; ++o) wacc[ty * K + tx] = fmaf(g[bq][o], win[2 * o + tx], wacc[ty * K + tx]);
             }
+            pin_registers(wacc);
         }
     }
 

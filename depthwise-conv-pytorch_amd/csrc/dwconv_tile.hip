@@ -97,17 +97,15 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
 #pragma unroll
             for (int o = 0; o < 4; ++o) acc[b][o] = 0.f;
 
+        // window rows are read one ahead of their use and the sums pinned after every row (see pin_registers)
+        float nxt[4 * NV];
+        load_window_row<NV>(base, nxt);
 #pragma unroll
         for (int wr = 0; wr < WIN_ROWS; ++wr) {
             float win[4 * NV];
 #pragma unroll
-            for (int v = 0; v < NV; ++v) {
-                const float4 q = *reinterpret_cast<const float4 *>(base + wr * p.st.pitch + 4 * v);
-                win[4 * v + 0] = q.x;
-                win[4 * v + 1] = q.y;
-                win[4 * v + 2] = q.z;
-                win[4 * v + 3] = q.w;
-            }
+            for (int i = 0; i < 4 * NV; ++i) win[i] = nxt[i];
+            if (wr + 1 < WIN_ROWS) load_window_row<NV>(base + (wr + 1) * p.st.pitch, nxt);
 #pragma unroll
             for (int b = 0; b < BH; ++b) {
                 const int ty = wr - b * S;
@@ -118,6 +116,7 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
                     for (int o = 0; o < 4; ++o)
                         acc[b][o] = fmaf(win[o * S + tx], tapv[ty * K + tx], acc[b][o]);
             }
+            pin_registers(acc);
         }
 
         const int ox = 4 * cb;
@@ -182,15 +181,14 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
 #pragma unroll
             for (int o = 0; o < 4; ++o) acc[b][o] = 0.f;
 
+        float nxt[NW];
+        load_window_row2<NW / 2>(base, nxt);
 #pragma unroll
         for (int wr = 0; wr < WIN_ROWS; ++wr) {
             float win[NW];
 #pragma unroll
-            for (int v = 0; v < NW / 2; ++v) {
-                const float2 q = *reinterpret_cast<const float2 *>(base + wr * p.st.pitch + 2 * v);
-                win[2 * v] = q.x;
-                win[2 * v + 1] = q.y;
-            }
+            for (int i = 0; i < NW; ++i) win[i] = nxt[i];
+            if (wr + 1 < WIN_ROWS) load_window_row2<NW / 2>(base + (wr + 1) * p.st.pitch, nxt);
 #pragma unroll
             for (int bq = 0; bq < BQ; ++bq)
 #pragma unroll
@@ -211,6 +209,7 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
                                     fmaf(win[xq + rx + ax], tapv[fy * K + fx], acc[2 * bq + r][2 * xq + rx]);
                             }
                 }
+            pin_registers(acc);
         }
 
         const int ox = 4 * cb;

@@ -185,6 +185,32 @@ __device__ __forceinline__ void pin_registers(float (&a)[R][C])
         for (int c = 0; c < C; ++c) asm volatile("" : "+v"(a[r][c]) : : "memory");
 }
 
+// NV aligned float4s of an LDS row into registers.
+template <int NV>
+__device__ __forceinline__ void load_window_row(const float *row, float (&w)[4 * NV])
+{
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const float4 q = reinterpret_cast<const float4 *>(row)[v];
+        w[4 * v + 0] = q.x;
+        w[4 * v + 1] = q.y;
+        w[4 * v + 2] = q.z;
+        w[4 * v + 3] = q.w;
+    }
+}
+
+// NV2 aligned float2s of an LDS row into registers.
+template <int NV2>
+__device__ __forceinline__ void load_window_row2(const float *row, float (&w)[2 * NV2])
+{
+#pragma unroll
+    for (int v = 0; v < NV2; ++v) {
+        const float2 q = reinterpret_cast<const float2 *>(row)[v];
+        w[2 * v + 0] = q.x;
+        w[2 * v + 1] = q.y;
+    }
+}
+
 inline int floor_div(int a, int b)
 {
     int q = a / b;

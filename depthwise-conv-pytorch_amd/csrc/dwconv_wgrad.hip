@@ -185,17 +185,14 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
             for (int b = 0; b < BH; ++b)
 #pragma unroll
                 for (int o = 0; o < 4; ++o) xacc[b][o] = 0.f;
+            float nxt[4 * NV];
+            load_window_row<NV>(base + p.g_base, nxt);
 #pragma unroll
             for (int wr = 0; wr < WIN_ROWS; ++wr) {
                 float win[4 * NV];
 #pragma unroll
-                for (int v = 0; v < NV; ++v) {
-                    const float4 q = *reinterpret_cast<const float4 *>(base + p.g_base + wr * p.st.pitch + 4 * v);
-                    win[4 * v + 0] = q.x;
-                    win[4 * v + 1] = q.y;
-                    win[4 * v + 2] = q.z;
-                    win[4 * v + 3] = q.w;
-                }
+                for (int i = 0; i < 4 * NV; ++i) win[i] = nxt[i];
+                if (wr + 1 < WIN_ROWS) load_window_row<NV>(base + p.g_base + (wr + 1) * p.st.pitch, nxt);
                 const int gb = wr - PC;
                 if (gb >= 0 && gb < BH) {
 #pragma unroll
@@ -210,6 +207,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
 #pragma unroll
                         for (int o = 0; o < 4; ++o) xacc[b][o] = fmaf(win[o + tx], rot[ty * K + tx], xacc[b][o]);
                 }
+                pin_registers(xacc);
             }
             if (has_item) {
                 float *dst = p.gx + (plane0 + pl) * p.st.in_plane + ox;
@@ -229,17 +227,14 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
             }
         }
 
+        float nxt[4 * NV];
+        load_window_row<NV>(base, nxt);
 #pragma unroll
         for (int wr = 0; wr < WIN_ROWS; ++wr) {
             float win[4 * NV];
 #pragma unroll
-            for (int v = 0; v < NV; ++v) {
-                const float4 q = *reinterpret_cast<const float4 *>(base + wr * p.st.pitch + 4 * v);
-                win[4 * v + 0] = q.x;
-                win[4 * v + 1] = q.y;
-                win[4 * v + 2] = q.z;
-                win[4 * v + 3] = q.w;
-            }
+            for (int i = 0; i < 4 * NV; ++i) win[i] = nxt[i];
+            if (wr + 1 < WIN_ROWS) load_window_row<NV>(base + (wr + 1) * p.st.pitch, nxt);
 #pragma unroll
             for (int b = 0; b < BH; ++b) {
                 const int ty = wr - b * S;
@@ -250,6 +245,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
                     for (int o = 0; o < 4; ++o)
                         acc[ty * K + tx] = fmaf(g[b][o], win[o * S + tx], acc[ty * K + tx]);
             }
+            pin_registers(acc);
         }
     }
 
