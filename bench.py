@@ -25,6 +25,7 @@ for _p in (ROOT, os.path.join(ROOT, "depthwise-conv-pytorch_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X fp32 vector peak (packed); the kernels use unpacked FMAs (half of it)
 
 # (C, H_in, k, stride), batch 128, padding k//2
 EFFNET_B0 = [
@@ -286,6 +287,9 @@ def main():
                                f"{len(calls)} C-ABI calls per step",
                    "layers": [l.name for l in layers], "algorithmic_bytes_per_step": step_bytes},
         "frac_of_hbm_roofline": round(step_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, 4),
+        # arithmetic side (matters for the 7x7-filter shapes): nominal FLOPs 2*|y|*k^2 per pass, three passes
+        "tflops": round(3 * sum(l.flops for l in layers) / ms_per_step / 1e9, 2),
+        "frac_of_fp32_vector_peak": round(3 * sum(l.flops for l in layers) / ms_per_step / 1e9 / FP32_VECTOR_PEAK_TFLOPS, 4),
         "host_wall_ms_per_step": round(wall_ms, 4),
         "sum_of_launch_us": round(sum(r["us"] for r in rows), 1),
         "roofline": roofline,

@@ -254,7 +254,15 @@ template <int W, int K>
 int launch_small_down_any(SmallPlan &p, int S, bool rot, hipStream_t stream)
 {
     constexpr int BH1 = W == 7 ? 7 : 2;
-    if (S == 1) return rot ? launch_small_down<W, K, 1, true, BH1>(p, stream) : launch_small_down<W, K, 1, false, BH1>(p, stream);
+    if (S == 1) {
+        if constexpr (W == 7) {
+            // one lane per plane needs 64 planes per wavefront: with few planes that leaves most CUs idle,
+            // so give a plane four lanes (two rows each) instead
+            if (p.planes < 64l * 2048)
+                return rot ? launch_small_down<W, K, 1, true, 2>(p, stream) : launch_small_down<W, K, 1, false, 2>(p, stream);
+        }
+        return rot ? launch_small_down<W, K, 1, true, BH1>(p, stream) : launch_small_down<W, K, 1, false, BH1>(p, stream);
+    }
     if constexpr (W % 2 == 0) {
         if (S == 2 && !rot) return launch_small_down<W, K, 2, false, 1>(p, stream);
     }
