@@ -57,7 +57,9 @@ __device__ __forceinline__ void run_commit(const float *__restrict__ g, float *l
     if (tail < n) lds[tail] = g[tail];
 }
 
-template <int W, int K, int S, int BH, bool GX>
+// PF: the runs of the next image are fetched into registers while the current image is processed
+// (56 registers; dropped for the 7x7 filter, whose sums and taps already take 98).
+template <int W, int K, int S, int BH, bool GX, bool PF = (K < 7)>
 __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -92,7 +94,7 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
     if constexpr (GX) load_taps<KK, true>(p.taps, c0 + pl, tapv);
 
     float4 rx[kRunRegs], rg[kRunRegs];
-    {
+    if constexpr (PF) {
         const long plane0 = static_cast<long>(n0) * p.channel + c0;
         run_fetch(p.x + plane0 * in_plane, nx, rx);
         run_fetch(p.gy + plane0 * out_plane, ng, rg);
@@ -101,10 +103,14 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
     for (int n = n0; n < n1; ++n) {
         const long plane0 = static_cast<long>(n) * p.channel + c0;
         if (n != n0) __syncthreads();  // the previous image is done with the LDS runs
+        if constexpr (!PF) {
+            run_fetch(p.x + plane0 * in_plane, nx, rx);
+            run_fetch(p.gy + plane0 * out_plane, ng, rg);
+        }
         run_commit(p.x + plane0 * in_plane, lds_x, nx, rx);
         run_commit(p.gy + plane0 * out_plane, lds_g, ng, rg);
         __syncthreads();
-        if (n + 1 < n1) {
+        if (PF && n + 1 < n1) {
             const long plane1 = plane0 + p.channel;
             run_fetch(p.x + plane1 * in_plane, nx, rx);
             run_fetch(p.gy + plane1 * out_plane, ng, rg);
