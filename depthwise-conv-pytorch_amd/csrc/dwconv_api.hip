@@ -320,7 +320,9 @@ size_t dwconv2d_backward_kernel_workspace_bytes(int batch, int channel, int in_h
     if (batch <= 0 || channel <= 0 || kernel_h < 1 || kernel_w < 1 || down_h < 1 || down_w < 1) return 0;
     const WgradGeometry g{batch, channel, in_h, in_w, out_h, out_w, kernel_h, kernel_w,
                           down_h, down_w, pad_h, pad_w};
-    return elem_size == 8 ? wgrad_workspace<double>(g) : wgrad_workspace<float>(g);
+    if (elem_size == 8) return wgrad_workspace<double>(g);
+    if (elem_size == 2) return wgrad_workspace<half_t>(g);
+    return wgrad_workspace<float>(g);
 }
 
 int dwconv2d_backward_kernel_f32(const float *input, const float *out_grad, float *kernel_grad,
@@ -344,6 +346,39 @@ int dwconv2d_backward_kernel_f64(const double *input, const double *out_grad, do
                              in_h, in_w, out_h, out_w, kernel_h, kernel_w, up_h, up_w, down_h, down_w,
                              pad_h, pad_w, stream);
 }
+
+// ---- 16-bit element types (storage passed as unsigned short) ----
+#define DWCONV_16BIT_ENTRY_POINTS(SUFFIX, TYPE)                                                                       \
+    int dwconv2d_##SUFFIX(const unsigned short *input, const unsigned short *kernel, unsigned short *out, int batch,   \
+                          int channel, int in_h, int in_w, int kernel_h, int kernel_w, int up_h, int up_w, int down_h, \
+                          int down_w, int pad_h0, int pad_h1, int pad_w0, int pad_w1, int forward, void *stream)       \
+    {                                                                                                                  \
+        return dwconv2d_any<TYPE>(reinterpret_cast<const TYPE *>(input), reinterpret_cast<const TYPE *>(kernel),       \
+                                  reinterpret_cast<TYPE *>(out), batch, channel, in_h, in_w, kernel_h, kernel_w, up_h, \
+                                  up_w, down_h, down_w, pad_h0, pad_h1, pad_w0, pad_w1, forward, stream);              \
+    }                                                                                                                  \
+    int dwconv2d_small_##SUFFIX(const unsigned short *input, const unsigned short *kernel, unsigned short *out,        \
+                                int batch, int channel, int in_h, int in_w, int kernel_h, int kernel_w, int up_h,      \
+                                int up_w, int down_h, int down_w, int pad_h, int pad_w, int forward, void *stream)     \
+    {                                                                                                                  \
+        return dwconv2d_small_any<TYPE>(reinterpret_cast<const TYPE *>(input), reinterpret_cast<const TYPE *>(kernel), \
+                                        reinterpret_cast<TYPE *>(out), batch, channel, in_h, in_w, kernel_h, kernel_w, \
+                                        up_h, up_w, down_h, down_w, pad_h, pad_w, forward, stream);                    \
+    }                                                                                                                  \
+    int dwconv2d_backward_kernel_##SUFFIX(const unsigned short *input, const unsigned short *out_grad,                 \
+                                          unsigned short *kernel_grad, void *workspace, size_t workspace_bytes,        \
+                                          int batch, int channel, int in_h, int in_w, int out_h, int out_w,            \
+                                          int kernel_h, int kernel_w, int up_h, int up_w, int down_h, int down_w,      \
+                                          int pad_h, int pad_w, void *stream)                                          \
+    {                                                                                                                  \
+        return wgrad_any<TYPE>(reinterpret_cast<const TYPE *>(input), reinterpret_cast<const TYPE *>(out_grad),        \
+                               reinterpret_cast<TYPE *>(kernel_grad), workspace, workspace_bytes, batch, channel,      \
+                               in_h, in_w, out_h, out_w, kernel_h, kernel_w, up_h, up_w, down_h, down_w, pad_h, pad_w, \
+                               stream);                                                                                \
+    }
+DWCONV_16BIT_ENTRY_POINTS(f16, half_t)
+DWCONV_16BIT_ENTRY_POINTS(bf16, bf16_t)
+#undef DWCONV_16BIT_ENTRY_POINTS
 
 int dwconv2d_backward_f32(const float *input, const float *out_grad, const float *kernel, float *in_grad,
                           float *kernel_grad, void *workspace, size_t workspace_bytes, int batch, int channel,

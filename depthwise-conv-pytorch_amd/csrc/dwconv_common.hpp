@@ -11,6 +11,46 @@
 
 namespace dwconv {
 
+// ---- element types at the boundary --------------------------------------------------------------------
+// fp16 and bf16 tensors are read and written as such; all arithmetic and every partial sum is fp32
+// (the reference accumulates halves in half, torch_dwconv/dwconv_kernel.cu:749 `AT_DISPATCH_..._AND_HALF`
+// with `scalar_t v`; fp32 accumulation is strictly more accurate).
+using half_t = _Float16;
+struct bf16_t {
+    uint16_t bits;
+};
+
+template <typename T>
+struct Io {
+    using acc_t = float;
+    __host__ __device__ static float in(T v) { return static_cast<float>(v); }
+    __host__ __device__ static T out(float v) { return static_cast<T>(v); }
+};
+template <>
+struct Io<double> {
+    using acc_t = double;
+    __host__ __device__ static double in(double v) { return v; }
+    __host__ __device__ static double out(double v) { return v; }
+};
+template <>
+struct Io<bf16_t> {
+    using acc_t = float;
+    __host__ __device__ static float in(bf16_t v)
+    {
+        union { uint32_t u; float f; } c;
+        c.u = static_cast<uint32_t>(v.bits) << 16;
+        return c.f;
+    }
+    __host__ __device__ static bf16_t out(float v)
+    {
+        union { uint32_t u; float f; } c;
+        c.f = v;
+        if ((c.u & 0x7fffffffu) > 0x7f800000u) return bf16_t{static_cast<uint16_t>((c.u >> 16) | 0x40u)};  // NaN stays NaN
+        c.u += 0x7fffu + ((c.u >> 16) & 1u);  // round to nearest even
+        return bf16_t{static_cast<uint16_t>(c.u >> 16)};
+    }
+};
+
 // Geometry of one up/FIR/down call on dense NCHW planes.  The same fields as the
 // reference's DWConv2dKernelParams (torch_dwconv/dwconv_kernel.cu:42-67), with the
 // batch and channel extents folded into `planes` where a kernel does not need them.

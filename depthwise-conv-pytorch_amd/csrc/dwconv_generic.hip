@@ -30,7 +30,7 @@ __global__ __launch_bounds__(kDirectThreads) void fir_direct_kernel(
         const int c = static_cast<int>(plane % g.channel);
         const T *src = in + plane * g.in_h * g.in_w;
         const T *f = taps + static_cast<long>(c) * g.kernel_h * g.kernel_w;
-        T acc = 0;
+        typename Io<T>::acc_t acc = 0;
         for (int ty = 0; ty < g.kernel_h; ++ty) {
             const int uy = oy * g.down_h - g.pad_h0 + ty;
             if (uy < 0 || uy % g.up_h != 0) continue;
@@ -43,10 +43,10 @@ __global__ __launch_bounds__(kDirectThreads) void fir_direct_kernel(
                 if (ix >= g.in_w) continue;
                 const T fv = g.forward ? f[ty * g.kernel_w + tx]
                                        : f[(g.kernel_h - 1 - ty) * g.kernel_w + (g.kernel_w - 1 - tx)];
-                acc += fv * src[static_cast<long>(iy) * g.in_w + ix];
+                acc += Io<T>::in(fv) * Io<T>::in(src[static_cast<long>(iy) * g.in_w + ix]);
             }
         }
-        out[idx] = acc;
+        out[idx] = Io<T>::out(acc);
     }
 }
 
@@ -65,10 +65,11 @@ __device__ inline T wave_sum(T v)
 // K*K partial sums.  (Sum of torch_dwconv/dwconv_kernel.cu:269-297.)
 template <typename T>
 __global__ __launch_bounds__(kDirectThreads) void wgrad_direct_partial_kernel(
-    const T *__restrict__ in, const T *__restrict__ gy, T *__restrict__ partial,
+    const T *__restrict__ in, const T *__restrict__ gy, typename Io<T>::acc_t *__restrict__ partial,
     const WgradGeometry g, const int chunks, const int images_per_chunk)
 {
-    __shared__ T wave_part[kDirectThreads / 64];
+    using A = typename Io<T>::acc_t;
+    __shared__ A wave_part[kDirectThreads / 64];
     const int c = blockIdx.x;
     const int chunk = blockIdx.y;
     const int n0 = chunk * images_per_chunk;
@@ -77,7 +78,7 @@ __global__ __launch_bounds__(kDirectThreads) void wgrad_direct_partial_kernel(
     const int taps = g.kernel_h * g.kernel_w;
     for (int tap = 0; tap < taps; ++tap) {
         const int i = tap / g.kernel_w, j = tap - i * g.kernel_w;
-        T acc = 0;
+        A acc = 0;
         for (int n = n0; n < n1; ++n) {
             const long plane = static_cast<long>(n) * g.channel + c;
             const T *x = in + plane * g.in_h * g.in_w;
@@ -87,14 +88,14 @@ __global__ __launch_bounds__(kDirectThreads) void wgrad_direct_partial_kernel(
                 const int iy = oy * g.down_h - g.pad_h + i;
                 const int ix = ox * g.down_w - g.pad_w + j;
                 if (iy >= 0 && iy < g.in_h && ix >= 0 && ix < g.in_w)
-                    acc += d[p] * x[static_cast<long>(iy) * g.in_w + ix];
+                    acc += Io<T>::in(d[p]) * Io<T>::in(x[static_cast<long>(iy) * g.in_w + ix]);
             }
         }
         acc = wave_sum(acc);
         if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = acc;
         __syncthreads();
         if (threadIdx.x == 0) {
-            T s = wave_part[0];
+            A s = wave_part[0];
             for (int w = 1; w < kDirectThreads / 64; ++w) s += wave_part[w];
             partial[(static_cast<long>(c) * chunks + chunk) * taps + tap] = s;
         }
@@ -104,16 +105,16 @@ __global__ __launch_bounds__(kDirectThreads) void wgrad_direct_partial_kernel(
 
 // Pass 2: one lane per (c, tap) adds the chunk partials front to back.
 template <typename T>
-__global__ void wgrad_direct_final_kernel(const T *__restrict__ partial, T *__restrict__ gw,
+__global__ void wgrad_direct_final_kernel(const typename Io<T>::acc_t *__restrict__ partial, T *__restrict__ gw,
                                           const int channel_taps, const int taps, const int chunks)
 {
     const int e = blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= channel_taps) return;
     const int c = e / taps, tap = e - c * taps;
-    const T *p = partial + static_cast<long>(c) * chunks * taps + tap;
-    T s = 0;
+    const typename Io<T>::acc_t *p = partial + static_cast<long>(c) * chunks * taps + tap;
+    typename Io<T>::acc_t s = 0;
     for (int k = 0; k < chunks; ++k) s += p[static_cast<long>(k) * taps];
-    gw[e] = s;
+    gw[e] = Io<T>::out(s);
 }
 
 __global__ void fill_zero_kernel(uint32_t *p, const size_t words)
@@ -152,14 +153,14 @@ int launch_fir_direct(const T *in, const T *taps, T *out, const Geometry &g, hip
     if (blocks > 1 << 20) blocks = 1 << 20;
     hipLaunchKernelGGL(fir_direct_kernel<T>, dim3(static_cast<unsigned>(blocks)),
                        dim3(kDirectThreads), 0, stream, in, taps, out, g, total);
-    note_variant("direct_%s", sizeof(T) == 4 ? "f32" : "f64");
+    note_variant("direct_%s", sizeof(T) == 4 ? "f32" : (sizeof(T) == 8 ? "f64" : "16"));
     return check_launch("fir_direct_kernel");
 }
 
 template <typename T>
 size_t wgrad_direct_workspace(const WgradGeometry &g)
 {
-    return static_cast<size_t>(g.channel) * direct_chunks(g) * g.kernel_h * g.kernel_w * sizeof(T);
+    return static_cast<size_t>(g.channel) * direct_chunks(g) * g.kernel_h * g.kernel_w * sizeof(typename Io<T>::acc_t);
 }
 
 template <typename T>
@@ -173,7 +174,7 @@ int launch_wgrad_direct(const T *in, const T *gy, T *gw, void *ws, size_t ws_byt
     const int chunks = direct_chunks(g);
     const int per = ceil_div(g.batch, chunks);
     const int taps = g.kernel_h * g.kernel_w;
-    T *partial = static_cast<T *>(ws);
+    auto *partial = static_cast<typename Io<T>::acc_t *>(ws);
     hipLaunchKernelGGL(wgrad_direct_partial_kernel<T>, dim3(g.channel, chunks), dim3(kDirectThreads),
                        0, stream, in, gy, partial, g, chunks, per);
     int rc = check_launch("wgrad_direct_partial_kernel");
@@ -181,12 +182,20 @@ int launch_wgrad_direct(const T *in, const T *gy, T *gw, void *ws, size_t ws_byt
     const int total = g.channel * taps;
     hipLaunchKernelGGL(wgrad_direct_final_kernel<T>, dim3(ceil_div(total, 256)), dim3(256), 0, stream,
                        partial, gw, total, taps, chunks);
-    note_variant("wgrad_direct_%s", sizeof(T) == 4 ? "f32" : "f64");
+    note_variant("wgrad_direct_%s", sizeof(T) == 4 ? "f32" : (sizeof(T) == 8 ? "f64" : "16"));
     return check_launch("wgrad_direct_final_kernel");
 }
 
 template int launch_fir_direct<float>(const float *, const float *, float *, const Geometry &,
                                       hipStream_t);
+template int launch_fir_direct<half_t>(const half_t *, const half_t *, half_t *, const Geometry &, hipStream_t);
+template int launch_fir_direct<bf16_t>(const bf16_t *, const bf16_t *, bf16_t *, const Geometry &, hipStream_t);
+template size_t wgrad_direct_workspace<half_t>(const WgradGeometry &);
+template size_t wgrad_direct_workspace<bf16_t>(const WgradGeometry &);
+template int launch_wgrad_direct<half_t>(const half_t *, const half_t *, half_t *, void *, size_t,
+                                         const WgradGeometry &, hipStream_t);
+template int launch_wgrad_direct<bf16_t>(const bf16_t *, const bf16_t *, bf16_t *, void *, size_t,
+                                         const WgradGeometry &, hipStream_t);
 template int launch_fir_direct<double>(const double *, const double *, double *, const Geometry &,
                                        hipStream_t);
 template size_t wgrad_direct_workspace<float>(const WgradGeometry &);

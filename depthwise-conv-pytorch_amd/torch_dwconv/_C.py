@@ -34,22 +34,23 @@ _lib.dwconv_out_size.restype = _i
 _lib.dwconv_out_size.argtypes = [_i] * 6
 _lib.dwconv_use_dwconv2d_small.restype = _i
 _lib.dwconv_use_dwconv2d_small.argtypes = [_i] * 10
-for _name in ("dwconv2d_f32", "dwconv2d_f64"):
+for _name in ("dwconv2d_f32", "dwconv2d_f64", "dwconv2d_f16", "dwconv2d_bf16"):
     getattr(_lib, _name).restype = _i
     getattr(_lib, _name).argtypes = [_p, _p, _p] + [_i] * 15 + [_p]
-for _name in ("dwconv2d_small_f32", "dwconv2d_small_f64"):
+for _name in ("dwconv2d_small_f32", "dwconv2d_small_f64", "dwconv2d_small_f16", "dwconv2d_small_bf16"):
     getattr(_lib, _name).restype = _i
     getattr(_lib, _name).argtypes = [_p, _p, _p] + [_i] * 13 + [_p]
 _lib.dwconv2d_backward_kernel_workspace_bytes.restype = _z
 _lib.dwconv2d_backward_kernel_workspace_bytes.argtypes = [_i] * 13
-for _name in ("dwconv2d_backward_kernel_f32", "dwconv2d_backward_kernel_f64"):
+for _name in ("dwconv2d_backward_kernel_f32", "dwconv2d_backward_kernel_f64", "dwconv2d_backward_kernel_f16",
+              "dwconv2d_backward_kernel_bf16"):
     getattr(_lib, _name).restype = _i
     getattr(_lib, _name).argtypes = [_p, _p, _p, _p, _z] + [_i] * 14 + [_p]
 
 _lib.dwconv2d_backward_f32.restype = _i
 _lib.dwconv2d_backward_f32.argtypes = [_p, _p, _p, _p, _p, _p, _z] + [_i] * 12 + [_p]
 
-_SUFFIX = {torch.float32: "f32", torch.float64: "f64"}
+_SUFFIX = {torch.float32: "f32", torch.float64: "f64", torch.float16: "f16", torch.bfloat16: "bf16"}
 
 
 def version():
@@ -69,7 +70,7 @@ def _check_cuda(t, name):
 def _suffix(*tensors):
     dtype = tensors[0].dtype
     if dtype not in _SUFFIX:
-        raise RuntimeError(f"torch_dwconv supports float32 and float64 tensors, got {dtype}")
+        raise RuntimeError(f"torch_dwconv supports float32, float64, float16 and bfloat16 tensors, got {dtype}")
     for t in tensors[1:]:
         if t.dtype != dtype:
             raise RuntimeError(f"torch_dwconv needs tensors of one dtype, got {dtype} and {t.dtype}")

@@ -100,7 +100,7 @@ int dwconv2d_small_f64(const double *input, const double *kernel, double *out,
  * geometry (0 is possible).  The reference allocates its own zero-filled
  * result and accumulates into it with atomics (dwconv_kernel.cu:1026, :304,
  * :583); here the caller lends a workspace for per-workgroup partial sums that
- * a second kernel adds up in a fixed order.  `elem_size` is 4 or 8. */
+ * a second kernel adds up in a fixed order.  `elem_size` is 2 (fp16/bf16), 4 or 8. */
 size_t dwconv2d_backward_kernel_workspace_bytes(int batch, int channel,
                                                 int in_h, int in_w,
                                                 int out_h, int out_w,
@@ -130,6 +130,38 @@ int dwconv2d_backward_kernel_f64(const double *input, const double *out_grad,
                                  int kernel_h, int kernel_w, int up_h, int up_w,
                                  int down_h, int down_w, int pad_h, int pad_w,
                                  void *stream);
+
+/* fp16 (`_f16`) and bfloat16 (`_bf16`) twins of the three operations above: tensors hold 16-bit elements
+ * (passed as `unsigned short` storage), every product and partial sum is fp32, results are rounded to
+ * nearest-even once when stored.  The reference dispatches half for `_C.dwconv2d`, `_C.dwconv2d_small` and
+ * the general grad-weight kernel (torch_dwconv/dwconv_kernel.cu:749, :860, :999) and accumulates in half.
+ * Workspace for grad-weight: dwconv2d_backward_kernel_workspace_bytes(..., elem_size = 2). */
+int dwconv2d_f16(const unsigned short *input, const unsigned short *kernel, unsigned short *out,
+                 int batch, int channel, int in_h, int in_w, int kernel_h, int kernel_w,
+                 int up_h, int up_w, int down_h, int down_w, int pad_h0, int pad_h1,
+                 int pad_w0, int pad_w1, int forward, void *stream);
+int dwconv2d_bf16(const unsigned short *input, const unsigned short *kernel, unsigned short *out,
+                  int batch, int channel, int in_h, int in_w, int kernel_h, int kernel_w,
+                  int up_h, int up_w, int down_h, int down_w, int pad_h0, int pad_h1,
+                  int pad_w0, int pad_w1, int forward, void *stream);
+int dwconv2d_small_f16(const unsigned short *input, const unsigned short *kernel,
+                       unsigned short *out, int batch, int channel, int in_h, int in_w,
+                       int kernel_h, int kernel_w, int up_h, int up_w, int down_h, int down_w,
+                       int pad_h, int pad_w, int forward, void *stream);
+int dwconv2d_small_bf16(const unsigned short *input, const unsigned short *kernel,
+                        unsigned short *out, int batch, int channel, int in_h, int in_w,
+                        int kernel_h, int kernel_w, int up_h, int up_w, int down_h, int down_w,
+                        int pad_h, int pad_w, int forward, void *stream);
+int dwconv2d_backward_kernel_f16(const unsigned short *input, const unsigned short *out_grad,
+                                 unsigned short *kernel_grad, void *workspace,
+                                 size_t workspace_bytes, int batch, int channel, int in_h, int in_w,
+                                 int out_h, int out_w, int kernel_h, int kernel_w, int up_h, int up_w,
+                                 int down_h, int down_w, int pad_h, int pad_w, void *stream);
+int dwconv2d_backward_kernel_bf16(const unsigned short *input, const unsigned short *out_grad,
+                                  unsigned short *kernel_grad, void *workspace,
+                                  size_t workspace_bytes, int batch, int channel, int in_h, int in_w,
+                                  int out_h, int out_w, int kernel_h, int kernel_w, int up_h, int up_w,
+                                  int down_h, int down_w, int pad_h, int pad_w, void *stream);
 
 /* Both gradients of one layer in one call: in_grad (batch*channel*in_h*in_w) and kernel_grad
  * (channel*kernel_h*kernel_w), from the forward input, the output gradient and the taps.

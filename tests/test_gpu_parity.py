@@ -320,6 +320,34 @@ def test_c_entry_points_directly(dw, gpu):
         _C.dwconv2d(x, torch.randn(3, 1, 3, 3, device=gpu), 1, 1, 1, 1, 1, 1, 1, 1, True)
 
 
+HALF_SHAPES = [(2, 6, 14, 14, 3, 1, 1), (2, 5, 28, 28, 5, 2, 2), (2, 4, 56, 56, 3, 1, 1), (2, 3, 57, 59, 5, 2, 2),
+               (1, 8, 7, 7, 5, 1, 2), (2, 4, 112, 112, 3, 2, 1), (1, 2, 33, 35, 7, 1, 3), (2, 8, 14, 14, 5, 2, 2)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("shape", HALF_SHAPES, ids=shape_id)
+def test_half_precision_io(dw, gpu, shape, dtype):
+    """16-bit tensors in and out, fp32 arithmetic inside: the only error is the final rounding of each result.
+    The oracle runs in fp64 on the already rounded inputs; tolerance = one rounding step of the 16-bit format
+    (2^-11 for fp16, 2^-8 for bf16) plus the fp32 bounds used elsewhere."""
+    n, c, h, w, k, s, p = shape
+    x, wt, gy = (t.to(dtype) for t in make_inputs(shape, seed=17))
+    y, gx, gw, variant = run_three_passes(dw, x.to(gpu), wt.to(gpu), gy.to(gpu), s, p)
+    _announce(shape_id(shape), str(dtype), variant)
+    assert y.dtype == dtype and gx.dtype == dtype and gw.dtype == dtype
+    xr, wr, gr = (_np(t.double()) for t in (x, wt, gy))
+    step = 2.0 ** -11 if dtype == torch.float16 else 2.0 ** -8
+    y_ref = oracle.forward(xr, wr, s, p)
+    gx_ref = oracle.grad_input(gr, wr, (h, w), s, p)
+    gw_ref = oracle.grad_weight(xr, gr, wt.shape, s, p)
+    np.testing.assert_allclose(_np(y.double()), y_ref, rtol=step, atol=1e-5 + step * 1e-2)
+    np.testing.assert_allclose(_np(gx.double()), gx_ref, rtol=step, atol=1e-5 + step * 1e-2)
+    np.testing.assert_allclose(_np(gw.double()), gw_ref, rtol=step + 1e-4, atol=(step + 1e-4) * float(np.abs(gw_ref).max()))
+    # bit-identical grad-weight from run to run here too
+    _, _, gw2, _ = run_three_passes(dw, x.to(gpu), wt.to(gpu), gy.to(gpu), s, p)
+    assert torch.equal(gw, gw2)
+
+
 def test_combined_backward_entry_point(dw, gpu):
     """dwconv2d_backward: fused kernels where they exist, the two separate passes otherwise; errors as status codes."""
     from torch_dwconv import _C
