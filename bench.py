@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the depthwise conv2d hot path on one MI355X.
 
-Workload (BASELINE.json, configs[2]): the 12 depthwise layers of EfficientNet-B0,
+Workload: the 12 depthwise layers of EfficientNet-B0,
 fp32 NCHW, batch 128, padding k//2.  One "step" = forward of layers 1..12, then
 grad-input and grad-weight of layers 12..1 (training order): 24 calls into the
 C ABI of libdwconv_hip (12 forward, 12 combined backward; --separate-backward
@@ -9,7 +9,7 @@ makes it 36), all tensors resident in HBM before the clock starts.
 
 Prints one JSON line.  `value` is achieved HBM GB/s = algorithmic bytes of the
 step (every tensor of every pass touched exactly once: 12(|x|+|y|+|w|) bytes per
-layer) / step time; `ms_per_step` carries the fwd+bwd time itself.
+layer, 6 per element with --dtype f16/bf16) / step time; `ms_per_step` carries the fwd+bwd time itself.
 """
 import argparse
 import ctypes
@@ -47,22 +47,27 @@ WORKLOADS = {
 class Layer:
     """Device tensors and the three C-ABI calls of one depthwise layer."""
 
-    def __init__(self, shape, lib, torch, dev, gen):
+    def __init__(self, shape, lib, torch, dev, gen, dtype="f32"):
         n, c, h, w, k, s, p = shape
+        tdtype = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype]
+        es = 4 if dtype == "f32" else 2
+        self.fn_fir = getattr(lib, "dwconv2d_" + dtype)
+        self.fn_wgrad = getattr(lib, "dwconv2d_backward_kernel_" + dtype)
+        self.fn_bwd = getattr(lib, "dwconv2d_backward_" + dtype)
         self.shape = shape
         self.lib = lib
         oh, ow = (h + 2 * p - k) // s + 1, (w + 2 * p - k) // s + 1
         self.geom = (n, c, h, w, oh, ow, k, s, p)
-        self.x = torch.randn(n, c, h, w, generator=gen).to(dev)
-        self.w = (torch.randn(c, 1, k, k, generator=gen) / k).to(dev)
-        self.gy = torch.randn(n, c, oh, ow, generator=gen).to(dev)
-        self.y = torch.empty(n, c, oh, ow, device=dev)
+        self.x = torch.randn(n, c, h, w, generator=gen).to(dev, tdtype)
+        self.w = (torch.randn(c, 1, k, k, generator=gen) / k).to(dev, tdtype)
+        self.gy = torch.randn(n, c, oh, ow, generator=gen).to(dev, tdtype)
+        self.y = torch.empty(n, c, oh, ow, device=dev, dtype=tdtype)
         self.gx = torch.empty_like(self.x)
         self.gw = torch.empty_like(self.w)
-        self.ws_bytes = lib.dwconv2d_backward_kernel_workspace_bytes(n, c, h, w, oh, ow, k, k, s, s, p, p, 4)
+        self.ws_bytes = lib.dwconv2d_backward_kernel_workspace_bytes(n, c, h, w, oh, ow, k, k, s, s, p, p, es)
         self.ws = torch.empty(max(self.ws_bytes, 16), dtype=torch.uint8, device=dev)
         nx, ny, nw = n * c * h * w, n * c * oh * ow, c * k * k
-        self.bytes = {"fwd": 4 * (nx + ny + nw), "gx": 4 * (ny + nx + nw), "gw": 4 * (nx + ny + nw)}
+        self.bytes = {"fwd": es * (nx + ny + nw), "gx": es * (ny + nx + nw), "gw": es * (nx + ny + nw)}
         # the combined backward call is credited with the bytes of the two passes it replaces
         self.bytes["bwd"] = self.bytes["gx"] + self.bytes["gw"]
         self.flops = 2 * ny * k * k
@@ -76,25 +81,25 @@ class Layer:
 
     def fwd(self, stream):
         n, c, h, w, oh, ow, k, s, p = self.geom
-        self._check(self.lib.dwconv2d_f32(self.x.data_ptr(), self.w.data_ptr(), self.y.data_ptr(), n, c, h, w, k, k,
+        self._check(self.fn_fir(self.x.data_ptr(), self.w.data_ptr(), self.y.data_ptr(), n, c, h, w, k, k,
                                           1, 1, s, s, p, p, p, p, 1, stream))
 
     def bwd_input(self, stream):
         n, c, h, w, oh, ow, k, s, p = self.geom
         g = self.g_pad
-        self._check(self.lib.dwconv2d_f32(self.gy.data_ptr(), self.w.data_ptr(), self.gx.data_ptr(), n, c, oh, ow, k, k,
+        self._check(self.fn_fir(self.gy.data_ptr(), self.w.data_ptr(), self.gx.data_ptr(), n, c, oh, ow, k, k,
                                           s, s, 1, 1, g[0], g[1], g[2], g[3], 0, stream))
 
     def bwd_filter(self, stream):
         n, c, h, w, oh, ow, k, s, p = self.geom
-        self._check(self.lib.dwconv2d_backward_kernel_f32(
+        self._check(self.fn_wgrad(
             self.x.data_ptr(), self.gy.data_ptr(), self.gw.data_ptr(), self.ws.data_ptr(), self.ws_bytes,
             n, c, h, w, oh, ow, k, k, 1, 1, s, s, p, p, stream))
 
 
     def bwd(self, stream):
         n, c, h, w, oh, ow, k, s, p = self.geom
-        self._check(self.lib.dwconv2d_backward_f32(
+        self._check(self.fn_bwd(
             self.x.data_ptr(), self.gy.data_ptr(), self.w.data_ptr(), self.gx.data_ptr(), self.gw.data_ptr(),
             self.ws.data_ptr(), self.ws_bytes, n, c, h, w, oh, ow, k, k, s, s, p, p, stream))
 
@@ -172,6 +177,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="effnet_b0", choices=sorted(WORKLOADS))
     ap.add_argument("--batch", type=int, default=128)
+    ap.add_argument("--dtype", default="f32", choices=["f32", "f16", "bf16"],
+                    help="element type of the tensors (the headline metric is f32; 16-bit types accumulate in fp32)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-miopen", action="store_true")
     ap.add_argument("--separate-backward", action="store_true",
@@ -195,7 +202,7 @@ def main():
     lib = _C._lib
     shapes = WORKLOADS[args.workload](args.batch)
     gen = torch.Generator("cpu").manual_seed(0)
-    layers = [Layer(s, lib, torch, dev, gen) for s in shapes]
+    layers = [Layer(s, lib, torch, dev, gen, args.dtype) for s in shapes]
     calls = schedule(layers, args.separate_backward)
     stream_obj = torch.cuda.current_stream(dev)
     stream = ctypes.c_void_p(stream_obj.cuda_stream)
@@ -280,9 +287,10 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": args.dtype,
         "data": "synthetic",
-        "config": {"workload": f"{args.workload}: {len(layers)} depthwise layers, fp32 NCHW, batch {shapes[0][0]}, "
+        "config": {"workload": f"{args.workload}: {len(layers)} depthwise layers, "
+                               f"{'fp32' if args.dtype == 'f32' else args.dtype} NCHW, batch {shapes[0][0]}, "
                                "fwd + grad-input + grad-weight per layer, training order, "
                                f"{len(calls)} C-ABI calls per step",
                    "layers": [l.name for l in layers], "algorithmic_bytes_per_step": step_bytes},
@@ -306,7 +314,7 @@ def main():
             result["speedup_vs_miopen_native"] = round(sum(per_layer) / ms_per_step, 2)
         except Exception as e:  # the comparison is informative only
             result["miopen_native_ms_per_step"] = f"failed: {type(e).__name__}"
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.dtype == "f32":
         result["cpu_baseline"] = cpu_baseline(shapes, torch)
     print(json.dumps(result))
 

@@ -2,6 +2,8 @@
 // argument checks, kernel-family selection, error strings.
 #include "dwconv_common.hpp"
 
+#include <type_traits>
+
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -86,11 +88,11 @@ int run_fir(const T *in, const T *taps, T *out, const Geometry &g, hipStream_t s
         note_variant("empty");
         return DWCONV_OK;
     }
-    if constexpr (sizeof(T) == 4) {
+    if constexpr (!std::is_same<T, double>::value) {
         if (!force_generic()) {
-            int rc = try_launch_fir_small(in, taps, out, g, stream);
+            int rc = try_launch_fir_small<T>(in, taps, out, g, stream);
             if (rc >= 0) return rc;
-            rc = try_launch_fir_tiled(in, taps, out, g, stream);
+            rc = try_launch_fir_tiled<T>(in, taps, out, g, stream);
             if (rc >= 0) return rc;
         }
     }
@@ -163,7 +165,7 @@ template <typename T>
 size_t wgrad_workspace(const WgradGeometry &g)
 {
     size_t need = wgrad_direct_workspace<T>(g);
-    if constexpr (sizeof(T) == 4) {
+    if constexpr (!std::is_same<T, double>::value) {
         const size_t t = wgrad_tiled_workspace(g);
         if (t > need) need = t;
         const size_t sm = wgrad_small_workspace(g);
@@ -195,14 +197,14 @@ int wgrad_any(const T *in, const T *gy, T *gw, void *ws, size_t ws_bytes, int ba
         note_variant("zero");
         return launch_fill_zero(gw, static_cast<size_t>(taps) * sizeof(T), stream);
     }
-    if constexpr (sizeof(T) == 4) {
+    if constexpr (!std::is_same<T, double>::value) {
         if (!force_generic()) {
             if (wgrad_small_workspace(g) > 0) {
-                const int r = try_launch_wgrad_small(in, gy, gw, ws, ws_bytes, g, stream);
+                const int r = try_launch_wgrad_small<T>(in, gy, gw, ws, ws_bytes, g, stream);
                 if (r >= 0) return r;
             }
             if (wgrad_tiled_workspace(g) > 0) {
-                const int r = try_launch_wgrad_tiled(in, gy, gw, ws, ws_bytes, g, stream);
+                const int r = try_launch_wgrad_tiled<T>(in, gy, gw, ws, ws_bytes, g, stream);
                 if (r >= 0) return r;
             }
         }
@@ -211,9 +213,10 @@ int wgrad_any(const T *in, const T *gy, T *gw, void *ws, size_t ws_bytes, int ba
 }
 
 // Both gradients of one layer.  Fused kernels where they exist; otherwise the two separate passes.
-int backward_f32(const float *in, const float *gy, const float *taps, float *gx, float *gw, void *ws,
-                 size_t ws_bytes, int batch, int channel, int in_h, int in_w, int out_h, int out_w, int kernel_h,
-                 int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w, void *stream_)
+template <typename T>  // float, half_t or bf16_t
+int backward_any(const T *in, const T *gy, const T *taps, T *gx, T *gw, void *ws, size_t ws_bytes, int batch,
+                 int channel, int in_h, int in_w, int out_h, int out_w, int kernel_h, int kernel_w, int stride_h,
+                 int stride_w, int pad_h, int pad_w, void *stream_)
 {
     WgradGeometry g;
     int rc = make_wgrad_geometry(g, in, gy, gw, batch, channel, in_h, in_w, out_h, out_w, kernel_h, kernel_w, 1, 1,
@@ -227,21 +230,21 @@ int backward_f32(const float *in, const float *gy, const float *taps, float *gx,
     const bool has_work = 1ll * batch * channel * out_h * out_w > 0 && in_h > 0 && in_w > 0;
     if (has_work && !force_generic()) {
         if (taps == nullptr || gx == nullptr) return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");
-        rc = try_launch_bwd_small(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+        rc = try_launch_bwd_small<T>(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
         if (rc >= 0) return rc;
-        rc = try_launch_bwd_tiled(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+        rc = try_launch_bwd_tiled<T>(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
         if (rc >= 0) return rc;
-        rc = try_launch_bwd_s2(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+        rc = try_launch_bwd_s2<T>(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
         if (rc >= 0) return rc;
     }
     // grad-input as the transposed problem (torch_dwconv/dwconv.py:39-44, :61-64), then grad-weight
-    rc = dwconv2d_any<float>(gy, taps, gx, batch, channel, out_h, out_w, kernel_h, kernel_w, stride_h, stride_w, 1, 1,
+    rc = dwconv2d_any<T>(gy, taps, gx, batch, channel, out_h, out_w, kernel_h, kernel_w, stride_h, stride_w, 1, 1,
                              kernel_h - pad_h - 1, in_h - out_h * stride_h + pad_h, kernel_w - pad_w - 1,
                              in_w - out_w * stride_w + pad_w, 0, stream_);
     if (rc != DWCONV_OK) return rc;
     char first[sizeof(g_variant)];
     std::snprintf(first, sizeof(first), "%s", g_variant);
-    rc = wgrad_any<float>(in, gy, gw, ws, ws_bytes, batch, channel, in_h, in_w, out_h, out_w, kernel_h, kernel_w, 1, 1,
+    rc = wgrad_any<T>(in, gy, gw, ws, ws_bytes, batch, channel, in_h, in_w, out_h, out_w, kernel_h, kernel_w, 1, 1,
                           stride_h, stride_w, pad_h, pad_w, stream_);
     if (rc == DWCONV_OK) {
         char second[sizeof(g_variant)];
@@ -375,6 +378,18 @@ int dwconv2d_backward_kernel_f64(const double *input, const double *out_grad, do
                                reinterpret_cast<TYPE *>(kernel_grad), workspace, workspace_bytes, batch, channel,      \
                                in_h, in_w, out_h, out_w, kernel_h, kernel_w, up_h, up_w, down_h, down_w, pad_h, pad_w, \
                                stream);                                                                                \
+    }                                                                                                                  \
+    int dwconv2d_backward_##SUFFIX(const unsigned short *input, const unsigned short *out_grad,                        \
+                                   const unsigned short *kernel, unsigned short *in_grad,                              \
+                                   unsigned short *kernel_grad, void *workspace, size_t workspace_bytes, int batch,    \
+                                   int channel, int in_h, int in_w, int out_h, int out_w, int kernel_h, int kernel_w,  \
+                                   int stride_h, int stride_w, int pad_h, int pad_w, void *stream)                     \
+    {                                                                                                                  \
+        return backward_any<TYPE>(reinterpret_cast<const TYPE *>(input), reinterpret_cast<const TYPE *>(out_grad),     \
+                                  reinterpret_cast<const TYPE *>(kernel), reinterpret_cast<TYPE *>(in_grad),           \
+                                  reinterpret_cast<TYPE *>(kernel_grad), workspace, workspace_bytes, batch, channel,   \
+                                  in_h, in_w, out_h, out_w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w,      \
+                                  stream);                                                                             \
     }
 DWCONV_16BIT_ENTRY_POINTS(f16, half_t)
 DWCONV_16BIT_ENTRY_POINTS(bf16, bf16_t)
@@ -385,8 +400,9 @@ int dwconv2d_backward_f32(const float *input, const float *out_grad, const float
                           int in_h, int in_w, int out_h, int out_w, int kernel_h, int kernel_w, int stride_h,
                           int stride_w, int pad_h, int pad_w, void *stream)
 {
-    return backward_f32(input, out_grad, kernel, in_grad, kernel_grad, workspace, workspace_bytes, batch, channel,
-                        in_h, in_w, out_h, out_w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, stream);
+    return backward_any<float>(input, out_grad, kernel, in_grad, kernel_grad, workspace, workspace_bytes, batch,
+                               channel, in_h, in_w, out_h, out_w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w,
+                               stream);
 }
 
 }  // extern "C"

@@ -24,10 +24,10 @@ constexpr int kUx = 8, kUg = 2;               // float4 slots per lane that hold
 struct BwdS2Plan {
     StageLayout sx;   // x image: row r holds x row 2*q0 - pad + r, column c holds x column c - pad
     StageLayout sg;   // gy image: row r holds gy row q0 - m + r, column c holds gy column c - m
-    const float *x;
-    const float *gy;
-    const float *taps;
-    float *gx;
+    const void *x;    // element type IO of the kernel template
+    const void *gy;
+    const void *taps;
+    void *gx;
     float *partial;
     int channel;
     int pad;          // forward padding (both axes)
@@ -67,11 +67,13 @@ __device__ __forceinline__ float wave_sum_to_last_lane(float v)
 // PF: keep the next tile's bands in flight in registers (worth its ~50 registers for the 3x3 kernel only;
 // with more taps the lower occupancy costs more than the overlap brings).
 // BQ: half-resolution rows per lane (4; 2 for planes too low to give every lane a block of 4).
-template <int K, int E, bool PF, int BQ>
+template <typename IO, int K, int E, bool PF, int BQ>
 __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
 {
     extern __shared__ float4 lds_raw[];
     float *lds = reinterpret_cast<float *>(lds_raw);
+    const IO *const x = static_cast<const IO *>(p.x);
+    const IO *const gy = static_cast<const IO *>(p.gy);
     constexpr int KK = K * K;
     constexpr int KA = (K + E + 1) / 2;
     constexpr int GW_ROWS = BQ + KA;                  // gy window rows
@@ -91,7 +93,7 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
 
     float rot[KK];
 #pragma unroll
-    for (int t = 0; t < KK; ++t) rot[t] = p.taps[c * KK + KK - 1 - t];
+    for (int t = 0; t < KK; ++t) rot[t] = Io<IO>::in(static_cast<const IO *>(p.taps)[c * KK + KK - 1 - t]);
     float wacc[KK];
 #pragma unroll
     for (int t = 0; t < KK; ++t) wacc[t] = 0.f;
@@ -102,8 +104,8 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
         if (chunk < p.tiles_per_group) {
         const int n = chunk / p.row_tiles, rt = chunk - n * p.row_tiles;
         const long plane0 = static_cast<long>(n) * p.channel + c;
-        stage_fetch(p.sx, p.x, plane0, 1, 2 * rt * p.rows_per_tile - p.pad, tx);
-        stage_fetch(p.sg, p.gy, plane0, 1, rt * p.rows_per_tile - p.m, tg);
+        stage_fetch(p.sx, x, plane0, 1, 2 * rt * p.rows_per_tile - p.pad, tx);
+        stage_fetch(p.sg, gy, plane0, 1, rt * p.rows_per_tile - p.m, tg);
         }
     }
 
@@ -117,8 +119,8 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
             stage_commit(p.sx, lds, 1, tx);
             stage_commit(p.sg, lds + p.g_base, 1, tg);
         } else {
-            stage_tile(p.sx, p.x, lds, plane0, 1, 2 * q0 - p.pad);
-            stage_tile(p.sg, p.gy, lds + p.g_base, plane0, 1, q0 - p.m);
+            stage_tile(p.sx, x, lds, plane0, 1, 2 * q0 - p.pad);
+            stage_tile(p.sg, gy, lds + p.g_base, plane0, 1, q0 - p.m);
         }
         __syncthreads();
         if constexpr (PF) {
@@ -127,8 +129,8 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
             const int t1 = tile + p.chunks;
             const int n1 = t1 / p.row_tiles, rt1 = t1 - n1 * p.row_tiles;
             const long plane1 = static_cast<long>(n1) * p.channel + c;
-            stage_fetch(p.sx, p.x, plane1, 1, 2 * rt1 * p.rows_per_tile - p.pad, tx);
-            stage_fetch(p.sg, p.gy, plane1, 1, rt1 * p.rows_per_tile - p.m, tg);
+            stage_fetch(p.sx, x, plane1, 1, 2 * rt1 * p.rows_per_tile - p.pad, tx);
+            stage_fetch(p.sg, gy, plane1, 1, rt1 * p.rows_per_tile - p.m, tg);
           }
         }
 
@@ -180,19 +182,18 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
         }
         if (has_item) {
             const int ox = 4 * cb;
-            float *dst = p.gx + plane0 * p.sx.in_plane + ox;
+            IO *dst = static_cast<IO *>(p.gx) + plane0 * p.sx.in_plane + ox;
 #pragma unroll
             for (int b = 0; b < 2 * BQ; ++b) {
                 const int oy = 2 * (q0 + rb * BQ) + b;
                 if (oy >= p.sx.in_h) continue;
-                float *row = dst + static_cast<long>(oy) * p.sx.in_w;
+                IO *row = dst + static_cast<long>(oy) * p.sx.in_w;
                 if (p.vec_gx) {
-                    if (ox < p.sx.in_w)
-                        *reinterpret_cast<float4 *>(row) = make_float4(xacc[b][0], xacc[b][1], xacc[b][2], xacc[b][3]);
+                    if (ox < p.sx.in_w) store4<IO>(row, xacc[b][0], xacc[b][1], xacc[b][2], xacc[b][3]);
                 } else {
 #pragma unroll
                     for (int o = 0; o < 4; ++o)
-                        if (ox + o < p.sx.in_w) row[o] = xacc[b][o];
+                        if (ox + o < p.sx.in_w) row[o] = Io<IO>::out(xacc[b][o]);
                 }
             }
         }
@@ -292,8 +293,8 @@ bool plan_bwd_s2(BwdS2Plan &p, const WgradGeometry &g, int kBq)
     return true;
 }
 
-template <int K>
-long bwd_s2_case(int mode, const float *x, const float *gy, const float *taps, float *gx, float *gw, void *ws,
+template <typename IO, int K>
+long bwd_s2_case(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws,
                  size_t ws_bytes, const WgradGeometry &g, hipStream_t stream)
 {
     // blocks of 4 half-resolution rows, or of 2 when that is what it takes to give most lanes an item
@@ -310,9 +311,9 @@ long bwd_s2_case(int mode, const float *x, const float *gy, const float *taps, f
     p.taps = taps;
     p.gx = gx;
     p.partial = static_cast<float *>(ws);
-    p.sx.vec_in = (g.in_w % 4 == 0) && aligned16(x);
-    p.sg.vec_in = (g.out_w % 4 == 0) && aligned16(gy);
-    p.vec_gx = (g.in_w % 4 == 0) && aligned16(gx);
+    p.sx.vec_in = (g.in_w % 4 == 0) && aligned4(x);
+    p.sg.vec_in = (g.out_w % 4 == 0) && aligned4(gy);
+    p.vec_gx = (g.in_w % 4 == 0) && aligned4(gx);
     // all 256 lanes stage the images even when the tile has fewer items than that
     const int threads = kThreads;
     p.prefetch = bq == 4 && K == 3 && env_int("DWCONV_PREFETCH", 1) && p.sx.lds_rows * p.sx.spr <= kUx * threads &&
@@ -323,20 +324,21 @@ long bwd_s2_case(int mode, const float *x, const float *gy, const float *taps, f
     const int E = (K - 1 - g.pad_h) & 1;
     const dim3 grid(g.channel * p.chunks), block(threads);
     if (bq == 2) {
-        if (E) hipLaunchKernelGGL((bwd_s2_kernel<K, 1, false, 2>), grid, block, shmem, stream, p);
-        else hipLaunchKernelGGL((bwd_s2_kernel<K, 0, false, 2>), grid, block, shmem, stream, p);
-    } else if (E && p.prefetch) hipLaunchKernelGGL((bwd_s2_kernel<K, 1, true, 4>), grid, block, shmem, stream, p);
-    else if (E) hipLaunchKernelGGL((bwd_s2_kernel<K, 1, false, 4>), grid, block, shmem, stream, p);
-    else if (p.prefetch) hipLaunchKernelGGL((bwd_s2_kernel<K, 0, true, 4>), grid, block, shmem, stream, p);
-    else hipLaunchKernelGGL((bwd_s2_kernel<K, 0, false, 4>), grid, block, shmem, stream, p);
+        if (E) hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 1, false, 2>), grid, block, shmem, stream, p);
+        else hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 0, false, 2>), grid, block, shmem, stream, p);
+    } else if (E && p.prefetch) hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 1, true, 4>), grid, block, shmem, stream, p);
+    else if (E) hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 1, false, 4>), grid, block, shmem, stream, p);
+    else if (p.prefetch) hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 0, true, 4>), grid, block, shmem, stream, p);
+    else hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 0, false, 4>), grid, block, shmem, stream, p);
     const int rc = check_launch("bwd_s2_kernel");
     if (rc != DWCONV_OK) return rc;
-    note_variant("bwd_tile_s2<k%d,e%d,bq%d> rows%d chunks%d vin%d vgy%d vgx%d pf%d", K, E, bq, p.rows_per_tile, p.chunks, p.sx.vec_in,
-                 p.sg.vec_in, p.vec_gx, p.prefetch);
+    note_variant("bwd_tile_s2%s<k%d,e%d,bq%d> rows%d chunks%d vin%d vgy%d vgx%d pf%d", sizeof(IO) == 2 ? "16" : "", K, E, bq,
+                 p.rows_per_tile, p.chunks, p.sx.vec_in, p.sg.vec_in, p.vec_gx, p.prefetch);
     return launch_wgrad_final(p.partial, gw, g.channel, K * K, p.chunks, stream);
 }
 
-long bwd_s2_any(int mode, const float *x, const float *gy, const float *taps, float *gx, float *gw, void *ws,
+template <typename IO>
+long bwd_s2_any(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws,
                 size_t ws_bytes, const WgradGeometry &g, hipStream_t stream)
 {
     if (env_int("DWCONV_NO_FUSED_TILE", 0)) return -1;
@@ -345,9 +347,9 @@ long bwd_s2_any(int mode, const float *x, const float *gy, const float *taps, fl
     if (g.pad_h != g.pad_w || g.pad_h < 0 || g.pad_h > K - 1) return -1;
     if (g.in_h < 1 || g.in_w < 1 || g.out_h < 1 || g.out_w < 1) return -1;
     if (static_cast<long>(g.in_h) * g.in_w >= (1l << 30)) return -1;
-    if (K == 3) return bwd_s2_case<3>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
-    if (K == 5) return bwd_s2_case<5>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
-    if (K == 7) return bwd_s2_case<7>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+    if (K == 3) return bwd_s2_case<IO, 3>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+    if (K == 5) return bwd_s2_case<IO, 5>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+    if (K == 7) return bwd_s2_case<IO, 7>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
     return -1;
 }
 
@@ -355,14 +357,23 @@ long bwd_s2_any(int mode, const float *x, const float *gy, const float *taps, fl
 
 size_t bwd_s2_workspace(const WgradGeometry &g)
 {
-    const long n = bwd_s2_any(0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, g, nullptr);
+    // partial sums are fp32 whatever the element type
+    const long n = bwd_s2_any<float>(0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, g, nullptr);
     return n > 0 ? static_cast<size_t>(n) : 0;
 }
 
-int try_launch_bwd_s2(const float *in, const float *gy, const float *taps, float *gx, float *gw, void *ws,
-                      size_t ws_bytes, const WgradGeometry &g, hipStream_t stream)
+template <typename IO>
+int try_launch_bwd_s2(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
+                      const WgradGeometry &g, hipStream_t stream)
 {
-    return static_cast<int>(bwd_s2_any(1, in, gy, taps, gx, gw, ws, ws_bytes, g, stream));
+    return static_cast<int>(bwd_s2_any<IO>(1, in, gy, taps, gx, gw, ws, ws_bytes, g, stream));
 }
+
+template int try_launch_bwd_s2<float>(const float *, const float *, const float *, float *, float *, void *, size_t,
+                                      const WgradGeometry &, hipStream_t);
+template int try_launch_bwd_s2<half_t>(const half_t *, const half_t *, const half_t *, half_t *, half_t *, void *, size_t,
+                                       const WgradGeometry &, hipStream_t);
+template int try_launch_bwd_s2<bf16_t>(const bf16_t *, const bf16_t *, const bf16_t *, bf16_t *, bf16_t *, void *, size_t,
+                                       const WgradGeometry &, hipStream_t);
 
 }  // namespace dwconv

@@ -104,34 +104,41 @@ int launch_wgrad_direct(const T *in, const T *gy, T *gw, void *ws, size_t ws_byt
 // Return DWCONV_OK after launching, a negative value (-1) when the geometry is
 // outside what the tiled kernels cover (the caller then uses the generic kernel),
 // or a positive dwconv_status on a launch error.
-int try_launch_fir_tiled(const float *in, const float *taps, float *out, const Geometry &g,
-                         hipStream_t stream);
+template <typename IO>  // float, half_t or bf16_t
+int try_launch_fir_tiled(const IO *in, const IO *taps, IO *out, const Geometry &g, hipStream_t stream);
 
-// ---- whole-plane fp32 kernels for maps 7, 14 or 28 wide: dwconv_small.hip (same return convention) ----
-int try_launch_fir_small(const float *in, const float *taps, float *out, const Geometry &g,
-                         hipStream_t stream);
+// ---- whole-plane kernels for maps 7, 14 or 28 wide: dwconv_small.hip (same return convention) ----
+template <typename IO>  // float, half_t or bf16_t
+int try_launch_fir_small(const IO *in, const IO *taps, IO *out, const Geometry &g, hipStream_t stream);
 
 size_t wgrad_small_workspace(const WgradGeometry &g);  // 0 when the whole-plane kernel does not cover g
-int try_launch_wgrad_small(const float *in, const float *gy, float *gw, void *ws, size_t ws_bytes,
-                           const WgradGeometry &g, hipStream_t stream);
+template <typename IO>
+int try_launch_wgrad_small(const IO *in, const IO *gy, IO *gw, void *ws, size_t ws_bytes, const WgradGeometry &g,
+                           hipStream_t stream);
 // Fused grad-weight + grad-input for the same maps (gy read once); same return convention.
-int try_launch_bwd_small(const float *in, const float *gy, const float *taps, float *gx, float *gw, void *ws,
-                         size_t ws_bytes, const WgradGeometry &g, hipStream_t stream);
-// Pass 2 shared by the fp32 grad-weight kernels: gw[c][tap] = sum over chunks of partial[c][chunk][tap].
-int launch_wgrad_final(const float *partial, float *gw, int channel, int taps, int chunks, hipStream_t stream);
+template <typename IO>
+int try_launch_bwd_small(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
+                         const WgradGeometry &g, hipStream_t stream);
+// Pass 2 shared by the tiled and whole-plane grad-weight kernels:
+// gw[c][tap] = sum over chunks of partial[c][chunk][tap] (fp32 partial sums, added in fp64 in a fixed order).
+template <typename IO>
+int launch_wgrad_final(const float *partial, IO *gw, int channel, int taps, int chunks, hipStream_t stream);
 
-// ---- fp32 grad-weight with LDS tiles and a fixed-order two-pass reduction: dwconv_wgrad.hip ----
+// ---- grad-weight with LDS tiles and a fixed-order two-pass reduction: dwconv_wgrad.hip ----
 size_t wgrad_tiled_workspace(const WgradGeometry &g);  // 0 when the tiled kernel does not cover g
-int try_launch_wgrad_tiled(const float *in, const float *gy, float *gw, void *ws, size_t ws_bytes,
-                           const WgradGeometry &g, hipStream_t stream);
+template <typename IO>
+int try_launch_wgrad_tiled(const IO *in, const IO *gy, IO *gw, void *ws, size_t ws_bytes, const WgradGeometry &g,
+                           hipStream_t stream);
 
 // Fused grad-weight + grad-input with LDS tiles (stride 1, "same" padding); same return convention.
-int try_launch_bwd_tiled(const float *in, const float *gy, const float *taps, float *gx, float *gw, void *ws,
-                         size_t ws_bytes, const WgradGeometry &g, hipStream_t stream);
+template <typename IO>
+int try_launch_bwd_tiled(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
+                         const WgradGeometry &g, hipStream_t stream);
 
 // The same for stride-2 layers: dwconv_bwd_s2.hip.
 size_t bwd_s2_workspace(const WgradGeometry &g);  // 0 when that kernel does not cover g
-int try_launch_bwd_s2(const float *in, const float *gy, const float *taps, float *gx, float *gw, void *ws,
-                      size_t ws_bytes, const WgradGeometry &g, hipStream_t stream);
+template <typename IO>
+int try_launch_bwd_s2(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
+                      const WgradGeometry &g, hipStream_t stream);
 
 }  // namespace dwconv

@@ -25,9 +25,9 @@ namespace dwconv {
 namespace {
 
 struct SmallPlan {
-    const float *in;
-    const float *taps;
-    float *out;
+    const void *in;    // element type IO of the kernel template
+    const void *taps;
+    void *out;
     long planes;
     int channel;
     int in_h, out_h;
@@ -38,7 +38,7 @@ struct SmallPlan {
 };
 
 // out[oy,ox] = sum_{ty,tx} in[oy*S - pad_h + ty, ox*S - K/2 + tx] * f[ty,tx], planes W wide.
-template <int W, int K, int S, bool FLIP, int BH>
+template <typename IO, int W, int K, int S, bool FLIP, int BH>
 __global__ __launch_bounds__(kWave) void small_down_kernel(const SmallPlan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -57,8 +57,8 @@ __global__ __launch_bounds__(kWave) void small_down_kernel(const SmallPlan p)
     const int pl = active ? pl_raw : 0;
 
     float tapv[K * K];
-    load_taps<K * K, FLIP>(p.taps, static_cast<int>((plane0 + pl) % p.channel), tapv);
-    run_to_lds(p.in + plane0 * in_plane, lds, nplanes * in_plane);
+    load_taps<K * K, FLIP>(static_cast<const IO *>(p.taps), static_cast<int>((plane0 + pl) % p.channel), tapv);
+    run_to_lds(static_cast<const IO *>(p.in) + plane0 * in_plane, lds, nplanes * in_plane);
     __syncthreads();
 
     float acc[BH][OW];
@@ -111,13 +111,13 @@ __global__ __launch_bounds__(kWave) void small_down_kernel(const SmallPlan p)
             if (oy0 + b < p.out_h) lds_store_row<OW>(dst + (oy0 + b) * OW, acc[b]);
     }
     __syncthreads();
-    lds_to_run(p.out + plane0 * out_plane, lds, nplanes * out_plane);
+    lds_to_run(static_cast<IO *>(p.out) + plane0 * out_plane, lds, nplanes * out_plane);
 }
 
 // up = 2, taps rotated, "same" padding of the forward conv (leading pad of the transposed problem = K/2):
 //   out[2q + r] = sum_a in[q - m + r + a] * g'[r + 2a],  g'[t] = g[t - E],  E = (K/2) & 1,  m = (K/2 + E) / 2.
 // Input planes are W wide, output planes 2W wide; a lane owns output rows 2q, 2q+1.
-template <int W, int K>
+template <typename IO, int W, int K>
 __global__ __launch_bounds__(kWave) void small_up2_kernel(const SmallPlan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -138,8 +138,8 @@ __global__ __launch_bounds__(kWave) void small_up2_kernel(const SmallPlan p)
     const int pl = active ? pl_raw : 0;
 
     float tapv[K * K];
-    load_taps<K * K, true>(p.taps, static_cast<int>((plane0 + pl) % p.channel), tapv);
-    run_to_lds(p.in + plane0 * in_plane, lds, nplanes * in_plane);
+    load_taps<K * K, true>(static_cast<const IO *>(p.taps), static_cast<int>((plane0 + pl) % p.channel), tapv);
+    run_to_lds(static_cast<const IO *>(p.in) + plane0 * in_plane, lds, nplanes * in_plane);
     __syncthreads();
 
     float acc[2][OW];
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(kWave) void small_up2_kernel(const SmallPlan p)
             if (2 * q + r < p.out_h) lds_store_row<OW>(dst + (2 * q + r) * OW, acc[r]);
     }
     __syncthreads();
-    lds_to_run(p.out + plane0 * out_plane, lds, nplanes * out_plane);
+    lds_to_run(static_cast<IO *>(p.out) + plane0 * out_plane, lds, nplanes * out_plane);
 }
 
 size_t small_lds_bytes(int planes, int in_plane, int out_plane)
@@ -204,7 +204,7 @@ size_t small_lds_bytes(int planes, int in_plane, int out_plane)
 }
 
 // Planes per wavefront: as many as there are lane slots, a multiple of 4 when a plane is not a
-// multiple of 4 floats (so that every run starts on a 16-byte boundary), within the LDS budget.
+// multiple of 4 elements (so that every run starts on a 4-element boundary), within the LDS budget.
 int planes_per_run(int lanes_per_plane, int in_plane, int out_plane, long planes)
 {
     int P = kWave / lanes_per_plane;
@@ -214,7 +214,7 @@ int planes_per_run(int lanes_per_plane, int in_plane, int out_plane, long planes
     return P;
 }
 
-template <int W, int K, int S, bool FLIP, int BH>
+template <typename IO, int W, int K, int S, bool FLIP, int BH>
 int launch_small_down(SmallPlan &p, hipStream_t stream)
 {
     constexpr int OW = (W - 1) / S + 1;
@@ -227,13 +227,14 @@ int launch_small_down(SmallPlan &p, hipStream_t stream)
     const long runs = (p.planes + p.planes_per_run - 1) / p.planes_per_run;
     if (runs > 0x7fffffffL) return -1;
     const size_t shmem = small_lds_bytes(p.planes_per_run, in_plane, out_plane);
-    hipLaunchKernelGGL((small_down_kernel<W, K, S, FLIP, BH>), dim3(static_cast<unsigned>(runs)), dim3(kWave), shmem,
+    hipLaunchKernelGGL((small_down_kernel<IO, W, K, S, FLIP, BH>), dim3(static_cast<unsigned>(runs)), dim3(kWave), shmem,
                        stream, p);
-    note_variant("small_down<w%d,k%d,s%d,%s,bh%d> P%d", W, K, S, FLIP ? "rot" : "fwd", BH, p.planes_per_run);
+    note_variant("small_down%s<w%d,k%d,s%d,%s,bh%d> P%d", sizeof(IO) == 2 ? "16" : "", W, K, S, FLIP ? "rot" : "fwd", BH,
+                 p.planes_per_run);
     return check_launch("small_down_kernel");
 }
 
-template <int W, int K>
+template <typename IO, int W, int K>
 int launch_small_up2(SmallPlan &p, hipStream_t stream)
 {
     p.lanes_per_plane = ceil_div(p.out_h, 2);
@@ -245,12 +246,12 @@ int launch_small_up2(SmallPlan &p, hipStream_t stream)
     const long runs = (p.planes + p.planes_per_run - 1) / p.planes_per_run;
     if (runs > 0x7fffffffL) return -1;
     const size_t shmem = small_lds_bytes(p.planes_per_run, in_plane, out_plane);
-    hipLaunchKernelGGL((small_up2_kernel<W, K>), dim3(static_cast<unsigned>(runs)), dim3(kWave), shmem, stream, p);
-    note_variant("small_up2<w%d,k%d> P%d", W, K, p.planes_per_run);
+    hipLaunchKernelGGL((small_up2_kernel<IO, W, K>), dim3(static_cast<unsigned>(runs)), dim3(kWave), shmem, stream, p);
+    note_variant("small_up2%s<w%d,k%d> P%d", sizeof(IO) == 2 ? "16" : "", W, K, p.planes_per_run);
     return check_launch("small_up2_kernel");
 }
 
-template <int W, int K>
+template <typename IO, int W, int K>
 int launch_small_down_any(SmallPlan &p, int S, bool rot, hipStream_t stream)
 {
     constexpr int BH1 = W == 7 ? 7 : 2;
@@ -259,43 +260,44 @@ int launch_small_down_any(SmallPlan &p, int S, bool rot, hipStream_t stream)
             // one lane per plane needs 64 planes per wavefront: with few planes that leaves most CUs idle,
             // so give a plane four lanes (two rows each) instead
             if (p.planes < 64l * 2048)
-                return rot ? launch_small_down<W, K, 1, true, 2>(p, stream) : launch_small_down<W, K, 1, false, 2>(p, stream);
+                return rot ? launch_small_down<IO, W, K, 1, true, 2>(p, stream) : launch_small_down<IO, W, K, 1, false, 2>(p, stream);
         }
-        return rot ? launch_small_down<W, K, 1, true, BH1>(p, stream) : launch_small_down<W, K, 1, false, BH1>(p, stream);
+        return rot ? launch_small_down<IO, W, K, 1, true, BH1>(p, stream) : launch_small_down<IO, W, K, 1, false, BH1>(p, stream);
     }
     if constexpr (W % 2 == 0) {
-        if (S == 2 && !rot) return launch_small_down<W, K, 2, false, 1>(p, stream);
+        if (S == 2 && !rot) return launch_small_down<IO, W, K, 2, false, 1>(p, stream);
     }
     return -1;
 }
 
-template <int W>
+template <typename IO, int W>
 int launch_small_down_k(SmallPlan &p, int K, int S, bool rot, hipStream_t stream)
 {
-    if (K == 3) return launch_small_down_any<W, 3>(p, S, rot, stream);
-    if (K == 5) return launch_small_down_any<W, 5>(p, S, rot, stream);
-    if (K == 7) return launch_small_down_any<W, 7>(p, S, rot, stream);
+    if (K == 3) return launch_small_down_any<IO, W, 3>(p, S, rot, stream);
+    if (K == 5) return launch_small_down_any<IO, W, 5>(p, S, rot, stream);
+    if (K == 7) return launch_small_down_any<IO, W, 7>(p, S, rot, stream);
     return -1;
 }
 
-template <int W>
+template <typename IO, int W>
 int launch_small_up2_k(SmallPlan &p, int K, hipStream_t stream)
 {
-    if (K == 3) return launch_small_up2<W, 3>(p, stream);
-    if (K == 5) return launch_small_up2<W, 5>(p, stream);
-    if (K == 7) return launch_small_up2<W, 7>(p, stream);
+    if (K == 3) return launch_small_up2<IO, W, 3>(p, stream);
+    if (K == 5) return launch_small_up2<IO, W, 5>(p, stream);
+    if (K == 7) return launch_small_up2<IO, W, 7>(p, stream);
     return -1;
 }
 
 
 }  // namespace
 
-int try_launch_fir_small(const float *in, const float *taps, float *out, const Geometry &g, hipStream_t stream)
+template <typename IO>
+int try_launch_fir_small(const IO *in, const IO *taps, IO *out, const Geometry &g, hipStream_t stream)
 {
     if (env_int("DWCONV_NO_SMALL", 0)) return -1;
     const int K = g.kernel_h;
     if (g.kernel_w != K || (K != 3 && K != 5 && K != 7)) return -1;
-    if (!aligned16(in) || !aligned16(out)) return -1;
+    if (!aligned4(in) || !aligned4(out)) return -1;
     if (g.in_h < 1 || g.in_h > 64 || g.out_h < 1 || g.out_h > 128) return -1;
     SmallPlan p{};
     p.in = in;
@@ -312,20 +314,24 @@ int try_launch_fir_small(const float *in, const float *taps, float *out, const G
         if (g.pad_w0 != K / 2 || g.out_w != (W - 1) / S + 1) return -1;
         if (g.pad_h0 < 0 || g.pad_h0 > 7) return -1;
         p.pad_h = g.pad_h0;
-        if (W == 7) return launch_small_down_k<7>(p, K, S, !g.forward, stream);
-        if (W == 14) return launch_small_down_k<14>(p, K, S, !g.forward, stream);
-        if (W == 28) return launch_small_down_k<28>(p, K, S, !g.forward, stream);
+        if (W == 7) return launch_small_down_k<IO, 7>(p, K, S, !g.forward, stream);
+        if (W == 14) return launch_small_down_k<IO, 14>(p, K, S, !g.forward, stream);
+        if (W == 28) return launch_small_down_k<IO, 28>(p, K, S, !g.forward, stream);
         return -1;
     }
     if (g.up_h == 2 && g.up_w == 2 && g.down_h == 1 && g.down_w == 1 && !g.forward) {
         if (g.pad_w0 != K / 2 || g.pad_h0 != K / 2 || g.out_w != 2 * W) return -1;
         const int E = (K / 2) & 1;
         p.pad_h = (K / 2 + E) / 2;
-        if (W == 7) return launch_small_up2_k<7>(p, K, stream);
-        if (W == 14) return launch_small_up2_k<14>(p, K, stream);
+        if (W == 7) return launch_small_up2_k<IO, 7>(p, K, stream);
+        if (W == 14) return launch_small_up2_k<IO, 14>(p, K, stream);
         return -1;
     }
     return -1;
 }
+
+template int try_launch_fir_small<float>(const float *, const float *, float *, const Geometry &, hipStream_t);
+template int try_launch_fir_small<half_t>(const half_t *, const half_t *, half_t *, const Geometry &, hipStream_t);
+template int try_launch_fir_small<bf16_t>(const bf16_t *, const bf16_t *, bf16_t *, const Geometry &, hipStream_t);
 
 }  // namespace dwconv

@@ -22,10 +22,10 @@ constexpr int kRunFloats = kRunRegs * kWave * 4;
 constexpr int kSmallRedPitch = kWave + 1;
 
 struct SmallBwdPlan {
-    const float *x;
-    const float *gy;
-    const float *taps;
-    float *gx;
+    const void *x;    // element type IO of the kernel template
+    const void *gy;
+    const void *taps;
+    void *gx;
     float *partial;
     int batch, channel;
     int in_h, out_h;
@@ -36,30 +36,33 @@ struct SmallBwdPlan {
     int chunks, images_per_chunk;
 };
 
-// Issues the loads of a run of n floats (n >= 4, g 16-byte aligned); slots past the end re-read the last float4.
-__device__ __forceinline__ void run_fetch(const float *__restrict__ g, int n, float4 (&v)[kRunRegs])
+// Issues the loads of a run of n elements (n >= 4, g aligned to four elements); slots past the end re-read the
+// last group of four.
+template <typename IO>
+__device__ __forceinline__ void run_fetch(const IO *__restrict__ g, int n, typename Raw4<IO>::type (&v)[kRunRegs])
 {
     const int n4 = n >> 2;
 #pragma unroll
-    for (int u = 0; u < kRunRegs; ++u)
-        v[u] = reinterpret_cast<const float4 *>(g)[min(static_cast<int>(threadIdx.x) + u * kWave, n4 - 1)];
+    for (int u = 0; u < kRunRegs; ++u) v[u] = load4_raw<IO>(g + 4 * min(static_cast<int>(threadIdx.x) + u * kWave, n4 - 1));
 }
 
-__device__ __forceinline__ void run_commit(const float *__restrict__ g, float *lds, int n, const float4 (&v)[kRunRegs])
+template <typename IO>
+__device__ __forceinline__ void run_commit(const IO *__restrict__ g, float *lds, int n,
+                                           const typename Raw4<IO>::type (&v)[kRunRegs])
 {
     const int n4 = n >> 2;
 #pragma unroll
     for (int u = 0; u < kRunRegs; ++u) {
-        const float4 t = v[u];  // read outside the condition: a conditional copy keeps the array out of registers
+        const float4 t = widen4<IO>(v[u]);  // read outside the condition: a conditional copy keeps the array out of registers
         if (static_cast<int>(threadIdx.x) + u * kWave < n4) reinterpret_cast<float4 *>(lds)[threadIdx.x + u * kWave] = t;
     }
     const int tail = n4 * 4 + threadIdx.x;
-    if (tail < n) lds[tail] = g[tail];
+    if (tail < n) lds[tail] = Io<IO>::in(g[tail]);
 }
 
 // PF: the runs of the next image are fetched into registers while the current image is processed
-// (56 registers; dropped for the 7x7 filter, whose sums and taps already take 98).
-template <int W, int K, int S, int BH, bool GX, bool PF = (K < 7)>
+// (56 registers in fp32, 28 for 16-bit elements; dropped for the fp32 7x7 filter, whose sums and taps already take 98).
+template <typename IO, int W, int K, int S, int BH, bool GX, bool PF = (K < 7 || sizeof(IO) == 2)>
 __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -91,29 +94,31 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
 #pragma unroll
     for (int t = 0; t < KK; ++t) wacc[t] = 0.f;
     float tapv[GX ? KK : 1];
-    if constexpr (GX) load_taps<KK, true>(p.taps, c0 + pl, tapv);
+    if constexpr (GX) load_taps<KK, true>(static_cast<const IO *>(p.taps), c0 + pl, tapv);
 
-    float4 rx[kRunRegs], rg[kRunRegs];
+    const IO *const x = static_cast<const IO *>(p.x);
+    const IO *const gy = static_cast<const IO *>(p.gy);
+    typename Raw4<IO>::type rx[kRunRegs], rg[kRunRegs];
     if constexpr (PF) {
         const long plane0 = static_cast<long>(n0) * p.channel + c0;
-        run_fetch(p.x + plane0 * in_plane, nx, rx);
-        run_fetch(p.gy + plane0 * out_plane, ng, rg);
+        run_fetch(x + plane0 * in_plane, nx, rx);
+        run_fetch(gy + plane0 * out_plane, ng, rg);
     }
 
     for (int n = n0; n < n1; ++n) {
         const long plane0 = static_cast<long>(n) * p.channel + c0;
         if (n != n0) __syncthreads();  // the previous image is done with the LDS runs
         if constexpr (!PF) {
-            run_fetch(p.x + plane0 * in_plane, nx, rx);
-            run_fetch(p.gy + plane0 * out_plane, ng, rg);
+            run_fetch(x + plane0 * in_plane, nx, rx);
+            run_fetch(gy + plane0 * out_plane, ng, rg);
         }
-        run_commit(p.x + plane0 * in_plane, lds_x, nx, rx);
-        run_commit(p.gy + plane0 * out_plane, lds_g, ng, rg);
+        run_commit(x + plane0 * in_plane, lds_x, nx, rx);
+        run_commit(gy + plane0 * out_plane, lds_g, ng, rg);
         __syncthreads();
         if (PF && n + 1 < n1) {
             const long plane1 = plane0 + p.channel;
-            run_fetch(p.x + plane1 * in_plane, nx, rx);
-            run_fetch(p.gy + plane1 * out_plane, ng, rg);
+            run_fetch(x + plane1 * in_plane, nx, rx);
+            run_fetch(gy + plane1 * out_plane, ng, rg);
         }
 
         // ---- grad-weight: this lane's gy rows against the x rows they touch
@@ -257,7 +262,7 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
                     if (row0 + b < p.in_h) lds_store_row<W>(dst + (row0 + b) * W, xacc[b]);
             }
             __syncthreads();
-            lds_to_run(p.gx + plane0 * in_plane, lds_x, nx);
+            lds_to_run(static_cast<IO *>(p.gx) + plane0 * in_plane, lds_x, nx);
         }
     }
 
@@ -287,7 +292,7 @@ bool plan_small_bwd(SmallBwdPlan &p, const WgradGeometry &g)
     if (p.lanes_per_plane > kWave) return false;
     const int in_plane = g.in_h * W, out_plane = g.out_h * OW;
     const bool odd = in_plane % 4 != 0 || out_plane % 4 != 0;
-    if (odd && g.channel % 4 != 0) return false;  // runs of every image must start on a 16-byte boundary
+    if (odd && g.channel % 4 != 0) return false;  // runs of every image must start on a 4-element boundary
     int P = kWave / p.lanes_per_plane;
     if (P > g.channel) P = g.channel;
     // a run must fit the registers that prefetch it
@@ -307,8 +312,8 @@ bool plan_small_bwd(SmallBwdPlan &p, const WgradGeometry &g)
 
 // mode 0: report the workspace bytes; mode 1: grad-weight; mode 2: grad-weight + grad-input.
 // Returns -1 when this family does not cover g.
-template <int W, int K, int S, int BH>
-long small_bwd_case(int mode, const float *x, const float *gy, const float *taps, float *gx, float *gw, void *ws,
+template <typename IO, int W, int K, int S, int BH>
+long small_bwd_case(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws,
                     size_t ws_bytes, const WgradGeometry &g, hipStream_t stream)
 {
     constexpr int OW = (W - 1) / S + 1;
@@ -328,39 +333,40 @@ long small_bwd_case(int mode, const float *x, const float *gy, const float *taps
     const size_t shmem = runs > red ? runs : red;
     const int groups = ceil_div(g.channel, p.planes_per_run);
     if (mode == 2)
-        hipLaunchKernelGGL((small_bwd_kernel<W, K, S, BH, true>), dim3(groups * p.chunks), dim3(kWave), shmem, stream, p);
+        hipLaunchKernelGGL((small_bwd_kernel<IO, W, K, S, BH, true>), dim3(groups * p.chunks), dim3(kWave), shmem, stream, p);
     else
-        hipLaunchKernelGGL((small_bwd_kernel<W, K, S, BH, false>), dim3(groups * p.chunks), dim3(kWave), shmem, stream, p);
+        hipLaunchKernelGGL((small_bwd_kernel<IO, W, K, S, BH, false>), dim3(groups * p.chunks), dim3(kWave), shmem, stream, p);
     const int rc = check_launch("small_bwd_kernel");
     if (rc != DWCONV_OK) return rc;
-    note_variant("%s<w%d,k%d,s%d,bh%d> P%d chunks%d", mode == 2 ? "small_bwd" : "small_wgrad", W, K, S, BH,
-                 p.planes_per_run, p.chunks);
+    note_variant("%s%s<w%d,k%d,s%d,bh%d> P%d chunks%d", mode == 2 ? "small_bwd" : "small_wgrad",
+                 sizeof(IO) == 2 ? "16" : "", W, K, S, BH, p.planes_per_run, p.chunks);
     return launch_wgrad_final(p.partial, gw, g.channel, K * K, p.chunks, stream);
 }
 
-template <int W, int K>
-long small_bwd_s(int mode, const float *x, const float *gy, const float *taps, float *gx, float *gw, void *ws,
+template <typename IO, int W, int K>
+long small_bwd_s(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws,
                  size_t ws_bytes, const WgradGeometry &g, hipStream_t stream)
 {
     constexpr int BH1 = W == 7 ? 4 : (W == 14 ? 2 : 1);
-    if (g.down_h == 1) return small_bwd_case<W, K, 1, BH1>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+    if (g.down_h == 1) return small_bwd_case<IO, W, K, 1, BH1>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
     if constexpr (W % 2 == 0) {
-        if (g.down_h == 2) return small_bwd_case<W, K, 2, 1>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+        if (g.down_h == 2) return small_bwd_case<IO, W, K, 2, 1>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
     }
     return -1;
 }
 
-template <int W>
-long small_bwd_k(int mode, const float *x, const float *gy, const float *taps, float *gx, float *gw, void *ws,
+template <typename IO, int W>
+long small_bwd_k(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws,
                  size_t ws_bytes, const WgradGeometry &g, hipStream_t stream)
 {
-    if (g.kernel_h == 3) return small_bwd_s<W, 3>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
-    if (g.kernel_h == 5) return small_bwd_s<W, 5>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
-    if (g.kernel_h == 7) return small_bwd_s<W, 7>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+    if (g.kernel_h == 3) return small_bwd_s<IO, W, 3>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+    if (g.kernel_h == 5) return small_bwd_s<IO, W, 5>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+    if (g.kernel_h == 7) return small_bwd_s<IO, W, 7>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
     return -1;
 }
 
-long small_bwd_any(int mode, const float *x, const float *gy, const float *taps, float *gx, float *gw, void *ws,
+template <typename IO>
+long small_bwd_any(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws,
                    size_t ws_bytes, const WgradGeometry &g, hipStream_t stream)
 {
     if (env_int("DWCONV_NO_SMALL", 0)) return -1;
@@ -374,12 +380,12 @@ long small_bwd_any(int mode, const float *x, const float *gy, const float *taps,
         if (g.pad_h != K / 2) return -1;
         if (S == 1 && g.out_h != g.in_h) return -1;
         if (S == 2 && (g.in_h != 2 * g.out_h || g.in_w != 2 * g.out_w)) return -1;
-        if (!aligned16(gx)) return -1;
+        if (!aligned4(gx)) return -1;
     }
-    if (mode != 0 && (!aligned16(x) || !aligned16(gy))) return -1;
-    if (g.in_w == 7) return small_bwd_k<7>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
-    if (g.in_w == 14) return small_bwd_k<14>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
-    if (g.in_w == 28) return small_bwd_k<28>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+    if (mode != 0 && (!aligned4(x) || !aligned4(gy))) return -1;
+    if (g.in_w == 7) return small_bwd_k<IO, 7>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+    if (g.in_w == 14) return small_bwd_k<IO, 14>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+    if (g.in_w == 28) return small_bwd_k<IO, 28>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
     return -1;
 }
 
@@ -387,20 +393,33 @@ long small_bwd_any(int mode, const float *x, const float *gy, const float *taps,
 
 size_t wgrad_small_workspace(const WgradGeometry &g)
 {
-    const long n = small_bwd_any(0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, g, nullptr);
+    // partial sums are fp32 whatever the element type
+    const long n = small_bwd_any<float>(0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, g, nullptr);
     return n > 0 ? static_cast<size_t>(n) : 0;
 }
 
-int try_launch_wgrad_small(const float *in, const float *gy, float *gw, void *ws, size_t ws_bytes,
-                           const WgradGeometry &g, hipStream_t stream)
+template <typename IO>
+int try_launch_wgrad_small(const IO *in, const IO *gy, IO *gw, void *ws, size_t ws_bytes, const WgradGeometry &g,
+                           hipStream_t stream)
 {
-    return static_cast<int>(small_bwd_any(1, in, gy, nullptr, nullptr, gw, ws, ws_bytes, g, stream));
+    return static_cast<int>(small_bwd_any<IO>(1, in, gy, nullptr, nullptr, gw, ws, ws_bytes, g, stream));
 }
 
-int try_launch_bwd_small(const float *in, const float *gy, const float *taps, float *gx, float *gw, void *ws,
-                         size_t ws_bytes, const WgradGeometry &g, hipStream_t stream)
+template <typename IO>
+int try_launch_bwd_small(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
+                         const WgradGeometry &g, hipStream_t stream)
 {
-    return static_cast<int>(small_bwd_any(2, in, gy, taps, gx, gw, ws, ws_bytes, g, stream));
+    return static_cast<int>(small_bwd_any<IO>(2, in, gy, taps, gx, gw, ws, ws_bytes, g, stream));
 }
+
+#define DWCONV_INSTANTIATE(IO)                                                                                        \
+    template int try_launch_wgrad_small<IO>(const IO *, const IO *, IO *, void *, size_t, const WgradGeometry &,      \
+                                            hipStream_t);                                                             \
+    template int try_launch_bwd_small<IO>(const IO *, const IO *, const IO *, IO *, IO *, void *, size_t,             \
+                                          const WgradGeometry &, hipStream_t);
+DWCONV_INSTANTIATE(float)
+DWCONV_INSTANTIATE(half_t)
+DWCONV_INSTANTIATE(bf16_t)
+#undef DWCONV_INSTANTIATE
 
 }  // namespace dwconv

@@ -47,11 +47,13 @@ __device__ __forceinline__ void lds_store_row(float *p, const float *r)
 }
 
 // ---- flat runs between global memory and LDS ---------------------------------------------------
-// `g` is 16-byte aligned; n floats; the last partial float4 (only at the very end of a tensor) goes scalar.
+// `g` is aligned to four elements; n elements; the last partial group of four (only at the very end of a
+// tensor) goes scalar.  LDS always holds fp32.
 // Loads are issued kRunBatch at a time before any of them is consumed, so their latencies overlap.
 constexpr int kRunBatch = 8;
 
-__device__ __forceinline__ void run_to_lds(const float *__restrict__ g, float *lds, int n)
+template <typename IO>
+__device__ __forceinline__ void run_to_lds(const IO *__restrict__ g, float *lds, int n)
 {
     const int n4 = n >> 2;
     for (int base = threadIdx.x; base < n4; base += kWave * kRunBatch) {
@@ -59,18 +61,19 @@ __device__ __forceinline__ void run_to_lds(const float *__restrict__ g, float *l
         // out-of-range slots re-read the last float4 of the run (always a valid address) and are not stored
 #pragma unroll
         for (int u = 0; u < kRunBatch; ++u)
-            v[u] = reinterpret_cast<const float4 *>(g)[min(base + u * kWave, n4 - 1)];
+            v[u] = load4<IO>(g + 4 * min(base + u * kWave, n4 - 1));
 #pragma unroll
         for (int u = 0; u < kRunBatch; ++u)
             if (base + u * kWave < n4) reinterpret_cast<float4 *>(lds)[base + u * kWave] = v[u];
     }
     const int tail = n4 * 4 + threadIdx.x;
-    if (tail < n) lds[tail] = g[tail];
+    if (tail < n) lds[tail] = Io<IO>::in(g[tail]);
 }
 
 // Two runs at once (grad-weight: x and gy of the same planes): all loads of a batch of both runs fly together.
-__device__ __forceinline__ void runs_to_lds(const float *__restrict__ ga, float *la, int na,
-                                            const float *__restrict__ gb, float *lb, int nb)
+template <typename IO>
+__device__ __forceinline__ void runs_to_lds(const IO *__restrict__ ga, float *la, int na,
+                                            const IO *__restrict__ gb, float *lb, int nb)
 {
     const int na4 = na >> 2, nb4 = nb >> 2;
     const int nmax = na4 > nb4 ? na4 : nb4;
@@ -79,8 +82,8 @@ __device__ __forceinline__ void runs_to_lds(const float *__restrict__ ga, float 
         float4 va[U], vb[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            va[u] = reinterpret_cast<const float4 *>(ga)[min(base + u * kWave, na4 - 1)];
-            vb[u] = reinterpret_cast<const float4 *>(gb)[min(base + u * kWave, nb4 - 1)];
+            va[u] = load4<IO>(ga + 4 * min(base + u * kWave, na4 - 1));
+            vb[u] = load4<IO>(gb + 4 * min(base + u * kWave, nb4 - 1));
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -89,11 +92,12 @@ __device__ __forceinline__ void runs_to_lds(const float *__restrict__ ga, float 
         }
     }
     const int ta = na4 * 4 + threadIdx.x, tb = nb4 * 4 + threadIdx.x;
-    if (ta < na) la[ta] = ga[ta];
-    if (tb < nb) lb[tb] = gb[tb];
+    if (ta < na) la[ta] = Io<IO>::in(ga[ta]);
+    if (tb < nb) lb[tb] = Io<IO>::in(gb[tb]);
 }
 
-__device__ __forceinline__ void lds_to_run(float *__restrict__ g, const float *lds, int n)
+template <typename IO>
+__device__ __forceinline__ void lds_to_run(IO *__restrict__ g, const float *lds, int n)
 {
     const int n4 = n >> 2;
     constexpr int U = 4;
@@ -103,18 +107,18 @@ __device__ __forceinline__ void lds_to_run(float *__restrict__ g, const float *l
         for (int u = 0; u < U; ++u) v[u] = reinterpret_cast<const float4 *>(lds)[min(base + u * kWave, n4 - 1)];
 #pragma unroll
         for (int u = 0; u < U; ++u)
-            if (base + u * kWave < n4) reinterpret_cast<float4 *>(g)[base + u * kWave] = v[u];
+            if (base + u * kWave < n4) store4<IO>(g + 4 * (base + u * kWave), v[u].x, v[u].y, v[u].z, v[u].w);
     }
     const int tail = n4 * 4 + threadIdx.x;
-    if (tail < n) g[tail] = lds[tail];
+    if (tail < n) g[tail] = Io<IO>::out(lds[tail]);
 }
 
 // This lane's K*K taps straight from global memory (the lanes of one plane read the same addresses).
-template <int KK, bool FLIP>
-__device__ __forceinline__ void load_taps(const float *__restrict__ taps, int c, float (&t)[KK])
+template <int KK, bool FLIP, typename IO>
+__device__ __forceinline__ void load_taps(const IO *__restrict__ taps, int c, float (&t)[KK])
 {
 #pragma unroll
-    for (int i = 0; i < KK; ++i) t[i] = taps[c * KK + (FLIP ? KK - 1 - i : i)];
+    for (int i = 0; i < KK; ++i) t[i] = Io<IO>::in(taps[c * KK + (FLIP ? KK - 1 - i : i)]);
 }
 
 }  // namespace dwconv

@@ -29,9 +29,9 @@ namespace {
 
 struct TilePlan {
     StageLayout st;
-    const float *in;
-    const float *taps;
-    float *out;
+    const void *in;    // element type IO of the kernel template
+    const void *taps;
+    void *out;
     long planes;
     int channel;
     int out_h, out_w, out_plane;
@@ -49,18 +49,18 @@ struct TilePlan {
 };
 
 // Copies the tap tables of the tile's planes into LDS, rotated by 180 degrees if FLIP.
-template <int KK, bool FLIP>
+template <typename IO, int KK, bool FLIP>
 __device__ __forceinline__ void stage_taps(const TilePlan &p, float *lds, long plane0, int nplanes)
 {
     for (int i = threadIdx.x; i < nplanes * KK; i += blockDim.x) {
         const int pl = i / KK, t = i - pl * KK;
         const int c = static_cast<int>((plane0 + pl) % p.channel);
-        lds[p.tap_base + i] = p.taps[c * KK + (FLIP ? KK - 1 - t : t)];
+        lds[p.tap_base + i] = Io<IO>::in(static_cast<const IO *>(p.taps)[c * KK + (FLIP ? KK - 1 - t : t)]);
     }
 }
 
 // up = 1, decimation S.  out[oy,ox] = sum_{ty,tx} in[oy*S - pad_h0 + ty, ox*S - pad_w0 + tx] * f[ty,tx].
-template <int K, int S, bool FLIP, int BH>
+template <typename IO, int K, int S, bool FLIP, int BH>
 __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -75,8 +75,8 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
     const int nplanes = static_cast<int>(min(static_cast<long>(p.planes_per_tile), p.planes - plane0));
     const int oy0 = rt * p.rows_per_tile;
 
-    stage_taps<KK, FLIP>(p, lds, plane0, nplanes);
-    stage_tile(p.st, p.in, lds, plane0, nplanes, oy0 * S - p.row_shift);
+    stage_taps<IO, KK, FLIP>(p, lds, plane0, nplanes);
+    stage_tile(p.st, static_cast<const IO *>(p.in), lds, plane0, nplanes, oy0 * S - p.row_shift);
     __syncthreads();
 
     const int n_items = nplanes * p.items_per_plane;
@@ -120,18 +120,18 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
         }
 
         const int ox = 4 * cb;
-        float *dst = p.out + (plane0 + pl) * p.out_plane + ox;
+        IO *dst = static_cast<IO *>(p.out) + (plane0 + pl) * p.out_plane + ox;
 #pragma unroll
         for (int b = 0; b < BH; ++b) {
             const int oy = oy0 + rb * BH + b;
             if (oy >= p.out_h) continue;
-            float *row = dst + static_cast<long>(oy) * p.out_w;
+            IO *row = dst + static_cast<long>(oy) * p.out_w;
             if (p.vec_out) {
-                *reinterpret_cast<float4 *>(row) = make_float4(acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+                store4<IO>(row, acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
             } else {
 #pragma unroll
                 for (int o = 0; o < 4; ++o)
-                    if (ox + o < p.out_w) row[o] = acc[b][o];
+                    if (ox + o < p.out_w) row[o] = Io<IO>::out(acc[b][o]);
             }
         }
     }
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
 // i.e. a stride-1 correlation per output parity r with every other tap.
 // A lane owns 2*BQ output rows x 4 output columns (BQ x 2 half-resolution positions), so that the
 // 128-bit stores of consecutive lanes are contiguous in memory.
-template <int K, int EY, int EX, int BQ>
+template <typename IO, int K, int EY, int EX, int BQ>
 __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -159,8 +159,8 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
     const int nplanes = static_cast<int>(min(static_cast<long>(p.planes_per_tile), p.planes - plane0));
     const int qy0 = rt * p.rows_per_tile;
 
-    stage_taps<KK, true>(p, lds, plane0, nplanes);
-    stage_tile(p.st, p.in, lds, plane0, nplanes, qy0 - p.row_shift);
+    stage_taps<IO, KK, true>(p, lds, plane0, nplanes);
+    stage_tile(p.st, static_cast<const IO *>(p.in), lds, plane0, nplanes, qy0 - p.row_shift);
     __syncthreads();
 
     const int n_items = nplanes * p.items_per_plane;
@@ -213,18 +213,18 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
         }
 
         const int ox = 4 * cb;
-        float *dst = p.out + (plane0 + pl) * p.out_plane + ox;
+        IO *dst = static_cast<IO *>(p.out) + (plane0 + pl) * p.out_plane + ox;
 #pragma unroll
         for (int b = 0; b < 2 * BQ; ++b) {
             const int oy = 2 * (qy0 + rb * BQ) + b;
             if (oy >= p.out_h) continue;
-            float *row = dst + static_cast<long>(oy) * p.out_w;
+            IO *row = dst + static_cast<long>(oy) * p.out_w;
             if (p.vec_out) {
-                *reinterpret_cast<float4 *>(row) = make_float4(acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+                store4<IO>(row, acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
             } else {
 #pragma unroll
                 for (int o = 0; o < 4; ++o)
-                    if (ox + o < p.out_w) row[o] = acc[b][o];
+                    if (ox + o < p.out_w) row[o] = Io<IO>::out(acc[b][o]);
             }
         }
     }
@@ -291,7 +291,7 @@ size_t lds_bytes(const TilePlan &p, int taps_per_plane)
     return static_cast<size_t>(p.planes_per_tile) * (p.st.plane_pitch + taps_per_plane) * 4;
 }
 
-template <int K, int S, bool FLIP, int BH>
+template <typename IO, int K, int S, bool FLIP, int BH>
 int launch_down(TilePlan &p, hipStream_t stream)
 {
     constexpr int NV = (3 * S + K + 3) / 4;
@@ -299,22 +299,22 @@ int launch_down(TilePlan &p, hipStream_t stream)
     const int used_cols = 4 * (p.ncb - 1) * S + 4 * NV;
     auto rows_for = [](int units) { return (units * BH - 1) * S + K; };
     if (!plan_tiles(p, ceil_div(p.out_h, BH), BH, used_cols, K * K, rows_for)) return -1;
-    hipLaunchKernelGGL((fir_down_kernel<K, S, FLIP, BH>), dim3(p.n_tiles), dim3(env_int("DWCONV_TILE_THREADS", kThreads)), lds_bytes(p, K * K),
+    hipLaunchKernelGGL((fir_down_kernel<IO, K, S, FLIP, BH>), dim3(p.n_tiles), dim3(env_int("DWCONV_TILE_THREADS", kThreads)), lds_bytes(p, K * K),
                        stream, p);
-    note_variant("tile_down<k%d,s%d,%s,bh%d> P%d rows%d vin%d vout%d", K, S, FLIP ? "rot" : "fwd", BH,
+    note_variant("tile_down%s<k%d,s%d,%s,bh%d> P%d rows%d vin%d vout%d", sizeof(IO) == 2 ? "16" : "", K, S, FLIP ? "rot" : "fwd", BH,
                  p.planes_per_tile, p.rows_per_tile, p.st.vec_in, p.vec_out);
     return check_launch("fir_down_kernel");
 }
 
-template <int K, int S, bool FLIP>
+template <typename IO, int K, int S, bool FLIP>
 int launch_down_bh(TilePlan &p, hipStream_t stream)
 {
     const int forced = env_int("DWCONV_TILE_BH", 0);
     const bool seven = forced ? forced == 7 : (p.out_h % 7 == 0 || p.out_h > 64) && p.out_h % 4 != 0;
-    return seven ? launch_down<K, S, FLIP, 7>(p, stream) : launch_down<K, S, FLIP, 4>(p, stream);
+    return seven ? launch_down<IO, K, S, FLIP, 7>(p, stream) : launch_down<IO, K, S, FLIP, 4>(p, stream);
 }
 
-template <int K, int EY, int EX>
+template <typename IO, int K, int EY, int EX>
 int launch_up2(TilePlan &p, hipStream_t stream)
 {
     constexpr int BQ = 4;
@@ -324,25 +324,26 @@ int launch_up2(TilePlan &p, hipStream_t stream)
     const int used_cols = 2 * (p.ncb - 1) + NW;
     auto rows_for = [](int units) { return units * BQ + KAY; };
     if (!plan_tiles(p, ceil_div(ceil_div(p.out_h, 2), BQ), BQ, used_cols, K * K, rows_for)) return -1;
-    hipLaunchKernelGGL((fir_up2_kernel<K, EY, EX, BQ>), dim3(p.n_tiles), dim3(env_int("DWCONV_TILE_THREADS", kThreads)), lds_bytes(p, K * K), stream,
+    hipLaunchKernelGGL((fir_up2_kernel<IO, K, EY, EX, BQ>), dim3(p.n_tiles), dim3(env_int("DWCONV_TILE_THREADS", kThreads)), lds_bytes(p, K * K), stream,
                        p);
-    note_variant("tile_up2<k%d,e%d%d,bq%d> P%d rows%d vin%d vout%d", K, EY, EX, BQ, p.planes_per_tile,
+    note_variant("tile_up2%s<k%d,e%d%d,bq%d> P%d rows%d vin%d vout%d", sizeof(IO) == 2 ? "16" : "", K, EY, EX, BQ, p.planes_per_tile,
                  p.rows_per_tile, p.st.vec_in, p.vec_out);
     return check_launch("fir_up2_kernel");
 }
 
-template <int K>
+template <typename IO, int K>
 int launch_up2_parity(TilePlan &p, int ey, int ex, hipStream_t stream)
 {
-    if (ey == 0 && ex == 0) return launch_up2<K, 0, 0>(p, stream);
-    if (ey == 0 && ex == 1) return launch_up2<K, 0, 1>(p, stream);
-    if (ey == 1 && ex == 0) return launch_up2<K, 1, 0>(p, stream);
-    return launch_up2<K, 1, 1>(p, stream);
+    if (ey == 0 && ex == 0) return launch_up2<IO, K, 0, 0>(p, stream);
+    if (ey == 0 && ex == 1) return launch_up2<IO, K, 0, 1>(p, stream);
+    if (ey == 1 && ex == 0) return launch_up2<IO, K, 1, 0>(p, stream);
+    return launch_up2<IO, K, 1, 1>(p, stream);
 }
 
 }  // namespace
 
-int try_launch_fir_tiled(const float *in, const float *taps, float *out, const Geometry &g, hipStream_t stream)
+template <typename IO>
+int try_launch_fir_tiled(const IO *in, const IO *taps, IO *out, const Geometry &g, hipStream_t stream)
 {
     const int K = g.kernel_h;
     if (g.kernel_w != K || (K != 3 && K != 5 && K != 7)) return -1;
@@ -364,32 +365,36 @@ int try_launch_fir_tiled(const float *in, const float *taps, float *out, const G
     p.out_w = g.out_w;
     p.st.in_plane = g.in_h * g.in_w;
     p.out_plane = g.out_h * g.out_w;
-    p.st.vec_in = (g.in_w % 4 == 0) && aligned16(in);
-    p.vec_out = (g.out_w % 4 == 0) && aligned16(out);
+    p.st.vec_in = (g.in_w % 4 == 0) && aligned4(in);
+    p.vec_out = (g.out_w % 4 == 0) && aligned4(out);
 
     if (g.up_h == 1 && g.up_w == 1 && g.down_h == g.down_w && (g.down_h == 1 || g.down_h == 2)) {
         p.row_shift = g.pad_h0;
         p.st.col_shift = g.pad_w0;
         const bool rot = !g.forward;
         if (g.down_h == 1) {
-            if (K == 3) return rot ? launch_down_bh<3, 1, true>(p, stream) : launch_down_bh<3, 1, false>(p, stream);
-            if (K == 5) return rot ? launch_down_bh<5, 1, true>(p, stream) : launch_down_bh<5, 1, false>(p, stream);
-            return rot ? launch_down_bh<7, 1, true>(p, stream) : launch_down_bh<7, 1, false>(p, stream);
+            if (K == 3) return rot ? launch_down_bh<IO, 3, 1, true>(p, stream) : launch_down_bh<IO, 3, 1, false>(p, stream);
+            if (K == 5) return rot ? launch_down_bh<IO, 5, 1, true>(p, stream) : launch_down_bh<IO, 5, 1, false>(p, stream);
+            return rot ? launch_down_bh<IO, 7, 1, true>(p, stream) : launch_down_bh<IO, 7, 1, false>(p, stream);
         }
         if (rot) return -1;
-        if (K == 3) return launch_down_bh<3, 2, false>(p, stream);
-        if (K == 5) return launch_down_bh<5, 2, false>(p, stream);
-        return launch_down_bh<7, 2, false>(p, stream);
+        if (K == 3) return launch_down_bh<IO, 3, 2, false>(p, stream);
+        if (K == 5) return launch_down_bh<IO, 5, 2, false>(p, stream);
+        return launch_down_bh<IO, 7, 2, false>(p, stream);
     }
     if (g.up_h == 2 && g.up_w == 2 && g.down_h == 1 && g.down_w == 1 && !g.forward) {
         const int ey = g.pad_h0 & 1, ex = g.pad_w0 & 1;
         p.row_shift = (g.pad_h0 + ey) / 2;
         p.st.col_shift = (g.pad_w0 + ex) / 2;
-        if (K == 3) return launch_up2_parity<3>(p, ey, ex, stream);
-        if (K == 5) return launch_up2_parity<5>(p, ey, ex, stream);
-        return launch_up2_parity<7>(p, ey, ex, stream);
+        if (K == 3) return launch_up2_parity<IO, 3>(p, ey, ex, stream);
+        if (K == 5) return launch_up2_parity<IO, 5>(p, ey, ex, stream);
+        return launch_up2_parity<IO, 7>(p, ey, ex, stream);
     }
     return -1;
 }
+
+template int try_launch_fir_tiled<float>(const float *, const float *, float *, const Geometry &, hipStream_t);
+template int try_launch_fir_tiled<half_t>(const half_t *, const half_t *, half_t *, const Geometry &, hipStream_t);
+template int try_launch_fir_tiled<bf16_t>(const bf16_t *, const bf16_t *, bf16_t *, const Geometry &, hipStream_t);
 
 }  // namespace dwconv

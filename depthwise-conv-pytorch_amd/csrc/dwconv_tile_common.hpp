@@ -26,8 +26,107 @@ struct StageLayout {
     unsigned spr_magic;
     int pitch;        // floats per LDS row, slack included
     int plane_pitch;  // floats per plane image
-    int vec_in;       // 128-bit global loads are legal (in_w % 4 == 0, 16-byte aligned base)
+    int vec_in;       // four elements may be loaded at once (in_w % 4 == 0, base aligned to four elements)
 };
+
+// Four consecutive elements (aligned to four elements) as fp32, and back.
+template <typename IO>
+__device__ __forceinline__ float4 load4(const IO *p);
+template <>
+__device__ __forceinline__ float4 load4<float>(const float *p)
+{
+    return *reinterpret_cast<const float4 *>(p);
+}
+template <>
+__device__ __forceinline__ float4 load4<half_t>(const half_t *p)
+{
+    const uint2 raw = *reinterpret_cast<const uint2 *>(p);
+    union { uint32_t u; half_t h[2]; } a, b;
+    a.u = raw.x;
+    b.u = raw.y;
+    return make_float4(static_cast<float>(a.h[0]), static_cast<float>(a.h[1]), static_cast<float>(b.h[0]),
+                       static_cast<float>(b.h[1]));
+}
+template <>
+__device__ __forceinline__ float4 load4<bf16_t>(const bf16_t *p)
+{
+    const uint2 raw = *reinterpret_cast<const uint2 *>(p);
+    return make_float4(__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u), __uint_as_float(raw.y << 16),
+                       __uint_as_float(raw.y & 0xffff0000u));
+}
+
+template <typename IO>
+__device__ __forceinline__ void store4(IO *p, float a, float b, float c, float d);
+template <>
+__device__ __forceinline__ void store4<float>(float *p, float a, float b, float c, float d)
+{
+    *reinterpret_cast<float4 *>(p) = make_float4(a, b, c, d);
+}
+template <>
+__device__ __forceinline__ void store4<half_t>(half_t *p, float a, float b, float c, float d)
+{
+    union { uint32_t u; half_t h[2]; } lo, hi;
+    lo.h[0] = static_cast<half_t>(a);
+    lo.h[1] = static_cast<half_t>(b);
+    hi.h[0] = static_cast<half_t>(c);
+    hi.h[1] = static_cast<half_t>(d);
+    *reinterpret_cast<uint2 *>(p) = make_uint2(lo.u, hi.u);
+}
+template <>
+__device__ __forceinline__ void store4<bf16_t>(bf16_t *p, float a, float b, float c, float d)
+{
+    const uint32_t lo = Io<bf16_t>::out(a).bits | (static_cast<uint32_t>(Io<bf16_t>::out(b).bits) << 16);
+    const uint32_t hi = Io<bf16_t>::out(c).bits | (static_cast<uint32_t>(Io<bf16_t>::out(d).bits) << 16);
+    *reinterpret_cast<uint2 *>(p) = make_uint2(lo, hi);
+}
+
+// The same four elements as loaded, not yet widened: half the registers for the 16-bit types.
+template <typename IO>
+struct Raw4 {
+    using type = float4;
+};
+template <>
+struct Raw4<half_t> {
+    using type = uint2;
+};
+template <>
+struct Raw4<bf16_t> {
+    using type = uint2;
+};
+template <typename IO>
+__device__ __forceinline__ typename Raw4<IO>::type load4_raw(const IO *p)
+{
+    return *reinterpret_cast<const typename Raw4<IO>::type *>(p);
+}
+template <typename IO>
+__device__ __forceinline__ float4 widen4(const typename Raw4<IO>::type &raw);
+template <>
+__device__ __forceinline__ float4 widen4<float>(const float4 &raw)
+{
+    return raw;
+}
+template <>
+__device__ __forceinline__ float4 widen4<half_t>(const uint2 &raw)
+{
+    union { uint32_t u; half_t h[2]; } a, b;
+    a.u = raw.x;
+    b.u = raw.y;
+    return make_float4(static_cast<float>(a.h[0]), static_cast<float>(a.h[1]), static_cast<float>(b.h[0]),
+                       static_cast<float>(b.h[1]));
+}
+template <>
+__device__ __forceinline__ float4 widen4<bf16_t>(const uint2 &raw)
+{
+    return make_float4(__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u), __uint_as_float(raw.y << 16),
+                       __uint_as_float(raw.y & 0xffff0000u));
+}
+
+// True when groups of four elements starting at `p` may be moved with one vector access.
+template <typename IO>
+inline bool aligned4(const IO *p)
+{
+    return (reinterpret_cast<uintptr_t>(p) & (4 * sizeof(IO) - 1)) == 0;
+}
 
 // n / d through the reciprocal made by magic_u16(d); a zero reciprocal stands for d == 1.
 __device__ __forceinline__ int fast_div(int n, unsigned magic)
@@ -51,7 +150,8 @@ __device__ __forceinline__ int xcd_contiguous_tile(int bid, int n_tiles)
 // their latencies overlap instead of adding up.
 constexpr int kStageBatch = 4;
 
-__device__ __forceinline__ void stage_tile(const StageLayout &s, const float *__restrict__ in, float *lds,
+template <typename IO>
+__device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__restrict__ in, float *lds,
                                            long plane0, int nplanes, int iy0)
 {
     const int total = nplanes * s.lds_rows * s.spr;
@@ -71,14 +171,14 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const float *__
                 const int ix = 4 * (s.g_lo + sc);
                 const int iy = iy0 + r;
                 const bool row_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(s.in_h);
-                const float *src = in + (plane0 + pl) * s.in_plane + static_cast<long>(iy) * s.in_w + ix;
+                const IO *src = in + (plane0 + pl) * s.in_plane + static_cast<long>(iy) * s.in_w + ix;
                 if (s.vec_in) {
-                    if (row_ok && ix >= 0 && ix < s.in_w) v[u] = *reinterpret_cast<const float4 *>(src);
+                    if (row_ok && ix >= 0 && ix < s.in_w) v[u] = load4<IO>(src);
                 } else if (row_ok) {
-                    if (static_cast<unsigned>(ix + 0) < static_cast<unsigned>(s.in_w)) v[u].x = src[0];
-                    if (static_cast<unsigned>(ix + 1) < static_cast<unsigned>(s.in_w)) v[u].y = src[1];
-                    if (static_cast<unsigned>(ix + 2) < static_cast<unsigned>(s.in_w)) v[u].z = src[2];
-                    if (static_cast<unsigned>(ix + 3) < static_cast<unsigned>(s.in_w)) v[u].w = src[3];
+                    if (static_cast<unsigned>(ix + 0) < static_cast<unsigned>(s.in_w)) v[u].x = Io<IO>::in(src[0]);
+                    if (static_cast<unsigned>(ix + 1) < static_cast<unsigned>(s.in_w)) v[u].y = Io<IO>::in(src[1]);
+                    if (static_cast<unsigned>(ix + 2) < static_cast<unsigned>(s.in_w)) v[u].z = Io<IO>::in(src[2]);
+                    if (static_cast<unsigned>(ix + 3) < static_cast<unsigned>(s.in_w)) v[u].w = Io<IO>::in(src[3]);
                 }
                 dst[u] = pl * s.plane_pitch + r * s.pitch + kSlack + ix + s.col_shift;
             }
@@ -116,8 +216,8 @@ __device__ __forceinline__ int stage_slot_offset(const StageLayout &s, int slot,
     return pl * s.plane_pitch + r * s.pitch + kSlack + 4 * (s.g_lo + sc) + s.col_shift;
 }
 
-template <int U>
-__device__ __forceinline__ void stage_fetch(const StageLayout &s, const float *__restrict__ in, long plane0,
+template <int U, typename IO>
+__device__ __forceinline__ void stage_fetch(const StageLayout &s, const IO *__restrict__ in, long plane0,
                                             int nplanes, int iy0, StagedTile<U> &t)
 {
     const int total = nplanes * s.lds_rows * s.spr;
@@ -133,14 +233,14 @@ __device__ __forceinline__ void stage_fetch(const StageLayout &s, const float *_
             const int ix = 4 * (s.g_lo + sc);
             const int iy = iy0 + r;
             const bool row_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(s.in_h);
-            const float *src = in + (plane0 + pl) * s.in_plane + static_cast<long>(iy) * s.in_w + ix;
+            const IO *src = in + (plane0 + pl) * s.in_plane + static_cast<long>(iy) * s.in_w + ix;
             if (s.vec_in) {
-                if (row_ok && ix >= 0 && ix < s.in_w) v = *reinterpret_cast<const float4 *>(src);
+                if (row_ok && ix >= 0 && ix < s.in_w) v = load4<IO>(src);
             } else if (row_ok) {
-                if (static_cast<unsigned>(ix + 0) < static_cast<unsigned>(s.in_w)) v.x = src[0];
-                if (static_cast<unsigned>(ix + 1) < static_cast<unsigned>(s.in_w)) v.y = src[1];
-                if (static_cast<unsigned>(ix + 2) < static_cast<unsigned>(s.in_w)) v.z = src[2];
-                if (static_cast<unsigned>(ix + 3) < static_cast<unsigned>(s.in_w)) v.w = src[3];
+                if (static_cast<unsigned>(ix + 0) < static_cast<unsigned>(s.in_w)) v.x = Io<IO>::in(src[0]);
+                if (static_cast<unsigned>(ix + 1) < static_cast<unsigned>(s.in_w)) v.y = Io<IO>::in(src[1]);
+                if (static_cast<unsigned>(ix + 2) < static_cast<unsigned>(s.in_w)) v.z = Io<IO>::in(src[2]);
+                if (static_cast<unsigned>(ix + 3) < static_cast<unsigned>(s.in_w)) v.w = Io<IO>::in(src[3]);
             }
         }
         t.v[u] = v;

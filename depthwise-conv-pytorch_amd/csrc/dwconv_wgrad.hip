@@ -24,8 +24,8 @@ namespace {
 
 struct WgradPlan {
     StageLayout st;
-    const float *x;
-    const float *gy;
+    const void *x;    // element type IO of the kernel template
+    const void *gy;
     float *partial;
     int batch, channel;
     int out_h, out_w, out_plane;
@@ -42,8 +42,8 @@ struct WgradPlan {
     unsigned ipp_magic;
     int vec_gy;
     // fused grad-input (stride 1, "same" padding): taps, destination, and where the gy image sits in LDS
-    const float *taps;
-    float *gx;
+    const void *taps;
+    void *gx;
     int g_base;            // float offset of the gy image (same layout as the x image)
     int vec_gx;
     int strided;           // chunk k takes tiles k, k+chunks, ... instead of a contiguous range
@@ -77,7 +77,7 @@ constexpr int kRedPitch = kThreads + 1;  // odd pitch: lanes of one wave reading
 // PF: the band(s) of the next tile are fetched into registers while the current tile is computed.
 constexpr int kPrefetchSlots = 4;  // float4 slots per lane and image
 
-template <int K, int S, int BH, bool GX, bool PF>
+template <typename IO, int K, int S, int BH, bool GX, bool PF>
 __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -86,6 +86,8 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
     constexpr int WIN_ROWS = (BH - 1) * S + K;
     constexpr int NV = (3 * S + K + 3) / 4;
     static_assert(!GX || S == 1, "the fused variant is the stride-1 one");
+    const IO *const x = static_cast<const IO *>(p.x);
+    const IO *const gy = static_cast<const IO *>(p.gy);
 
     const int group = blockIdx.x / p.chunks;
     const int chunk = blockIdx.x - group * p.chunks;
@@ -115,7 +117,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
     float rot[GX ? KK : 1];
     if constexpr (GX) {
 #pragma unroll
-        for (int t = 0; t < KK; ++t) rot[t] = p.taps[(c0 + pl) * KK + KK - 1 - t];
+        for (int t = 0; t < KK; ++t) rot[t] = Io<IO>::in(static_cast<const IO *>(p.taps)[(c0 + pl) * KK + KK - 1 - t]);
     }
 
     StagedTile<PF ? kPrefetchSlots : 1> tx, tg;
@@ -123,8 +125,8 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
         if (t_begin < t_end) {
             const int n = t_begin / p.row_tiles, rt = t_begin - n * p.row_tiles;
             const long plane0 = static_cast<long>(n) * p.channel + c0;
-            stage_fetch(p.st, p.x, plane0, nplanes, rt * p.rows_per_tile * S - p.pad_h, tx);
-            if constexpr (GX) stage_fetch(p.st, p.gy, plane0, nplanes, rt * p.rows_per_tile - p.pad_h, tg);
+            stage_fetch(p.st, x, plane0, nplanes, rt * p.rows_per_tile * S - p.pad_h, tx);
+            if constexpr (GX) stage_fetch(p.st, gy, plane0, nplanes, rt * p.rows_per_tile - p.pad_h, tg);
         }
     }
 
@@ -136,21 +138,21 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
         // this lane's block of gy (zero where it hangs over the edge of the plane); issued before the
         // x band is staged so that both sets of loads are in flight together
         float g[BH][4];
-        const float *gsrc = p.gy + (plane0 + pl) * p.out_plane + ox;
+        const IO *gsrc = gy + (plane0 + pl) * p.out_plane + ox;
 #pragma unroll
         for (int b = 0; b < BH; ++b) {
             if constexpr (GX) break;
             const int oy = oy0 + rb * BH + b;
-            const float *row = gsrc + static_cast<long>(oy) * p.out_w;
+            const IO *row = gsrc + static_cast<long>(oy) * p.out_w;
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
             if (has_item && oy < p.out_h) {
                 if (p.vec_gy) {
-                    v = *reinterpret_cast<const float4 *>(row);
+                    v = load4<IO>(row);
                 } else {
-                    if (ox + 0 < p.out_w) v.x = row[0];
-                    if (ox + 1 < p.out_w) v.y = row[1];
-                    if (ox + 2 < p.out_w) v.z = row[2];
-                    if (ox + 3 < p.out_w) v.w = row[3];
+                    if (ox + 0 < p.out_w) v.x = Io<IO>::in(row[0]);
+                    if (ox + 1 < p.out_w) v.y = Io<IO>::in(row[1]);
+                    if (ox + 2 < p.out_w) v.z = Io<IO>::in(row[2]);
+                    if (ox + 3 < p.out_w) v.w = Io<IO>::in(row[3]);
                 }
             }
             g[b][0] = v.x;
@@ -164,8 +166,8 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
             stage_commit(p.st, lds, nplanes, tx);
             if constexpr (GX) stage_commit(p.st, lds + p.g_base, nplanes, tg);
         } else {
-            stage_tile(p.st, p.x, lds, plane0, nplanes, oy0 * S - p.pad_h);
-            if constexpr (GX) stage_tile(p.st, p.gy, lds + p.g_base, plane0, nplanes, oy0 - p.pad_h);
+            stage_tile(p.st, x, lds, plane0, nplanes, oy0 * S - p.pad_h);
+            if constexpr (GX) stage_tile(p.st, gy, lds + p.g_base, plane0, nplanes, oy0 - p.pad_h);
         }
         __syncthreads();
         if constexpr (PF) {
@@ -173,8 +175,8 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
                 const int t1 = tile + t_step;
                 const int n1 = t1 / p.row_tiles, rt1 = t1 - n1 * p.row_tiles;
                 const long plane1 = static_cast<long>(n1) * p.channel + c0;
-                stage_fetch(p.st, p.x, plane1, nplanes, rt1 * p.rows_per_tile * S - p.pad_h, tx);
-                if constexpr (GX) stage_fetch(p.st, p.gy, plane1, nplanes, rt1 * p.rows_per_tile - p.pad_h, tg);
+                stage_fetch(p.st, x, plane1, nplanes, rt1 * p.rows_per_tile * S - p.pad_h, tx);
+                if constexpr (GX) stage_fetch(p.st, gy, plane1, nplanes, rt1 * p.rows_per_tile - p.pad_h, tg);
             }
         }
 
@@ -210,18 +212,18 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
                 pin_registers(xacc);
             }
             if (has_item) {
-                float *dst = p.gx + (plane0 + pl) * p.st.in_plane + ox;
+                IO *dst = static_cast<IO *>(p.gx) + (plane0 + pl) * p.st.in_plane + ox;
 #pragma unroll
                 for (int b = 0; b < BH; ++b) {
                     const int oy = oy0 + rb * BH + b;
                     if (oy >= p.st.in_h) continue;
-                    float *row = dst + static_cast<long>(oy) * p.st.in_w;
+                    IO *row = dst + static_cast<long>(oy) * p.st.in_w;
                     if (p.vec_gx) {
-                        *reinterpret_cast<float4 *>(row) = make_float4(xacc[b][0], xacc[b][1], xacc[b][2], xacc[b][3]);
+                        store4<IO>(row, xacc[b][0], xacc[b][1], xacc[b][2], xacc[b][3]);
                     } else {
 #pragma unroll
                         for (int o = 0; o < 4; ++o)
-                            if (ox + o < p.st.in_w) row[o] = xacc[b][o];
+                            if (ox + o < p.st.in_w) row[o] = Io<IO>::out(xacc[b][o]);
                     }
                 }
             }
@@ -286,8 +288,9 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
 // sums are combined by a fixed butterfly.
 constexpr int kFinalLanes = 8;
 
+template <typename IO>
 __global__ __launch_bounds__(256) void wgrad_tile_final_kernel(const float *__restrict__ partial,
-                                                               float *__restrict__ gw, const int channel_taps,
+                                                               IO *__restrict__ gw, const int channel_taps,
                                                                const int taps, const int chunks)
 {
     const int gid = blockIdx.x * blockDim.x + threadIdx.x;
@@ -310,7 +313,7 @@ __global__ __launch_bounds__(256) void wgrad_tile_final_kernel(const float *__re
     for (; k < k1; ++k) s += static_cast<double>(p[static_cast<long>(k) * taps]);
 #pragma unroll
     for (int off = 1; off < kFinalLanes; off <<= 1) s += __shfl_xor(s, off, 64);
-    if (live && part == 0) gw[e] = static_cast<float>(s);
+    if (live && part == 0) gw[e] = Io<IO>::out(static_cast<float>(s));
 }
 
 template <int K, int S, int BH>
@@ -434,16 +437,17 @@ struct WorkspaceQuery {
     }
 };
 
+template <typename IO>
 struct Launcher {
-    const float *x;
-    const float *gy;
-    float *gw;
+    const IO *x;
+    const IO *gy;
+    IO *gw;
     void *ws;
     size_t ws_bytes;
     const WgradGeometry &g;
     hipStream_t stream;
-    const float *taps = nullptr;  // with gx: also produce grad-input (stride 1, "same" padding)
-    float *gx = nullptr;
+    const IO *taps = nullptr;  // with gx: also produce grad-input (stride 1, "same" padding)
+    IO *gx = nullptr;
     int rc = -1;
     template <int K, int S, int BH>
     void operator()()
@@ -460,12 +464,12 @@ struct Launcher {
         p.x = x;
         p.gy = gy;
         p.partial = static_cast<float *>(ws);
-        p.st.vec_in = (g.in_w % 4 == 0) && aligned16(x);
-        p.vec_gy = (g.out_w % 4 == 0) && aligned16(gy);
+        p.st.vec_in = (g.in_w % 4 == 0) && aligned4(x);
+        p.vec_gy = (g.out_w % 4 == 0) && aligned4(gy);
         p.strided = env_int("DWCONV_WGRAD_STRIDED", 1);
         p.taps = taps;
         p.gx = gx;
-        p.vec_gx = (g.in_w % 4 == 0) && aligned16(gx);
+        p.vec_gx = (g.in_w % 4 == 0) && aligned4(gx);
         const size_t shmem = lds_bytes<K, S, BH>(p, fused);
         const dim3 grid(p.groups * p.chunks), block(kThreads);
         // prefetching costs ~35 registers: worth it for the 3x3 kernels, whose tiles also fit the slots
@@ -474,34 +478,35 @@ struct Launcher {
         if constexpr (S == 1) {
             if (fused) {
                 // the gy image is staged with the x image's layout: it needs the same 128-bit rule
-                p.st.vec_in = p.st.vec_in && aligned16(gy);
+                p.st.vec_in = p.st.vec_in && aligned4(gy);
                 if constexpr (K == 3) {
-                    if (pf) hipLaunchKernelGGL((wgrad_tile_kernel<K, S, BH, true, true>), grid, block, shmem, stream, p);
+                    if (pf) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, true, true>), grid, block, shmem, stream, p);
                 }
-                if (!pf) hipLaunchKernelGGL((wgrad_tile_kernel<K, S, BH, true, false>), grid, block, shmem, stream, p);
+                if (!pf) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, true, false>), grid, block, shmem, stream, p);
             }
         }
         if (!fused) {
             if constexpr (K == 3 && S == 1) {
-                if (pf) hipLaunchKernelGGL((wgrad_tile_kernel<K, S, BH, false, true>), grid, block, shmem, stream, p);
+                if (pf) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, false, true>), grid, block, shmem, stream, p);
             }
             if (!(pf && K == 3 && S == 1))
-                hipLaunchKernelGGL((wgrad_tile_kernel<K, S, BH, false, false>), grid, block, shmem, stream, p);
+                hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, false, false>), grid, block, shmem, stream, p);
         }
         rc = check_launch("wgrad_tile_kernel");
         if (rc != DWCONV_OK) return;
-        note_variant("%s<k%d,s%d,bh%d> P%d rows%d chunks%d vin%d vgy%d pf%d", fused ? "bwd_tile" : "wgrad_tile", K, S, BH,
-                     p.planes_per_tile, p.rows_per_tile, p.chunks, p.st.vec_in, p.vec_gy, pf && S == 1 ? 1 : 0);
+        note_variant("%s%s<k%d,s%d,bh%d> P%d rows%d chunks%d vin%d vgy%d pf%d", fused ? "bwd_tile" : "wgrad_tile",
+                     sizeof(IO) == 2 ? "16" : "", K, S, BH, p.planes_per_tile, p.rows_per_tile, p.chunks, p.st.vec_in, p.vec_gy, pf && S == 1 ? 1 : 0);
         rc = launch_wgrad_final(static_cast<const float *>(ws), gw, g.channel, K * K, p.chunks, stream);
     }
 };
 
 }  // namespace
 
-int launch_wgrad_final(const float *partial, float *gw, int channel, int taps, int chunks, hipStream_t stream)
+template <typename IO>
+int launch_wgrad_final(const float *partial, IO *gw, int channel, int taps, int chunks, hipStream_t stream)
 {
     const int total = channel * taps;
-    hipLaunchKernelGGL(wgrad_tile_final_kernel, dim3(ceil_div(total * kFinalLanes, 256)), dim3(256), 0, stream, partial,
+    hipLaunchKernelGGL(wgrad_tile_final_kernel<IO>, dim3(ceil_div(total * kFinalLanes, 256)), dim3(256), 0, stream, partial,
                        gw, total, taps, chunks);
     return check_launch("wgrad_tile_final_kernel");
 }
@@ -513,16 +518,18 @@ size_t wgrad_tiled_workspace(const WgradGeometry &g)
     return q.bytes;
 }
 
-int try_launch_wgrad_tiled(const float *in, const float *gy, float *gw, void *ws, size_t ws_bytes,
-                           const WgradGeometry &g, hipStream_t stream)
+template <typename IO>
+int try_launch_wgrad_tiled(const IO *in, const IO *gy, IO *gw, void *ws, size_t ws_bytes, const WgradGeometry &g,
+                           hipStream_t stream)
 {
-    Launcher l{in, gy, gw, ws, ws_bytes, g, stream};
+    Launcher<IO> l{in, gy, gw, ws, ws_bytes, g, stream};
     if (!dispatch(g, l)) return -1;
     return l.rc;
 }
 
-int try_launch_bwd_tiled(const float *in, const float *gy, const float *taps, float *gx, float *gw, void *ws,
-                         size_t ws_bytes, const WgradGeometry &g, hipStream_t stream)
+template <typename IO>
+int try_launch_bwd_tiled(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
+                         const WgradGeometry &g, hipStream_t stream)
 {
     if (env_int("DWCONV_NO_FUSED_TILE", 0)) return -1;
     const int K = g.kernel_h;
@@ -530,9 +537,20 @@ int try_launch_bwd_tiled(const float *in, const float *gy, const float *taps, fl
     // the x band's LDS layout
     if (g.down_h != 1 || g.down_w != 1 || g.kernel_w != K || g.pad_h != K / 2 || g.pad_w != K / 2) return -1;
     if (g.out_h != g.in_h || g.out_w != g.in_w) return -1;
-    Launcher l{in, gy, gw, ws, ws_bytes, g, stream, taps, gx};
+    Launcher<IO> l{in, gy, gw, ws, ws_bytes, g, stream, taps, gx};
     if (!dispatch(g, l)) return -1;
     return l.rc;
 }
+
+#define DWCONV_INSTANTIATE(IO)                                                                                        \
+    template int launch_wgrad_final<IO>(const float *, IO *, int, int, int, hipStream_t);                             \
+    template int try_launch_wgrad_tiled<IO>(const IO *, const IO *, IO *, void *, size_t, const WgradGeometry &,      \
+                                            hipStream_t);                                                             \
+    template int try_launch_bwd_tiled<IO>(const IO *, const IO *, const IO *, IO *, IO *, void *, size_t,             \
+                                          const WgradGeometry &, hipStream_t);
+DWCONV_INSTANTIATE(float)
+DWCONV_INSTANTIATE(half_t)
+DWCONV_INSTANTIATE(bf16_t)
+#undef DWCONV_INSTANTIATE
 
 }  // namespace dwconv

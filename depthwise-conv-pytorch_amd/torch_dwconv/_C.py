@@ -47,8 +47,9 @@ for _name in ("dwconv2d_backward_kernel_f32", "dwconv2d_backward_kernel_f64", "d
     getattr(_lib, _name).restype = _i
     getattr(_lib, _name).argtypes = [_p, _p, _p, _p, _z] + [_i] * 14 + [_p]
 
-_lib.dwconv2d_backward_f32.restype = _i
-_lib.dwconv2d_backward_f32.argtypes = [_p, _p, _p, _p, _p, _p, _z] + [_i] * 12 + [_p]
+for _name in ("dwconv2d_backward_f32", "dwconv2d_backward_f16", "dwconv2d_backward_bf16"):
+    getattr(_lib, _name).restype = _i
+    getattr(_lib, _name).argtypes = [_p, _p, _p, _p, _p, _p, _z] + [_i] * 12 + [_p]
 
 _SUFFIX = {torch.float32: "f32", torch.float64: "f64", torch.float16: "f16", torch.bfloat16: "bf16"}
 
@@ -179,7 +180,7 @@ def dwconv2d_backward_kernel(input, out_grad, kernel, up_h, up_w, down_h, down_w
 
 
 def dwconv2d_backward(input, out_grad, kernel, stride_h, stride_w, pad_h, pad_w):
-    """Both gradients of ``depthwise_conv2d(input, kernel, stride, pad)`` for float32 tensors.
+    """Both gradients of ``depthwise_conv2d(input, kernel, stride, pad)`` for float32, float16 or bfloat16 tensors.
 
     One call for the two the reference's backward makes (torch_dwconv/dwconv.py:56-68); the library reads
     ``out_grad`` once where a fused kernel covers the geometry.  Returns ``(grad_input, grad_kernel)``.
@@ -190,8 +191,9 @@ def dwconv2d_backward(input, out_grad, kernel, stride_h, stride_w, pad_h, pad_w)
     _check_shapes(input, kernel)
     if out_grad.dim() != 4 or out_grad.shape[:2] != input.shape[:2]:
         raise RuntimeError(f"out_grad of shape {tuple(out_grad.shape)} does not belong to input {tuple(input.shape)}")
-    if _suffix(input, out_grad, kernel) != "f32":
-        raise RuntimeError("dwconv2d_backward is a float32 entry point")
+    suffix = _suffix(input, out_grad, kernel)
+    if suffix == "f64":
+        raise RuntimeError("dwconv2d_backward has no float64 entry point")
     x, gy, k = input.contiguous(), out_grad.contiguous(), kernel.contiguous()
     n, c, h, w = x.shape
     oh, ow = gy.shape[2], gy.shape[3]
@@ -199,10 +201,10 @@ def dwconv2d_backward(input, out_grad, kernel, stride_h, stride_w, pad_h, pad_w)
     gx = torch.empty_like(x)
     gw = torch.empty_like(k)
     geom = (n, c, h, w, oh, ow, kh, kw)
-    ws_bytes = _lib.dwconv2d_backward_kernel_workspace_bytes(*geom, stride_h, stride_w, pad_h, pad_w, 4)
+    ws_bytes = _lib.dwconv2d_backward_kernel_workspace_bytes(*geom, stride_h, stride_w, pad_h, pad_w, x.element_size())
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):
-        rc = _lib.dwconv2d_backward_f32(
+        rc = getattr(_lib, "dwconv2d_backward_" + suffix)(
             x.data_ptr(), gy.data_ptr(), k.data_ptr(), gx.data_ptr(), gw.data_ptr(), ws.data_ptr(), ws_bytes,
             *geom, stride_h, stride_w, pad_h, pad_w, _stream(x),
         )

@@ -97,7 +97,7 @@ class DepthwiseConv2dFunction(Function):
         input, kernel = ctx.saved_tensors
         stride, pad, g_pad = ctx.stride, ctx.pad, ctx.g_pad
         # The reference always computes both gradients (:48-70).
-        if input.dtype == torch.float32 and grad_output.dtype == torch.float32 and kernel.dtype == torch.float32:
+        if input.dtype != torch.float64:
             # one library call for the pair of calls below; same values, out_grad read once where fused
             grad_input, grad_kernel = _C.dwconv2d_backward(
                 input, grad_output, kernel, stride[0], stride[1], pad[0], pad[1]

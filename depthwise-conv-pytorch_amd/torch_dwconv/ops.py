@@ -36,7 +36,7 @@ def _(input, weight, stride, padding):
 @torch.library.custom_op("torch_dwconv::depthwise_conv2d_backward", mutates_args=())
 def depthwise_conv2d_backward_op(input: torch.Tensor, grad_output: torch.Tensor, weight: torch.Tensor,
                                  stride: List[int], padding: List[int]) -> Tuple[torch.Tensor, torch.Tensor]:
-    if input.dtype == torch.float32:
+    if input.dtype != torch.float64:
         return _C.dwconv2d_backward(input, grad_output, weight, stride[0], stride[1], padding[0], padding[1])
     kh, kw = weight.shape[2], weight.shape[3]
     g_pad = (kh - padding[0] - 1, input.shape[2] - grad_output.shape[2] * stride[0] + padding[0],

@@ -177,6 +177,20 @@ int dwconv2d_backward_f32(const float *input, const float *out_grad, const float
                           int out_h, int out_w, int kernel_h, int kernel_w, int stride_h,
                           int stride_w, int pad_h, int pad_w, void *stream);
 
+/* fp16 / bfloat16 twins (fp32 products and sums, one rounding on store). */
+int dwconv2d_backward_f16(const unsigned short *input, const unsigned short *out_grad,
+                          const unsigned short *kernel, unsigned short *in_grad,
+                          unsigned short *kernel_grad, void *workspace, size_t workspace_bytes,
+                          int batch, int channel, int in_h, int in_w, int out_h, int out_w,
+                          int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+                          void *stream);
+int dwconv2d_backward_bf16(const unsigned short *input, const unsigned short *out_grad,
+                           const unsigned short *kernel, unsigned short *in_grad,
+                           unsigned short *kernel_grad, void *workspace, size_t workspace_bytes,
+                           int batch, int channel, int in_h, int in_w, int out_h, int out_w,
+                           int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+                           void *stream);
+
 /* Tuning/diagnostic hook: name of the kernel variant the last successful call
  * on this thread launched (e.g. "tile_f32<k3,s1,v4>"), for benchmarks and tests. */
 const char *dwconv_last_variant(void);

@@ -321,7 +321,9 @@ def test_c_entry_points_directly(dw, gpu):
 
 
 HALF_SHAPES = [(2, 6, 14, 14, 3, 1, 1), (2, 5, 28, 28, 5, 2, 2), (2, 4, 56, 56, 3, 1, 1), (2, 3, 57, 59, 5, 2, 2),
-               (1, 8, 7, 7, 5, 1, 2), (2, 4, 112, 112, 3, 2, 1), (1, 2, 33, 35, 7, 1, 3), (2, 8, 14, 14, 5, 2, 2)]
+               (1, 8, 7, 7, 5, 1, 2), (2, 4, 112, 112, 3, 2, 1), (1, 2, 33, 35, 7, 1, 3), (2, 8, 14, 14, 5, 2, 2),
+               (3, 4, 28, 28, 7, 1, 3), (2, 8, 7, 7, 7, 1, 3), (2, 3, 64, 64, 5, 2, 2), (2, 3, 40, 44, 7, 2, 3),
+               (3, 5, 14, 14, 7, 1, 3), (1, 3, 9, 11, 4, 2, 1)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
@@ -346,6 +348,35 @@ def test_half_precision_io(dw, gpu, shape, dtype):
     # bit-identical grad-weight from run to run here too
     _, _, gw2, _ = run_three_passes(dw, x.to(gpu), wt.to(gpu), gy.to(gpu), s, p)
     assert torch.equal(gw, gw2)
+    # the two entry points the reference's backward calls, and tensors whose base is not aligned to four elements
+    gx_s, gw_s = run_separate_backward(x.to(gpu), wt.to(gpu), gy.to(gpu), s, p)
+    np.testing.assert_allclose(_np(gx_s.double()), gx_ref, rtol=step, atol=1e-5 + step * 1e-2)
+    np.testing.assert_allclose(_np(gw_s.double()), gw_ref, rtol=step + 1e-4, atol=(step + 1e-4) * float(np.abs(gw_ref).max()))
+
+    def shifted(t):
+        flat = torch.empty(t.numel() + 1, dtype=t.dtype, device=gpu)
+        flat[1:] = t.to(gpu).reshape(-1)
+        return flat[1:].view(t.shape)
+
+    y_u, gx_u, gw_u, _ = run_three_passes(dw, shifted(x), wt.to(gpu), shifted(gy), s, p)
+    assert torch.equal(y_u, y) and torch.equal(gx_u, gx)
+    np.testing.assert_allclose(_np(gw_u.double()), gw_ref, rtol=step + 1e-4, atol=(step + 1e-4) * float(np.abs(gw_ref).max()))
+
+
+def test_half_precision_uses_the_fast_kernels(dw, gpu):
+    """fp16 tensors of the benchmark's layer shapes go through the tiled / whole-plane kernels, not the generic one."""
+    from torch_dwconv import _C
+
+    for shape, fwd, bwd in [((2, 8, 112, 112, 3, 1, 1), "tile_down16", "bwd_tile16"),
+                            ((2, 8, 112, 112, 3, 2, 1), "tile_down16", "bwd_tile_s216"),
+                            ((2, 8, 14, 14, 5, 1, 2), "small_down16", "small_bwd16"),
+                            ((2, 8, 28, 28, 3, 1, 1), "small_down16", "small_bwd16")]:
+        n, c, h, w, k, s, p = shape
+        x, wt, gy = (t.to(torch.float16).to(gpu) for t in make_inputs(shape, seed=3))
+        dw.depthwise_conv2d(x, wt, stride=s, padding=p)
+        assert _C.last_variant().startswith(fwd), _C.last_variant()
+        _C.dwconv2d_backward(x, gy, wt, s, s, p, p)
+        assert _C.last_variant().startswith(bwd), _C.last_variant()
 
 
 def test_combined_backward_entry_point(dw, gpu):
