@@ -47,13 +47,18 @@ WORKLOADS = {
 class Layer:
     """Device tensors and the three C-ABI calls of one depthwise layer."""
 
-    def __init__(self, shape, lib, torch, dev, gen, dtype="f32"):
+    def __init__(self, shape, lib, torch, dev, gen, dtype="f32", layout="nchw"):
         n, c, h, w, k, s, p = shape
         tdtype = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype]
         es = 4 if dtype == "f32" else 2
         self.fn_fir = getattr(lib, "dwconv2d_" + dtype)
         self.fn_wgrad = getattr(lib, "dwconv2d_backward_kernel_" + dtype)
         self.fn_bwd = getattr(lib, "dwconv2d_backward_" + dtype)
+        self.layout = layout
+        if layout == "nhwc":
+            self.fn_fir = self.fn_wgrad = None
+            self.fn_fwd_nhwc = getattr(lib, "dwconv2d_nhwc_" + dtype)
+            self.fn_bwd = getattr(lib, "dwconv2d_backward_nhwc_" + dtype)
         self.shape = shape
         self.lib = lib
         oh, ow = (h + 2 * p - k) // s + 1, (w + 2 * p - k) // s + 1
@@ -64,7 +69,9 @@ class Layer:
         self.y = torch.empty(n, c, oh, ow, device=dev, dtype=tdtype)
         self.gx = torch.empty_like(self.x)
         self.gw = torch.empty_like(self.w)
-        self.ws_bytes = lib.dwconv2d_backward_kernel_workspace_bytes(n, c, h, w, oh, ow, k, k, s, s, p, p, es)
+        # channels-last: the same element counts, stored (N,H,W,C); values are random either way
+        self.ws_bytes = (lib.dwconv2d_backward_nhwc_workspace_bytes(n, c, h, w, k, k, s, s, p, p, es) if layout == "nhwc"
+                         else lib.dwconv2d_backward_kernel_workspace_bytes(n, c, h, w, oh, ow, k, k, s, s, p, p, es))
         self.ws = torch.empty(max(self.ws_bytes, 16), dtype=torch.uint8, device=dev)
         nx, ny, nw = n * c * h * w, n * c * oh * ow, c * k * k
         self.bytes = {"fwd": es * (nx + ny + nw), "gx": es * (ny + nx + nw), "gw": es * (nx + ny + nw)}
@@ -81,6 +88,10 @@ class Layer:
 
     def fwd(self, stream):
         n, c, h, w, oh, ow, k, s, p = self.geom
+        if self.layout == "nhwc":
+            self._check(self.fn_fwd_nhwc(self.x.data_ptr(), self.w.data_ptr(), self.y.data_ptr(), n, c, h, w, k, k,
+                                         s, s, p, p, stream))
+            return
         self._check(self.fn_fir(self.x.data_ptr(), self.w.data_ptr(), self.y.data_ptr(), n, c, h, w, k, k,
                                           1, 1, s, s, p, p, p, p, 1, stream))
 
@@ -179,6 +190,8 @@ def main():
     ap.add_argument("--batch", type=int, default=128)
     ap.add_argument("--dtype", default="f32", choices=["f32", "f16", "bf16"],
                     help="element type of the tensors (the headline metric is f32; 16-bit types accumulate in fp32)")
+    ap.add_argument("--layout", default="nchw", choices=["nchw", "nhwc"],
+                    help="memory layout of the activations (the headline metric is nchw, the reference's layout)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-miopen", action="store_true")
     ap.add_argument("--separate-backward", action="store_true",
@@ -202,7 +215,9 @@ def main():
     lib = _C._lib
     shapes = WORKLOADS[args.workload](args.batch)
     gen = torch.Generator("cpu").manual_seed(0)
-    layers = [Layer(s, lib, torch, dev, gen, args.dtype) for s in shapes]
+    if args.layout == "nhwc" and args.separate_backward:
+        sys.exit("--separate-backward applies to the nchw entry points")
+    layers = [Layer(s, lib, torch, dev, gen, args.dtype, args.layout) for s in shapes]
     calls = schedule(layers, args.separate_backward)
     stream_obj = torch.cuda.current_stream(dev)
     stream = ctypes.c_void_p(stream_obj.cuda_stream)
@@ -290,7 +305,7 @@ def main():
         "dtype": args.dtype,
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: {len(layers)} depthwise layers, "
-                               f"{'fp32' if args.dtype == 'f32' else args.dtype} NCHW, batch {shapes[0][0]}, "
+                               f"{'fp32' if args.dtype == 'f32' else args.dtype} {args.layout.upper()}, batch {shapes[0][0]}, "
                                "fwd + grad-input + grad-weight per layer, training order, "
                                f"{len(calls)} C-ABI calls per step",
                    "layers": [l.name for l in layers], "algorithmic_bytes_per_step": step_bytes},
@@ -307,14 +322,14 @@ def main():
             print(f"{r['layer']:>18} {r['pass']:>3} {r['us']:9.1f} us {r['GBs']:8.1f} GB/s  {r['variant']}", file=sys.stderr)
     result["per_pass_us"] = {k: round(sum(r["us"] for r in rows if r["pass"] == k), 1)
                              for k in ("fwd", "gx", "gw", "bwd") if any(r["pass"] == k for r in rows)}
-    if not args.no_miopen:
+    if not args.no_miopen and args.layout == "nchw":
         try:
             per_layer = miopen_native(layers, torch)
             result["miopen_native_ms_per_step"] = round(sum(per_layer), 3)
             result["speedup_vs_miopen_native"] = round(sum(per_layer) / ms_per_step, 2)
         except Exception as e:  # the comparison is informative only
             result["miopen_native_ms_per_step"] = f"failed: {type(e).__name__}"
-    if not args.no_cpu_baseline and args.dtype == "f32":
+    if not args.no_cpu_baseline and args.dtype == "f32" and args.layout == "nchw":
         result["cpu_baseline"] = cpu_baseline(shapes, torch)
     print(json.dumps(result))
 

@@ -2,6 +2,7 @@
 // argument checks, kernel-family selection, error strings.
 #include "dwconv_common.hpp"
 
+#include <algorithm>
 #include <type_traits>
 
 #include <cstdarg>
@@ -254,6 +255,74 @@ int backward_any(const T *in, const T *gy, const T *taps, T *gx, T *gw, void *ws
     return rc;
 }
 
+// ---- channels-last entry points ----
+int make_nhwc_geometry(NhwcGeometry &g, int batch, int channel, int in_h, int in_w, int kernel_h, int kernel_w,
+                       int stride_h, int stride_w, int pad_h, int pad_w)
+{
+    if (batch < 0 || channel < 0 || in_h < 0 || in_w < 0)
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "negative tensor extent (batch %d, channel %d, input %dx%d)", batch,
+                    channel, in_h, in_w);
+    if (kernel_h < 1 || kernel_w < 1)
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "kernel extent must be >= 1, got %dx%d", kernel_h, kernel_w);
+    if (stride_h < 1 || stride_w < 1)
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "stride must be >= 1, got %dx%d", stride_h, stride_w);
+    if (pad_h < 0 || pad_w < 0) return fail(DWCONV_ERR_INVALID_ARGUMENT, "padding must be >= 0, got %dx%d", pad_h, pad_w);
+    g = NhwcGeometry{batch, channel, in_h, in_w, 0, 0, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w};
+    g.out_h = std::max(0, dwconv_out_size(in_h, 1, stride_h, pad_h, pad_h, kernel_h));
+    g.out_w = std::max(0, dwconv_out_size(in_w, 1, stride_w, pad_w, pad_w, kernel_w));
+    if (1ll * batch * channel * in_h * in_w >= (1ll << 40) || 1ll * batch * channel * g.out_h * g.out_w >= (1ll << 40))
+        return fail(DWCONV_ERR_UNSUPPORTED, "tensor too large");
+    return DWCONV_OK;
+}
+
+template <typename T>
+int nhwc_forward_any(const T *in, const T *taps, T *out, int batch, int channel, int in_h, int in_w, int kernel_h,
+                     int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w, void *stream)
+{
+    NhwcGeometry g;
+    const int rc = make_nhwc_geometry(g, batch, channel, in_h, in_w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w);
+    if (rc != DWCONV_OK) return rc;
+    const long long out_elems = 1ll * batch * channel * g.out_h * g.out_w;
+    if (out_elems > 0 && (in == nullptr || taps == nullptr || out == nullptr))
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");
+    return nhwc_forward<T>(in, taps, out, g, static_cast<hipStream_t>(stream));
+}
+
+template <typename T>
+int nhwc_backward_any(const T *in, const T *gy, const T *taps, T *gx, T *gw, void *ws, size_t ws_bytes, int batch,
+                      int channel, int in_h, int in_w, int out_h, int out_w, int kernel_h, int kernel_w, int stride_h,
+                      int stride_w, int pad_h, int pad_w, void *stream_)
+{
+    NhwcGeometry g;
+    int rc = make_nhwc_geometry(g, batch, channel, in_h, in_w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w);
+    if (rc != DWCONV_OK) return rc;
+    if (g.out_h != std::max(0, out_h) || g.out_w != std::max(0, out_w))
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "out_grad extent %dx%d does not match the convolution geometry", out_h,
+                    out_w);
+    if (gx == nullptr && gw == nullptr) return fail(DWCONV_ERR_INVALID_ARGUMENT, "neither in_grad nor kernel_grad given");
+    const bool has_out = 1ll * batch * channel * g.out_h * g.out_w > 0;
+    if (has_out && gy == nullptr) return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    char first[sizeof(g_variant)] = "";
+    if (gx != nullptr) {
+        if (has_out && taps == nullptr) return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");
+        rc = nhwc_grad_input<T>(gy, taps, gx, g, stream);
+        if (rc != DWCONV_OK) return rc;
+        std::snprintf(first, sizeof(first), "%s", g_variant);
+    }
+    if (gw != nullptr) {
+        if (has_out && in_h > 0 && in_w > 0 && in == nullptr) return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");
+        rc = nhwc_grad_weight<T>(in, gy, gw, ws, ws_bytes, g, stream);
+        if (rc != DWCONV_OK) return rc;
+        if (gx != nullptr) {
+            char second[sizeof(g_variant)];
+            std::snprintf(second, sizeof(second), "%s", g_variant);
+            note_variant("%.60s + %.60s", first, second);
+        }
+    }
+    return DWCONV_OK;
+}
+
 }  // namespace
 }  // namespace dwconv
 
@@ -404,5 +473,44 @@ int dwconv2d_backward_f32(const float *input, const float *out_grad, const float
                                channel, in_h, in_w, out_h, out_w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w,
                                stream);
 }
+
+// ---- channels-last tensors ----
+size_t dwconv2d_backward_nhwc_workspace_bytes(int batch, int channel, int in_h, int in_w, int kernel_h, int kernel_w,
+                                              int stride_h, int stride_w, int pad_h, int pad_w, int elem_size)
+{
+    NhwcGeometry g;
+    if (make_nhwc_geometry(g, batch, channel, in_h, in_w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w) != DWCONV_OK)
+        return 0;
+    if (batch == 0 || channel == 0) return 0;
+    if (elem_size == 8) return nhwc_grad_weight_workspace<double>(g);
+    if (elem_size == 2) return nhwc_grad_weight_workspace<half_t>(g);
+    return nhwc_grad_weight_workspace<float>(g);
+}
+
+#define DWCONV_NHWC_ENTRY_POINTS(SUFFIX, CTYPE, TYPE)                                                                  \
+    int dwconv2d_nhwc_##SUFFIX(const CTYPE *input, const CTYPE *kernel, CTYPE *out, int batch, int channel, int in_h,  \
+                               int in_w, int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w, \
+                               void *stream)                                                                           \
+    {                                                                                                                  \
+        return nhwc_forward_any<TYPE>(reinterpret_cast<const TYPE *>(input), reinterpret_cast<const TYPE *>(kernel),   \
+                                      reinterpret_cast<TYPE *>(out), batch, channel, in_h, in_w, kernel_h, kernel_w,   \
+                                      stride_h, stride_w, pad_h, pad_w, stream);                                       \
+    }                                                                                                                  \
+    int dwconv2d_backward_nhwc_##SUFFIX(const CTYPE *input, const CTYPE *out_grad, const CTYPE *kernel, CTYPE *in_grad, \
+                                        CTYPE *kernel_grad, void *workspace, size_t workspace_bytes, int batch,        \
+                                        int channel, int in_h, int in_w, int out_h, int out_w, int kernel_h,           \
+                                        int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w, void *stream)  \
+    {                                                                                                                  \
+        return nhwc_backward_any<TYPE>(reinterpret_cast<const TYPE *>(input), reinterpret_cast<const TYPE *>(out_grad), \
+                                       reinterpret_cast<const TYPE *>(kernel), reinterpret_cast<TYPE *>(in_grad),      \
+                                       reinterpret_cast<TYPE *>(kernel_grad), workspace, workspace_bytes, batch,       \
+                                       channel, in_h, in_w, out_h, out_w, kernel_h, kernel_w, stride_h, stride_w,      \
+                                       pad_h, pad_w, stream);                                                          \
+    }
+DWCONV_NHWC_ENTRY_POINTS(f32, float, float)
+DWCONV_NHWC_ENTRY_POINTS(f64, double, double)
+DWCONV_NHWC_ENTRY_POINTS(f16, unsigned short, half_t)
+DWCONV_NHWC_ENTRY_POINTS(bf16, unsigned short, bf16_t)
+#undef DWCONV_NHWC_ENTRY_POINTS
 
 }  // extern "C"

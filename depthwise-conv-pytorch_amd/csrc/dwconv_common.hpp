@@ -76,6 +76,16 @@ struct WgradGeometry {
     int pad_h, pad_w;
 };
 
+// Geometry of a channels-last call: input (N,H,W,C), output (N,OH,OW,C), taps (C,1,KH,KW).
+struct NhwcGeometry {
+    int batch, channel;
+    int in_h, in_w;
+    int out_h, out_w;
+    int kernel_h, kernel_w;
+    int stride_h, stride_w;
+    int pad_h, pad_w;
+};
+
 // Thread-local error/variant strings behind dwconv_last_error()/dwconv_last_variant().
 int fail(dwconv_status code, const char *fmt, ...);
 void note_variant(const char *fmt, ...);
@@ -140,5 +150,16 @@ size_t bwd_s2_workspace(const WgradGeometry &g);  // 0 when that kernel does not
 template <typename IO>
 int try_launch_bwd_s2(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
                       const WgradGeometry &g, hipStream_t stream);
+
+// ---- channels-last kernels: dwconv_nhwc.hip (T = float, double, half_t or bf16_t) ----
+template <typename T>
+int nhwc_forward(const T *in, const T *taps, T *out, const NhwcGeometry &g, hipStream_t stream);
+template <typename T>
+int nhwc_grad_input(const T *gy, const T *taps, T *gx, const NhwcGeometry &g, hipStream_t stream);
+template <typename T>
+size_t nhwc_grad_weight_workspace(const NhwcGeometry &g);
+template <typename T>
+int nhwc_grad_weight(const T *x, const T *gy, T *gw, void *ws, size_t ws_bytes, const NhwcGeometry &g,
+                     hipStream_t stream);
 
 }  // namespace dwconv

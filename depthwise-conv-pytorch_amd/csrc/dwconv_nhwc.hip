@@ -1,0 +1,787 @@
+// Depthwise conv2d on channels-last tensors: input (N,H,W,C), taps (C,1,KH,KW) as everywhere else, output (N,OH,OW,C).
+//
+// The reference makes every tensor NCHW-contiguous before its kernels run (torch_dwconv/dwconv_kernel.cu:741,
+// :855, :1023), which costs a layout-conversion pass either side of the op for a channels-last network.  These
+// kernels read and write channels-last directly.  Channels are the fastest dimension, so lanes run along C:
+//   * a lane owns CV consecutive channels (one vector access per pixel) and a BH x TW block of output pixels;
+//     it walks the input rows of its block once, keeps one row of the window in registers and feeds every
+//     output row that the input row touches; neighbouring lanes (next channels) read neighbouring addresses;
+//   * taps are transposed once per workgroup into LDS as [tap][channel], so a lane reads the taps of its
+//     channels as one vector;
+//   * grad-weight keeps K*K*CV sums per lane over a chunk of pixel blocks, adds the lanes of a workgroup that
+//     share channels through LDS in a fixed order, and leaves partial[chunk][tap][C] for a second kernel that
+//     adds the chunks in a fixed order: bit-identical from run to run, no atomics.
+// Geometries outside the fast kernels (C not a multiple of 4, filters other than 3/5/7, fp64) take the
+// one-lane-per-element kernels at the end of the file.
+#include "dwconv_tile_common.hpp"
+
+#include <algorithm>
+#include <type_traits>
+
+namespace dwconv {
+
+namespace {
+
+constexpr int kNhwcThreads = 256;
+constexpr int kNhwcTapLds = 48 * 1024;
+
+struct NhwcPlan {
+    const void *in;    // element type IO of the kernel template
+    const void *in2;   // grad-weight: out_grad
+    const void *taps;
+    void *out;
+    float *partial;
+    int batch, channel;
+    int in_h, in_w, out_h, out_w;
+    int pad_h, pad_w;        // leading zeros (down kernels); floor(pad / 2) for the stride-2 transposed kernel
+    int lanes_c;             // channel lanes per workgroup (each CV channels wide)
+    unsigned lanes_c_magic;
+    int blocks_per_wg;       // pixel blocks per workgroup = 256 / lanes_c
+    int blocks_x, blocks_y;  // pixel blocks per image
+    long blocks_total;       // batch * blocks_y * blocks_x
+    int groups;              // grad-weight: workgroups along the pixel-block axis (= chunks)
+};
+
+template <typename IO, int CV>
+__device__ __forceinline__ void load_cv(const IO *p, float (&v)[CV])
+{
+    if constexpr (CV == 4) {
+        const float4 t = load4<IO>(p);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    } else if constexpr (CV == 2 && sizeof(IO) == 4) {
+        const float2 t = *reinterpret_cast<const float2 *>(p);
+        v[0] = t.x; v[1] = t.y;
+    } else {
+#pragma unroll
+        for (int i = 0; i < CV; ++i) v[i] = Io<IO>::in(p[i]);
+    }
+}
+
+// One row of a lane's window: COLS pixels x CV channels from row iy, columns ix0.. of an image with C channels.
+// Pixels outside the image read a valid (clamped) address and are zeroed afterwards.
+template <typename IO, int COLS, int CV = 4>
+__device__ __forceinline__ void nhwc_load_row(const IO *src, int iy, int ix0, int in_h, int in_w, int C,
+                                              float (&row)[COLS * CV])
+{
+    const bool row_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(in_h);
+    const long row_off = static_cast<long>(min(max(iy, 0), in_h - 1)) * in_w;
+#pragma unroll
+    for (int j = 0; j < COLS; ++j) {
+        const int ix = ix0 + j;
+        const bool ok = row_ok && static_cast<unsigned>(ix) < static_cast<unsigned>(in_w);
+        float t[CV];
+        load_cv<IO, CV>(src + (row_off + min(max(ix, 0), in_w - 1)) * C, t);
+#pragma unroll
+        for (int v = 0; v < CV; ++v) row[CV * j + v] = ok ? t[v] : 0.f;
+    }
+}
+
+// Transposes the taps of channels [c0, c0 + nch) into LDS as [tap][channel] (rotated by 180 degrees when FLIP).
+template <typename IO, int KK, bool FLIP>
+__device__ __forceinline__ void nhwc_stage_taps(const IO *__restrict__ taps, float *lds, int c0, int nch)
+{
+    for (int i = threadIdx.x; i < nch * KK; i += blockDim.x) {
+        const int cl = i / KK, t = i - cl * KK;
+        lds[(FLIP ? KK - 1 - t : t) * nch + cl] = Io<IO>::in(taps[static_cast<long>(c0) * KK + i]);
+    }
+}
+
+// out[n,oy,ox,c] = sum_{ty,tx} in[n, oy*S - pad_h + ty, ox*S - pad_w + tx, c] * f[c,ty,tx]
+template <typename IO, int K, int S, bool FLIP, int BH, int TW>
+__global__ __launch_bounds__(kNhwcThreads) void nhwc_down_kernel(const NhwcPlan p)
+{
+    extern __shared__ float4 lds_raw[];
+    float *lds = reinterpret_cast<float *>(lds_raw);
+    constexpr int KK = K * K;
+    constexpr int ROWS = (BH - 1) * S + K, COLS = (TW - 1) * S + K;
+    const int C = p.channel;
+    const int c0 = blockIdx.y * p.lanes_c * 4;
+    const int nch = min(p.lanes_c * 4, C - c0);
+    nhwc_stage_taps<IO, KK, FLIP>(static_cast<const IO *>(p.taps), lds, c0, nch);
+    __syncthreads();
+
+    const int pb_local = fast_div(threadIdx.x, p.lanes_c_magic);
+    const int lane_c = threadIdx.x - pb_local * p.lanes_c;
+    const long pb = static_cast<long>(blockIdx.x) * p.blocks_per_wg + pb_local;
+    if (pb_local >= p.blocks_per_wg || pb >= p.blocks_total || 4 * lane_c >= nch) return;
+    const int per_image = p.blocks_x * p.blocks_y;
+    const int n = static_cast<int>(pb / per_image);
+    const int rem = static_cast<int>(pb - static_cast<long>(n) * per_image);
+    const int by = rem / p.blocks_x, bx = rem - by * p.blocks_x;
+    const int oy0 = by * BH, ox0 = bx * TW;
+    const int iy0 = oy0 * S - p.pad_h, ix0 = ox0 * S - p.pad_w;
+    const int c = c0 + 4 * lane_c;
+    const IO *src = static_cast<const IO *>(p.in) + static_cast<long>(n) * p.in_h * p.in_w * C + c;
+    const float *wl = lds + 4 * lane_c;
+
+    float acc[BH][TW * 4];
+#pragma unroll
+    for (int b = 0; b < BH; ++b)
+#pragma unroll
+        for (int o = 0; o < TW * 4; ++o) acc[b][o] = 0.f;
+
+    // Rows are loaded one ahead of their use and the sums pinned after every row: otherwise the compiler
+    // hoists the loads of the whole window to the top and keeps all of it in registers.
+    float cur[COLS * 4], nxt[COLS * 4];
+    nhwc_load_row<IO, COLS>(src, iy0, ix0, p.in_h, p.in_w, C, cur);
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        if (r + 1 < ROWS) nhwc_load_row<IO, COLS>(src, iy0 + r + 1, ix0, p.in_h, p.in_w, C, nxt);
+#pragma unroll
+        for (int b = 0; b < BH; ++b) {
+            const int ty = r - b * S;
+            if (ty < 0 || ty >= K) continue;
+#pragma unroll
+            for (int tx = 0; tx < K; ++tx) {
+                const float4 w = *reinterpret_cast<const float4 *>(wl + (ty * K + tx) * nch);
+#pragma unroll
+                for (int o = 0; o < TW; ++o) {
+                    acc[b][4 * o + 0] = fmaf(cur[4 * (o * S + tx) + 0], w.x, acc[b][4 * o + 0]);
+                    acc[b][4 * o + 1] = fmaf(cur[4 * (o * S + tx) + 1], w.y, acc[b][4 * o + 1]);
+                    acc[b][4 * o + 2] = fmaf(cur[4 * (o * S + tx) + 2], w.z, acc[b][4 * o + 2]);
+                    acc[b][4 * o + 3] = fmaf(cur[4 * (o * S + tx) + 3], w.w, acc[b][4 * o + 3]);
+                }
+            }
+        }
+        pin_registers(acc);
+#pragma unroll
+        for (int j = 0; j < COLS * 4; ++j) cur[j] = nxt[j];
+    }
+
+    IO *dst = static_cast<IO *>(p.out) + static_cast<long>(n) * p.out_h * p.out_w * C + c;
+#pragma unroll
+    for (int b = 0; b < BH; ++b) {
+        const int oy = oy0 + b;
+        if (oy >= p.out_h) continue;
+#pragma unroll
+        for (int o = 0; o < TW; ++o) {
+            const int ox = ox0 + o;
+            if (ox < p.out_w)
+                store4<IO>(dst + (static_cast<long>(oy) * p.out_w + ox) * C, acc[b][4 * o], acc[b][4 * o + 1],
+                           acc[b][4 * o + 2], acc[b][4 * o + 3]);
+        }
+    }
+}
+
+// Grad-input of a stride-2 convolution with padding 2*p.pad_h + PE (same for both axes), taps as stored:
+//   gx[iy,ix] = sum over (ty,tx) with iy + pad - ty and ix + pad - tx even of gy[(iy+pad-ty)/2, (ix+pad-tx)/2] * w[ty,tx].
+// A lane owns a BH x TW block of gx that starts on even coordinates, so which taps meet which gy sample is
+// known at compile time: row b of the block and gy row d (relative to iy0/2 + floor(pad/2)) meet in tap
+// ty = b + PE - 2d.  The zero-stuffed intermediate of the reference (torch_dwconv/dwconv_kernel.cu:822-832) never exists.
+template <typename IO, int K, int PE, int BH, int TW>
+__global__ __launch_bounds__(kNhwcThreads) void nhwc_up2_kernel(const NhwcPlan p)
+{
+    extern __shared__ float4 lds_raw[];
+    float *lds = reinterpret_cast<float *>(lds_raw);
+    constexpr int KK = K * K;
+    static_assert(BH % 2 == 0 && TW % 2 == 0, "blocks start on even coordinates");
+    constexpr int DMIN = -((K - 1 - PE) / 2);
+    constexpr int GROWS = (BH - 1 + PE) / 2 - DMIN + 1, GCOLS = (TW - 1 + PE) / 2 - DMIN + 1;
+    const int C = p.channel;
+    const int c0 = blockIdx.y * p.lanes_c * 4;
+    const int nch = min(p.lanes_c * 4, C - c0);
+    nhwc_stage_taps<IO, KK, false>(static_cast<const IO *>(p.taps), lds, c0, nch);
+    __syncthreads();
+
+    const int pb_local = fast_div(threadIdx.x, p.lanes_c_magic);
+    const int lane_c = threadIdx.x - pb_local * p.lanes_c;
+    const long pb = static_cast<long>(blockIdx.x) * p.blocks_per_wg + pb_local;
+    if (pb_local >= p.blocks_per_wg || pb >= p.blocks_total || 4 * lane_c >= nch) return;
+    const int per_image = p.blocks_x * p.blocks_y;
+    const int n = static_cast<int>(pb / per_image);
+    const int rem = static_cast<int>(pb - static_cast<long>(n) * per_image);
+    const int by = rem / p.blocks_x, bx = rem - by * p.blocks_x;
+    // here "out" is gx (extent out_h x out_w) and "in" is gy (extent in_h x in_w)
+    const int iy0 = by * BH, ix0 = bx * TW;
+    const int gy0 = iy0 / 2 + p.pad_h + DMIN, gx0 = ix0 / 2 + p.pad_w + DMIN;
+    const int c = c0 + 4 * lane_c;
+    const IO *src = static_cast<const IO *>(p.in) + static_cast<long>(n) * p.in_h * p.in_w * C + c;
+    const float *wl = lds + 4 * lane_c;
+
+    float acc[BH][TW * 4];
+#pragma unroll
+    for (int b = 0; b < BH; ++b)
+#pragma unroll
+        for (int o = 0; o < TW * 4; ++o) acc[b][o] = 0.f;
+
+    float cur[GCOLS * 4], nxt[GCOLS * 4];
+    nhwc_load_row<IO, GCOLS>(src, gy0, gx0, p.in_h, p.in_w, C, cur);
+#pragma unroll
+    for (int g = 0; g < GROWS; ++g) {
+        if (g + 1 < GROWS) nhwc_load_row<IO, GCOLS>(src, gy0 + g + 1, gx0, p.in_h, p.in_w, C, nxt);
+#pragma unroll
+        for (int b = 0; b < BH; ++b) {
+            const int ty = b + PE - 2 * (DMIN + g);
+            if (ty < 0 || ty >= K) continue;
+#pragma unroll
+            for (int o = 0; o < TW; ++o) {
+#pragma unroll
+                for (int j = 0; j < GCOLS; ++j) {
+                    const int tx = o + PE - 2 * (DMIN + j);
+                    if (tx < 0 || tx >= K) continue;
+                    const float4 w = *reinterpret_cast<const float4 *>(wl + (ty * K + tx) * nch);
+                    acc[b][4 * o + 0] = fmaf(cur[4 * j + 0], w.x, acc[b][4 * o + 0]);
+                    acc[b][4 * o + 1] = fmaf(cur[4 * j + 1], w.y, acc[b][4 * o + 1]);
+                    acc[b][4 * o + 2] = fmaf(cur[4 * j + 2], w.z, acc[b][4 * o + 2]);
+                    acc[b][4 * o + 3] = fmaf(cur[4 * j + 3], w.w, acc[b][4 * o + 3]);
+                }
+            }
+        }
+        pin_registers(acc);
+#pragma unroll
+        for (int j = 0; j < GCOLS * 4; ++j) cur[j] = nxt[j];
+    }
+
+    IO *dst = static_cast<IO *>(p.out) + static_cast<long>(n) * p.out_h * p.out_w * C + c;
+#pragma unroll
+    for (int b = 0; b < BH; ++b) {
+        const int iy = iy0 + b;
+        if (iy >= p.out_h) continue;
+#pragma unroll
+        for (int o = 0; o < TW; ++o) {
+            const int ix = ix0 + o;
+            if (ix < p.out_w)
+                store4<IO>(dst + (static_cast<long>(iy) * p.out_w + ix) * C, acc[b][4 * o], acc[b][4 * o + 1],
+                           acc[b][4 * o + 2], acc[b][4 * o + 3]);
+        }
+    }
+}
+
+// Grad-weight, pass 1.  in = x (in_h x in_w), in2 = gy (out_h x out_w).  Workgroup (chunk, channel group):
+// the lane walks the pixel blocks chunk, chunk + groups, ... with its K*K*CV sums in registers.
+template <typename IO, int K, int S, int CV, int BH, int TW>
+__global__ __launch_bounds__(kNhwcThreads) void nhwc_wgrad_kernel(const NhwcPlan p)
+{
+    extern __shared__ float4 lds_raw[];
+    float *lds = reinterpret_cast<float *>(lds_raw);
+    constexpr int KK = K * K;
+    constexpr int ROWS = (BH - 1) * S + K, COLS = (TW - 1) * S + K;
+    const int C = p.channel;
+    const int c0 = blockIdx.y * p.lanes_c * CV;
+    const int nch = min(p.lanes_c * CV, C - c0);
+    const int pb_local = fast_div(threadIdx.x, p.lanes_c_magic);
+    const int lane_c = threadIdx.x - pb_local * p.lanes_c;
+    const bool lane_ok = pb_local < p.blocks_per_wg && CV * lane_c < nch;
+    const int c = c0 + (lane_ok ? CV * lane_c : 0);
+    const int per_image = p.blocks_x * p.blocks_y;
+
+    float acc[KK][CV];
+#pragma unroll
+    for (int t = 0; t < KK; ++t)
+#pragma unroll
+        for (int v = 0; v < CV; ++v) acc[t][v] = 0.f;
+
+    for (long grp = blockIdx.x; grp * p.blocks_per_wg < p.blocks_total; grp += p.groups) {
+        const long pb = grp * p.blocks_per_wg + pb_local;
+        if (!lane_ok || pb >= p.blocks_total) continue;
+        const int n = static_cast<int>(pb / per_image);
+        const int rem = static_cast<int>(pb - static_cast<long>(n) * per_image);
+        const int by = rem / p.blocks_x, bx = rem - by * p.blocks_x;
+        const int oy0 = by * BH, ox0 = bx * TW;
+        const int iy0 = oy0 * S - p.pad_h, ix0 = ox0 * S - p.pad_w;
+        const IO *xs = static_cast<const IO *>(p.in) + static_cast<long>(n) * p.in_h * p.in_w * C + c;
+        const IO *gs = static_cast<const IO *>(p.in2) + static_cast<long>(n) * p.out_h * p.out_w * C + c;
+
+        float g[BH][TW][CV];
+#pragma unroll
+        for (int b = 0; b < BH; ++b) {
+            const int oy = oy0 + b;
+#pragma unroll
+            for (int o = 0; o < TW; ++o) {
+                const int ox = ox0 + o;
+                const bool ok = oy < p.out_h && ox < p.out_w;
+                float t[CV];
+                load_cv<IO, CV>(gs + (static_cast<long>(min(oy, p.out_h - 1)) * p.out_w + min(ox, p.out_w - 1)) * C, t);
+#pragma unroll
+                for (int v = 0; v < CV; ++v) g[b][o][v] = ok ? t[v] : 0.f;
+            }
+        }
+        float cur[COLS * CV], nxt[COLS * CV];
+        nhwc_load_row<IO, COLS, CV>(xs, iy0, ix0, p.in_h, p.in_w, C, cur);
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            if (r + 1 < ROWS) nhwc_load_row<IO, COLS, CV>(xs, iy0 + r + 1, ix0, p.in_h, p.in_w, C, nxt);
+#pragma unroll
+            for (int b = 0; b < BH; ++b) {
+                const int ty = r - b * S;
+                if (ty < 0 || ty >= K) continue;
+#pragma unroll
+                for (int tx = 0; tx < K; ++tx)
+#pragma unroll
+                    for (int o = 0; o < TW; ++o)
+#pragma unroll
+                        for (int v = 0; v < CV; ++v)
+                            acc[ty * K + tx][v] = fmaf(g[b][o][v], cur[CV * (o * S + tx) + v], acc[ty * K + tx][v]);
+            }
+            pin_registers(acc);
+#pragma unroll
+            for (int j = 0; j < COLS * CV; ++j) cur[j] = nxt[j];
+        }
+    }
+
+    // Lanes that share channels (same lane_c, different pixel block) are added front to back, one tap row at a time.
+    const int width = p.lanes_c * CV;  // floats per (pixel block, tap) line in LDS
+    float *out = p.partial + static_cast<long>(blockIdx.x) * KK * C;
+#pragma unroll
+    for (int ty = 0; ty < K; ++ty) {
+        if (ty) __syncthreads();
+        if (pb_local < p.blocks_per_wg) {
+#pragma unroll
+            for (int tx = 0; tx < K; ++tx)
+#pragma unroll
+                for (int v = 0; v < CV; ++v) lds[(pb_local * K + tx) * width + CV * lane_c + v] = lane_ok ? acc[ty * K + tx][v] : 0.f;
+        }
+        __syncthreads();
+        for (int e = threadIdx.x; e < K * nch; e += blockDim.x) {
+            const int tx = e / nch, cl = e - tx * nch;
+            float s = 0.f;
+            for (int q = 0; q < p.blocks_per_wg; ++q) s += lds[(q * K + tx) * width + cl];
+            out[static_cast<long>(ty * K + tx) * C + c0 + cl] = s;
+        }
+    }
+}
+
+// Grad-weight, pass 2: gw[c][t] = sum over chunks of partial[chunk][t][c].  16 lanes per output add contiguous
+// sixteenths of the chunks in fp64; the sixteen sums are then added in order: bit-identical from run to run.
+constexpr int kNhwcFinalParts = 16;
+template <typename T>
+__global__ __launch_bounds__(256) void nhwc_wgrad_final_kernel(const float *__restrict__ partial, T *__restrict__ gw,
+                                                               const int channel, const int taps, const int chunks)
+{
+    __shared__ double red[kNhwcFinalParts][16];
+    const int el = threadIdx.x & 15, part = threadIdx.x >> 4;
+    const int e = blockIdx.x * 16 + el;  // e = t * C + c: neighbouring lanes read neighbouring floats
+    const bool live = e < channel * taps;
+    const long stride = static_cast<long>(channel) * taps;
+    const int per = (chunks + kNhwcFinalParts - 1) / kNhwcFinalParts;
+    const int k0 = part * per, k1 = min(chunks, k0 + per);
+    const float *src = partial + (live ? e : 0);
+    double s = 0.0;
+    int k = k0;
+    for (; k + 8 <= k1; k += 8) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = src[(k + j) * stride];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s += static_cast<double>(v[j]);
+    }
+    for (; k < k1; ++k) s += static_cast<double>(src[k * stride]);
+    red[part][el] = s;
+    __syncthreads();
+    if (part == 0 && live) {
+        double total = 0.0;
+#pragma unroll
+        for (int q = 0; q < kNhwcFinalParts; ++q) total += red[q][el];
+        const int t = e / channel, c = e - t * channel;
+        gw[static_cast<long>(c) * taps + t] = Io<T>::out(static_cast<typename Io<T>::acc_t>(total));
+    }
+}
+
+// ---- one lane per element: any geometry, any element type ------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void nhwc_fwd_direct_kernel(const T *__restrict__ in, const T *__restrict__ taps,
+                                                              T *__restrict__ out, const NhwcGeometry g, const long total)
+{
+    using acc_t = typename Io<T>::acc_t;
+    const long e = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (e >= total) return;
+    const int c = static_cast<int>(e % g.channel);
+    long r = e / g.channel;
+    const int ox = static_cast<int>(r % g.out_w);
+    r /= g.out_w;
+    const int oy = static_cast<int>(r % g.out_h);
+    const long n = r / g.out_h;
+    acc_t s = 0;
+    for (int ty = 0; ty < g.kernel_h; ++ty) {
+        const int iy = oy * g.stride_h - g.pad_h + ty;
+        if (iy < 0 || iy >= g.in_h) continue;
+        for (int tx = 0; tx < g.kernel_w; ++tx) {
+            const int ix = ox * g.stride_w - g.pad_w + tx;
+            if (ix < 0 || ix >= g.in_w) continue;
+            s += static_cast<acc_t>(Io<T>::in(in[((n * g.in_h + iy) * g.in_w + ix) * g.channel + c])) *
+                 static_cast<acc_t>(Io<T>::in(taps[(static_cast<long>(c) * g.kernel_h + ty) * g.kernel_w + tx]));
+        }
+    }
+    out[e] = Io<T>::out(s);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void nhwc_gx_direct_kernel(const T *__restrict__ gy, const T *__restrict__ taps,
+                                                             T *__restrict__ gx, const NhwcGeometry g, const long total)
+{
+    using acc_t = typename Io<T>::acc_t;
+    const long e = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (e >= total) return;
+    const int c = static_cast<int>(e % g.channel);
+    long r = e / g.channel;
+    const int ix = static_cast<int>(r % g.in_w);
+    r /= g.in_w;
+    const int iy = static_cast<int>(r % g.in_h);
+    const long n = r / g.in_h;
+    acc_t s = 0;
+    for (int ty = 0; ty < g.kernel_h; ++ty) {
+        const int ny = iy + g.pad_h - ty;
+        if (ny < 0 || ny % g.stride_h != 0) continue;
+        const int oy = ny / g.stride_h;
+        if (oy >= g.out_h) continue;
+        for (int tx = 0; tx < g.kernel_w; ++tx) {
+            const int nx = ix + g.pad_w - tx;
+            if (nx < 0 || nx % g.stride_w != 0) continue;
+            const int ox = nx / g.stride_w;
+            if (ox >= g.out_w) continue;
+            s += static_cast<acc_t>(Io<T>::in(gy[((n * g.out_h + oy) * g.out_w + ox) * g.channel + c])) *
+                 static_cast<acc_t>(Io<T>::in(taps[(static_cast<long>(c) * g.kernel_h + ty) * g.kernel_w + tx]));
+        }
+    }
+    gx[e] = Io<T>::out(s);
+}
+
+// partial[chunk][t][c]: lane = (t, c) with c fastest, loops over the output pixels of its chunk.
+template <typename T>
+__global__ __launch_bounds__(256) void nhwc_gw_direct_kernel(const T *__restrict__ x, const T *__restrict__ gy,
+                                                             float *__restrict__ partial_f, const NhwcGeometry g,
+                                                             const long pixels, const int chunks)
+{
+    using acc_t = typename Io<T>::acc_t;
+    acc_t *partial = reinterpret_cast<acc_t *>(partial_f);
+    const int taps = g.kernel_h * g.kernel_w;
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= taps * g.channel) return;
+    const int t = e / g.channel, c = e - t * g.channel;
+    const int ty = t / g.kernel_w, tx = t - ty * g.kernel_w;
+    const int chunk = blockIdx.y;
+    const long per = (pixels + chunks - 1) / chunks;
+    const long p0 = chunk * per, p1 = min(pixels, p0 + per);
+    acc_t s = 0;
+    for (long q = p0; q < p1; ++q) {
+        const int ox = static_cast<int>(q % g.out_w);
+        const long r = q / g.out_w;
+        const int oy = static_cast<int>(r % g.out_h);
+        const long n = r / g.out_h;
+        const int iy = oy * g.stride_h - g.pad_h + ty, ix = ox * g.stride_w - g.pad_w + tx;
+        if (iy < 0 || iy >= g.in_h || ix < 0 || ix >= g.in_w) continue;
+        s += static_cast<acc_t>(Io<T>::in(gy[q * g.channel + c])) *
+             static_cast<acc_t>(Io<T>::in(x[((n * g.in_h + iy) * g.in_w + ix) * g.channel + c]));
+    }
+    partial[static_cast<long>(chunk) * taps * g.channel + e] = s;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void nhwc_gw_direct_final_kernel(const float *__restrict__ partial_f, T *__restrict__ gw,
+                                                                   const int channel, const int taps, const int chunks)
+{
+    using acc_t = typename Io<T>::acc_t;
+    const acc_t *partial = reinterpret_cast<const acc_t *>(partial_f);
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= channel * taps) return;
+    const int t = e / channel, c = e - t * channel;
+    double s = 0.0;
+    for (int k = 0; k < chunks; ++k) s += static_cast<double>(partial[static_cast<long>(k) * channel * taps + e]);
+    gw[static_cast<long>(c) * taps + t] = Io<T>::out(static_cast<acc_t>(s));
+}
+
+// ---- planning -------------------------------------------------------------------------------------------
+// Channel lanes per workgroup: the largest divisor of `lanes` (= C / CV) that is at most `cap`, so that no
+// workgroup straddles the end of the channel axis; at least 8 (half a 128-byte line of fp32 float4 lanes)
+// or the cap itself when the divisors are all tiny.
+int pick_lanes_c(int lanes, int cap)
+{
+    if (lanes <= cap) return lanes;
+    int best = 1;
+    for (int d = cap; d >= 1; --d)
+        if (lanes % d == 0) {
+            best = d;
+            break;
+        }
+    return best >= 8 ? best : cap;
+}
+
+template <int K, int CV>
+bool plan_nhwc(NhwcPlan &p, const NhwcGeometry &g, int bh, int tw, int blocks_h, int blocks_w)
+{
+    p.batch = g.batch;
+    p.channel = g.channel;
+    int cap = 64;
+    while (cap > 1 && static_cast<size_t>(cap) * CV * K * K * 4 > static_cast<size_t>(kNhwcTapLds)) --cap;
+    p.lanes_c = pick_lanes_c(g.channel / CV, cap);
+    p.lanes_c_magic = magic_u16(p.lanes_c);
+    p.blocks_per_wg = kNhwcThreads / p.lanes_c;
+    p.blocks_y = ceil_div(blocks_h, bh);
+    p.blocks_x = ceil_div(blocks_w, tw);
+    p.blocks_total = static_cast<long>(g.batch) * p.blocks_y * p.blocks_x;
+    if (p.blocks_total <= 0 || ceil_div(g.channel / CV, p.lanes_c) > 65535) return false;
+    if ((p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg > 0x7fffffffL) return false;
+    return true;
+}
+
+bool nhwc_fast_ok(const NhwcGeometry &g)
+{
+    if (env_int("DWCONV_FORCE_GENERIC", 0) || env_int("DWCONV_NO_NHWC_FAST", 0)) return false;
+    const int K = g.kernel_h;
+    if (g.kernel_w != K || (K != 3 && K != 5 && K != 7)) return false;
+    if (g.stride_h != g.stride_w || (g.stride_h != 1 && g.stride_h != 2)) return false;
+    if (g.channel % 4 != 0) return false;
+    if (g.pad_h < 0 || g.pad_w < 0 || g.pad_h >= K || g.pad_w >= K) return false;
+    if (g.in_h < 1 || g.in_w < 1 || g.out_h < 1 || g.out_w < 1) return false;
+    if (static_cast<long>(g.in_h) * g.in_w * g.channel >= (1l << 31)) return false;
+    return true;
+}
+
+template <typename IO, int K, int S, bool FLIP>
+int launch_nhwc_down(const IO *in, const IO *taps, IO *out, const NhwcGeometry &g, int in_h, int in_w, int out_h,
+                     int out_w, int pad_h, int pad_w, hipStream_t stream)
+{
+    constexpr int BH = 4, TW = K == 3 ? 4 : 2;
+    NhwcPlan p{};
+    if (!plan_nhwc<K, 4>(p, g, BH, TW, out_h, out_w)) return -1;
+    p.in = in;
+    p.taps = taps;
+    p.out = out;
+    p.in_h = in_h;
+    p.in_w = in_w;
+    p.out_h = out_h;
+    p.out_w = out_w;
+    p.pad_h = pad_h;
+    p.pad_w = pad_w;
+    const dim3 grid(static_cast<unsigned>((p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg),
+                    ceil_div(g.channel / 4, p.lanes_c));
+    const size_t shmem = static_cast<size_t>(p.lanes_c) * 4 * K * K * 4;
+    hipLaunchKernelGGL((nhwc_down_kernel<IO, K, S, FLIP, BH, TW>), grid, dim3(kNhwcThreads), shmem, stream, p);
+    note_variant("nhwc_down%s<k%d,s%d,%s,%dx%d> lanes_c%d", sizeof(IO) == 2 ? "16" : "", K, S, FLIP ? "rot" : "fwd", BH, TW,
+                 p.lanes_c);
+    return check_launch("nhwc_down_kernel");
+}
+
+template <typename IO, int K, int PE>
+int launch_nhwc_up2(const IO *gy, const IO *taps, IO *gx, const NhwcGeometry &g, hipStream_t stream)
+{
+    constexpr int BH = 4, TW = K == 3 ? 4 : 2;
+    NhwcPlan p{};
+    if (!plan_nhwc<K, 4>(p, g, BH, TW, g.in_h, g.in_w)) return -1;
+    p.in = gy;
+    p.taps = taps;
+    p.out = gx;
+    p.in_h = g.out_h;
+    p.in_w = g.out_w;
+    p.out_h = g.in_h;
+    p.out_w = g.in_w;
+    p.pad_h = g.pad_h / 2;
+    p.pad_w = g.pad_w / 2;
+    const dim3 grid(static_cast<unsigned>((p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg),
+                    ceil_div(g.channel / 4, p.lanes_c));
+    const size_t shmem = static_cast<size_t>(p.lanes_c) * 4 * K * K * 4;
+    hipLaunchKernelGGL((nhwc_up2_kernel<IO, K, PE, BH, TW>), grid, dim3(kNhwcThreads), shmem, stream, p);
+    note_variant("nhwc_up2%s<k%d,e%d,%dx%d> lanes_c%d", sizeof(IO) == 2 ? "16" : "", K, PE, BH, TW, p.lanes_c);
+    return check_launch("nhwc_up2_kernel");
+}
+
+template <int K>
+struct WgradShape {
+    static constexpr int CV = K == 7 ? 2 : 4;
+    static constexpr int BH = K == 3 ? 4 : 2;
+    static constexpr int TW = 4;
+};
+
+// mode 0: workspace bytes; mode 1: launch.  -1 when the fast kernel does not cover g.
+template <typename IO, int K, int S>
+long nhwc_wgrad_case(int mode, const IO *x, const IO *gy, IO *gw, void *ws, size_t ws_bytes, const NhwcGeometry &g,
+                     hipStream_t stream)
+{
+    constexpr int CV = WgradShape<K>::CV, BH = WgradShape<K>::BH, TW = WgradShape<K>::TW;
+    NhwcPlan p{};
+    if (!plan_nhwc<1, CV>(p, g, BH, TW, g.out_h, g.out_w)) return -1;
+    const int cgroups = ceil_div(g.channel / CV, p.lanes_c);
+    const long wg_iters = (p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg;
+    long groups = env_int("DWCONV_NHWC_WGRAD_WGS", 1024) / cgroups;
+    groups = std::max(1l, std::min(groups, wg_iters));
+    p.groups = static_cast<int>(groups);
+    const size_t need = static_cast<size_t>(groups) * K * K * g.channel * sizeof(float);
+    if (mode == 0) return static_cast<long>(need);
+    if (ws == nullptr || ws_bytes < need)
+        return fail(DWCONV_ERR_WORKSPACE, "grad-weight needs a workspace of %zu bytes, got %zu", need, ws_bytes);
+    p.in = x;
+    p.in2 = gy;
+    p.partial = static_cast<float *>(ws);
+    p.in_h = g.in_h;
+    p.in_w = g.in_w;
+    p.out_h = g.out_h;
+    p.out_w = g.out_w;
+    p.pad_h = g.pad_h;
+    p.pad_w = g.pad_w;
+    const size_t shmem = static_cast<size_t>(p.blocks_per_wg) * K * p.lanes_c * CV * 4;
+    hipLaunchKernelGGL((nhwc_wgrad_kernel<IO, K, S, CV, BH, TW>), dim3(p.groups, cgroups), dim3(kNhwcThreads), shmem, stream, p);
+    int rc = check_launch("nhwc_wgrad_kernel");
+    if (rc != DWCONV_OK) return rc;
+    note_variant("nhwc_wgrad%s<k%d,s%d,cv%d,%dx%d> lanes_c%d chunks%d", sizeof(IO) == 2 ? "16" : "", K, S, CV, BH, TW,
+                 p.lanes_c, p.groups);
+    hipLaunchKernelGGL(nhwc_wgrad_final_kernel<IO>, dim3(ceil_div(g.channel * K * K, 16)), dim3(256), 0, stream,
+                       p.partial, gw, g.channel, K * K, p.groups);
+    return check_launch("nhwc_wgrad_final_kernel");
+}
+
+template <typename IO>
+long nhwc_wgrad_fast(int mode, const IO *x, const IO *gy, IO *gw, void *ws, size_t ws_bytes, const NhwcGeometry &g,
+                     hipStream_t stream)
+{
+    if (!nhwc_fast_ok(g)) return -1;
+    const int K = g.kernel_h, S = g.stride_h;
+#define DWCONV_NHWC_WGRAD(KV, SV) \
+    if (K == KV && S == SV) return nhwc_wgrad_case<IO, KV, SV>(mode, x, gy, gw, ws, ws_bytes, g, stream);
+    DWCONV_NHWC_WGRAD(3, 1)
+    DWCONV_NHWC_WGRAD(3, 2)
+    DWCONV_NHWC_WGRAD(5, 1)
+    DWCONV_NHWC_WGRAD(5, 2)
+    DWCONV_NHWC_WGRAD(7, 1)
+    DWCONV_NHWC_WGRAD(7, 2)
+#undef DWCONV_NHWC_WGRAD
+    return -1;
+}
+
+template <typename T>
+int direct_chunks(const NhwcGeometry &g)
+{
+    const long pixels = static_cast<long>(g.batch) * g.out_h * g.out_w;
+    return static_cast<int>(std::max(1l, std::min(256l, pixels / 64)));
+}
+
+template <typename T>
+size_t nhwc_wgrad_direct_bytes(const NhwcGeometry &g)
+{
+    return static_cast<size_t>(direct_chunks<T>(g)) * g.kernel_h * g.kernel_w * g.channel * sizeof(typename Io<T>::acc_t);
+}
+
+}  // namespace
+
+template <typename T>
+int nhwc_forward(const T *in, const T *taps, T *out, const NhwcGeometry &g, hipStream_t stream)
+{
+    const long total = static_cast<long>(g.batch) * g.out_h * g.out_w * g.channel;
+    if (total == 0) {
+        note_variant("empty");
+        return DWCONV_OK;
+    }
+    if constexpr (!std::is_same<T, double>::value) {
+        if (nhwc_fast_ok(g) && aligned4(in) && aligned4(out)) {
+            const int K = g.kernel_h, S = g.stride_h;
+            int rc = -1;
+#define DWCONV_NHWC_DOWN(KV, SV)                                                                                       \
+    if (K == KV && S == SV)                                                                                            \
+        rc = launch_nhwc_down<T, KV, SV, false>(in, taps, out, g, g.in_h, g.in_w, g.out_h, g.out_w, g.pad_h, g.pad_w, stream);
+            DWCONV_NHWC_DOWN(3, 1)
+            DWCONV_NHWC_DOWN(3, 2)
+            DWCONV_NHWC_DOWN(5, 1)
+            DWCONV_NHWC_DOWN(5, 2)
+            DWCONV_NHWC_DOWN(7, 1)
+            DWCONV_NHWC_DOWN(7, 2)
+#undef DWCONV_NHWC_DOWN
+            if (rc >= 0) return rc;
+        }
+    }
+    if ((total + 255) / 256 > 0x7fffffffL) return fail(DWCONV_ERR_UNSUPPORTED, "tensor too large");
+    hipLaunchKernelGGL(nhwc_fwd_direct_kernel<T>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream, in,
+                       taps, out, g, total);
+    note_variant("nhwc_fwd_direct");
+    return check_launch("nhwc_fwd_direct_kernel");
+}
+
+template <typename T>
+int nhwc_grad_input(const T *gy, const T *taps, T *gx, const NhwcGeometry &g, hipStream_t stream)
+{
+    const long total = static_cast<long>(g.batch) * g.in_h * g.in_w * g.channel;
+    if (total == 0) {
+        note_variant("empty");
+        return DWCONV_OK;
+    }
+    if (static_cast<long>(g.batch) * g.out_h * g.out_w == 0) {
+        note_variant("zero");
+        return launch_fill_zero(gx, static_cast<size_t>(total) * sizeof(T), stream);
+    }
+    if constexpr (!std::is_same<T, double>::value) {
+        if (nhwc_fast_ok(g) && aligned4(gy) && aligned4(gx)) {
+            const int K = g.kernel_h, S = g.stride_h;
+            int rc = -1;
+            if (S == 1) {
+                // the transposed problem is a stride-1 correlation with the rotated taps and pad K - 1 - pad
+#define DWCONV_NHWC_ROT(KV)                                                                                            \
+    if (K == KV)                                                                                                       \
+        rc = launch_nhwc_down<T, KV, 1, true>(gy, taps, gx, g, g.out_h, g.out_w, g.in_h, g.in_w, KV - 1 - g.pad_h,     \
+                                              KV - 1 - g.pad_w, stream);
+                DWCONV_NHWC_ROT(3)
+                DWCONV_NHWC_ROT(5)
+                DWCONV_NHWC_ROT(7)
+#undef DWCONV_NHWC_ROT
+            } else if (((g.pad_h ^ g.pad_w) & 1) == 0) {  // one parity class serves both axes
+                const int pe = g.pad_h & 1;
+#define DWCONV_NHWC_UP2(KV)                                                                                            \
+    if (K == KV) rc = pe ? launch_nhwc_up2<T, KV, 1>(gy, taps, gx, g, stream) : launch_nhwc_up2<T, KV, 0>(gy, taps, gx, g, stream);
+                DWCONV_NHWC_UP2(3)
+                DWCONV_NHWC_UP2(5)
+                DWCONV_NHWC_UP2(7)
+#undef DWCONV_NHWC_UP2
+            }
+            if (rc >= 0) return rc;
+        }
+    }
+    if ((total + 255) / 256 > 0x7fffffffL) return fail(DWCONV_ERR_UNSUPPORTED, "tensor too large");
+    hipLaunchKernelGGL(nhwc_gx_direct_kernel<T>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream, gy,
+                       taps, gx, g, total);
+    note_variant("nhwc_gx_direct");
+    return check_launch("nhwc_gx_direct_kernel");
+}
+
+template <typename T>
+size_t nhwc_grad_weight_workspace(const NhwcGeometry &g)
+{
+    size_t need = nhwc_wgrad_direct_bytes<T>(g);
+    if constexpr (!std::is_same<T, double>::value) {
+        const long fast = nhwc_wgrad_fast<T>(0, nullptr, nullptr, nullptr, nullptr, 0, g, nullptr);
+        if (fast > 0 && static_cast<size_t>(fast) > need) need = static_cast<size_t>(fast);
+    }
+    return need;
+}
+
+template <typename T>
+int nhwc_grad_weight(const T *x, const T *gy, T *gw, void *ws, size_t ws_bytes, const NhwcGeometry &g, hipStream_t stream)
+{
+    const int taps = g.kernel_h * g.kernel_w;
+    if (static_cast<long>(g.channel) * taps == 0) {
+        note_variant("empty");
+        return DWCONV_OK;
+    }
+    const long pixels = static_cast<long>(g.batch) * g.out_h * g.out_w;
+    if (pixels == 0 || g.in_h == 0 || g.in_w == 0) {
+        note_variant("zero");
+        return launch_fill_zero(gw, static_cast<size_t>(g.channel) * taps * sizeof(T), stream);
+    }
+    if constexpr (!std::is_same<T, double>::value) {
+        if (aligned4(x) && aligned4(gy)) {
+            const long rc = nhwc_wgrad_fast<T>(1, x, gy, gw, ws, ws_bytes, g, stream);
+            if (rc >= 0) return static_cast<int>(rc);
+        }
+    }
+    const size_t need = nhwc_wgrad_direct_bytes<T>(g);
+    if (ws == nullptr || ws_bytes < need)
+        return fail(DWCONV_ERR_WORKSPACE, "grad-weight needs a workspace of %zu bytes, got %zu", need, ws_bytes);
+    const int chunks = direct_chunks<T>(g);
+    hipLaunchKernelGGL(nhwc_gw_direct_kernel<T>, dim3(ceil_div(taps * g.channel, 256), chunks), dim3(256), 0, stream, x, gy,
+                       static_cast<float *>(ws), g, pixels, chunks);
+    int rc = check_launch("nhwc_gw_direct_kernel");
+    if (rc != DWCONV_OK) return rc;
+    hipLaunchKernelGGL(nhwc_gw_direct_final_kernel<T>, dim3(ceil_div(taps * g.channel, 256)), dim3(256), 0, stream,
+                       static_cast<const float *>(ws), gw, g.channel, taps, chunks);
+    note_variant("nhwc_gw_direct chunks%d", chunks);
+    return check_launch("nhwc_gw_direct_final_kernel");
+}
+
+#define DWCONV_INSTANTIATE(T)                                                                                          \
+    template int nhwc_forward<T>(const T *, const T *, T *, const NhwcGeometry &, hipStream_t);                        \
+    template int nhwc_grad_input<T>(const T *, const T *, T *, const NhwcGeometry &, hipStream_t);                     \
+    template size_t nhwc_grad_weight_workspace<T>(const NhwcGeometry &);                                               \
+    template int nhwc_grad_weight<T>(const T *, const T *, T *, void *, size_t, const NhwcGeometry &, hipStream_t);
+DWCONV_INSTANTIATE(float)
+DWCONV_INSTANTIATE(double)
+DWCONV_INSTANTIATE(half_t)
+DWCONV_INSTANTIATE(bf16_t)
+#undef DWCONV_INSTANTIATE
+
+}  // namespace dwconv

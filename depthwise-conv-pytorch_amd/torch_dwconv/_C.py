@@ -51,6 +51,16 @@ for _name in ("dwconv2d_backward_f32", "dwconv2d_backward_f16", "dwconv2d_backwa
     getattr(_lib, _name).restype = _i
     getattr(_lib, _name).argtypes = [_p, _p, _p, _p, _p, _p, _z] + [_i] * 12 + [_p]
 
+for _name in ("dwconv2d_nhwc_f32", "dwconv2d_nhwc_f64", "dwconv2d_nhwc_f16", "dwconv2d_nhwc_bf16"):
+    getattr(_lib, _name).restype = _i
+    getattr(_lib, _name).argtypes = [_p, _p, _p] + [_i] * 10 + [_p]
+_lib.dwconv2d_backward_nhwc_workspace_bytes.restype = _z
+_lib.dwconv2d_backward_nhwc_workspace_bytes.argtypes = [_i] * 11
+for _name in ("dwconv2d_backward_nhwc_f32", "dwconv2d_backward_nhwc_f64", "dwconv2d_backward_nhwc_f16",
+              "dwconv2d_backward_nhwc_bf16"):
+    getattr(_lib, _name).restype = _i
+    getattr(_lib, _name).argtypes = [_p, _p, _p, _p, _p, _p, _z] + [_i] * 12 + [_p]
+
 _SUFFIX = {torch.float32: "f32", torch.float64: "f64", torch.float16: "f16", torch.bfloat16: "bf16"}
 
 
@@ -207,6 +217,66 @@ def dwconv2d_backward(input, out_grad, kernel, stride_h, stride_w, pad_h, pad_w)
         rc = getattr(_lib, "dwconv2d_backward_" + suffix)(
             x.data_ptr(), gy.data_ptr(), k.data_ptr(), gx.data_ptr(), gw.data_ptr(), ws.data_ptr(), ws_bytes,
             *geom, stride_h, stride_w, pad_h, pad_w, _stream(x),
+        )
+    if rc != 0:
+        _raise(rc)
+    return gx, gw
+
+
+# ---- channels-last tensors -----------------------------------------------------------------------------
+def is_channels_last(t):
+    """True when ``t`` (logical shape N,C,H,W) is laid out N,H,W,C in memory and not also N,C,H,W."""
+    return t.dim() == 4 and t.is_contiguous(memory_format=torch.channels_last) and not t.is_contiguous()
+
+
+def dwconv2d_nhwc(input, kernel, stride_h, stride_w, pad_h, pad_w):
+    """Forward convolution of a channels-last ``input`` (logical shape N,C,H,W); the result is channels-last too.
+
+    The reference has no such path: it makes ``input`` NCHW-contiguous first (torch_dwconv/dwconv_kernel.cu:855).
+    """
+    _check_cuda(input, "input")
+    _check_cuda(kernel, "kernel")
+    _check_shapes(input, kernel)
+    sfx = _suffix(input, kernel)
+    x, k = input.contiguous(memory_format=torch.channels_last), kernel.contiguous()
+    n, c, h, w = x.shape
+    kh, kw = k.shape[2], k.shape[3]
+    oh = max(_lib.dwconv_out_size(h, 1, stride_h, pad_h, pad_h, kh), 0)
+    ow = max(_lib.dwconv_out_size(w, 1, stride_w, pad_w, pad_w, kw), 0)
+    out = torch.empty((n, c, oh, ow), dtype=x.dtype, device=x.device, memory_format=torch.channels_last)
+    with torch.cuda.device(x.device):
+        rc = getattr(_lib, "dwconv2d_nhwc_" + sfx)(
+            x.data_ptr(), k.data_ptr(), out.data_ptr(), n, c, h, w, kh, kw, stride_h, stride_w, pad_h, pad_w, _stream(x),
+        )
+    if rc != 0:
+        _raise(rc)
+    return out
+
+
+def dwconv2d_backward_nhwc(input, out_grad, kernel, stride_h, stride_w, pad_h, pad_w):
+    """Both gradients for channels-last ``input`` / ``out_grad``; ``grad_input`` comes back channels-last."""
+    _check_cuda(input, "input")
+    _check_cuda(out_grad, "out_grad")
+    _check_cuda(kernel, "kernel")
+    _check_shapes(input, kernel)
+    if out_grad.dim() != 4 or out_grad.shape[:2] != input.shape[:2]:
+        raise RuntimeError(f"out_grad of shape {tuple(out_grad.shape)} does not belong to input {tuple(input.shape)}")
+    sfx = _suffix(input, out_grad, kernel)
+    x = input.contiguous(memory_format=torch.channels_last)
+    gy = out_grad.contiguous(memory_format=torch.channels_last)
+    k = kernel.contiguous()
+    n, c, h, w = x.shape
+    oh, ow = gy.shape[2], gy.shape[3]
+    kh, kw = k.shape[2], k.shape[3]
+    gx = torch.empty_like(x, memory_format=torch.channels_last)
+    gw = torch.empty_like(k)
+    ws_bytes = _lib.dwconv2d_backward_nhwc_workspace_bytes(n, c, h, w, kh, kw, stride_h, stride_w, pad_h, pad_w,
+                                                           x.element_size())
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = getattr(_lib, "dwconv2d_backward_nhwc_" + sfx)(
+            x.data_ptr(), gy.data_ptr(), k.data_ptr(), gx.data_ptr(), gw.data_ptr(), ws.data_ptr(), ws_bytes,
+            n, c, h, w, oh, ow, kh, kw, stride_h, stride_w, pad_h, pad_w, _stream(x),
         )
     if rc != 0:
         _raise(rc)

@@ -3,7 +3,9 @@ errors as the reference's torch_dwconv/dwconv.py, on top of the HIP library.
 
 ``depthwise_conv2d(input, weight, bias=None, stride=1, padding=0, dilation=1,
 groups=None)`` computes what ``F.conv2d(input, weight, stride=stride,
-padding=padding, groups=C)`` computes, for GPU tensors in float32 or float64.
+padding=padding, groups=C)`` computes, for GPU tensors in float32, float64,
+float16 or bfloat16, NCHW-contiguous or channels-last (the output then is
+channels-last as well).
 
 One deliberate difference: the reference hands planes of at most 32x32 that its
 small kernel cannot take (stride 2, or a filter too large for the plane) to
@@ -75,6 +77,12 @@ class DepthwiseConv2dFunction(Function):
     def forward(ctx, input, kernel, stride, pad, small):
         ctx.save_for_backward(input, kernel)
         ctx.stride, ctx.pad, ctx.use_small = stride, pad, small
+        # Channels-last activations stay channels-last (the reference converts them to NCHW,
+        # torch_dwconv/dwconv_kernel.cu:855): same values, no layout-conversion pass either side of the op.
+        ctx.channels_last = _C.is_channels_last(input)
+        if ctx.channels_last:
+            ctx.g_pad = None
+            return _C.dwconv2d_nhwc(input, kernel, stride[0], stride[1], pad[0], pad[1])
         if small:
             out = _C.dwconv2d_small(input, kernel, 1, 1, stride[0], stride[1], pad[0], pad[1], True)
         else:
@@ -97,6 +105,11 @@ class DepthwiseConv2dFunction(Function):
         input, kernel = ctx.saved_tensors
         stride, pad, g_pad = ctx.stride, ctx.pad, ctx.g_pad
         # The reference always computes both gradients (:48-70).
+        if ctx.channels_last:
+            grad_input, grad_kernel = _C.dwconv2d_backward_nhwc(
+                input, grad_output, kernel, stride[0], stride[1], pad[0], pad[1]
+            )
+            return grad_input, grad_kernel, None, None, None, None
         if input.dtype != torch.float64:
             # one library call for the pair of calls below; same values, out_grad read once where fused
             grad_input, grad_kernel = _C.dwconv2d_backward(

@@ -191,6 +191,56 @@ int dwconv2d_backward_bf16(const unsigned short *input, const unsigned short *ou
                            int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
                            void *stream);
 
+/* ---- channels-last (NHWC) tensors -------------------------------------------------------------
+ * No counterpart in the reference, which makes every tensor NCHW-contiguous before its kernels run
+ * (torch_dwconv/dwconv_kernel.cu:741, :855, :1023): these entry points serve callers whose activations are
+ * channels-last, so that no layout conversion is needed either side of the op.  input is (N,H,W,C), out and
+ * out_grad are (N,OH,OW,C) with OH = dwconv_out_size(H, 1, stride_h, pad_h, pad_h, kernel_h); kernel and
+ * kernel_grad are (C,1,KH,KW) as everywhere else.  Same arithmetic as dwconv2d_* with up = 1,
+ * down = stride, pad0 = pad1 = pad (forward) and as the reference's backward pair (dwconv.py:56-68). */
+int dwconv2d_nhwc_f32(const float *input, const float *kernel, float *out, int batch, int channel,
+                      int in_h, int in_w, int kernel_h, int kernel_w, int stride_h, int stride_w,
+                      int pad_h, int pad_w, void *stream);
+int dwconv2d_nhwc_f64(const double *input, const double *kernel, double *out, int batch, int channel,
+                      int in_h, int in_w, int kernel_h, int kernel_w, int stride_h, int stride_w,
+                      int pad_h, int pad_w, void *stream);
+int dwconv2d_nhwc_f16(const unsigned short *input, const unsigned short *kernel, unsigned short *out,
+                      int batch, int channel, int in_h, int in_w, int kernel_h, int kernel_w,
+                      int stride_h, int stride_w, int pad_h, int pad_w, void *stream);
+int dwconv2d_nhwc_bf16(const unsigned short *input, const unsigned short *kernel, unsigned short *out,
+                       int batch, int channel, int in_h, int in_w, int kernel_h, int kernel_w,
+                       int stride_h, int stride_w, int pad_h, int pad_w, void *stream);
+
+/* Workspace (bytes) for dwconv2d_backward_nhwc_*; elem_size 2, 4 or 8. */
+size_t dwconv2d_backward_nhwc_workspace_bytes(int batch, int channel, int in_h, int in_w,
+                                              int kernel_h, int kernel_w, int stride_h, int stride_w,
+                                              int pad_h, int pad_w, int elem_size);
+
+/* Both gradients (either of in_grad, kernel_grad may be NULL to skip it).  kernel_grad is overwritten
+ * and bit-identical from run to run. */
+int dwconv2d_backward_nhwc_f32(const float *input, const float *out_grad, const float *kernel,
+                               float *in_grad, float *kernel_grad, void *workspace,
+                               size_t workspace_bytes, int batch, int channel, int in_h, int in_w,
+                               int out_h, int out_w, int kernel_h, int kernel_w, int stride_h,
+                               int stride_w, int pad_h, int pad_w, void *stream);
+int dwconv2d_backward_nhwc_f64(const double *input, const double *out_grad, const double *kernel,
+                               double *in_grad, double *kernel_grad, void *workspace,
+                               size_t workspace_bytes, int batch, int channel, int in_h, int in_w,
+                               int out_h, int out_w, int kernel_h, int kernel_w, int stride_h,
+                               int stride_w, int pad_h, int pad_w, void *stream);
+int dwconv2d_backward_nhwc_f16(const unsigned short *input, const unsigned short *out_grad,
+                               const unsigned short *kernel, unsigned short *in_grad,
+                               unsigned short *kernel_grad, void *workspace, size_t workspace_bytes,
+                               int batch, int channel, int in_h, int in_w, int out_h, int out_w,
+                               int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h,
+                               int pad_w, void *stream);
+int dwconv2d_backward_nhwc_bf16(const unsigned short *input, const unsigned short *out_grad,
+                                const unsigned short *kernel, unsigned short *in_grad,
+                                unsigned short *kernel_grad, void *workspace, size_t workspace_bytes,
+                                int batch, int channel, int in_h, int in_w, int out_h, int out_w,
+                                int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h,
+                                int pad_w, void *stream);
+
 /* Tuning/diagnostic hook: name of the kernel variant the last successful call
  * on this thread launched (e.g. "tile_f32<k3,s1,v4>"), for benchmarks and tests. */
 const char *dwconv_last_variant(void);

@@ -436,3 +436,145 @@ def test_runs_on_the_current_stream(dw, gpu):
         out = dw.depthwise_conv2d(x, w, padding=1)
     side.synchronize()
     assert torch.equal(out, ref)
+
+
+# ---- channels-last tensors ---------------------------------------------------------------------------------
+NHWC_SHAPES = [
+    # (N, C, H, W, k, stride, pad): C % 4 == 0 and k in {3,5,7} take the vector kernels, the rest the per-element ones
+    (2, 8, 14, 14, 3, 1, 1), (2, 32, 20, 24, 3, 1, 1), (1, 96, 17, 19, 3, 2, 1), (2, 144, 9, 11, 5, 2, 2),
+    (2, 240, 7, 7, 5, 1, 2), (1, 12, 28, 28, 7, 1, 3), (2, 16, 15, 13, 7, 2, 3), (2, 8, 12, 12, 3, 1, 0),
+    (2, 8, 12, 12, 5, 2, 0), (1, 4, 10, 9, 3, 2, 2), (2, 20, 6, 5, 5, 1, 4), (1, 260, 5, 5, 3, 1, 1),
+    (3, 1152, 7, 7, 3, 1, 1), (2, 8, 1, 9, 3, 1, 1), (2, 8, 9, 1, 3, 2, 1), (2, 4, 33, 35, 5, 2, 1),
+    (2, 3, 9, 11, 3, 1, 1), (1, 6, 8, 8, 4, 2, 1), (2, 5, 7, 7, 1, 1, 0), (1, 2, 12, 10, 9, 1, 4),
+]
+
+
+def _channels_last(t, gpu):
+    return t.to(gpu).contiguous(memory_format=torch.channels_last)
+
+
+@pytest.mark.parametrize("shape", NHWC_SHAPES, ids=shape_id)
+def test_channels_last_matches_oracle(dw, gpu, shape):
+    """Channels-last input: same values as the NCHW oracle, channels-last results, bit-identical grad-weight."""
+    from torch_dwconv import _C
+
+    n, c, h, w, k, s, p = shape
+    x, wt, gy = make_inputs(shape, seed=23)
+    xg = _channels_last(x, gpu).requires_grad_(True)
+    wg = wt.to(gpu).requires_grad_(True)
+    y = dw.depthwise_conv2d(xg, wg, stride=s, padding=p)
+    v_fwd = _C.last_variant()
+    gx, gw = torch.autograd.grad(y, (xg, wg), _channels_last(gy, gpu))
+    _announce(shape_id(shape), v_fwd, "|", _C.last_variant())
+    assert v_fwd.startswith("nhwc_"), v_fwd
+    fast = c % 4 == 0 and k in (3, 5, 7)
+    assert v_fwd.startswith("nhwc_down") == fast, v_fwd
+    if c > 1 and y.shape[2] * y.shape[3] > 1:
+        assert y.is_contiguous(memory_format=torch.channels_last)
+    if c > 1 and h * w > 1:
+        assert gx.is_contiguous(memory_format=torch.channels_last)
+    y_ref = oracle.forward(_np(x), _np(wt), s, p)
+    gx_ref = oracle.grad_input(_np(gy), _np(wt), (h, w), s, p)
+    gw_ref = oracle.grad_weight(_np(x), _np(gy), wt.shape, s, p)
+    np.testing.assert_allclose(_np(y.detach()).astype(np.float64), y_ref, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(_np(gx).astype(np.float64), gx_ref, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(_np(gw).astype(np.float64), gw_ref, rtol=1e-4, atol=1e-4 * np.abs(gw_ref).max())
+    _, gw2 = torch.autograd.grad(dw.depthwise_conv2d(xg, wg, stride=s, padding=p), (xg, wg), _channels_last(gy, gpu))
+    assert torch.equal(gw, gw2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float16, torch.bfloat16], ids=["f64", "f16", "bf16"])
+def test_channels_last_other_dtypes(dw, gpu, dtype):
+    step = {torch.float64: 0.0, torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[dtype]
+    for shape in [(2, 16, 14, 14, 3, 1, 1), (2, 8, 13, 15, 5, 2, 2), (1, 12, 9, 9, 7, 1, 3), (2, 6, 9, 8, 3, 2, 1)]:
+        n, c, h, w, k, s, p = shape
+        x, wt, gy = (t.to(dtype) for t in make_inputs(shape, seed=29))
+        xg = _channels_last(x, gpu).requires_grad_(True)
+        wg = wt.to(gpu).requires_grad_(True)
+        y = dw.depthwise_conv2d(xg, wg, stride=s, padding=p)
+        gx, gw = torch.autograd.grad(y, (xg, wg), _channels_last(gy, gpu))
+        assert y.dtype == dtype and gx.dtype == dtype and gw.dtype == dtype
+        xr, wr, gr = (_np(t.double()) for t in (x, wt, gy))
+        y_ref = oracle.forward(xr, wr, s, p)
+        gx_ref = oracle.grad_input(gr, wr, (h, w), s, p)
+        gw_ref = oracle.grad_weight(xr, gr, wt.shape, s, p)
+        tol = dict(rtol=max(step, 1e-12), atol=(1e-5 + step * 1e-2) if step else 1e-12)
+        np.testing.assert_allclose(_np(y.detach().double()), y_ref, **tol)
+        np.testing.assert_allclose(_np(gx.double()), gx_ref, **tol)
+        gtol = (step + 1e-4) if step else 1e-12
+        np.testing.assert_allclose(_np(gw.double()), gw_ref, rtol=gtol, atol=gtol * float(np.abs(gw_ref).max()))
+
+
+def test_channels_last_entry_points(dw, gpu):
+    """The C entry points directly: rectangular filters and strides, one gradient at a time, status codes."""
+    from torch_dwconv import _C
+
+    g = torch.Generator("cpu").manual_seed(31)
+    x = torch.randn(2, 8, 11, 13, generator=g)
+    wt = torch.randn(8, 1, 3, 5, generator=g)
+    xg, wg = _channels_last(x, gpu), wt.to(gpu)
+    ref = torch.nn.functional.conv2d(x.double(), wt.double(), stride=(2, 1), padding=(1, 2), groups=8)
+    out = torch.empty(ref.shape, device=gpu).contiguous(memory_format=torch.channels_last)
+    lib = _C._lib
+    rc = lib.dwconv2d_nhwc_f32(xg.data_ptr(), wg.data_ptr(), out.data_ptr(), 2, 8, 11, 13, 3, 5, 2, 1, 1, 2, None)
+    assert rc == 0, lib.dwconv_last_error()
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(_np(out).astype(np.float64), ref.numpy(), rtol=1e-5, atol=1e-5)
+    # grad-weight alone (in_grad = NULL), then grad-input alone
+    gy = torch.randn(ref.shape, generator=g)
+    gyg = _channels_last(gy, gpu)
+    xr = x.double().requires_grad_(True)
+    wr = wt.double().requires_grad_(True)
+    gx_ref, gw_ref = torch.autograd.grad(torch.nn.functional.conv2d(xr, wr, stride=(2, 1), padding=(1, 2), groups=8),
+                                         (xr, wr), gy.double())
+    ws_bytes = lib.dwconv2d_backward_nhwc_workspace_bytes(2, 8, 11, 13, 3, 5, 2, 1, 1, 2, 4)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=gpu)
+    gw = torch.empty_like(wg)
+    gx = torch.empty_like(xg)
+    geom = (2, 8, 11, 13, ref.shape[2], ref.shape[3], 3, 5, 2, 1, 1, 2)
+    assert lib.dwconv2d_backward_nhwc_f32(xg.data_ptr(), gyg.data_ptr(), None, None, gw.data_ptr(), ws.data_ptr(),
+                                          ws_bytes, *geom, None) == 0
+    assert lib.dwconv2d_backward_nhwc_f32(None, gyg.data_ptr(), wg.data_ptr(), gx.data_ptr(), None, None, 0,
+                                          *geom, None) == 0
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(_np(gw).astype(np.float64), gw_ref.numpy(), rtol=1e-4, atol=1e-4 * float(gw_ref.abs().max()))
+    np.testing.assert_allclose(_np(gx).astype(np.float64), gx_ref.numpy(), rtol=1e-5, atol=1e-5)
+    # errors come back as status codes
+    assert lib.dwconv2d_backward_nhwc_f32(xg.data_ptr(), gyg.data_ptr(), wg.data_ptr(), None, None, None, 0, *geom, None) == 1
+    assert lib.dwconv2d_backward_nhwc_f32(xg.data_ptr(), gyg.data_ptr(), wg.data_ptr(), gx.data_ptr(), gw.data_ptr(),
+                                          ws.data_ptr(), 4, *geom, None) == 3
+    bad = list(geom)
+    bad[4] += 1
+    assert lib.dwconv2d_backward_nhwc_f32(xg.data_ptr(), gyg.data_ptr(), wg.data_ptr(), gx.data_ptr(), gw.data_ptr(),
+                                          ws.data_ptr(), ws_bytes, *bad, None) == 1
+    # empty batch
+    e = dw.depthwise_conv2d(torch.empty(0, 8, 5, 5, device=gpu).contiguous(memory_format=torch.channels_last), wg[:, :, :, :3].contiguous(), padding=1)
+    assert e.shape == (0, 8, 5, 5)
+
+
+def test_channels_last_full_size_layers(dw, gpu):
+    """Two EfficientNet-B0 layers at batch 128, channels-last: adjoint identities over the whole tensors,
+    sampled channels against the oracle, bit-identical grad-weight."""
+    for shape in [(128, 144, 56, 56, 5, 2, 2), (128, 672, 14, 14, 5, 1, 2)]:
+        n, c, h, w, k, s, p = shape
+        x, wt, gy = make_inputs(shape, seed=37)
+        xg = _channels_last(x, gpu).requires_grad_(True)
+        wg = wt.to(gpu).requires_grad_(True)
+        gyg = _channels_last(gy, gpu)
+        y = dw.depthwise_conv2d(xg, wg, stride=s, padding=p)
+        gx, gw = torch.autograd.grad(y, (xg, wg), gyg)
+        lhs = (y.detach().double() * gyg.double()).sum().item()
+        assert abs(lhs - (xg.detach().double() * gx.double()).sum().item()) <= 1e-6 * abs(lhs) + 1e-3
+        assert abs(lhs - (wg.detach().double() * gw.double()).sum().item()) <= 1e-6 * abs(lhs) + 1e-3
+        for ch in (0, c // 2 + 1, c - 1):
+            sl = slice(ch, ch + 1)
+            xs, ws_, gs = x[:4, sl].contiguous(), wt[sl].contiguous(), gy[:4, sl].contiguous()
+            np.testing.assert_allclose(_np(y.detach()[:4, sl]).astype(np.float64), oracle.forward(_np(xs), _np(ws_), s, p),
+                                       rtol=1e-5, atol=1e-5)
+            np.testing.assert_allclose(_np(gx[:4, sl]).astype(np.float64),
+                                       oracle.grad_input(_np(gs), _np(ws_), (h, w), s, p), rtol=1e-5, atol=1e-5)
+            gw_ref = oracle.grad_weight(_np(x[:, sl].contiguous()), _np(gy[:, sl].contiguous()), ws_.shape, s, p)
+            np.testing.assert_allclose(_np(gw[sl]).astype(np.float64), gw_ref, rtol=1e-4, atol=1e-4 * np.abs(gw_ref).max())
+        _, gw2 = torch.autograd.grad(dw.depthwise_conv2d(xg, wg, stride=s, padding=p), (xg, wg), gyg)
+        assert torch.equal(gw, gw2)
+
