@@ -192,6 +192,7 @@ def main():
                     help="element type of the tensors (the headline metric is f32; 16-bit types accumulate in fp32)")
     ap.add_argument("--layout", default="nchw", choices=["nchw", "nhwc"],
                     help="memory layout of the activations (the headline metric is nchw, the reference's layout)")
+    ap.add_argument("--only", default="", help="comma-separated layer indices of the workload to run (profiling aid)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-miopen", action="store_true")
     ap.add_argument("--separate-backward", action="store_true",
@@ -214,6 +215,8 @@ def main():
     torch.cuda.set_device(dev)
     lib = _C._lib
     shapes = WORKLOADS[args.workload](args.batch)
+    if args.only:
+        shapes = [shapes[int(i)] for i in args.only.split(",")]
     gen = torch.Generator("cpu").manual_seed(0)
     if args.layout == "nhwc" and args.separate_backward:
         sys.exit("--separate-backward applies to the nchw entry points")

@@ -40,6 +40,8 @@ struct NhwcPlan {
     int blocks_x, blocks_y;  // pixel blocks per image
     long blocks_total;       // batch * blocks_y * blocks_x
     int groups;              // grad-weight: workgroups along the pixel-block axis (= chunks)
+    int cgroups;             // workgroups along the channel axis
+    int wgs;                 // forward / grad-input: workgroups in all (1-D grid)
 };
 
 template <typename IO, int CV>
@@ -57,22 +59,41 @@ __device__ __forceinline__ void load_cv(const IO *p, float (&v)[CV])
     }
 }
 
-// One row of a lane's window: COLS pixels x CV channels from row iy, columns ix0.. of an image with C channels.
-// Pixels outside the image read a valid (clamped) address and are zeroed afterwards.
-template <typename IO, int COLS, int CV = 4>
-__device__ __forceinline__ void nhwc_load_row(const IO *src, int iy, int ix0, int in_h, int in_w, int C,
-                                              float (&row)[COLS * CV])
+// Column part of a lane's window addresses, computed once per pixel block: element offset of each of the COLS
+// columns (clamped into the image) and one validity bit per column.
+template <int COLS>
+struct NhwcCols {
+    int off[COLS];
+    unsigned ok;
+};
+template <int COLS>
+__device__ __forceinline__ void nhwc_cols(int ix0, int in_w, int C, NhwcCols<COLS> &c)
 {
-    const bool row_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(in_h);
-    const long row_off = static_cast<long>(min(max(iy, 0), in_h - 1)) * in_w;
+    c.ok = 0;
 #pragma unroll
     for (int j = 0; j < COLS; ++j) {
         const int ix = ix0 + j;
-        const bool ok = row_ok && static_cast<unsigned>(ix) < static_cast<unsigned>(in_w);
-        float t[CV];
-        load_cv<IO, CV>(src + (row_off + min(max(ix, 0), in_w - 1)) * C, t);
+        c.off[j] = min(max(ix, 0), in_w - 1) * C;
+        c.ok |= (static_cast<unsigned>(ix) < static_cast<unsigned>(in_w) ? 1u : 0u) << j;
+    }
+}
+
+// One row of a lane's window: COLS pixels x CV channels of row iy.  `img` points at this lane's channels of
+// pixel (0,0) of its image; in-image offsets are 32-bit.  Pixels outside the image read a valid (clamped)
+// address and are zeroed afterwards.
+template <typename IO, int COLS, int CV = 4>
+__device__ __forceinline__ void nhwc_load_row(const IO *img, int iy, int in_h, int row_pitch, const NhwcCols<COLS> &cols,
+                                              float (&row)[COLS * CV])
+{
+    const unsigned ok = static_cast<unsigned>(iy) < static_cast<unsigned>(in_h) ? cols.ok : 0u;
+    const int rbase = min(max(iy, 0), in_h - 1) * row_pitch;
 #pragma unroll
-        for (int v = 0; v < CV; ++v) row[CV * j + v] = ok ? t[v] : 0.f;
+    for (int j = 0; j < COLS; ++j) {
+        float t[CV];
+        load_cv<IO, CV>(img + (rbase + cols.off[j]), t);
+        const bool keep = (ok >> j) & 1u;
+#pragma unroll
+        for (int v = 0; v < CV; ++v) row[CV * j + v] = keep ? t[v] : 0.f;
     }
 }
 
@@ -95,14 +116,18 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_down_kernel(const NhwcPlan 
     constexpr int KK = K * K;
     constexpr int ROWS = (BH - 1) * S + K, COLS = (TW - 1) * S + K;
     const int C = p.channel;
-    const int c0 = blockIdx.y * p.lanes_c * 4;
+    // 1-D grid, channel group fastest; every XCD (own L2) gets a contiguous run of workgroups, so that pixel
+    // groups that share halo rows, and the channel groups of one pixel group (neighbouring addresses), meet there
+    const int wg = xcd_contiguous_tile(blockIdx.x, p.wgs);
+    const int pg = wg / p.cgroups;
+    const int c0 = (wg - pg * p.cgroups) * p.lanes_c * 4;
     const int nch = min(p.lanes_c * 4, C - c0);
     nhwc_stage_taps<IO, KK, FLIP>(static_cast<const IO *>(p.taps), lds, c0, nch);
     __syncthreads();
 
     const int pb_local = fast_div(threadIdx.x, p.lanes_c_magic);
     const int lane_c = threadIdx.x - pb_local * p.lanes_c;
-    const long pb = static_cast<long>(blockIdx.x) * p.blocks_per_wg + pb_local;
+    const long pb = static_cast<long>(pg) * p.blocks_per_wg + pb_local;
     if (pb_local >= p.blocks_per_wg || pb >= p.blocks_total || 4 * lane_c >= nch) return;
     const int per_image = p.blocks_x * p.blocks_y;
     const int n = static_cast<int>(pb / per_image);
@@ -123,10 +148,13 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_down_kernel(const NhwcPlan 
     // Rows are loaded one ahead of their use and the sums pinned after every row: otherwise the compiler
     // hoists the loads of the whole window to the top and keeps all of it in registers.
     float cur[COLS * 4], nxt[COLS * 4];
-    nhwc_load_row<IO, COLS>(src, iy0, ix0, p.in_h, p.in_w, C, cur);
+    NhwcCols<COLS> cols;
+    nhwc_cols<COLS>(ix0, p.in_w, C, cols);
+    const int row_pitch = p.in_w * C;
+    nhwc_load_row<IO, COLS>(src, iy0, p.in_h, row_pitch, cols, cur);
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
-        if (r + 1 < ROWS) nhwc_load_row<IO, COLS>(src, iy0 + r + 1, ix0, p.in_h, p.in_w, C, nxt);
+        if (r + 1 < ROWS) nhwc_load_row<IO, COLS>(src, iy0 + r + 1, p.in_h, row_pitch, cols, nxt);
 #pragma unroll
         for (int b = 0; b < BH; ++b) {
             const int ty = r - b * S;
@@ -178,14 +206,18 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_up2_kernel(const NhwcPlan p
     constexpr int DMIN = -((K - 1 - PE) / 2);
     constexpr int GROWS = (BH - 1 + PE) / 2 - DMIN + 1, GCOLS = (TW - 1 + PE) / 2 - DMIN + 1;
     const int C = p.channel;
-    const int c0 = blockIdx.y * p.lanes_c * 4;
+    // 1-D grid, channel group fastest; every XCD (own L2) gets a contiguous run of workgroups, so that pixel
+    // groups that share halo rows, and the channel groups of one pixel group (neighbouring addresses), meet there
+    const int wg = xcd_contiguous_tile(blockIdx.x, p.wgs);
+    const int pg = wg / p.cgroups;
+    const int c0 = (wg - pg * p.cgroups) * p.lanes_c * 4;
     const int nch = min(p.lanes_c * 4, C - c0);
     nhwc_stage_taps<IO, KK, false>(static_cast<const IO *>(p.taps), lds, c0, nch);
     __syncthreads();
 
     const int pb_local = fast_div(threadIdx.x, p.lanes_c_magic);
     const int lane_c = threadIdx.x - pb_local * p.lanes_c;
-    const long pb = static_cast<long>(blockIdx.x) * p.blocks_per_wg + pb_local;
+    const long pb = static_cast<long>(pg) * p.blocks_per_wg + pb_local;
     if (pb_local >= p.blocks_per_wg || pb >= p.blocks_total || 4 * lane_c >= nch) return;
     const int per_image = p.blocks_x * p.blocks_y;
     const int n = static_cast<int>(pb / per_image);
@@ -205,10 +237,13 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_up2_kernel(const NhwcPlan p
         for (int o = 0; o < TW * 4; ++o) acc[b][o] = 0.f;
 
     float cur[GCOLS * 4], nxt[GCOLS * 4];
-    nhwc_load_row<IO, GCOLS>(src, gy0, gx0, p.in_h, p.in_w, C, cur);
+    NhwcCols<GCOLS> cols;
+    nhwc_cols<GCOLS>(gx0, p.in_w, C, cols);
+    const int row_pitch = p.in_w * C;
+    nhwc_load_row<IO, GCOLS>(src, gy0, p.in_h, row_pitch, cols, cur);
 #pragma unroll
     for (int g = 0; g < GROWS; ++g) {
-        if (g + 1 < GROWS) nhwc_load_row<IO, GCOLS>(src, gy0 + g + 1, gx0, p.in_h, p.in_w, C, nxt);
+        if (g + 1 < GROWS) nhwc_load_row<IO, GCOLS>(src, gy0 + g + 1, p.in_h, row_pitch, cols, nxt);
 #pragma unroll
         for (int b = 0; b < BH; ++b) {
             const int ty = b + PE - 2 * (DMIN + g);
@@ -291,16 +326,19 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_wgrad_kernel(const NhwcPlan
                 const int ox = ox0 + o;
                 const bool ok = oy < p.out_h && ox < p.out_w;
                 float t[CV];
-                load_cv<IO, CV>(gs + (static_cast<long>(min(oy, p.out_h - 1)) * p.out_w + min(ox, p.out_w - 1)) * C, t);
+                load_cv<IO, CV>(gs + (min(oy, p.out_h - 1) * p.out_w + min(ox, p.out_w - 1)) * C, t);
 #pragma unroll
                 for (int v = 0; v < CV; ++v) g[b][o][v] = ok ? t[v] : 0.f;
             }
         }
         float cur[COLS * CV], nxt[COLS * CV];
-        nhwc_load_row<IO, COLS, CV>(xs, iy0, ix0, p.in_h, p.in_w, C, cur);
+        NhwcCols<COLS> cols;
+        nhwc_cols<COLS>(ix0, p.in_w, C, cols);
+        const int row_pitch = p.in_w * C;
+        nhwc_load_row<IO, COLS, CV>(xs, iy0, p.in_h, row_pitch, cols, cur);
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) {
-            if (r + 1 < ROWS) nhwc_load_row<IO, COLS, CV>(xs, iy0 + r + 1, ix0, p.in_h, p.in_w, C, nxt);
+            if (r + 1 < ROWS) nhwc_load_row<IO, COLS, CV>(xs, iy0 + r + 1, p.in_h, row_pitch, cols, nxt);
 #pragma unroll
             for (int b = 0; b < BH; ++b) {
                 const int ty = r - b * S;
@@ -501,7 +539,12 @@ bool plan_nhwc(NhwcPlan &p, const NhwcGeometry &g, int bh, int tw, int blocks_h,
 {
     p.batch = g.batch;
     p.channel = g.channel;
-    int cap = 64;
+    // Few channel lanes per workgroup make its pixel blocks cover a compact patch of the image (or whole small
+    // images), so halo pixels are shared inside the workgroup's L1 instead of between workgroups.  Measured on
+    // the EfficientNet-B0 layers: 8 lanes win on 7x7 and 14x14 maps, 16 on 28x28, 64 on larger ones.
+    const long pixels = static_cast<long>(g.in_h) * g.in_w;
+    int cap = env_int("DWCONV_NHWC_LANES", pixels <= 256 ? 8 : pixels <= 1024 ? 16 : 64);
+    cap = std::max(1, std::min(cap, 64));
     while (cap > 1 && static_cast<size_t>(cap) * CV * K * K * 4 > static_cast<size_t>(kNhwcTapLds)) --cap;
     p.lanes_c = pick_lanes_c(g.channel / CV, cap);
     p.lanes_c_magic = magic_u16(p.lanes_c);
@@ -509,8 +552,10 @@ bool plan_nhwc(NhwcPlan &p, const NhwcGeometry &g, int bh, int tw, int blocks_h,
     p.blocks_y = ceil_div(blocks_h, bh);
     p.blocks_x = ceil_div(blocks_w, tw);
     p.blocks_total = static_cast<long>(g.batch) * p.blocks_y * p.blocks_x;
-    if (p.blocks_total <= 0 || ceil_div(g.channel / CV, p.lanes_c) > 65535) return false;
-    if ((p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg > 0x7fffffffL) return false;
+    p.cgroups = ceil_div(g.channel / CV, p.lanes_c);
+    const long wgs = (p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg * p.cgroups;
+    if (p.blocks_total <= 0 || p.cgroups > 65535 || wgs > 0x7fffffffL) return false;
+    p.wgs = static_cast<int>(wgs);
     return true;
 }
 
@@ -523,15 +568,22 @@ bool nhwc_fast_ok(const NhwcGeometry &g)
     if (g.channel % 4 != 0) return false;
     if (g.pad_h < 0 || g.pad_w < 0 || g.pad_h >= K || g.pad_w >= K) return false;
     if (g.in_h < 1 || g.in_w < 1 || g.out_h < 1 || g.out_w < 1) return false;
-    if (static_cast<long>(g.in_h) * g.in_w * g.channel >= (1l << 31)) return false;
+    // in-image element offsets are 32-bit
+    if (static_cast<long>(g.in_h) * g.in_w * g.channel >= (1l << 31) ||
+        static_cast<long>(g.out_h) * g.out_w * g.channel >= (1l << 31))
+        return false;
     return true;
 }
 
-template <typename IO, int K, int S, bool FLIP>
+template <typename IO, int K, int S, bool FLIP, int TW = 4>
 int launch_nhwc_down(const IO *in, const IO *taps, IO *out, const NhwcGeometry &g, int in_h, int in_w, int out_h,
                      int out_w, int pad_h, int pad_w, hipStream_t stream)
 {
-    constexpr int BH = 4, TW = K == 3 ? 4 : 2;
+    constexpr int BH = 4;
+    if constexpr (K > 3 && TW == 4) {
+        if (env_int("DWCONV_NHWC_TW", 4) == 2)
+            return launch_nhwc_down<IO, K, S, FLIP, 2>(in, taps, out, g, in_h, in_w, out_h, out_w, pad_h, pad_w, stream);
+    }
     NhwcPlan p{};
     if (!plan_nhwc<K, 4>(p, g, BH, TW, out_h, out_w)) return -1;
     p.in = in;
@@ -543,8 +595,7 @@ int launch_nhwc_down(const IO *in, const IO *taps, IO *out, const NhwcGeometry &
     p.out_w = out_w;
     p.pad_h = pad_h;
     p.pad_w = pad_w;
-    const dim3 grid(static_cast<unsigned>((p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg),
-                    ceil_div(g.channel / 4, p.lanes_c));
+    const dim3 grid(p.wgs);
     const size_t shmem = static_cast<size_t>(p.lanes_c) * 4 * K * K * 4;
     hipLaunchKernelGGL((nhwc_down_kernel<IO, K, S, FLIP, BH, TW>), grid, dim3(kNhwcThreads), shmem, stream, p);
     note_variant("nhwc_down%s<k%d,s%d,%s,%dx%d> lanes_c%d", sizeof(IO) == 2 ? "16" : "", K, S, FLIP ? "rot" : "fwd", BH, TW,
@@ -567,8 +618,7 @@ int launch_nhwc_up2(const IO *gy, const IO *taps, IO *gx, const NhwcGeometry &g,
     p.out_w = g.in_w;
     p.pad_h = g.pad_h / 2;
     p.pad_w = g.pad_w / 2;
-    const dim3 grid(static_cast<unsigned>((p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg),
-                    ceil_div(g.channel / 4, p.lanes_c));
+    const dim3 grid(p.wgs);
     const size_t shmem = static_cast<size_t>(p.lanes_c) * 4 * K * K * 4;
     hipLaunchKernelGGL((nhwc_up2_kernel<IO, K, PE, BH, TW>), grid, dim3(kNhwcThreads), shmem, stream, p);
     note_variant("nhwc_up2%s<k%d,e%d,%dx%d> lanes_c%d", sizeof(IO) == 2 ? "16" : "", K, PE, BH, TW, p.lanes_c);
@@ -577,8 +627,9 @@ int launch_nhwc_up2(const IO *gy, const IO *taps, IO *gx, const NhwcGeometry &g,
 
 template <int K>
 struct WgradShape {
-    static constexpr int CV = K == 7 ? 2 : 4;
-    static constexpr int BH = K == 3 ? 4 : 2;
+    // K*K*CV sums live in registers: 36 for 3x3 with four channels per lane, 50 / 98 with two for 5x5 / 7x7
+    static constexpr int CV = K == 3 ? 4 : 2;
+    static constexpr int BH = K == 7 ? 2 : 4;
     static constexpr int TW = 4;
 };
 
@@ -590,7 +641,7 @@ long nhwc_wgrad_case(int mode, const IO *x, const IO *gy, IO *gw, void *ws, size
     constexpr int CV = WgradShape<K>::CV, BH = WgradShape<K>::BH, TW = WgradShape<K>::TW;
     NhwcPlan p{};
     if (!plan_nhwc<1, CV>(p, g, BH, TW, g.out_h, g.out_w)) return -1;
-    const int cgroups = ceil_div(g.channel / CV, p.lanes_c);
+    const int cgroups = p.cgroups;
     const long wg_iters = (p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg;
     long groups = env_int("DWCONV_NHWC_WGRAD_WGS", 1024) / cgroups;
     groups = std::max(1l, std::min(groups, wg_iters));
