@@ -181,6 +181,52 @@ def miopen_native(layers, torch, iters=3):
     return per_layer
 
 
+def epilogue_comparison(layers, lib, torch, stream, dtype, layout, iters=10):
+    """Forward + folded batch-norm + SiLU over the workload: one fused C-ABI call per layer against the plain forward
+    call followed by PyTorch's elementwise ops on its output.  Returns (fused ms, unfused ms, convolution-only ms) per pass over the layers."""
+    import torch.nn.functional as F
+
+    fn = getattr(lib, ("dwconv2d_fused_nhwc_" if layout == "nhwc" else "dwconv2d_fused_") + dtype)
+    prepared = []
+    for l in layers:
+        n, c, h, w, oh, ow, k, s, p = l.geom
+        scale = torch.rand(c, device=l.x.device) + 0.5
+        shift = torch.randn(c, device=l.x.device)
+        shape = (1, 1, 1, c) if layout == "nhwc" else (1, c, 1, 1)
+        y = l.y.view(n, oh, ow, c) if layout == "nhwc" else l.y
+        prepared.append((l, scale, shift, scale.view(shape).to(l.y.dtype), shift.view(shape).to(l.y.dtype), y))
+
+    def call(l, scale, shift, act):
+        n, c, h, w, oh, ow, k, s, p = l.geom
+        l._check(fn(l.x.data_ptr(), l.w.data_ptr(), scale, shift, l.y.data_ptr(), n, c, h, w, k, k, s, s, p, p, act, stream))
+
+    def fused():
+        for l, scale, shift, _, _, _ in prepared:
+            call(l, scale.data_ptr(), shift.data_ptr(), 3)
+
+    def unfused():
+        for l, _, _, scale_b, shift_b, y in prepared:
+            call(l, None, None, 0)
+            F.silu(y * scale_b + shift_b)
+
+    def conv_only():
+        for l, _, _, _, _, _ in prepared:
+            call(l, None, None, 0)
+
+    out = []
+    for run in (fused, unfused, conv_only):
+        run()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        out.append(e0.elapsed_time(e1) / iters)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -193,6 +239,9 @@ def main():
     ap.add_argument("--layout", default="nchw", choices=["nchw", "nhwc"],
                     help="memory layout of the activations (the headline metric is nchw, the reference's layout)")
     ap.add_argument("--only", default="", help="comma-separated layer indices of the workload to run (profiling aid)")
+    ap.add_argument("--epilogue", action="store_true",
+                    help="also time forward + folded batch-norm + SiLU, fused into the convolution against separate "
+                         "elementwise passes (reported under 'fused_epilogue')")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-miopen", action="store_true")
     ap.add_argument("--separate-backward", action="store_true",
@@ -332,6 +381,11 @@ def main():
             result["speedup_vs_miopen_native"] = round(sum(per_layer) / ms_per_step, 2)
         except Exception as e:  # the comparison is informative only
             result["miopen_native_ms_per_step"] = f"failed: {type(e).__name__}"
+    if args.epilogue:
+        fused_ms, unfused_ms, conv_ms = epilogue_comparison(layers, lib, torch, stream, args.dtype, args.layout)
+        result["fused_epilogue"] = {"what": "forward + per-channel scale/shift + SiLU over the workload's layers",
+                                    "fused_ms": round(fused_ms, 4), "conv_then_torch_elementwise_ms": round(unfused_ms, 4),
+                                    "conv_only_ms": round(conv_ms, 4)}
     if not args.no_cpu_baseline and args.dtype == "f32" and args.layout == "nchw":
         result["cpu_baseline"] = cpu_baseline(shapes, torch)
     print(json.dumps(result))

@@ -100,15 +100,23 @@ int run_fir(const T *in, const T *taps, T *out, const Geometry &g, hipStream_t s
     return launch_fir_direct<T>(in, taps, out, g, stream);
 }
 
+int check_activation(int act)
+{
+    if (act < DWCONV_ACT_NONE || act > DWCONV_ACT_SILU)
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "unknown activation %d", act);
+    return DWCONV_OK;
+}
+
 template <typename T>
 int dwconv2d_any(const T *in, const T *taps, T *out, int batch, int channel, int in_h, int in_w,
                  int kernel_h, int kernel_w, int up_h, int up_w, int down_h, int down_w, int pad_h0,
-                 int pad_h1, int pad_w0, int pad_w1, int forward, void *stream)
+                 int pad_h1, int pad_w0, int pad_w1, int forward, void *stream, const Epilogue &epi = Epilogue{})
 {
     Geometry g;
     const int rc = make_geometry(g, in, taps, out, batch, channel, in_h, in_w, kernel_h, kernel_w,
                                  up_h, up_w, down_h, down_w, pad_h0, pad_h1, pad_w0, pad_w1, forward);
     if (rc != DWCONV_OK) return rc;
+    g.epi = epi;
     return run_fir<T>(in, taps, out, g, static_cast<hipStream_t>(stream));
 }
 
@@ -277,11 +285,13 @@ int make_nhwc_geometry(NhwcGeometry &g, int batch, int channel, int in_h, int in
 
 template <typename T>
 int nhwc_forward_any(const T *in, const T *taps, T *out, int batch, int channel, int in_h, int in_w, int kernel_h,
-                     int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w, void *stream)
+                     int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w, void *stream,
+                     const Epilogue &epi = Epilogue{})
 {
     NhwcGeometry g;
     const int rc = make_nhwc_geometry(g, batch, channel, in_h, in_w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w);
     if (rc != DWCONV_OK) return rc;
+    g.epi = epi;
     const long long out_elems = 1ll * batch * channel * g.out_h * g.out_w;
     if (out_elems > 0 && (in == nullptr || taps == nullptr || out == nullptr))
         return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");
@@ -512,5 +522,40 @@ DWCONV_NHWC_ENTRY_POINTS(f64, double, double)
 DWCONV_NHWC_ENTRY_POINTS(f16, unsigned short, half_t)
 DWCONV_NHWC_ENTRY_POINTS(bf16, unsigned short, bf16_t)
 #undef DWCONV_NHWC_ENTRY_POINTS
+
+// ---- forward with a fused per-channel scale / shift and activation ----
+#define DWCONV_FUSED_ENTRY_POINTS(SUFFIX, CTYPE, TYPE, PTYPE)                                                          \
+    int dwconv2d_fused_##SUFFIX(const CTYPE *input, const CTYPE *kernel, const PTYPE *scale, const PTYPE *shift,       \
+                                CTYPE *out, int batch, int channel, int in_h, int in_w, int kernel_h, int kernel_w,    \
+                                int stride_h, int stride_w, int pad_h, int pad_w, int activation, void *stream)        \
+    {                                                                                                                  \
+        if (check_activation(activation) != DWCONV_OK) return DWCONV_ERR_INVALID_ARGUMENT;                             \
+        Epilogue epi;                                                                                                  \
+        epi.scale = scale;                                                                                             \
+        epi.shift = shift;                                                                                             \
+        epi.act = activation;                                                                                          \
+        return dwconv2d_any<TYPE>(reinterpret_cast<const TYPE *>(input), reinterpret_cast<const TYPE *>(kernel),       \
+                                  reinterpret_cast<TYPE *>(out), batch, channel, in_h, in_w, kernel_h, kernel_w, 1, 1, \
+                                  stride_h, stride_w, pad_h, pad_h, pad_w, pad_w, 1, stream, epi);                     \
+    }                                                                                                                  \
+    int dwconv2d_fused_nhwc_##SUFFIX(const CTYPE *input, const CTYPE *kernel, const PTYPE *scale, const PTYPE *shift,  \
+                                     CTYPE *out, int batch, int channel, int in_h, int in_w, int kernel_h,             \
+                                     int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w, int activation,   \
+                                     void *stream)                                                                     \
+    {                                                                                                                  \
+        if (check_activation(activation) != DWCONV_OK) return DWCONV_ERR_INVALID_ARGUMENT;                             \
+        Epilogue epi;                                                                                                  \
+        epi.scale = scale;                                                                                             \
+        epi.shift = shift;                                                                                             \
+        epi.act = activation;                                                                                          \
+        return nhwc_forward_any<TYPE>(reinterpret_cast<const TYPE *>(input), reinterpret_cast<const TYPE *>(kernel),   \
+                                      reinterpret_cast<TYPE *>(out), batch, channel, in_h, in_w, kernel_h, kernel_w,   \
+                                      stride_h, stride_w, pad_h, pad_w, stream, epi);                                  \
+    }
+DWCONV_FUSED_ENTRY_POINTS(f32, float, float, float)
+DWCONV_FUSED_ENTRY_POINTS(f64, double, double, double)
+DWCONV_FUSED_ENTRY_POINTS(f16, unsigned short, half_t, float)
+DWCONV_FUSED_ENTRY_POINTS(bf16, unsigned short, bf16_t, float)
+#undef DWCONV_FUSED_ENTRY_POINTS
 
 }  // extern "C"

@@ -51,6 +51,68 @@ struct Io<bf16_t> {
     }
 };
 
+// What a forward kernel applies to each sum before storing it: v * scale[c] + shift[c], then an activation.
+// scale / shift are per-channel arrays of the accumulation type (float; double for fp64 tensors) or null.
+struct Epilogue {
+    const void *scale = nullptr;
+    const void *shift = nullptr;
+    int act = DWCONV_ACT_NONE;  // dwconv_activation
+    __host__ __device__ bool enabled() const { return scale != nullptr || shift != nullptr || act != DWCONV_ACT_NONE; }
+};
+
+// v * sigmoid(v).  fp32: hardware exp2 and reciprocal (1 ulp each), two quarter-rate instructions instead of
+// the dozen of an IEEE division.
+__device__ __forceinline__ float epilogue_silu(float v) { return v * __builtin_amdgcn_rcpf(1.f + __expf(-v)); }
+__device__ __forceinline__ double epilogue_silu(double v) { return v / (1.0 + exp(-v)); }
+
+template <typename A>
+__device__ __forceinline__ A epilogue_apply(A v, const Epilogue &e, int c)
+{
+    if (e.scale != nullptr) v *= static_cast<const A *>(e.scale)[c];
+    if (e.shift != nullptr) v += static_cast<const A *>(e.shift)[c];
+    // comparisons written so that NaN passes through, as it does in torch
+    if (e.act == DWCONV_ACT_RELU) v = v < A(0) ? A(0) : v;
+    else if (e.act == DWCONV_ACT_RELU6) v = v < A(0) ? A(0) : (v > A(6) ? A(6) : v);
+    else if (e.act == DWCONV_ACT_SILU) v = epilogue_silu(v);
+    return v;
+}
+
+// The same for a lane's whole register block: the tests on the (uniform) options are made once, outside the
+// element loops, so that the independent exp/rcp chains of the elements can overlap.  Element [r][j] belongs
+// to channel c0 + (j % CPL) (CPL = 1: one channel for the whole block).
+template <int CPL, int R, int C>
+__device__ __forceinline__ void epilogue_apply_block(float (&acc)[R][C], const Epilogue &e, int c0)
+{
+    if (e.scale != nullptr || e.shift != nullptr) {
+        float sc[CPL], sh[CPL];
+#pragma unroll
+        for (int v = 0; v < CPL; ++v) {
+            sc[v] = e.scale != nullptr ? static_cast<const float *>(e.scale)[c0 + v] : 1.f;
+            sh[v] = e.shift != nullptr ? static_cast<const float *>(e.shift)[c0 + v] : 0.f;
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int j = 0; j < C; ++j) acc[r][j] = fmaf(acc[r][j], sc[j % CPL], sh[j % CPL]);
+    }
+    if (e.act == DWCONV_ACT_RELU) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int j = 0; j < C; ++j) acc[r][j] = acc[r][j] < 0.f ? 0.f : acc[r][j];
+    } else if (e.act == DWCONV_ACT_RELU6) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int j = 0; j < C; ++j) acc[r][j] = acc[r][j] < 0.f ? 0.f : (acc[r][j] > 6.f ? 6.f : acc[r][j]);
+    } else if (e.act == DWCONV_ACT_SILU) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int j = 0; j < C; ++j) acc[r][j] = epilogue_silu(acc[r][j]);
+    }
+}
+
 // Geometry of one up/FIR/down call on dense NCHW planes.  The same fields as the
 // reference's DWConv2dKernelParams (torch_dwconv/dwconv_kernel.cu:42-67), with the
 // batch and channel extents folded into `planes` where a kernel does not need them.
@@ -63,6 +125,7 @@ struct Geometry {
     int pad_h0, pad_h1, pad_w0, pad_w1;
     int out_h, out_w;
     int forward;
+    Epilogue epi;  // forward convolutions only
     long planes() const { return static_cast<long>(batch) * channel; }
 };
 
@@ -84,6 +147,7 @@ struct NhwcGeometry {
     int kernel_h, kernel_w;
     int stride_h, stride_w;
     int pad_h, pad_w;
+    Epilogue epi;  // nhwc_forward only
 };
 
 // Thread-local error/variant strings behind dwconv_last_error()/dwconv_last_variant().

@@ -46,6 +46,7 @@ __global__ __launch_bounds__(kDirectThreads) void fir_direct_kernel(
                 acc += Io<T>::in(fv) * Io<T>::in(src[static_cast<long>(iy) * g.in_w + ix]);
             }
         }
+        if (g.epi.enabled()) acc = epilogue_apply(acc, g.epi, c);
         out[idx] = Io<T>::out(acc);
     }
 }

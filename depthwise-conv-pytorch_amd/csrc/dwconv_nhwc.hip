@@ -40,6 +40,7 @@ struct NhwcPlan {
     int blocks_x, blocks_y;  // pixel blocks per image
     long blocks_total;       // batch * blocks_y * blocks_x
     int groups;              // grad-weight: workgroups along the pixel-block axis (= chunks)
+    Epilogue epi;            // forward kernel: applied to every sum before it is stored
     int cgroups;             // workgroups along the channel axis
     int wgs;                 // forward / grad-input: workgroups in all (1-D grid)
 };
@@ -176,6 +177,9 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_down_kernel(const NhwcPlan 
         for (int j = 0; j < COLS * 4; ++j) cur[j] = nxt[j];
     }
 
+    if constexpr (!FLIP) {
+        if (p.epi.enabled()) epilogue_apply_block<4>(acc, p.epi, c);
+    }
     IO *dst = static_cast<IO *>(p.out) + static_cast<long>(n) * p.out_h * p.out_w * C + c;
 #pragma unroll
     for (int b = 0; b < BH; ++b) {
@@ -440,6 +444,7 @@ __global__ __launch_bounds__(256) void nhwc_fwd_direct_kernel(const T *__restric
                  static_cast<acc_t>(Io<T>::in(taps[(static_cast<long>(c) * g.kernel_h + ty) * g.kernel_w + tx]));
         }
     }
+    if (g.epi.enabled()) s = epilogue_apply(s, g.epi, c);
     out[e] = Io<T>::out(s);
 }
 
@@ -589,6 +594,7 @@ int launch_nhwc_down(const IO *in, const IO *taps, IO *out, const NhwcGeometry &
     p.in = in;
     p.taps = taps;
     p.out = out;
+    if (!FLIP) p.epi = g.epi;
     p.in_h = in_h;
     p.in_w = in_w;
     p.out_h = out_h;

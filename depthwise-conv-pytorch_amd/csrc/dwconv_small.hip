@@ -35,6 +35,7 @@ struct SmallPlan {
     int planes_per_run;    // P
     int lanes_per_plane;   // LPP
     unsigned lpp_magic;
+    Epilogue epi;          // forward kernels: applied to every sum before it is stored
 };
 
 // out[oy,ox] = sum_{ty,tx} in[oy*S - pad_h + ty, ox*S - K/2 + tx] * f[ty,tx], planes W wide.
@@ -101,6 +102,11 @@ __global__ __launch_bounds__(kWave) void small_down_kernel(const SmallPlan p)
                 }
         }
         pin_registers(acc);
+    }
+    if constexpr (!FLIP) {
+        if (p.epi.enabled()) {
+            epilogue_apply_block<1>(acc, p.epi, static_cast<int>((plane0 + pl) % p.channel));
+        }
     }
     __syncthreads();  // every lane has read its input rows: the run can be overwritten in place
 
@@ -305,6 +311,7 @@ int try_launch_fir_small(const IO *in, const IO *taps, IO *out, const Geometry &
     p.out = out;
     p.planes = g.planes();
     p.channel = g.channel;
+    p.epi = g.epi;
     p.in_h = g.in_h;
     p.out_h = g.out_h;
     const int W = g.in_w;

@@ -46,6 +46,7 @@ struct TilePlan {
     unsigned ipp_magic;
     int tap_base;              // float offset of the tap table in LDS
     int vec_out;               // 128-bit global stores are legal
+    Epilogue epi;              // forward kernels: applied to every sum before it is stored
 };
 
 // Copies the tap tables of the tile's planes into LDS, rotated by 180 degrees if FLIP.
@@ -119,6 +120,11 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
             pin_registers(acc);
         }
 
+        if constexpr (!FLIP) {
+            if (p.epi.enabled()) {
+                epilogue_apply_block<1>(acc, p.epi, static_cast<int>((plane0 + pl) % p.channel));
+            }
+        }
         const int ox = 4 * cb;
         IO *dst = static_cast<IO *>(p.out) + (plane0 + pl) * p.out_plane + ox;
 #pragma unroll
@@ -359,6 +365,7 @@ int try_launch_fir_tiled(const IO *in, const IO *taps, IO *out, const Geometry &
     p.out = out;
     p.planes = g.planes();
     p.channel = g.channel;
+    p.epi = g.epi;
     p.st.in_h = g.in_h;
     p.st.in_w = g.in_w;
     p.out_h = g.out_h;

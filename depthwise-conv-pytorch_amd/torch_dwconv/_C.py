@@ -61,6 +61,13 @@ for _name in ("dwconv2d_backward_nhwc_f32", "dwconv2d_backward_nhwc_f64", "dwcon
     getattr(_lib, _name).restype = _i
     getattr(_lib, _name).argtypes = [_p, _p, _p, _p, _p, _p, _z] + [_i] * 12 + [_p]
 
+for _sfx in ("f32", "f64", "f16", "bf16"):
+    for _name in ("dwconv2d_fused_" + _sfx, "dwconv2d_fused_nhwc_" + _sfx):
+        getattr(_lib, _name).restype = _i
+        getattr(_lib, _name).argtypes = [_p, _p, _p, _p, _p] + [_i] * 11 + [_p]
+
+ACTIVATIONS = {None: 0, "none": 0, "relu": 1, "relu6": 2, "silu": 3}
+
 _SUFFIX = {torch.float32: "f32", torch.float64: "f64", torch.float16: "f16", torch.bfloat16: "bf16"}
 
 
@@ -281,3 +288,44 @@ def dwconv2d_backward_nhwc(input, out_grad, kernel, stride_h, stride_w, pad_h, p
     if rc != 0:
         _raise(rc)
     return gx, gw
+
+
+def dwconv2d_fused(input, kernel, scale, shift, activation, stride_h, stride_w, pad_h, pad_w):
+    """``act(conv(input, kernel) * scale[c] + shift[c])`` in one kernel; NCHW or channels-last (kept) input.
+
+    ``scale`` / ``shift``: per-channel tensors or ``None``; ``activation``: ``None``, ``'relu'``, ``'relu6'`` or
+    ``'silu'``.  The reference has no such entry point (it rejects a bias, torch_dwconv/dwconv.py:108-109).
+    """
+    _check_cuda(input, "input")
+    _check_cuda(kernel, "kernel")
+    _check_shapes(input, kernel)
+    sfx = _suffix(input, kernel)
+    if activation not in ACTIVATIONS:
+        raise ValueError(f"unknown activation {activation!r}; expected one of None, 'relu', 'relu6', 'silu'")
+    param_dtype = torch.float64 if input.dtype == torch.float64 else torch.float32
+    params = []
+    for name, t in (("scale", scale), ("shift", shift)):
+        if t is None:
+            params.append(None)
+            continue
+        _check_cuda(t, name)
+        if t.numel() != input.shape[1]:
+            raise RuntimeError(f"{name} must have one entry per channel ({input.shape[1]}), got {tuple(t.shape)}")
+        params.append(t.detach().reshape(-1).to(device=input.device, dtype=param_dtype).contiguous())
+    nhwc = is_channels_last(input)
+    x = input.contiguous(memory_format=torch.channels_last) if nhwc else input.contiguous()
+    k = kernel.contiguous()
+    n, c, h, w = x.shape
+    kh, kw = k.shape[2], k.shape[3]
+    oh = max(_lib.dwconv_out_size(h, 1, stride_h, pad_h, pad_h, kh), 0)
+    ow = max(_lib.dwconv_out_size(w, 1, stride_w, pad_w, pad_w, kw), 0)
+    out = torch.empty((n, c, oh, ow), dtype=x.dtype, device=x.device,
+                      memory_format=torch.channels_last if nhwc else torch.contiguous_format)
+    fn = getattr(_lib, ("dwconv2d_fused_nhwc_" if nhwc else "dwconv2d_fused_") + sfx)
+    with torch.cuda.device(x.device):
+        rc = fn(x.data_ptr(), k.data_ptr(), params[0].data_ptr() if params[0] is not None else None,
+                params[1].data_ptr() if params[1] is not None else None, out.data_ptr(), n, c, h, w, kh, kw,
+                stride_h, stride_w, pad_h, pad_w, ACTIVATIONS[activation], _stream(x))
+    if rc != 0:
+        _raise(rc)
+    return out

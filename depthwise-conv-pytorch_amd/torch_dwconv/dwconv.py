@@ -140,6 +140,36 @@ def depthwise_conv2d(input, weight, bias=None, stride=1, padding=0, dilation=1, 
     return depthwise_conv2d_fn(input, weight, stride, padding, small)
 
 
+_TORCH_ACTIVATIONS = {None: None, "none": None, "relu": F.relu, "relu6": F.relu6, "silu": F.silu}
+
+
+def depthwise_conv2d_fused(input, weight, bias=None, scale=None, activation=None, stride=1, padding=0):
+    """``act(depthwise_conv2d(input, weight) * scale[c] + bias[c])``: the convolution together with the step that
+    follows it in EfficientNet / MobileNet blocks (bias or folded batch-norm, then ReLU / ReLU6 / SiLU).
+
+    Not in the reference, whose ``check_options`` rejects a bias (torch_dwconv/dwconv.py:108-109).  Without
+    gradients (inference) this is one kernel; when a gradient is needed the same value is composed from
+    ``depthwise_conv2d`` and PyTorch's elementwise ops, so that autograd differentiates it.
+    """
+    if activation not in _TORCH_ACTIVATIONS:
+        raise ValueError(f"unknown activation {activation!r}; expected one of None, 'relu', 'relu6', 'silu'")
+    stride = make_tuple(stride, 2)
+    padding = make_tuple(padding, 2)
+    check_options(input.shape[1], weight.shape[0], 1, None, False)
+    needs_grad = torch.is_grad_enabled() and any(
+        t is not None and t.requires_grad for t in (input, weight, bias, scale)
+    )
+    if not needs_grad:
+        return _C.dwconv2d_fused(input, weight, scale, bias, activation, stride[0], stride[1], padding[0], padding[1])
+    out = depthwise_conv2d(input, weight, None, stride, padding)
+    if scale is not None:
+        out = out * scale.view(1, -1, 1, 1).to(out.dtype)
+    if bias is not None:
+        out = out + bias.view(1, -1, 1, 1).to(out.dtype)
+    act = _TORCH_ACTIVATIONS[activation]
+    return out if act is None else act(out)
+
+
 class DepthwiseConv2d(nn.Module):
     """Reference: torch_dwconv/dwconv.py:133-175.
 

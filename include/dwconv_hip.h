@@ -39,6 +39,14 @@ typedef enum dwconv_status {
     DWCONV_ERR_LAUNCH = 4            /* HIP reported an error at launch */
 } dwconv_status;
 
+/* Activation of the fused forward entry points (dwconv2d_fused_*). */
+typedef enum dwconv_activation {
+    DWCONV_ACT_NONE = 0,
+    DWCONV_ACT_RELU = 1,  /* max(v, 0) */
+    DWCONV_ACT_RELU6 = 2, /* min(max(v, 0), 6) */
+    DWCONV_ACT_SILU = 3   /* v * sigmoid(v) */
+} dwconv_activation;
+
 /* Message describing the last error returned to this thread ("" if none). */
 const char *dwconv_last_error(void);
 
@@ -240,6 +248,47 @@ int dwconv2d_backward_nhwc_bf16(const unsigned short *input, const unsigned shor
                                 int batch, int channel, int in_h, int in_w, int out_h, int out_w,
                                 int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h,
                                 int pad_w, void *stream);
+
+/* ---- forward convolution with a fused epilogue ---------------------------------------------------
+ *   out = act(conv(input, kernel) * scale[c] + shift[c])
+ * for the step that follows a depthwise convolution in EfficientNet / MobileNet / ConvNeXt blocks: bias
+ * (which the reference rejects, torch_dwconv/dwconv.py:108-109), a folded batch-norm (scale and shift) and
+ * ReLU / ReLU6 / SiLU.  No counterpart in the reference.  scale and shift are device arrays of `channel`
+ * entries in the accumulation type (float for f32/f16/bf16 tensors, double for f64); either may be NULL
+ * (factor 1 / offset 0).  Saves the separate elementwise pass over `out` (one read and one write of it).
+ * conv = dwconv2d_* with up = 1, down = stride, pad0 = pad1 = pad, forward = 1; `_nhwc`: channels-last tensors. */
+int dwconv2d_fused_f32(const float *input, const float *kernel, const float *scale,
+    const float *shift, float *out, int batch, int channel, int in_h, int in_w,
+    int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+    int activation, void *stream);
+int dwconv2d_fused_nhwc_f32(const float *input, const float *kernel, const float *scale,
+    const float *shift, float *out, int batch, int channel, int in_h, int in_w,
+    int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+    int activation, void *stream);
+int dwconv2d_fused_f64(const double *input, const double *kernel, const double *scale,
+    const double *shift, double *out, int batch, int channel, int in_h, int in_w,
+    int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+    int activation, void *stream);
+int dwconv2d_fused_nhwc_f64(const double *input, const double *kernel, const double *scale,
+    const double *shift, double *out, int batch, int channel, int in_h, int in_w,
+    int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+    int activation, void *stream);
+int dwconv2d_fused_f16(const unsigned short *input, const unsigned short *kernel, const float *scale,
+    const float *shift, unsigned short *out, int batch, int channel, int in_h, int in_w,
+    int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+    int activation, void *stream);
+int dwconv2d_fused_nhwc_f16(const unsigned short *input, const unsigned short *kernel, const float *scale,
+    const float *shift, unsigned short *out, int batch, int channel, int in_h, int in_w,
+    int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+    int activation, void *stream);
+int dwconv2d_fused_bf16(const unsigned short *input, const unsigned short *kernel, const float *scale,
+    const float *shift, unsigned short *out, int batch, int channel, int in_h, int in_w,
+    int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+    int activation, void *stream);
+int dwconv2d_fused_nhwc_bf16(const unsigned short *input, const unsigned short *kernel, const float *scale,
+    const float *shift, unsigned short *out, int batch, int channel, int in_h, int in_w,
+    int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+    int activation, void *stream);
 
 /* Tuning/diagnostic hook: name of the kernel variant the last successful call
  * on this thread launched (e.g. "tile_f32<k3,s1,v4>"), for benchmarks and tests. */

@@ -21,6 +21,20 @@ def torch_reference(x, w, gy=None, stride=1, padding=0):
     return y.detach(), gx, gw
 
 
+_ACTIVATIONS = {None: lambda v: v, "none": lambda v: v, "relu": F.relu, "relu6": F.relu6, "silu": F.silu}
+
+
+def torch_reference_fused(x, w, scale=None, shift=None, activation=None, stride=1, padding=0):
+    """fp64 CPU value of ``act(conv(x, w) * scale[c] + shift[c])``: PyTorch's conv followed by PyTorch's own
+    elementwise functions (the fused forward entry points have no counterpart in the reference)."""
+    y, _, _ = torch_reference(x, w, None, stride, padding)
+    if scale is not None:
+        y = y * scale.detach().to("cpu", torch.float64).view(1, -1, 1, 1)
+    if shift is not None:
+        y = y + shift.detach().to("cpu", torch.float64).view(1, -1, 1, 1)
+    return _ACTIVATIONS[activation](y)
+
+
 def torch_cpu_fp32_step(x, w, gy, stride, padding, iters=3, threads=None):
     """Time fp32 ``F.conv2d(groups=C)`` forward + both gradients on the host cores.
 

@@ -578,3 +578,82 @@ def test_channels_last_full_size_layers(dw, gpu):
         _, gw2 = torch.autograd.grad(dw.depthwise_conv2d(xg, wg, stride=s, padding=p), (xg, wg), gyg)
         assert torch.equal(gw, gw2)
 
+
+# ---- forward with a fused per-channel scale / shift and activation -------------------------------------------
+FUSED_CASES = [
+    # (shape, channels_last, expected kernel family)
+    ((2, 8, 56, 56, 3, 1, 1), False, "tile_down"), ((2, 6, 57, 44, 5, 2, 2), False, "tile_down"),
+    ((3, 8, 14, 14, 5, 1, 2), False, "small_down"), ((2, 12, 28, 28, 3, 2, 1), False, "small_down"),
+    ((2, 3, 9, 11, 4, 1, 1), False, "direct"), ((2, 16, 20, 24, 3, 1, 1), True, "nhwc_down"),
+    ((2, 8, 15, 13, 5, 2, 2), True, "nhwc_down"), ((2, 5, 9, 9, 3, 1, 1), True, "nhwc_fwd_direct"),
+]
+
+
+@pytest.mark.parametrize("activation", [None, "relu", "relu6", "silu"])
+@pytest.mark.parametrize("case", FUSED_CASES, ids=lambda c: shape_id(c[0]) + ("_nhwc" if c[1] else ""))
+def test_fused_epilogue(dw, gpu, case, activation):
+    from torch_dwconv import _C
+    from torch_dwconv.dwconv import depthwise_conv2d_fused
+
+    shape, nhwc, family = case
+    n, c, h, w, k, s, p = shape
+    x, wt, _ = make_inputs(shape, seed=43)
+    x = x * 2  # enough spread to reach both sides of relu6
+    g = torch.Generator("cpu").manual_seed(44)
+    scale = torch.randn(c, generator=g) + 1.5
+    shift = torch.randn(c, generator=g)
+    xg = _channels_last(x, gpu) if nhwc else x.to(gpu)
+    for sc, sh in [(scale, shift), (None, shift), (scale, None), (None, None)]:
+        y = depthwise_conv2d_fused(xg, wt.to(gpu), bias=None if sh is None else sh.to(gpu),
+                                   scale=None if sc is None else sc.to(gpu), activation=activation, stride=s, padding=p)
+        assert _C.last_variant().startswith(family), _C.last_variant()
+        assert y.is_contiguous(memory_format=torch.channels_last) == nhwc or y.is_contiguous()
+        ref = oracle.torch_reference_fused(x, wt, sc, sh, activation, s, p)
+        np.testing.assert_allclose(_np(y).astype(np.float64), ref.numpy(), rtol=1e-5, atol=1e-5)
+
+
+def test_fused_epilogue_other_dtypes_and_autograd(dw, gpu):
+    from torch_dwconv import _C
+    from torch_dwconv.dwconv import depthwise_conv2d_fused
+
+    shape = (2, 8, 14, 14, 3, 1, 1)
+    n, c, h, w, k, s, p = shape
+    x, wt, gy = make_inputs(shape, seed=45)
+    scale, shift = torch.linspace(0.5, 2.0, c), torch.linspace(-1.0, 1.0, c)
+    # fp64 (generic kernel, double parameters) to 1e-12; fp16 / bf16 to one rounding step
+    y64 = depthwise_conv2d_fused(x.double().to(gpu), wt.double().to(gpu), shift.to(gpu), scale.to(gpu), "silu", s, p)
+    ref64 = oracle.torch_reference_fused(x.double(), wt.double(), scale.double(), shift.double(), "silu", s, p)
+    np.testing.assert_allclose(_np(y64), ref64.numpy(), rtol=1e-12, atol=1e-12)
+    for dtype, step in [(torch.float16, 2.0 ** -11), (torch.bfloat16, 2.0 ** -8)]:
+        xs, ws = x.to(dtype), wt.to(dtype)
+        y = depthwise_conv2d_fused(xs.to(gpu), ws.to(gpu), shift.to(gpu), scale.to(gpu), "relu6", s, p)
+        assert y.dtype == dtype
+        ref = oracle.torch_reference_fused(xs, ws, scale, shift, "relu6", s, p)
+        np.testing.assert_allclose(_np(y.double()), ref.numpy(), rtol=step, atol=1e-5 + step * 1e-2)
+    # with gradients the value is composed from differentiable pieces: same value, gradients as torch's
+    xg = x.to(gpu).requires_grad_(True)
+    wg = wt.to(gpu).requires_grad_(True)
+    bg = shift.to(gpu).requires_grad_(True)
+    y = depthwise_conv2d_fused(xg, wg, bg, scale.to(gpu), "silu", s, p)
+    with torch.no_grad():
+        y_fused = depthwise_conv2d_fused(xg, wg, bg, scale.to(gpu), "silu", s, p)
+    assert _C.last_variant().startswith("small_down")
+    np.testing.assert_allclose(_np(y.detach()), _np(y_fused), rtol=1e-5, atol=1e-6)
+    gx, gw, gb = torch.autograd.grad(y, (xg, wg, bg), gy.to(gpu))
+    xr, wr, br = (t.double().requires_grad_(True) for t in (x, wt, shift))
+    yr = torch.nn.functional.silu(torch.nn.functional.conv2d(xr, wr, stride=s, padding=p, groups=c)
+                                  * scale.double().view(1, -1, 1, 1) + br.view(1, -1, 1, 1))
+    rx, rw, rb = torch.autograd.grad(yr, (xr, wr, br), gy.double())
+    np.testing.assert_allclose(_np(gx).astype(np.float64), rx.numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(_np(gw).astype(np.float64), rw.numpy(), rtol=1e-4, atol=1e-4 * float(rw.abs().max()))
+    np.testing.assert_allclose(_np(gb).astype(np.float64), rb.numpy(), rtol=1e-4, atol=1e-4 * float(rb.abs().max()))
+    # argument errors
+    with pytest.raises(ValueError, match="unknown activation"):
+        depthwise_conv2d_fused(xg, wg, activation="gelu")
+    with pytest.raises(RuntimeError, match="one entry per channel"):
+        with torch.no_grad():
+            depthwise_conv2d_fused(xg, wg, bias=torch.zeros(c + 1, device=gpu))
+    rc = _C._lib.dwconv2d_fused_f32(xg.data_ptr(), wg.data_ptr(), None, None, y_fused.data_ptr(), n, c, h, w, k, k,
+                                    s, s, p, p, 9, None)
+    assert rc == 1 and b"activation" in _C._lib.dwconv_last_error()
+

@@ -286,3 +286,22 @@ def test_golden_vectors_c_oracle_and_torch():
         np.testing.assert_allclose(_np(y_t), z[f"c{i}_y"], rtol=1e-12, atol=1e-12)
         np.testing.assert_allclose(_np(gx_t), z[f"c{i}_gx"], rtol=1e-12, atol=1e-12)
         np.testing.assert_allclose(_np(gw_t), z[f"c{i}_gw"], rtol=1e-12, atol=1e-11)
+
+
+def test_fused_reference_closed_forms():
+    """torch_reference_fused = torch's conv followed by torch's elementwise functions; pinned by numpy closed forms."""
+    g = torch.Generator("cpu").manual_seed(41)
+    x = torch.randn(2, 3, 9, 8, generator=g, dtype=torch.float64) * 3
+    w = torch.randn(3, 1, 3, 3, generator=g, dtype=torch.float64)
+    scale = torch.tensor([0.5, -2.0, 3.0], dtype=torch.float64)
+    shift = torch.tensor([1.0, 0.25, -4.0], dtype=torch.float64)
+    plain = oracle.torch_reference(x, w, None, 2, 1)[0].numpy()
+    assert np.array_equal(oracle.torch_reference_fused(x, w, None, None, None, 2, 1).numpy(), plain)
+    z = plain * scale.numpy().reshape(1, 3, 1, 1) + shift.numpy().reshape(1, 3, 1, 1)
+    np.testing.assert_allclose(oracle.torch_reference_fused(x, w, scale, shift, None, 2, 1).numpy(), z, rtol=1e-14)
+    np.testing.assert_allclose(oracle.torch_reference_fused(x, w, scale, shift, "relu", 2, 1).numpy(), np.maximum(z, 0), rtol=1e-14)
+    np.testing.assert_allclose(oracle.torch_reference_fused(x, w, scale, shift, "relu6", 2, 1).numpy(), np.clip(z, 0, 6), rtol=1e-14)
+    np.testing.assert_allclose(oracle.torch_reference_fused(x, w, scale, shift, "silu", 2, 1).numpy(), z / (1 + np.exp(-z)),
+                               rtol=1e-12, atol=1e-14)
+    assert (z < 0).any() and (z > 6).any()  # every branch of the activations is exercised
+
