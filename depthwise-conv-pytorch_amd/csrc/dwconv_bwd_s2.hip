@@ -1,4 +1,4 @@
-// Fused backward pass (grad-weight + grad-input) for stride-2 layers on large maps, fp32.
+// Fused backward pass (grad-weight + grad-input) for stride-2 layers on large maps (fp32, fp16 or bf16 tensors).
 //
 // Workgroup (channel c, chunk k) walks tiles (image n, band of rows).  Per tile two images are staged
 // in LDS: the band of x the grad-weight sums need, and the (four times smaller) band of gy.  A lane

@@ -1,4 +1,5 @@
-// Whole-plane fp32 kernels for small feature maps (width 7, 14 or 28, "same" padding).
+// Whole-plane kernels for small feature maps (width 7, 14 or 28, "same" padding); element type fp32, fp16 or
+// bf16, LDS and arithmetic fp32.
 //
 // Planes of a small map are tiny (196 B to 3 KiB) and sit back to back in memory,
 // so the only way to move them at HBM speed is to treat a run of P planes as one
@@ -17,7 +18,7 @@
 //
 //   small_down_kernel : up = 1, decimation S; forward, and grad-input of stride-1 layers (FLIP)
 //   small_up2_kernel  : up = 2, taps rotated; grad-input of stride-2 layers
-//   small_wgrad_kernel: grad-weight pass 1 (lane keeps its channel across the images of a chunk)
+// (grad-weight and the fused backward of these maps: dwconv_small_bwd.hip)
 #include "dwconv_small_common.hpp"
 
 namespace dwconv {

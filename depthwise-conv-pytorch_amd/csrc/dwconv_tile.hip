@@ -1,14 +1,15 @@
-// LDS-tiled fp32 kernels for the forward and grad-input passes.
+// LDS-tiled kernels for the forward and grad-input passes (element type fp32, fp16 or bf16; LDS and
+// arithmetic are fp32).
 //
 // Work decomposition (one workgroup of 256 lanes = 4 wavefronts per tile):
 //   tile  = P consecutive (n,c) planes x a band of output rows x the full width.
 //           Large maps use P = 1 and several row bands per plane; maps small
 //           enough use whole planes and P > 1, so a wavefront carries several
 //           channels.
-//   load  = the input band (with its halo rows) is fetched with 128-bit loads
-//           and scattered into an LDS image whose zero padding is materialised,
+//   load  = the input band (with its halo rows) is fetched four elements per
+//           load and scattered into an LDS image whose zero padding is materialised,
 //           so the arithmetic below needs no bounds checks.
-//   item  = a register block of BH x 4 outputs (8 wide for the stride-2
+//   item  = a register block of BH x 4 outputs (2*BQ x 4 for the stride-2
 //           transposed case) owned by one lane: per input row the lane reads
 //           aligned float4s from LDS once and reuses them for every tap and
 //           every output row that touches it.

@@ -1,4 +1,4 @@
-// fp32 grad-weight with LDS tiles and a fixed-order two-pass reduction.
+// Grad-weight with LDS tiles and a fixed-order two-pass reduction (fp32, fp16 or bf16 tensors; fp32 sums).
 //
 //   gw[c,i,j] = sum_{n,oy,ox} gy[n,c,oy,ox] * x[n,c, oy*S - pad_h + i, ox*S - pad_w + j]
 //
