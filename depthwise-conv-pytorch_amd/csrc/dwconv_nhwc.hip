@@ -45,56 +45,71 @@ struct NhwcPlan {
     int wgs;                 // forward / grad-input: workgroups in all (1-D grid)
 };
 
-template <typename IO, int CV>
-__device__ __forceinline__ void load_cv(const IO *p, float (&v)[CV])
+// ---- window loads through a buffer view ---------------------------------------------------------------------
+// The lanes of a workgroup read their windows through a raw buffer view that starts at the first image the
+// workgroup touches.  A load whose byte offset is at or beyond the view's extent returns zeros, so a tap that
+// falls outside the image costs no address clamp and no select: its row or column offset is replaced by kOob
+// once (per row / per block), and the saturating sum of the two stays out of range.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+constexpr unsigned kOob = 0x80000000u;  // extent of every view; the planner keeps real offsets below it
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t nhwc_view(const void *base)
 {
-    if constexpr (CV == 4) {
-        const float4 t = load4<IO>(p);
-        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-    } else if constexpr (CV == 2 && sizeof(IO) == 4) {
-        const float2 t = *reinterpret_cast<const float2 *>(p);
-        v[0] = t.x; v[1] = t.y;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, kOob, 0x00020000);
+}
+
+// CV consecutive channels at byte offset `off` of the view, widened to fp32.
+template <typename IO, int CV>
+__device__ __forceinline__ void view_load(__amdgpu_buffer_rsrc_t view, unsigned off, float (&v)[CV])
+{
+    if constexpr (CV * sizeof(IO) == 16) {
+        const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(view, off, 0, 0);
+        v[0] = __uint_as_float(t.x); v[1] = __uint_as_float(t.y); v[2] = __uint_as_float(t.z); v[3] = __uint_as_float(t.w);
+    } else if constexpr (CV * sizeof(IO) == 8) {
+        const u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(view, off, 0, 0);
+        if constexpr (sizeof(IO) == 4) {
+            v[0] = __uint_as_float(t.x); v[1] = __uint_as_float(t.y);
+        } else {
+            const float4 w = widen4<IO>(make_uint2(t.x, t.y));
+            v[0] = w.x; v[1] = w.y; v[2] = w.z; v[3] = w.w;
+        }
     } else {
-#pragma unroll
-        for (int i = 0; i < CV; ++i) v[i] = Io<IO>::in(p[i]);
+        static_assert(CV == 2 && sizeof(IO) == 2, "two 16-bit channels");
+        const unsigned t = __builtin_amdgcn_raw_buffer_load_b32(view, off, 0, 0);
+        const float4 w = widen4<IO>(make_uint2(t, 0u));
+        v[0] = w.x; v[1] = w.y;
     }
 }
 
-// Column part of a lane's window addresses, computed once per pixel block: element offset of each of the COLS
-// columns (clamped into the image) and one validity bit per column.
+// Column part of a lane's window offsets, computed once per pixel block: byte offset of this lane's channels
+// in each of the COLS columns (lane_off = image and channel part), kOob for columns outside the image.
 template <int COLS>
 struct NhwcCols {
-    int off[COLS];
-    unsigned ok;
+    unsigned off[COLS];
 };
 template <int COLS>
-__device__ __forceinline__ void nhwc_cols(int ix0, int in_w, int C, NhwcCols<COLS> &c)
+__device__ __forceinline__ void nhwc_cols(int ix0, int in_w, unsigned pixel_bytes, unsigned lane_off, NhwcCols<COLS> &c)
 {
-    c.ok = 0;
 #pragma unroll
     for (int j = 0; j < COLS; ++j) {
         const int ix = ix0 + j;
-        c.off[j] = min(max(ix, 0), in_w - 1) * C;
-        c.ok |= (static_cast<unsigned>(ix) < static_cast<unsigned>(in_w) ? 1u : 0u) << j;
+        c.off[j] = static_cast<unsigned>(ix) < static_cast<unsigned>(in_w) ? lane_off + ix * pixel_bytes : kOob;
     }
 }
 
-// One row of a lane's window: COLS pixels x CV channels of row iy.  `img` points at this lane's channels of
-// pixel (0,0) of its image; in-image offsets are 32-bit.  Pixels outside the image read a valid (clamped)
-// address and are zeroed afterwards.
+// One row of a lane's window: COLS pixels x CV channels of row iy (zeros outside the image).
 template <typename IO, int COLS, int CV = 4>
-__device__ __forceinline__ void nhwc_load_row(const IO *img, int iy, int in_h, int row_pitch, const NhwcCols<COLS> &cols,
-                                              float (&row)[COLS * CV])
+__device__ __forceinline__ void nhwc_load_row(__amdgpu_buffer_rsrc_t view, int iy, int in_h, unsigned row_bytes,
+                                              const NhwcCols<COLS> &cols, float (&row)[COLS * CV])
 {
-    const unsigned ok = static_cast<unsigned>(iy) < static_cast<unsigned>(in_h) ? cols.ok : 0u;
-    const int rbase = min(max(iy, 0), in_h - 1) * row_pitch;
+    const unsigned roff = static_cast<unsigned>(iy) < static_cast<unsigned>(in_h) ? iy * row_bytes : kOob;
 #pragma unroll
     for (int j = 0; j < COLS; ++j) {
         float t[CV];
-        load_cv<IO, CV>(img + (rbase + cols.off[j]), t);
-        const bool keep = (ok >> j) & 1u;
+        view_load<IO, CV>(view, __builtin_elementwise_add_sat(roff, cols.off[j]), t);
 #pragma unroll
-        for (int v = 0; v < CV; ++v) row[CV * j + v] = keep ? t[v] : 0.f;
+        for (int v = 0; v < CV; ++v) row[CV * j + v] = t[v];
     }
 }
 
@@ -137,8 +152,14 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_down_kernel(const NhwcPlan 
     const int oy0 = by * BH, ox0 = bx * TW;
     const int iy0 = oy0 * S - p.pad_h, ix0 = ox0 * S - p.pad_w;
     const int c = c0 + 4 * lane_c;
-    const IO *src = static_cast<const IO *>(p.in) + static_cast<long>(n) * p.in_h * p.in_w * C + c;
     const float *wl = lds + 4 * lane_c;
+    // view of the input from the first image this workgroup touches (uniform); this lane's image and channels
+    // are part of its column offsets
+    const int n0 = static_cast<int>(static_cast<long>(pg) * p.blocks_per_wg / per_image);
+    const unsigned pixel_bytes = C * sizeof(IO), row_bytes = p.in_w * pixel_bytes;
+    const __amdgpu_buffer_rsrc_t view =
+        nhwc_view(static_cast<const IO *>(p.in) + static_cast<long>(n0) * p.in_h * p.in_w * C);
+    const unsigned lane_off = (n - n0) * (p.in_h * row_bytes) + c * static_cast<unsigned>(sizeof(IO));
 
     float acc[BH][TW * 4];
 #pragma unroll
@@ -146,16 +167,16 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_down_kernel(const NhwcPlan 
 #pragma unroll
         for (int o = 0; o < TW * 4; ++o) acc[b][o] = 0.f;
 
-    // Rows are loaded one ahead of their use and the sums pinned after every row: otherwise the compiler
-    // hoists the loads of the whole window to the top and keeps all of it in registers.
-    float cur[COLS * 4], nxt[COLS * 4];
+    // Rows are loaded one ahead of their use (two row buffers, alternating) and the sums pinned after every
+    // row: otherwise the compiler hoists the loads of the whole window to the top and keeps all of it in registers.
+    float rows[2][COLS * 4];
     NhwcCols<COLS> cols;
-    nhwc_cols<COLS>(ix0, p.in_w, C, cols);
-    const int row_pitch = p.in_w * C;
-    nhwc_load_row<IO, COLS>(src, iy0, p.in_h, row_pitch, cols, cur);
+    nhwc_cols<COLS>(ix0, p.in_w, pixel_bytes, lane_off, cols);
+    nhwc_load_row<IO, COLS>(view, iy0, p.in_h, row_bytes, cols, rows[0]);
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
-        if (r + 1 < ROWS) nhwc_load_row<IO, COLS>(src, iy0 + r + 1, p.in_h, row_pitch, cols, nxt);
+        float(&cur)[COLS * 4] = rows[r & 1];
+        if (r + 1 < ROWS) nhwc_load_row<IO, COLS>(view, iy0 + r + 1, p.in_h, row_bytes, cols, rows[(r + 1) & 1]);
 #pragma unroll
         for (int b = 0; b < BH; ++b) {
             const int ty = r - b * S;
@@ -173,8 +194,6 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_down_kernel(const NhwcPlan 
             }
         }
         pin_registers(acc);
-#pragma unroll
-        for (int j = 0; j < COLS * 4; ++j) cur[j] = nxt[j];
     }
 
     if constexpr (!FLIP) {
@@ -231,8 +250,12 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_up2_kernel(const NhwcPlan p
     const int iy0 = by * BH, ix0 = bx * TW;
     const int gy0 = iy0 / 2 + p.pad_h + DMIN, gx0 = ix0 / 2 + p.pad_w + DMIN;
     const int c = c0 + 4 * lane_c;
-    const IO *src = static_cast<const IO *>(p.in) + static_cast<long>(n) * p.in_h * p.in_w * C + c;
     const float *wl = lds + 4 * lane_c;
+    const int n0 = static_cast<int>(static_cast<long>(pg) * p.blocks_per_wg / per_image);
+    const unsigned pixel_bytes = C * sizeof(IO), row_bytes = p.in_w * pixel_bytes;
+    const __amdgpu_buffer_rsrc_t view =
+        nhwc_view(static_cast<const IO *>(p.in) + static_cast<long>(n0) * p.in_h * p.in_w * C);
+    const unsigned lane_off = (n - n0) * (p.in_h * row_bytes) + c * static_cast<unsigned>(sizeof(IO));
 
     float acc[BH][TW * 4];
 #pragma unroll
@@ -240,14 +263,14 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_up2_kernel(const NhwcPlan p
 #pragma unroll
         for (int o = 0; o < TW * 4; ++o) acc[b][o] = 0.f;
 
-    float cur[GCOLS * 4], nxt[GCOLS * 4];
+    float rows[2][GCOLS * 4];
     NhwcCols<GCOLS> cols;
-    nhwc_cols<GCOLS>(gx0, p.in_w, C, cols);
-    const int row_pitch = p.in_w * C;
-    nhwc_load_row<IO, GCOLS>(src, gy0, p.in_h, row_pitch, cols, cur);
+    nhwc_cols<GCOLS>(gx0, p.in_w, pixel_bytes, lane_off, cols);
+    nhwc_load_row<IO, GCOLS>(view, gy0, p.in_h, row_bytes, cols, rows[0]);
 #pragma unroll
     for (int g = 0; g < GROWS; ++g) {
-        if (g + 1 < GROWS) nhwc_load_row<IO, GCOLS>(src, gy0 + g + 1, p.in_h, row_pitch, cols, nxt);
+        float(&cur)[GCOLS * 4] = rows[g & 1];
+        if (g + 1 < GROWS) nhwc_load_row<IO, GCOLS>(view, gy0 + g + 1, p.in_h, row_bytes, cols, rows[(g + 1) & 1]);
 #pragma unroll
         for (int b = 0; b < BH; ++b) {
             const int ty = b + PE - 2 * (DMIN + g);
@@ -267,8 +290,6 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_up2_kernel(const NhwcPlan p
             }
         }
         pin_registers(acc);
-#pragma unroll
-        for (int j = 0; j < GCOLS * 4; ++j) cur[j] = nxt[j];
     }
 
     IO *dst = static_cast<IO *>(p.out) + static_cast<long>(n) * p.out_h * p.out_w * C + c;
@@ -318,31 +339,30 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_wgrad_kernel(const NhwcPlan
         const int by = rem / p.blocks_x, bx = rem - by * p.blocks_x;
         const int oy0 = by * BH, ox0 = bx * TW;
         const int iy0 = oy0 * S - p.pad_h, ix0 = ox0 * S - p.pad_w;
-        const IO *xs = static_cast<const IO *>(p.in) + static_cast<long>(n) * p.in_h * p.in_w * C + c;
-        const IO *gs = static_cast<const IO *>(p.in2) + static_cast<long>(n) * p.out_h * p.out_w * C + c;
+        // views of x and gy from the first image of this group of pixel blocks (uniform)
+        const int n0 = static_cast<int>(grp * p.blocks_per_wg / per_image);
+        const unsigned pixel_bytes = C * sizeof(IO), row_bytes = p.in_w * pixel_bytes, grow_bytes = p.out_w * pixel_bytes;
+        const __amdgpu_buffer_rsrc_t xview =
+            nhwc_view(static_cast<const IO *>(p.in) + static_cast<long>(n0) * p.in_h * p.in_w * C);
+        const __amdgpu_buffer_rsrc_t gview =
+            nhwc_view(static_cast<const IO *>(p.in2) + static_cast<long>(n0) * p.out_h * p.out_w * C);
+        const unsigned chan_off = c * static_cast<unsigned>(sizeof(IO));
 
-        float g[BH][TW][CV];
+        float g[BH][TW * CV];
+        {
+            NhwcCols<TW> gcols;
+            nhwc_cols<TW>(ox0, p.out_w, pixel_bytes, (n - n0) * (p.out_h * grow_bytes) + chan_off, gcols);
 #pragma unroll
-        for (int b = 0; b < BH; ++b) {
-            const int oy = oy0 + b;
-#pragma unroll
-            for (int o = 0; o < TW; ++o) {
-                const int ox = ox0 + o;
-                const bool ok = oy < p.out_h && ox < p.out_w;
-                float t[CV];
-                load_cv<IO, CV>(gs + (min(oy, p.out_h - 1) * p.out_w + min(ox, p.out_w - 1)) * C, t);
-#pragma unroll
-                for (int v = 0; v < CV; ++v) g[b][o][v] = ok ? t[v] : 0.f;
-            }
+            for (int b = 0; b < BH; ++b) nhwc_load_row<IO, TW, CV>(gview, oy0 + b, p.out_h, grow_bytes, gcols, g[b]);
         }
-        float cur[COLS * CV], nxt[COLS * CV];
+        float rows[2][COLS * CV];
         NhwcCols<COLS> cols;
-        nhwc_cols<COLS>(ix0, p.in_w, C, cols);
-        const int row_pitch = p.in_w * C;
-        nhwc_load_row<IO, COLS, CV>(xs, iy0, p.in_h, row_pitch, cols, cur);
+        nhwc_cols<COLS>(ix0, p.in_w, pixel_bytes, (n - n0) * (p.in_h * row_bytes) + chan_off, cols);
+        nhwc_load_row<IO, COLS, CV>(xview, iy0, p.in_h, row_bytes, cols, rows[0]);
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) {
-            if (r + 1 < ROWS) nhwc_load_row<IO, COLS, CV>(xs, iy0 + r + 1, p.in_h, row_pitch, cols, nxt);
+            float(&cur)[COLS * CV] = rows[r & 1];
+            if (r + 1 < ROWS) nhwc_load_row<IO, COLS, CV>(xview, iy0 + r + 1, p.in_h, row_bytes, cols, rows[(r + 1) & 1]);
 #pragma unroll
             for (int b = 0; b < BH; ++b) {
                 const int ty = r - b * S;
@@ -353,11 +373,9 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_wgrad_kernel(const NhwcPlan
                     for (int o = 0; o < TW; ++o)
 #pragma unroll
                         for (int v = 0; v < CV; ++v)
-                            acc[ty * K + tx][v] = fmaf(g[b][o][v], cur[CV * (o * S + tx) + v], acc[ty * K + tx][v]);
+                            acc[ty * K + tx][v] = fmaf(g[b][CV * o + v], cur[CV * (o * S + tx) + v], acc[ty * K + tx][v]);
             }
             pin_registers(acc);
-#pragma unroll
-            for (int j = 0; j < COLS * CV; ++j) cur[j] = nxt[j];
         }
     }
 
@@ -557,6 +575,13 @@ bool plan_nhwc(NhwcPlan &p, const NhwcGeometry &g, int bh, int tw, int blocks_h,
     p.blocks_y = ceil_div(blocks_h, bh);
     p.blocks_x = ceil_div(blocks_w, tw);
     p.blocks_total = static_cast<long>(g.batch) * p.blocks_y * p.blocks_x;
+    // every view starts at the first image of a workgroup's pixel blocks and must reach its last one below kOob
+    {
+        const long per_image = static_cast<long>(p.blocks_y) * p.blocks_x;
+        const long span = (p.blocks_per_wg - 1) / per_image + 2;
+        const long image = std::max(static_cast<long>(g.in_h) * g.in_w, static_cast<long>(g.out_h) * g.out_w) * g.channel * 4;
+        if (image * span >= 0x80000000l) return false;
+    }
     p.cgroups = ceil_div(g.channel / CV, p.lanes_c);
     const long wgs = (p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg * p.cgroups;
     if (p.blocks_total <= 0 || p.cgroups > 65535 || wgs > 0x7fffffffL) return false;
@@ -573,10 +598,6 @@ bool nhwc_fast_ok(const NhwcGeometry &g)
     if (g.channel % 4 != 0) return false;
     if (g.pad_h < 0 || g.pad_w < 0 || g.pad_h >= K || g.pad_w >= K) return false;
     if (g.in_h < 1 || g.in_w < 1 || g.out_h < 1 || g.out_w < 1) return false;
-    // in-image element offsets are 32-bit
-    if (static_cast<long>(g.in_h) * g.in_w * g.channel >= (1l << 31) ||
-        static_cast<long>(g.out_h) * g.out_w * g.channel >= (1l << 31))
-        return false;
     return true;
 }
 
