@@ -45,43 +45,11 @@ struct NhwcPlan {
     int wgs;                 // forward / grad-input: workgroups in all (1-D grid)
 };
 
-// ---- window loads through a buffer view ---------------------------------------------------------------------
+// ---- window loads through a buffer view (nhwc_view / view_load, dwconv_tile_common.hpp) -----------------------
 // The lanes of a workgroup read their windows through a raw buffer view that starts at the first image the
-// workgroup touches.  A load whose byte offset is at or beyond the view's extent returns zeros, so a tap that
-// falls outside the image costs no address clamp and no select: its row or column offset is replaced by kOob
-// once (per row / per block), and the saturating sum of the two stays out of range.
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-constexpr unsigned kOob = 0x80000000u;  // extent of every view; the planner keeps real offsets below it
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t nhwc_view(const void *base)
-{
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, kOob, 0x00020000);
-}
-
-// CV consecutive channels at byte offset `off` of the view, widened to fp32.
-template <typename IO, int CV>
-__device__ __forceinline__ void view_load(__amdgpu_buffer_rsrc_t view, unsigned off, float (&v)[CV])
-{
-    if constexpr (CV * sizeof(IO) == 16) {
-        const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(view, off, 0, 0);
-        v[0] = __uint_as_float(t.x); v[1] = __uint_as_float(t.y); v[2] = __uint_as_float(t.z); v[3] = __uint_as_float(t.w);
-    } else if constexpr (CV * sizeof(IO) == 8) {
-        const u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(view, off, 0, 0);
-        if constexpr (sizeof(IO) == 4) {
-            v[0] = __uint_as_float(t.x); v[1] = __uint_as_float(t.y);
-        } else {
-            const float4 w = widen4<IO>(make_uint2(t.x, t.y));
-            v[0] = w.x; v[1] = w.y; v[2] = w.z; v[3] = w.w;
-        }
-    } else {
-        static_assert(CV == 2 && sizeof(IO) == 2, "two 16-bit channels");
-        const unsigned t = __builtin_amdgcn_raw_buffer_load_b32(view, off, 0, 0);
-        const float4 w = widen4<IO>(make_uint2(t, 0u));
-        v[0] = w.x; v[1] = w.y;
-    }
-}
-
+// workgroup touches.  A tap that falls outside the image costs no address clamp and no select: its row or
+// column offset is replaced by kOob once (per row / per block), and the saturating sum of the two stays out
+// of range, where loads return zeros.
 // Column part of a lane's window offsets, computed once per pixel block: byte offset of this lane's channels
 // in each of the COLS columns (lane_off = image and channel part), kOob for columns outside the image.
 template <int COLS>
@@ -158,7 +126,7 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_down_kernel(const NhwcPlan 
     const int n0 = static_cast<int>(static_cast<long>(pg) * p.blocks_per_wg / per_image);
     const unsigned pixel_bytes = C * sizeof(IO), row_bytes = p.in_w * pixel_bytes;
     const __amdgpu_buffer_rsrc_t view =
-        nhwc_view(static_cast<const IO *>(p.in) + static_cast<long>(n0) * p.in_h * p.in_w * C);
+        buffer_view(static_cast<const IO *>(p.in) + static_cast<long>(n0) * p.in_h * p.in_w * C);
     const unsigned lane_off = (n - n0) * (p.in_h * row_bytes) + c * static_cast<unsigned>(sizeof(IO));
 
     float acc[BH][TW * 4];
@@ -254,7 +222,7 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_up2_kernel(const NhwcPlan p
     const int n0 = static_cast<int>(static_cast<long>(pg) * p.blocks_per_wg / per_image);
     const unsigned pixel_bytes = C * sizeof(IO), row_bytes = p.in_w * pixel_bytes;
     const __amdgpu_buffer_rsrc_t view =
-        nhwc_view(static_cast<const IO *>(p.in) + static_cast<long>(n0) * p.in_h * p.in_w * C);
+        buffer_view(static_cast<const IO *>(p.in) + static_cast<long>(n0) * p.in_h * p.in_w * C);
     const unsigned lane_off = (n - n0) * (p.in_h * row_bytes) + c * static_cast<unsigned>(sizeof(IO));
 
     float acc[BH][TW * 4];
@@ -343,9 +311,9 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_wgrad_kernel(const NhwcPlan
         const int n0 = static_cast<int>(grp * p.blocks_per_wg / per_image);
         const unsigned pixel_bytes = C * sizeof(IO), row_bytes = p.in_w * pixel_bytes, grow_bytes = p.out_w * pixel_bytes;
         const __amdgpu_buffer_rsrc_t xview =
-            nhwc_view(static_cast<const IO *>(p.in) + static_cast<long>(n0) * p.in_h * p.in_w * C);
+            buffer_view(static_cast<const IO *>(p.in) + static_cast<long>(n0) * p.in_h * p.in_w * C);
         const __amdgpu_buffer_rsrc_t gview =
-            nhwc_view(static_cast<const IO *>(p.in2) + static_cast<long>(n0) * p.out_h * p.out_w * C);
+            buffer_view(static_cast<const IO *>(p.in2) + static_cast<long>(n0) * p.out_h * p.out_w * C);
         const unsigned chan_off = c * static_cast<unsigned>(sizeof(IO));
 
         float g[BH][TW * CV];

@@ -306,6 +306,7 @@ int launch_down(TilePlan &p, hipStream_t stream)
     const int used_cols = 4 * (p.ncb - 1) * S + 4 * NV;
     auto rows_for = [](int units) { return (units * BH - 1) * S + K; };
     if (!plan_tiles(p, ceil_div(p.out_h, BH), BH, used_cols, K * K, rows_for)) return -1;
+    if (p.st.vec_in) p.st.vec_in = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
     hipLaunchKernelGGL((fir_down_kernel<IO, K, S, FLIP, BH>), dim3(p.n_tiles), dim3(env_int("DWCONV_TILE_THREADS", kThreads)), lds_bytes(p, K * K),
                        stream, p);
     note_variant("tile_down%s<k%d,s%d,%s,bh%d> P%d rows%d vin%d vout%d", sizeof(IO) == 2 ? "16" : "", K, S, FLIP ? "rot" : "fwd", BH,
@@ -331,6 +332,7 @@ int launch_up2(TilePlan &p, hipStream_t stream)
     const int used_cols = 2 * (p.ncb - 1) + NW;
     auto rows_for = [](int units) { return units * BQ + KAY; };
     if (!plan_tiles(p, ceil_div(ceil_div(p.out_h, 2), BQ), BQ, used_cols, K * K, rows_for)) return -1;
+    if (p.st.vec_in) p.st.vec_in = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
     hipLaunchKernelGGL((fir_up2_kernel<IO, K, EY, EX, BQ>), dim3(p.n_tiles), dim3(env_int("DWCONV_TILE_THREADS", kThreads)), lds_bytes(p, K * K), stream,
                        p);
     note_variant("tile_up2%s<k%d,e%d%d,bq%d> P%d rows%d vin%d vout%d", sizeof(IO) == 2 ? "16" : "", K, EY, EX, BQ, p.planes_per_tile,

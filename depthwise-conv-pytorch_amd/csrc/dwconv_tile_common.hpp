@@ -26,7 +26,8 @@ struct StageLayout {
     unsigned spr_magic;
     int pitch;        // floats per LDS row, slack included
     int plane_pitch;  // floats per plane image
-    int vec_in;       // four elements may be loaded at once (in_w % 4 == 0, base aligned to four elements)
+    int vec_in;       // 0: element loads; 1: four elements per load (in_w % 4 == 0, base aligned to four elements);
+                      // 2: the same through a buffer view (the tile's planes span less than kOob bytes)
 };
 
 // Four consecutive elements (aligned to four elements) as fp32, and back.
@@ -121,6 +122,49 @@ __device__ __forceinline__ float4 widen4<bf16_t>(const uint2 &raw)
                        __uint_as_float(raw.y & 0xffff0000u));
 }
 
+// ---- loads through a buffer view ------------------------------------------------------------------------------
+// A raw buffer view of kOob bytes from `base` (uniform).  A load whose byte offset is at or beyond kOob returns
+// zeros, so an element outside the image needs no branch and no select: its offset is replaced by kOob.  The
+// planners keep every real offset below kOob.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+constexpr unsigned kOob = 0x80000000u;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_view(const void *base)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, kOob, 0x00020000);
+}
+
+// CV consecutive elements at byte offset `off` of the view, widened to fp32.
+template <typename IO, int CV>
+__device__ __forceinline__ void view_load(__amdgpu_buffer_rsrc_t view, unsigned off, float (&v)[CV])
+{
+    if constexpr (CV * sizeof(IO) == 16) {
+        const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(view, off, 0, 0);
+        v[0] = __uint_as_float(t.x); v[1] = __uint_as_float(t.y); v[2] = __uint_as_float(t.z); v[3] = __uint_as_float(t.w);
+    } else if constexpr (CV * sizeof(IO) == 8) {
+        const u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(view, off, 0, 0);
+        if constexpr (sizeof(IO) == 4) {
+            v[0] = __uint_as_float(t.x); v[1] = __uint_as_float(t.y);
+        } else {
+            const float4 w = widen4<IO>(make_uint2(t.x, t.y));
+            v[0] = w.x; v[1] = w.y; v[2] = w.z; v[3] = w.w;
+        }
+    } else {
+        static_assert(CV == 2 && sizeof(IO) == 2, "two 16-bit elements");
+        const unsigned t = __builtin_amdgcn_raw_buffer_load_b32(view, off, 0, 0);
+        const float4 w = widen4<IO>(make_uint2(t, 0u));
+        v[0] = w.x; v[1] = w.y;
+    }
+}
+template <typename IO>
+__device__ __forceinline__ float4 view_load4(__amdgpu_buffer_rsrc_t view, unsigned off)
+{
+    float v[4];
+    view_load<IO, 4>(view, off, v);
+    return make_float4(v[0], v[1], v[2], v[3]);
+}
+
 // True when groups of four elements starting at `p` may be moved with one vector access.
 template <typename IO>
 inline bool aligned4(const IO *p)
@@ -155,6 +199,41 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__res
                                            long plane0, int nplanes, int iy0)
 {
     const int total = nplanes * s.lds_rows * s.spr;
+    if (s.vec_in == 2) {
+        // groups of four elements through a view of the tile's planes: slots outside the image read zeros
+        const __amdgpu_buffer_rsrc_t view = buffer_view(in + plane0 * s.in_plane);
+        for (int base = threadIdx.x; base < total; base += blockDim.x * kStageBatch) {
+            float4 v[kStageBatch];
+            int dst[kStageBatch];
+#pragma unroll
+            for (int u = 0; u < kStageBatch; ++u) {
+                const int slot = min(base + u * static_cast<int>(blockDim.x), total - 1);
+                const int rowidx = fast_div(slot, s.spr_magic);
+                const int sc = slot - rowidx * s.spr;
+                const int pl = fast_div(rowidx, s.lds_rows_magic);
+                const int r = rowidx - pl * s.lds_rows;
+                const int ix = 4 * (s.g_lo + sc);
+                const int iy = iy0 + r;
+                const bool ok = static_cast<unsigned>(iy) < static_cast<unsigned>(s.in_h) &&
+                                static_cast<unsigned>(ix) < static_cast<unsigned>(s.in_w);
+                const unsigned off = (pl * s.in_plane + iy * s.in_w + ix) * static_cast<unsigned>(sizeof(IO));
+                v[u] = view_load4<IO>(view, ok ? off : kOob);
+                dst[u] = pl * s.plane_pitch + r * s.pitch + kSlack + ix + s.col_shift;
+            }
+#pragma unroll
+            for (int u = 0; u < kStageBatch; ++u) {
+                const float4 t = v[u];  // read outside the condition: a conditional copy keeps the array out of registers
+                if (base + u * static_cast<int>(blockDim.x) < total) {
+                    float *d = lds + dst[u];
+                    d[0] = t.x;
+                    d[1] = t.y;
+                    d[2] = t.z;
+                    d[3] = t.w;
+                }
+            }
+        }
+        return;
+    }
     for (int base = threadIdx.x; base < total; base += blockDim.x * kStageBatch) {
         float4 v[kStageBatch];
         int dst[kStageBatch];
@@ -221,6 +300,24 @@ __device__ __forceinline__ void stage_fetch(const StageLayout &s, const IO *__re
                                             int nplanes, int iy0, StagedTile<U> &t)
 {
     const int total = nplanes * s.lds_rows * s.spr;
+    if (s.vec_in == 2) {
+        const __amdgpu_buffer_rsrc_t view = buffer_view(in + plane0 * s.in_plane);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int slot = threadIdx.x + u * blockDim.x;
+            const int rowidx = fast_div(slot, s.spr_magic);
+            const int sc = slot - rowidx * s.spr;
+            const int pl = fast_div(rowidx, s.lds_rows_magic);
+            const int r = rowidx - pl * s.lds_rows;
+            const int ix = 4 * (s.g_lo + sc);
+            const int iy = iy0 + r;
+            const bool ok = slot < total && static_cast<unsigned>(iy) < static_cast<unsigned>(s.in_h) &&
+                            static_cast<unsigned>(ix) < static_cast<unsigned>(s.in_w);
+            const unsigned off = (pl * s.in_plane + iy * s.in_w + ix) * static_cast<unsigned>(sizeof(IO));
+            t.v[u] = view_load4<IO>(view, ok ? off : kOob);
+        }
+        return;
+    }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const int slot = threadIdx.x + u * blockDim.x;
@@ -323,6 +420,13 @@ inline int env_int(const char *name, int dflt)
     const char *e = std::getenv(name);
     if (e == nullptr || e[0] == '\0') return dflt;
     return std::atoi(e);
+}
+
+// vec_in for a tile of `planes` planes of `in_plane` elements of `esize` bytes whose rows allow vector loads.
+inline int vector_mode(long planes, long in_plane, size_t esize)
+{
+    const bool fits = planes * in_plane * static_cast<long>(esize) < static_cast<long>(kOob);
+    return fits && env_int("DWCONV_STAGE_VIEW", 1) ? 2 : 1;
 }
 
 // Row pitch and float4 slots of an image `used_cols` floats wide (col_shift must be set).

@@ -475,10 +475,10 @@ struct Launcher {
         // prefetching costs ~35 registers: worth it for the 3x3 kernels, whose tiles also fit the slots
         const bool pf = K == 3 && env_int("DWCONV_PREFETCH", 1) &&
                         p.planes_per_tile * p.st.lds_rows * p.st.spr <= kPrefetchSlots * kThreads;
+        if (fused) p.st.vec_in = p.st.vec_in && aligned4(gy);  // gy is staged with the x image's layout
+        if (p.st.vec_in) p.st.vec_in = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
         if constexpr (S == 1) {
             if (fused) {
-                // the gy image is staged with the x image's layout: it needs the same 128-bit rule
-                p.st.vec_in = p.st.vec_in && aligned4(gy);
                 if constexpr (K == 3) {
                     if (pf) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, true, true>), grid, block, shmem, stream, p);
                 }
