@@ -100,12 +100,18 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
 
     StagedTile<PF ? kUx : 1> tx;
     StagedTile<PF ? kUg : 1> tg;
+    StageSlots<PF ? kUx : 1> qx;
+    StageSlots<PF ? kUg : 1> qg;
+    if constexpr (PF) {
+        stage_slots<kUx, IO>(p.sx, 1, qx);
+        stage_slots<kUg, IO>(p.sg, 1, qg);
+    }
     if constexpr (PF) {
         if (chunk < p.tiles_per_group) {
         const int n = chunk / p.row_tiles, rt = chunk - n * p.row_tiles;
         const long plane0 = static_cast<long>(n) * p.channel + c;
-        stage_fetch(p.sx, x, plane0, 1, 2 * rt * p.rows_per_tile - p.pad, tx);
-        stage_fetch(p.sg, gy, plane0, 1, rt * p.rows_per_tile - p.m, tg);
+        stage_fetch(p.sx, x, plane0, 1, 2 * rt * p.rows_per_tile - p.pad, qx, tx);
+        stage_fetch(p.sg, gy, plane0, 1, rt * p.rows_per_tile - p.m, qg, tg);
         }
     }
 
@@ -116,8 +122,8 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
 
         if (tile != chunk) __syncthreads();  // the previous tile's window reads are done
         if constexpr (PF) {
-            stage_commit(p.sx, lds, 1, tx);
-            stage_commit(p.sg, lds + p.g_base, 1, tg);
+            stage_commit(lds, qx, tx);
+            stage_commit(lds + p.g_base, qg, tg);
         } else {
             stage_tile(p.sx, x, lds, plane0, 1, 2 * q0 - p.pad);
             stage_tile(p.sg, gy, lds + p.g_base, plane0, 1, q0 - p.m);
@@ -129,8 +135,8 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
             const int t1 = tile + p.chunks;
             const int n1 = t1 / p.row_tiles, rt1 = t1 - n1 * p.row_tiles;
             const long plane1 = static_cast<long>(n1) * p.channel + c;
-            stage_fetch(p.sx, x, plane1, 1, 2 * rt1 * p.rows_per_tile - p.pad, tx);
-            stage_fetch(p.sg, gy, plane1, 1, rt1 * p.rows_per_tile - p.m, tg);
+            stage_fetch(p.sx, x, plane1, 1, 2 * rt1 * p.rows_per_tile - p.pad, qx, tx);
+            stage_fetch(p.sg, gy, plane1, 1, rt1 * p.rows_per_tile - p.m, qg, tg);
           }
         }
 

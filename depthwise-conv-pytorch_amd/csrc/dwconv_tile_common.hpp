@@ -284,37 +284,47 @@ struct StagedTile {
     float4 v[U];
 };
 
-// LDS offset (floats) of slot `slot` of the image, or -1 past its end; tile-independent.
-__device__ __forceinline__ int stage_slot_offset(const StageLayout &s, int slot, int nplanes)
+// What does not change from tile to tile for the U slots of a lane: the row of the slot within the tile's
+// rows, its byte offset from the tile's first row, and its place in LDS.  Kernels that walk many tiles compute
+// this once, so that fetching a tile costs four instructions per slot.
+template <int U>
+struct StageSlots {
+    int r[U];          // row within the tile's rows; a hugely negative row for slots that always read zeros
+    unsigned off[U];   // ((plane * in_plane + r * in_w + column) * element size
+    int lds[U];        // float offset in the LDS image, -1 past the end of the image
+};
+
+template <int U, typename IO>
+__device__ __forceinline__ void stage_slots(const StageLayout &s, int nplanes, StageSlots<U> &q)
 {
-    if (slot >= nplanes * s.lds_rows * s.spr) return -1;
-    const int rowidx = fast_div(slot, s.spr_magic);
-    const int sc = slot - rowidx * s.spr;
-    const int pl = fast_div(rowidx, s.lds_rows_magic);
-    const int r = rowidx - pl * s.lds_rows;
-    return pl * s.plane_pitch + r * s.pitch + kSlack + 4 * (s.g_lo + sc) + s.col_shift;
+    const int total = nplanes * s.lds_rows * s.spr;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int slot = threadIdx.x + u * blockDim.x;
+        const int rowidx = fast_div(slot, s.spr_magic);
+        const int sc = slot - rowidx * s.spr;
+        const int pl = fast_div(rowidx, s.lds_rows_magic);
+        const int r = rowidx - pl * s.lds_rows;
+        const int ix = 4 * (s.g_lo + sc);
+        const bool reads = slot < total && static_cast<unsigned>(ix) < static_cast<unsigned>(s.in_w);
+        q.r[u] = reads ? r : -(1 << 30);
+        q.off[u] = (pl * s.in_plane + r * s.in_w + ix) * static_cast<unsigned>(sizeof(IO));
+        q.lds[u] = slot < total ? pl * s.plane_pitch + r * s.pitch + kSlack + ix + s.col_shift : -1;
+    }
 }
 
 template <int U, typename IO>
 __device__ __forceinline__ void stage_fetch(const StageLayout &s, const IO *__restrict__ in, long plane0,
-                                            int nplanes, int iy0, StagedTile<U> &t)
+                                            int nplanes, int iy0, const StageSlots<U> &q, StagedTile<U> &t)
 {
     const int total = nplanes * s.lds_rows * s.spr;
     if (s.vec_in == 2) {
         const __amdgpu_buffer_rsrc_t view = buffer_view(in + plane0 * s.in_plane);
+        const unsigned row_base = static_cast<unsigned>(iy0 * s.in_w) * static_cast<unsigned>(sizeof(IO));  // uniform
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int slot = threadIdx.x + u * blockDim.x;
-            const int rowidx = fast_div(slot, s.spr_magic);
-            const int sc = slot - rowidx * s.spr;
-            const int pl = fast_div(rowidx, s.lds_rows_magic);
-            const int r = rowidx - pl * s.lds_rows;
-            const int ix = 4 * (s.g_lo + sc);
-            const int iy = iy0 + r;
-            const bool ok = slot < total && static_cast<unsigned>(iy) < static_cast<unsigned>(s.in_h) &&
-                            static_cast<unsigned>(ix) < static_cast<unsigned>(s.in_w);
-            const unsigned off = (pl * s.in_plane + iy * s.in_w + ix) * static_cast<unsigned>(sizeof(IO));
-            t.v[u] = view_load4<IO>(view, ok ? off : kOob);
+            const bool ok = static_cast<unsigned>(iy0 + q.r[u]) < static_cast<unsigned>(s.in_h);
+            t.v[u] = view_load4<IO>(view, ok ? q.off[u] + row_base : kOob);
         }
         return;
     }
@@ -345,12 +355,12 @@ __device__ __forceinline__ void stage_fetch(const StageLayout &s, const IO *__re
 }
 
 template <int U>
-__device__ __forceinline__ void stage_commit(const StageLayout &s, float *lds, int nplanes, const StagedTile<U> &t)
+__device__ __forceinline__ void stage_commit(float *lds, const StageSlots<U> &q, const StagedTile<U> &t)
 {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const float4 v = t.v[u];
-        const int d = stage_slot_offset(s, threadIdx.x + u * blockDim.x, nplanes);
+        const int d = q.lds[u];
         if (d >= 0) {
             float *dst = lds + d;
             dst[0] = v.x;

@@ -121,12 +121,14 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
     }
 
     StagedTile<PF ? kPrefetchSlots : 1> tx, tg;
+    StageSlots<PF ? kPrefetchSlots : 1> slots;  // x and gy bands share one layout
+    if constexpr (PF) stage_slots<kPrefetchSlots, IO>(p.st, nplanes, slots);
     if constexpr (PF) {
         if (t_begin < t_end) {
             const int n = t_begin / p.row_tiles, rt = t_begin - n * p.row_tiles;
             const long plane0 = static_cast<long>(n) * p.channel + c0;
-            stage_fetch(p.st, x, plane0, nplanes, rt * p.rows_per_tile * S - p.pad_h, tx);
-            if constexpr (GX) stage_fetch(p.st, gy, plane0, nplanes, rt * p.rows_per_tile - p.pad_h, tg);
+            stage_fetch(p.st, x, plane0, nplanes, rt * p.rows_per_tile * S - p.pad_h, slots, tx);
+            if constexpr (GX) stage_fetch(p.st, gy, plane0, nplanes, rt * p.rows_per_tile - p.pad_h, slots, tg);
         }
     }
 
@@ -163,8 +165,8 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
 
         if (tile != t_begin) __syncthreads();  // the previous tile's window reads are done
         if constexpr (PF) {
-            stage_commit(p.st, lds, nplanes, tx);
-            if constexpr (GX) stage_commit(p.st, lds + p.g_base, nplanes, tg);
+            stage_commit(lds, slots, tx);
+            if constexpr (GX) stage_commit(lds + p.g_base, slots, tg);
         } else {
             stage_tile(p.st, x, lds, plane0, nplanes, oy0 * S - p.pad_h);
             if constexpr (GX) stage_tile(p.st, gy, lds + p.g_base, plane0, nplanes, oy0 - p.pad_h);
@@ -175,8 +177,8 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
                 const int t1 = tile + t_step;
                 const int n1 = t1 / p.row_tiles, rt1 = t1 - n1 * p.row_tiles;
                 const long plane1 = static_cast<long>(n1) * p.channel + c0;
-                stage_fetch(p.st, x, plane1, nplanes, rt1 * p.rows_per_tile * S - p.pad_h, tx);
-                if constexpr (GX) stage_fetch(p.st, gy, plane1, nplanes, rt1 * p.rows_per_tile - p.pad_h, tg);
+                stage_fetch(p.st, x, plane1, nplanes, rt1 * p.rows_per_tile * S - p.pad_h, slots, tx);
+                if constexpr (GX) stage_fetch(p.st, gy, plane1, nplanes, rt1 * p.rows_per_tile - p.pad_h, slots, tg);
             }
         }
 
