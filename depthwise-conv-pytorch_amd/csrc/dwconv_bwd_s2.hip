@@ -186,7 +186,19 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
                 }
             pin_registers(xacc);
         }
-        if (has_item) {
+        if (p.vec_gx == 2) {
+            // branch-free: rows and column blocks past the end of the plane store out of range
+            const int ox = 4 * cb;
+            const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.gx) + plane0 * p.sx.in_plane);
+            const bool col_ok = has_item && ox < p.sx.in_w;
+#pragma unroll
+            for (int b = 0; b < 2 * BQ; ++b) {
+                const int oy = 2 * (q0 + rb * BQ) + b;
+                const bool ok = col_ok && oy < p.sx.in_h;
+                view_store4<IO>(view, ok ? (oy * p.sx.in_w + ox) * static_cast<unsigned>(sizeof(IO)) : kOob, xacc[b][0],
+                                xacc[b][1], xacc[b][2], xacc[b][3]);
+            }
+        } else if (has_item) {
             const int ox = 4 * cb;
             IO *dst = static_cast<IO *>(p.gx) + plane0 * p.sx.in_plane + ox;
 #pragma unroll
@@ -322,6 +334,7 @@ long bwd_s2_case(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO
     p.vec_gx = (g.in_w % 4 == 0) && aligned4(gx);
     if (p.sx.vec_in) p.sx.vec_in = vector_mode(1, p.sx.in_plane, sizeof(IO));
     if (p.sg.vec_in) p.sg.vec_in = vector_mode(1, p.sg.in_plane, sizeof(IO));
+    if (p.vec_gx) p.vec_gx = vector_mode(1, p.sx.in_plane, sizeof(IO));
     // all 256 lanes stage the images even when the tile has fewer items than that
     const int threads = kThreads;
     p.prefetch = bq == 4 && K == 3 && env_int("DWCONV_PREFETCH", 1) && p.sx.lds_rows * p.sx.spr <= kUx * threads &&

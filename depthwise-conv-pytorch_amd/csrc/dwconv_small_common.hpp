@@ -101,13 +101,17 @@ __device__ __forceinline__ void lds_to_run(IO *__restrict__ g, const float *lds,
 {
     const int n4 = n >> 2;
     constexpr int U = 4;
+    const __amdgpu_buffer_rsrc_t view = buffer_view(g);  // g is uniform: one run per wavefront
     for (int base = threadIdx.x; base < n4; base += kWave * U) {
         float4 v[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) v[u] = reinterpret_cast<const float4 *>(lds)[min(base + u * kWave, n4 - 1)];
+        // branch-free: groups past the end of the run store out of range of the view and are dropped
 #pragma unroll
-        for (int u = 0; u < U; ++u)
-            if (base + u * kWave < n4) store4<IO>(g + 4 * (base + u * kWave), v[u].x, v[u].y, v[u].z, v[u].w);
+        for (int u = 0; u < U; ++u) {
+            const int i = base + u * kWave;
+            view_store4<IO>(view, i < n4 ? i * 4u * static_cast<unsigned>(sizeof(IO)) : kOob, v[u].x, v[u].y, v[u].z, v[u].w);
+        }
     }
     const int tail = n4 * 4 + threadIdx.x;
     if (tail < n) g[tail] = Io<IO>::out(lds[tail]);

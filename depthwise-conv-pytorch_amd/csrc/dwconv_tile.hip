@@ -127,6 +127,18 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
             }
         }
         const int ox = 4 * cb;
+        if (p.vec_out == 2) {
+            // branch-free: rows past the end of the plane store out of range
+            const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane);
+            const unsigned o0 = (pl * p.out_plane + ox) * static_cast<unsigned>(sizeof(IO));
+#pragma unroll
+            for (int b = 0; b < BH; ++b) {
+                const int oy = oy0 + rb * BH + b;
+                view_store4<IO>(view, oy < p.out_h ? o0 + oy * p.out_w * static_cast<unsigned>(sizeof(IO)) : kOob, acc[b][0],
+                                acc[b][1], acc[b][2], acc[b][3]);
+            }
+            continue;
+        }
         IO *dst = static_cast<IO *>(p.out) + (plane0 + pl) * p.out_plane + ox;
 #pragma unroll
         for (int b = 0; b < BH; ++b) {
@@ -307,6 +319,7 @@ int launch_down(TilePlan &p, hipStream_t stream)
     auto rows_for = [](int units) { return (units * BH - 1) * S + K; };
     if (!plan_tiles(p, ceil_div(p.out_h, BH), BH, used_cols, K * K, rows_for)) return -1;
     if (p.st.vec_in) p.st.vec_in = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
+    if (p.vec_out) p.vec_out = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
     hipLaunchKernelGGL((fir_down_kernel<IO, K, S, FLIP, BH>), dim3(p.n_tiles), dim3(env_int("DWCONV_TILE_THREADS", kThreads)), lds_bytes(p, K * K),
                        stream, p);
     note_variant("tile_down%s<k%d,s%d,%s,bh%d> P%d rows%d vin%d vout%d", sizeof(IO) == 2 ? "16" : "", K, S, FLIP ? "rot" : "fwd", BH,

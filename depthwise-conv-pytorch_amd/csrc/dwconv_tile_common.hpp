@@ -165,6 +165,21 @@ __device__ __forceinline__ float4 view_load4(__amdgpu_buffer_rsrc_t view, unsign
     return make_float4(v[0], v[1], v[2], v[3]);
 }
 
+// Four results as elements at byte offset `off` of the view; dropped when `off` is at or beyond kOob.
+template <typename IO>
+__device__ __forceinline__ void view_store4(__amdgpu_buffer_rsrc_t view, unsigned off, float a, float b, float c, float d)
+{
+    if constexpr (sizeof(IO) == 4) {
+        u32x4 t;
+        t.x = __float_as_uint(a); t.y = __float_as_uint(b); t.z = __float_as_uint(c); t.w = __float_as_uint(d);
+        __builtin_amdgcn_raw_buffer_store_b128(t, view, off, 0, 0);
+    } else {
+        union { IO e[4]; u32x2 u; } t;
+        t.e[0] = Io<IO>::out(a); t.e[1] = Io<IO>::out(b); t.e[2] = Io<IO>::out(c); t.e[3] = Io<IO>::out(d);
+        __builtin_amdgcn_raw_buffer_store_b64(t.u, view, off, 0, 0);
+    }
+}
+
 // True when groups of four elements starting at `p` may be moved with one vector access.
 template <typename IO>
 inline bool aligned4(const IO *p)

@@ -213,7 +213,18 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
                 }
                 pin_registers(xacc);
             }
-            if (has_item) {
+            if (p.vec_gx == 2) {
+                // branch-free: rows past the end of the plane (and lanes without an item) store out of range
+                const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.gx) + plane0 * p.st.in_plane);
+                const unsigned o0 = (pl * p.st.in_plane + ox) * static_cast<unsigned>(sizeof(IO));
+#pragma unroll
+                for (int b = 0; b < BH; ++b) {
+                    const int oy = oy0 + rb * BH + b;
+                    const bool ok = has_item && oy < p.st.in_h;
+                    view_store4<IO>(view, ok ? o0 + oy * p.st.in_w * static_cast<unsigned>(sizeof(IO)) : kOob, xacc[b][0],
+                                    xacc[b][1], xacc[b][2], xacc[b][3]);
+                }
+            } else if (has_item) {
                 IO *dst = static_cast<IO *>(p.gx) + (plane0 + pl) * p.st.in_plane + ox;
 #pragma unroll
                 for (int b = 0; b < BH; ++b) {
@@ -479,6 +490,7 @@ struct Launcher {
                         p.planes_per_tile * p.st.lds_rows * p.st.spr <= kPrefetchSlots * kThreads;
         if (fused) p.st.vec_in = p.st.vec_in && aligned4(gy);  // gy is staged with the x image's layout
         if (p.st.vec_in) p.st.vec_in = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
+        if (p.vec_gx) p.vec_gx = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
         if constexpr (S == 1) {
             if (fused) {
                 if constexpr (K == 3) {
