@@ -167,18 +167,20 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_down_kernel(const NhwcPlan 
     if constexpr (!FLIP) {
         if (p.epi.enabled()) epilogue_apply_block<4>(acc, p.epi, c);
     }
-    IO *dst = static_cast<IO *>(p.out) + static_cast<long>(n) * p.out_h * p.out_w * C + c;
+    // branch-free stores through a view of the output: pixels past the edge of the image store out of range
+    const unsigned out_row_bytes = p.out_w * pixel_bytes;
+    const __amdgpu_buffer_rsrc_t out_view =
+        buffer_view(static_cast<IO *>(p.out) + static_cast<long>(n0) * p.out_h * p.out_w * C);
+    NhwcCols<TW> ocols;
+    nhwc_cols<TW>(ox0, p.out_w, pixel_bytes, (n - n0) * (p.out_h * out_row_bytes) + c * static_cast<unsigned>(sizeof(IO)), ocols);
 #pragma unroll
     for (int b = 0; b < BH; ++b) {
         const int oy = oy0 + b;
-        if (oy >= p.out_h) continue;
+        const unsigned roff = oy < p.out_h ? oy * out_row_bytes : kOob;
 #pragma unroll
-        for (int o = 0; o < TW; ++o) {
-            const int ox = ox0 + o;
-            if (ox < p.out_w)
-                store4<IO>(dst + (static_cast<long>(oy) * p.out_w + ox) * C, acc[b][4 * o], acc[b][4 * o + 1],
-                           acc[b][4 * o + 2], acc[b][4 * o + 3]);
-        }
+        for (int o = 0; o < TW; ++o)
+            view_store4<IO>(out_view, __builtin_elementwise_add_sat(roff, ocols.off[o]), acc[b][4 * o], acc[b][4 * o + 1],
+                            acc[b][4 * o + 2], acc[b][4 * o + 3]);
     }
 }
 
@@ -260,18 +262,19 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_up2_kernel(const NhwcPlan p
         pin_registers(acc);
     }
 
-    IO *dst = static_cast<IO *>(p.out) + static_cast<long>(n) * p.out_h * p.out_w * C + c;
+    const unsigned out_row_bytes = p.out_w * pixel_bytes;
+    const __amdgpu_buffer_rsrc_t out_view =
+        buffer_view(static_cast<IO *>(p.out) + static_cast<long>(n0) * p.out_h * p.out_w * C);
+    NhwcCols<TW> ocols;
+    nhwc_cols<TW>(ix0, p.out_w, pixel_bytes, (n - n0) * (p.out_h * out_row_bytes) + c * static_cast<unsigned>(sizeof(IO)), ocols);
 #pragma unroll
     for (int b = 0; b < BH; ++b) {
         const int iy = iy0 + b;
-        if (iy >= p.out_h) continue;
+        const unsigned roff = iy < p.out_h ? iy * out_row_bytes : kOob;
 #pragma unroll
-        for (int o = 0; o < TW; ++o) {
-            const int ix = ix0 + o;
-            if (ix < p.out_w)
-                store4<IO>(dst + (static_cast<long>(iy) * p.out_w + ix) * C, acc[b][4 * o], acc[b][4 * o + 1],
-                           acc[b][4 * o + 2], acc[b][4 * o + 3]);
-        }
+        for (int o = 0; o < TW; ++o)
+            view_store4<IO>(out_view, __builtin_elementwise_add_sat(roff, ocols.off[o]), acc[b][4 * o], acc[b][4 * o + 1],
+                            acc[b][4 * o + 2], acc[b][4 * o + 3]);
     }
 }
 
