@@ -333,7 +333,7 @@ def main():
     # summary does not cover this variant)
     traffic = None
     try:
-        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json" if args.layout == "nchw" else "hbm_traffic_nhwc.json")) as f:
             traffic = json.load(f)["bytes_per_launch"].get(dom_name)
     except (OSError, ValueError, KeyError):
         traffic = None
