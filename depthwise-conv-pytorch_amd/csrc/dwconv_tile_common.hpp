@@ -222,6 +222,7 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__res
             int dst[kStageBatch];
 #pragma unroll
             for (int u = 0; u < kStageBatch; ++u) {
+                const bool live = base + u * static_cast<int>(blockDim.x) < total;
                 const int slot = min(base + u * static_cast<int>(blockDim.x), total - 1);
                 const int rowidx = fast_div(slot, s.spr_magic);
                 const int sc = slot - rowidx * s.spr;
@@ -229,22 +230,21 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__res
                 const int r = rowidx - pl * s.lds_rows;
                 const int ix = 4 * (s.g_lo + sc);
                 const int iy = iy0 + r;
-                const bool ok = static_cast<unsigned>(iy) < static_cast<unsigned>(s.in_h) &&
+                const bool ok = live && static_cast<unsigned>(iy) < static_cast<unsigned>(s.in_h) &&
                                 static_cast<unsigned>(ix) < static_cast<unsigned>(s.in_w);
                 const unsigned off = (pl * s.in_plane + iy * s.in_w + ix) * static_cast<unsigned>(sizeof(IO));
                 v[u] = view_load4<IO>(view, ok ? off : kOob);
-                dst[u] = pl * s.plane_pitch + r * s.pitch + kSlack + ix + s.col_shift;
+                // slots past the end of the image (they hold zeros) go to the spare floats that end the image:
+                // the right-hand slack of its last row, which no stored output depends on
+                dst[u] = live ? pl * s.plane_pitch + r * s.pitch + kSlack + ix + s.col_shift : nplanes * s.plane_pitch - 4;
             }
 #pragma unroll
             for (int u = 0; u < kStageBatch; ++u) {
-                const float4 t = v[u];  // read outside the condition: a conditional copy keeps the array out of registers
-                if (base + u * static_cast<int>(blockDim.x) < total) {
-                    float *d = lds + dst[u];
-                    d[0] = t.x;
-                    d[1] = t.y;
-                    d[2] = t.z;
-                    d[3] = t.w;
-                }
+                float *d = lds + dst[u];
+                d[0] = v[u].x;
+                d[1] = v[u].y;
+                d[2] = v[u].z;
+                d[3] = v[u].w;
             }
         }
         return;
@@ -306,7 +306,7 @@ template <int U>
 struct StageSlots {
     int r[U];          // row within the tile's rows; a hugely negative row for slots that always read zeros
     unsigned off[U];   // ((plane * in_plane + r * in_w + column) * element size
-    int lds[U];        // float offset in the LDS image, -1 past the end of the image
+    int lds[U];        // float offset in the LDS image; slots past its end: the spare floats that end the image
 };
 
 template <int U, typename IO>
@@ -324,7 +324,7 @@ __device__ __forceinline__ void stage_slots(const StageLayout &s, int nplanes, S
         const bool reads = slot < total && static_cast<unsigned>(ix) < static_cast<unsigned>(s.in_w);
         q.r[u] = reads ? r : -(1 << 30);
         q.off[u] = (pl * s.in_plane + r * s.in_w + ix) * static_cast<unsigned>(sizeof(IO));
-        q.lds[u] = slot < total ? pl * s.plane_pitch + r * s.pitch + kSlack + ix + s.col_shift : -1;
+        q.lds[u] = slot < total ? pl * s.plane_pitch + r * s.pitch + kSlack + ix + s.col_shift : nplanes * s.plane_pitch - 4;
     }
 }
 
@@ -375,14 +375,11 @@ __device__ __forceinline__ void stage_commit(float *lds, const StageSlots<U> &q,
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const float4 v = t.v[u];
-        const int d = q.lds[u];
-        if (d >= 0) {
-            float *dst = lds + d;
-            dst[0] = v.x;
-            dst[1] = v.y;
-            dst[2] = v.z;
-            dst[3] = v.w;
-        }
+        float *dst = lds + q.lds[u];
+        dst[0] = v.x;
+        dst[1] = v.y;
+        dst[2] = v.z;
+        dst[3] = v.w;
     }
 }
 
