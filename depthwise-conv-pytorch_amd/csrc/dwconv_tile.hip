@@ -232,6 +232,18 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
         }
 
         const int ox = 4 * cb;
+        if (p.vec_out == 2) {
+            // branch-free: rows past the end of the plane store out of range
+            const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane);
+            const unsigned o0 = (pl * p.out_plane + ox) * static_cast<unsigned>(sizeof(IO));
+#pragma unroll
+            for (int b = 0; b < 2 * BQ; ++b) {
+                const int oy = 2 * (qy0 + rb * BQ) + b;
+                view_store4<IO>(view, oy < p.out_h ? o0 + oy * p.out_w * static_cast<unsigned>(sizeof(IO)) : kOob, acc[b][0],
+                                acc[b][1], acc[b][2], acc[b][3]);
+            }
+            continue;
+        }
         IO *dst = static_cast<IO *>(p.out) + (plane0 + pl) * p.out_plane + ox;
 #pragma unroll
         for (int b = 0; b < 2 * BQ; ++b) {
@@ -346,6 +358,7 @@ int launch_up2(TilePlan &p, hipStream_t stream)
     auto rows_for = [](int units) { return units * BQ + KAY; };
     if (!plan_tiles(p, ceil_div(ceil_div(p.out_h, 2), BQ), BQ, used_cols, K * K, rows_for)) return -1;
     if (p.st.vec_in) p.st.vec_in = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
+    if (p.vec_out) p.vec_out = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
     hipLaunchKernelGGL((fir_up2_kernel<IO, K, EY, EX, BQ>), dim3(p.n_tiles), dim3(env_int("DWCONV_TILE_THREADS", kThreads)), lds_bytes(p, K * K), stream,
                        p);
     note_variant("tile_up2%s<k%d,e%d%d,bq%d> P%d rows%d vin%d vout%d", sizeof(IO) == 2 ? "16" : "", K, EY, EX, BQ, p.planes_per_tile,

@@ -147,7 +147,11 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
             const int oy = oy0 + rb * BH + b;
             const IO *row = gsrc + static_cast<long>(oy) * p.out_w;
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (has_item && oy < p.out_h) {
+            if (p.vec_gy == 2) {
+                // branch-free: rows past the plane (and lanes without an item) read zeros through the view
+                const unsigned off = ((pl * p.out_plane + ox) + oy * p.out_w) * static_cast<unsigned>(sizeof(IO));
+                v = view_load4<IO>(buffer_view(gy + plane0 * p.out_plane), has_item && oy < p.out_h ? off : kOob);
+            } else if (has_item && oy < p.out_h) {
                 if (p.vec_gy) {
                     v = load4<IO>(row);
                 } else {
@@ -491,6 +495,7 @@ struct Launcher {
         if (fused) p.st.vec_in = p.st.vec_in && aligned4(gy);  // gy is staged with the x image's layout
         if (p.st.vec_in) p.st.vec_in = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
         if (p.vec_gx) p.vec_gx = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
+        if (p.vec_gy) p.vec_gy = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
         if constexpr (S == 1) {
             if (fused) {
                 if constexpr (K == 3) {
