@@ -332,8 +332,8 @@ long bwd_s2_case(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO
     p.sx.vec_in = (g.in_w % 4 == 0) && aligned4(x);
     p.sg.vec_in = (g.out_w % 4 == 0) && aligned4(gy);
     p.vec_gx = (g.in_w % 4 == 0) && aligned4(gx);
-    if (p.sx.vec_in) p.sx.vec_in = vector_mode(1, p.sx.in_plane, sizeof(IO));
-    if (p.sg.vec_in) p.sg.vec_in = vector_mode(1, p.sg.in_plane, sizeof(IO));
+    if (p.sx.vec_in) p.sx.vec_in = stage_vector_mode(p.sx, 1, sizeof(IO));
+    if (p.sg.vec_in) p.sg.vec_in = stage_vector_mode(p.sg, 1, sizeof(IO));
     if (p.vec_gx) p.vec_gx = vector_mode(1, p.sx.in_plane, sizeof(IO));
     // all 256 lanes stage the images even when the tile has fewer items than that
     const int threads = kThreads;

@@ -83,16 +83,17 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
 
     const int n_items = nplanes * p.items_per_plane;
     for (int item = threadIdx.x; item < n_items; item += blockDim.x) {
+        // (24-bit multiplies: full rate, and every operand here is an LDS-sized quantity)
         const int pl = fast_div(item, p.ipp_magic);
-        const int rem = item - pl * p.items_per_plane;
+        const int rem = item - __mul24(pl, p.items_per_plane);
         const int rb = fast_div(rem, p.ncb_magic);
-        const int cb = rem - rb * p.ncb;
+        const int cb = rem - __mul24(rb, p.ncb);
 
         float tapv[KK];
 #pragma unroll
         for (int t = 0; t < KK; ++t) tapv[t] = lds[p.tap_base + pl * KK + t];
 
-        const float *base = lds + pl * p.st.plane_pitch + (rb * BH * S) * p.st.pitch + kSlack + 4 * cb * S;
+        const float *base = lds + __mul24(pl, p.st.plane_pitch) + __mul24(rb * BH * S, p.st.pitch) + kSlack + 4 * cb * S;
         float acc[BH][4];
 #pragma unroll
         for (int b = 0; b < BH; ++b)
@@ -330,7 +331,7 @@ int launch_down(TilePlan &p, hipStream_t stream)
     const int used_cols = 4 * (p.ncb - 1) * S + 4 * NV;
     auto rows_for = [](int units) { return (units * BH - 1) * S + K; };
     if (!plan_tiles(p, ceil_div(p.out_h, BH), BH, used_cols, K * K, rows_for)) return -1;
-    if (p.st.vec_in) p.st.vec_in = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
+    if (p.st.vec_in) p.st.vec_in = stage_vector_mode(p.st, p.planes_per_tile, sizeof(IO));
     if (p.vec_out) p.vec_out = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
     hipLaunchKernelGGL((fir_down_kernel<IO, K, S, FLIP, BH>), dim3(p.n_tiles), dim3(env_int("DWCONV_TILE_THREADS", kThreads)), lds_bytes(p, K * K),
                        stream, p);
@@ -357,7 +358,7 @@ int launch_up2(TilePlan &p, hipStream_t stream)
     const int used_cols = 2 * (p.ncb - 1) + NW;
     auto rows_for = [](int units) { return units * BQ + KAY; };
     if (!plan_tiles(p, ceil_div(ceil_div(p.out_h, 2), BQ), BQ, used_cols, K * K, rows_for)) return -1;
-    if (p.st.vec_in) p.st.vec_in = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
+    if (p.st.vec_in) p.st.vec_in = stage_vector_mode(p.st, p.planes_per_tile, sizeof(IO));
     if (p.vec_out) p.vec_out = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
     hipLaunchKernelGGL((fir_up2_kernel<IO, K, EY, EX, BQ>), dim3(p.n_tiles), dim3(env_int("DWCONV_TILE_THREADS", kThreads)), lds_bytes(p, K * K), stream,
                        p);

@@ -224,19 +224,22 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__res
             for (int u = 0; u < kStageBatch; ++u) {
                 const bool live = base + u * static_cast<int>(blockDim.x) < total;
                 const int slot = min(base + u * static_cast<int>(blockDim.x), total - 1);
+                // 24-bit multiplies run at full rate, 32-bit ones at a quarter of it; vector_mode() guarantees
+                // that the operands fit
                 const int rowidx = fast_div(slot, s.spr_magic);
-                const int sc = slot - rowidx * s.spr;
-                const int pl = fast_div(rowidx, s.lds_rows_magic);
-                const int r = rowidx - pl * s.lds_rows;
+                const int sc = slot - __mul24(rowidx, s.spr);
+                const int pl = nplanes == 1 ? 0 : fast_div(rowidx, s.lds_rows_magic);
+                const int r = rowidx - __mul24(pl, s.lds_rows);
                 const int ix = 4 * (s.g_lo + sc);
                 const int iy = iy0 + r;
                 const bool ok = live && static_cast<unsigned>(iy) < static_cast<unsigned>(s.in_h) &&
                                 static_cast<unsigned>(ix) < static_cast<unsigned>(s.in_w);
-                const unsigned off = (pl * s.in_plane + iy * s.in_w + ix) * static_cast<unsigned>(sizeof(IO));
+                const unsigned off = (__mul24(pl, s.in_plane) + __mul24(iy, s.in_w) + ix) * static_cast<unsigned>(sizeof(IO));
                 v[u] = view_load4<IO>(view, ok ? off : kOob);
                 // slots past the end of the image (they hold zeros) go to the spare floats that end the image:
                 // the right-hand slack of its last row, which no stored output depends on
-                dst[u] = live ? pl * s.plane_pitch + r * s.pitch + kSlack + ix + s.col_shift : nplanes * s.plane_pitch - 4;
+                dst[u] = live ? __mul24(pl, s.plane_pitch) + __mul24(r, s.pitch) + kSlack + ix + s.col_shift
+                              : nplanes * s.plane_pitch - 4;
             }
 #pragma unroll
             for (int u = 0; u < kStageBatch; ++u) {
@@ -449,6 +452,13 @@ inline int vector_mode(long planes, long in_plane, size_t esize)
 {
     const bool fits = planes * in_plane * static_cast<long>(esize) < static_cast<long>(kOob);
     return fits && env_int("DWCONV_STAGE_VIEW", 1) ? 2 : 1;
+}
+
+// vec_in of a staged image: the view path also needs operands that fit its 24-bit multiplies.
+inline int stage_vector_mode(const StageLayout &s, long planes, size_t esize)
+{
+    const bool dims = s.in_h < (1 << 23) && s.in_w < (1 << 23) && (planes == 1 || s.in_plane < (1 << 23));
+    return dims ? vector_mode(planes, s.in_plane, esize) : 1;
 }
 
 // Row pitch and float4 slots of an image `used_cols` floats wide (col_shift must be set).

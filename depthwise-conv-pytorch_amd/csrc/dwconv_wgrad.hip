@@ -493,7 +493,7 @@ struct Launcher {
         const bool pf = K == 3 && env_int("DWCONV_PREFETCH", 1) &&
                         p.planes_per_tile * p.st.lds_rows * p.st.spr <= kPrefetchSlots * kThreads;
         if (fused) p.st.vec_in = p.st.vec_in && aligned4(gy);  // gy is staged with the x image's layout
-        if (p.st.vec_in) p.st.vec_in = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
+        if (p.st.vec_in) p.st.vec_in = stage_vector_mode(p.st, p.planes_per_tile, sizeof(IO));
         if (p.vec_gx) p.vec_gx = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
         if (p.vec_gy) p.vec_gy = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
         if constexpr (S == 1) {
