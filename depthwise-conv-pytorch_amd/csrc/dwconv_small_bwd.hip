@@ -53,8 +53,8 @@ __device__ __forceinline__ void run_commit(const IO *__restrict__ g, float *lds,
     const int n4 = n >> 2;
 #pragma unroll
     for (int u = 0; u < kRunRegs; ++u) {
-        const float4 t = widen4<IO>(v[u]);  // read outside the condition: a conditional copy keeps the array out of registers
-        if (static_cast<int>(threadIdx.x) + u * kWave < n4) reinterpret_cast<float4 *>(lds)[threadIdx.x + u * kWave] = t;
+        // slots past the end of the run hold its last group of four again (run_fetch) and rewrite it in place
+        reinterpret_cast<float4 *>(lds)[min(static_cast<int>(threadIdx.x) + u * kWave, n4 - 1)] = widen4<IO>(v[u]);
     }
     const int tail = n4 * 4 + threadIdx.x;
     if (tail < n) lds[tail] = Io<IO>::in(g[tail]);

@@ -58,13 +58,13 @@ __device__ __forceinline__ void run_to_lds(const IO *__restrict__ g, float *lds,
     const int n4 = n >> 2;
     for (int base = threadIdx.x; base < n4; base += kWave * kRunBatch) {
         float4 v[kRunBatch];
-        // out-of-range slots re-read the last float4 of the run (always a valid address) and are not stored
+        // slots past the end of the run re-read its last group of four and write it to the same place again:
+        // no branch around either access
 #pragma unroll
         for (int u = 0; u < kRunBatch; ++u)
             v[u] = load4<IO>(g + 4 * min(base + u * kWave, n4 - 1));
 #pragma unroll
-        for (int u = 0; u < kRunBatch; ++u)
-            if (base + u * kWave < n4) reinterpret_cast<float4 *>(lds)[base + u * kWave] = v[u];
+        for (int u = 0; u < kRunBatch; ++u) reinterpret_cast<float4 *>(lds)[min(base + u * kWave, n4 - 1)] = v[u];
     }
     const int tail = n4 * 4 + threadIdx.x;
     if (tail < n) lds[tail] = Io<IO>::in(g[tail]);
@@ -87,8 +87,8 @@ __device__ __forceinline__ void runs_to_lds(const IO *__restrict__ ga, float *la
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            if (base + u * kWave < na4) reinterpret_cast<float4 *>(la)[base + u * kWave] = va[u];
-            if (base + u * kWave < nb4) reinterpret_cast<float4 *>(lb)[base + u * kWave] = vb[u];
+            reinterpret_cast<float4 *>(la)[min(base + u * kWave, na4 - 1)] = va[u];
+            reinterpret_cast<float4 *>(lb)[min(base + u * kWave, nb4 - 1)] = vb[u];
         }
     }
     const int ta = na4 * 4 + threadIdx.x, tb = nb4 * 4 + threadIdx.x;
