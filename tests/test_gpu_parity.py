@@ -657,3 +657,92 @@ def test_fused_epilogue_other_dtypes_and_autograd(dw, gpu):
                                     s, s, p, p, 9, None)
     assert rc == 1 and b"activation" in _C._lib.dwconv_last_error()
 
+
+def test_plane_beyond_two_gib(dw, gpu):
+    """One fp32 plane of more than 2 GiB: byte offsets inside it pass 2^31, where the kernels' 32-bit buffer-view
+    offsets end, so the library must take its 64-bit addressing path.  Corners (with their zero padding) and an
+    interior window are compared with the oracle on crops."""
+    from torch_dwconv import _C
+
+    hh, ww = 540000, 1024  # 540000 * 1024 * 4 B = 2.2 GB, narrow enough for the tiled kernels
+    free, _ = torch.cuda.mem_get_info()
+    if free < 12 * 1024 ** 3:
+        pytest.skip("needs 12 GiB of free device memory")
+    g = torch.Generator(device=gpu).manual_seed(5)
+    x = torch.randn(1, 1, hh, ww, device=gpu, generator=g)
+    wt = torch.randn(1, 1, 3, 3, generator=torch.Generator("cpu").manual_seed(6))
+    y = dw.depthwise_conv2d(x, wt.to(gpu), stride=1, padding=1)
+    variant = _C.last_variant()
+    _announce("2.2 GB plane", variant)
+    assert "vin1" in variant and "vout1" in variant, variant  # vector accesses, but not through a 2 GiB view
+    for (r0, c0) in [(0, 0), (hh - 64, ww - 64), (hh // 2 + 3, ww // 2 - 5), (hh - 64, 0)]:
+        # crop with a one-pixel halo where the plane has one
+        ra, rb_ = max(r0 - 1, 0), min(r0 + 64 + 1, hh)
+        ca, cb_ = max(c0 - 1, 0), min(c0 + 64 + 1, ww)
+        crop = x[:, :, ra:rb_, ca:cb_].cpu().contiguous()
+        ref = oracle.forward(_np(crop), _np(wt), 1, 1)
+        got = _np(y[:, :, r0:r0 + 64, c0:c0 + 64].cpu())
+        np.testing.assert_allclose(got.astype(np.float64), ref[:, :, r0 - ra:r0 - ra + 64, c0 - ca:c0 - ca + 64],
+                                   rtol=1e-5, atol=1e-5)
+    del y
+    # grad-input of the same plane (the transposed problem) on the same crops, grad-weight against an fp64 sum
+    gy = torch.randn(1, 1, hh, ww, device=gpu, generator=g)
+    gx, gw = _C.dwconv2d_backward(x, gy, wt.to(gpu), 1, 1, 1, 1)
+    _announce("2.2 GB plane backward", _C.last_variant())
+    for (r0, c0) in [(0, 0), (hh - 64, ww - 64)]:
+        ra, rb_ = max(r0 - 1, 0), min(r0 + 64 + 1, hh)
+        ca, cb_ = max(c0 - 1, 0), min(c0 + 64 + 1, ww)
+        crop = gy[:, :, ra:rb_, ca:cb_].cpu().contiguous()
+        ref = oracle.grad_input(_np(crop), _np(wt), crop.shape[2:], 1, 1)
+        got = _np(gx[:, :, r0:r0 + 64, c0:c0 + 64].cpu())
+        np.testing.assert_allclose(got.astype(np.float64), ref[:, :, r0 - ra:r0 - ra + 64, c0 - ca:c0 - ca + 64],
+                                   rtol=1e-5, atol=1e-5)
+    # gw[i,j] = <gy, x shifted by (i-1, j-1)>: torch's fp64 reductions on the device as the independent sum
+    ref_gw = torch.zeros(3, 3, dtype=torch.float64)
+    for i in range(3):
+        for j in range(3):
+            di, dj = i - 1, j - 1
+            ys = slice(max(0, -di), hh - max(0, di))
+            xs = slice(max(0, -dj), ww - max(0, dj))
+            yi = slice(max(0, di), hh - max(0, -di))
+            xi = slice(max(0, dj), ww - max(0, -dj))
+            ref_gw[i, j] = torch.sum(gy[0, 0, ys, xs].double() * x[0, 0, yi, xi].double()).item()
+    np.testing.assert_allclose(_np(gw.cpu())[0, 0].astype(np.float64), ref_gw.numpy(), rtol=1e-4,
+                               atol=1e-4 * float(ref_gw.abs().max()))
+
+
+@pytest.mark.parametrize("layout", ["nchw", "nhwc"])
+def test_tensor_beyond_two_gib(dw, gpu, layout):
+    """A batch whose input tensor exceeds 2 GiB (planes themselves are small): the buffer views start at the
+    workgroup's own planes / images, so their 32-bit offsets stay small while the bases pass 2^31 bytes.  The last
+    images (largest addresses) and the first are compared with the oracle; grad-weight over the whole batch is
+    checked through the adjoint identity."""
+    free, _ = torch.cuda.mem_get_info()
+    if free < 16 * 1024 ** 3:
+        pytest.skip("needs 16 GiB of free device memory")
+    n, c, h, w, k, s, p = 520, 96, 112, 112, 3, 2, 1  # 520 * 96 * 112 * 112 * 4 B = 2.5 GB
+    g = torch.Generator(device=gpu).manual_seed(9)
+    x = torch.randn(n, c, h, w, device=gpu, generator=g)
+    wt = (torch.randn(c, 1, k, k, generator=torch.Generator("cpu").manual_seed(10)) / k).to(gpu)
+    if layout == "nhwc":
+        x = x.contiguous(memory_format=torch.channels_last)
+    xg = x.requires_grad_(True)
+    wg = wt.clone().requires_grad_(True)
+    y = dw.depthwise_conv2d(xg, wg, stride=s, padding=p)
+    gy = torch.randn(y.shape, device=gpu, generator=g)
+    if layout == "nhwc":
+        gy = gy.contiguous(memory_format=torch.channels_last)
+    gx, gw = torch.autograd.grad(y, (xg, wg), gy)
+    for img in (0, n - 1):
+        for ch in (0, c - 1):
+            xs = x.detach()[img:img + 1, ch:ch + 1].cpu().contiguous()
+            ws = wt[ch:ch + 1].cpu().contiguous()
+            gs = gy[img:img + 1, ch:ch + 1].cpu().contiguous()
+            np.testing.assert_allclose(_np(y.detach()[img:img + 1, ch:ch + 1].cpu()).astype(np.float64),
+                                       oracle.forward(_np(xs), _np(ws), s, p), rtol=1e-5, atol=1e-5)
+            np.testing.assert_allclose(_np(gx[img:img + 1, ch:ch + 1].cpu()).astype(np.float64),
+                                       oracle.grad_input(_np(gs), _np(ws), (h, w), s, p), rtol=1e-5, atol=1e-5)
+    lhs = (y.detach().double() * gy.double()).sum().item()
+    assert abs(lhs - (wg.detach().double() * gw.double()).sum().item()) <= 1e-6 * abs(lhs) + 1e-2
+    assert abs(lhs - (x.detach().double() * gx.double()).sum().item()) <= 1e-6 * abs(lhs) + 1e-2
+
