@@ -333,6 +333,101 @@ int nhwc_backward_any(const T *in, const T *gy, const T *taps, T *gx, T *gw, voi
     return DWCONV_OK;
 }
 
+// ---- dilation and depth multiplier ----
+int make_general_geometry(GeneralGeometry &g, int batch, int channel, int in_h, int in_w, int multiplier, int kernel_h,
+                          int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w)
+{
+    if (batch < 0 || channel < 0 || in_h < 0 || in_w < 0)
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "negative tensor extent (batch %d, channel %d, input %dx%d)", batch,
+                    channel, in_h, in_w);
+    if (multiplier < 1) return fail(DWCONV_ERR_INVALID_ARGUMENT, "depth multiplier must be >= 1, got %d", multiplier);
+    if (kernel_h < 1 || kernel_w < 1)
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "kernel extent must be >= 1, got %dx%d", kernel_h, kernel_w);
+    if (stride_h < 1 || stride_w < 1 || dil_h < 1 || dil_w < 1)
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "stride and dilation must be >= 1, got stride %dx%d dilation %dx%d",
+                    stride_h, stride_w, dil_h, dil_w);
+    if (pad_h < 0 || pad_w < 0) return fail(DWCONV_ERR_INVALID_ARGUMENT, "padding must be >= 0, got %dx%d", pad_h, pad_w);
+    g = GeneralGeometry{batch, channel, multiplier, in_h, in_w, 0, 0, kernel_h, kernel_w, stride_h, stride_w,
+                        pad_h, pad_w, dil_h, dil_w};
+    const long span_h = 1l * dil_h * (kernel_h - 1) + 1, span_w = 1l * dil_w * (kernel_w - 1) + 1;
+    const long oh = in_h + 2l * pad_h - span_h, ow = in_w + 2l * pad_w - span_w;
+    g.out_h = oh < 0 ? 0 : static_cast<int>(oh / stride_h + 1);
+    g.out_w = ow < 0 ? 0 : static_cast<int>(ow / stride_w + 1);
+    if (1ll * batch * channel * in_h * in_w >= (1ll << 40) ||
+        1ll * batch * channel * multiplier * g.out_h * g.out_w >= (1ll << 40) ||
+        1ll * channel * multiplier * kernel_h * kernel_w >= (1ll << 31))
+        return fail(DWCONV_ERR_UNSUPPORTED, "tensor too large");
+    return DWCONV_OK;
+}
+
+inline bool is_plain(const GeneralGeometry &g) { return g.multiplier == 1 && g.dil_h == 1 && g.dil_w == 1; }
+
+template <typename T>
+int general_forward_any(const T *in, const T *taps, T *out, int batch, int channel, int in_h, int in_w, int multiplier,
+                        int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w, int dil_h,
+                        int dil_w, void *stream)
+{
+    GeneralGeometry g;
+    const int rc = make_general_geometry(g, batch, channel, in_h, in_w, multiplier, kernel_h, kernel_w, stride_h,
+                                         stride_w, pad_h, pad_w, dil_h, dil_w);
+    if (rc != DWCONV_OK) return rc;
+    if (is_plain(g))  // the tuned kernels
+        return dwconv2d_any<T>(in, taps, out, batch, channel, in_h, in_w, kernel_h, kernel_w, 1, 1, stride_h, stride_w,
+                               pad_h, pad_h, pad_w, pad_w, 1, stream);
+    const long long out_elems = 1ll * batch * channel * multiplier * g.out_h * g.out_w;
+    if (out_elems > 0 && (in == nullptr || taps == nullptr || out == nullptr))
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");
+    return general_forward<T>(in, taps, out, g, static_cast<hipStream_t>(stream));
+}
+
+template <typename T>
+size_t general_workspace_any(const GeneralGeometry &g)
+{
+    if (is_plain(g)) {
+        const WgradGeometry w{g.batch, g.channel, g.in_h, g.in_w, g.out_h, g.out_w, g.kernel_h, g.kernel_w,
+                              g.stride_h, g.stride_w, g.pad_h, g.pad_w};
+        return wgrad_workspace<T>(w);
+    }
+    return general_grad_weight_workspace<T>(g);
+}
+
+template <typename T>
+int general_backward_any(const T *in, const T *gy, const T *taps, T *gx, T *gw, void *ws, size_t ws_bytes, int batch,
+                         int channel, int in_h, int in_w, int out_h, int out_w, int multiplier, int kernel_h,
+                         int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w,
+                         void *stream_)
+{
+    GeneralGeometry g;
+    int rc = make_general_geometry(g, batch, channel, in_h, in_w, multiplier, kernel_h, kernel_w, stride_h, stride_w,
+                                   pad_h, pad_w, dil_h, dil_w);
+    if (rc != DWCONV_OK) return rc;
+    if (g.out_h != std::max(0, out_h) || g.out_w != std::max(0, out_w))
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "out_grad extent %dx%d does not match the convolution geometry", out_h,
+                    out_w);
+    if (gx == nullptr || gw == nullptr) return fail(DWCONV_ERR_INVALID_ARGUMENT, "null gradient pointer");
+    if (is_plain(g)) {
+        if constexpr (std::is_same<T, double>::value) {
+            // fp64 has no combined kernel: the two passes of the reference's backward (torch_dwconv/dwconv.py:56-68)
+            rc = dwconv2d_any<T>(gy, taps, gx, batch, channel, out_h, out_w, kernel_h, kernel_w, stride_h, stride_w, 1,
+                                 1, kernel_h - pad_h - 1, in_h - out_h * stride_h + pad_h, kernel_w - pad_w - 1,
+                                 in_w - out_w * stride_w + pad_w, 0, stream_);
+            if (rc != DWCONV_OK) return rc;
+            return wgrad_any<T>(in, gy, gw, ws, ws_bytes, batch, channel, in_h, in_w, out_h, out_w, kernel_h, kernel_w,
+                                1, 1, stride_h, stride_w, pad_h, pad_w, stream_);
+        } else {
+            return backward_any<T>(in, gy, taps, gx, gw, ws, ws_bytes, batch, channel, in_h, in_w, out_h, out_w,
+                                   kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, stream_);
+        }
+    }
+    const bool has_out = 1ll * batch * channel * multiplier * g.out_h * g.out_w > 0;
+    if (has_out && (gy == nullptr || taps == nullptr || (in_h > 0 && in_w > 0 && in == nullptr)))
+        return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    rc = general_grad_input<T>(gy, taps, gx, g, stream);
+    if (rc != DWCONV_OK) return rc;
+    return general_grad_weight<T>(in, gy, gw, ws, ws_bytes, g, stream);
+}
+
 }  // namespace
 }  // namespace dwconv
 
@@ -557,5 +652,48 @@ DWCONV_FUSED_ENTRY_POINTS(f64, double, double, double)
 DWCONV_FUSED_ENTRY_POINTS(f16, unsigned short, half_t, float)
 DWCONV_FUSED_ENTRY_POINTS(bf16, unsigned short, bf16_t, float)
 #undef DWCONV_FUSED_ENTRY_POINTS
+
+// ---- dilation and depth multiplier ----
+size_t dwconv2d_general_backward_workspace_bytes(int batch, int channel, int in_h, int in_w, int multiplier,
+                                                 int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h,
+                                                 int pad_w, int dil_h, int dil_w, int elem_size)
+{
+    GeneralGeometry g;
+    if (make_general_geometry(g, batch, channel, in_h, in_w, multiplier, kernel_h, kernel_w, stride_h, stride_w, pad_h,
+                              pad_w, dil_h, dil_w) != DWCONV_OK)
+        return 0;
+    if (batch == 0 || channel == 0) return 0;
+    if (elem_size == 8) return general_workspace_any<double>(g);
+    if (elem_size == 2) return general_workspace_any<half_t>(g);
+    return general_workspace_any<float>(g);
+}
+
+#define DWCONV_GENERAL_ENTRY_POINTS(SUFFIX, CTYPE, TYPE)                                                               \
+    int dwconv2d_general_##SUFFIX(const CTYPE *input, const CTYPE *kernel, CTYPE *out, int batch, int channel,         \
+                                  int in_h, int in_w, int multiplier, int kernel_h, int kernel_w, int stride_h,        \
+                                  int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void *stream)              \
+    {                                                                                                                  \
+        return general_forward_any<TYPE>(reinterpret_cast<const TYPE *>(input), reinterpret_cast<const TYPE *>(kernel), \
+                                         reinterpret_cast<TYPE *>(out), batch, channel, in_h, in_w, multiplier,        \
+                                         kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, stream);  \
+    }                                                                                                                  \
+    int dwconv2d_general_backward_##SUFFIX(const CTYPE *input, const CTYPE *out_grad, const CTYPE *kernel,             \
+                                           CTYPE *in_grad, CTYPE *kernel_grad, void *workspace,                        \
+                                           size_t workspace_bytes, int batch, int channel, int in_h, int in_w,         \
+                                           int out_h, int out_w, int multiplier, int kernel_h, int kernel_w,           \
+                                           int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w,     \
+                                           void *stream)                                                               \
+    {                                                                                                                  \
+        return general_backward_any<TYPE>(                                                                             \
+            reinterpret_cast<const TYPE *>(input), reinterpret_cast<const TYPE *>(out_grad),                           \
+            reinterpret_cast<const TYPE *>(kernel), reinterpret_cast<TYPE *>(in_grad),                                 \
+            reinterpret_cast<TYPE *>(kernel_grad), workspace, workspace_bytes, batch, channel, in_h, in_w, out_h,      \
+            out_w, multiplier, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, stream);            \
+    }
+DWCONV_GENERAL_ENTRY_POINTS(f32, float, float)
+DWCONV_GENERAL_ENTRY_POINTS(f64, double, double)
+DWCONV_GENERAL_ENTRY_POINTS(f16, unsigned short, half_t)
+DWCONV_GENERAL_ENTRY_POINTS(bf16, unsigned short, bf16_t)
+#undef DWCONV_GENERAL_ENTRY_POINTS
 
 }  // extern "C"

@@ -150,6 +150,18 @@ struct NhwcGeometry {
     Epilogue epi;  // nhwc_forward only
 };
 
+// Geometry of a call with dilation and depth multiplier (NCHW): input (N,C,H,W), taps (C*M,1,KH,KW),
+// output (N,C*M,OH,OW), OH = (H + 2*pad - dil*(KH-1) - 1) / stride + 1.
+struct GeneralGeometry {
+    int batch, channel, multiplier;
+    int in_h, in_w;
+    int out_h, out_w;
+    int kernel_h, kernel_w;
+    int stride_h, stride_w;
+    int pad_h, pad_w;
+    int dil_h, dil_w;
+};
+
 // Thread-local error/variant strings behind dwconv_last_error()/dwconv_last_variant().
 int fail(dwconv_status code, const char *fmt, ...);
 void note_variant(const char *fmt, ...);
@@ -225,5 +237,16 @@ size_t nhwc_grad_weight_workspace(const NhwcGeometry &g);
 template <typename T>
 int nhwc_grad_weight(const T *x, const T *gy, T *gw, void *ws, size_t ws_bytes, const NhwcGeometry &g,
                      hipStream_t stream);
+
+// ---- dilation and depth multiplier: dwconv_general.hip (T = float, double, half_t or bf16_t) ----
+template <typename T>
+int general_forward(const T *in, const T *taps, T *out, const GeneralGeometry &g, hipStream_t stream);
+template <typename T>
+int general_grad_input(const T *gy, const T *taps, T *gx, const GeneralGeometry &g, hipStream_t stream);
+template <typename T>
+size_t general_grad_weight_workspace(const GeneralGeometry &g);
+template <typename T>
+int general_grad_weight(const T *x, const T *gy, T *gw, void *ws, size_t ws_bytes, const GeneralGeometry &g,
+                        hipStream_t stream);
 
 }  // namespace dwconv

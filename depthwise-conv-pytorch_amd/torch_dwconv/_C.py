@@ -66,6 +66,14 @@ for _sfx in ("f32", "f64", "f16", "bf16"):
         getattr(_lib, _name).restype = _i
         getattr(_lib, _name).argtypes = [_p, _p, _p, _p, _p] + [_i] * 11 + [_p]
 
+_lib.dwconv2d_general_backward_workspace_bytes.restype = _z
+_lib.dwconv2d_general_backward_workspace_bytes.argtypes = [_i] * 14
+for _sfx in ("f32", "f64", "f16", "bf16"):
+    getattr(_lib, "dwconv2d_general_" + _sfx).restype = _i
+    getattr(_lib, "dwconv2d_general_" + _sfx).argtypes = [_p, _p, _p] + [_i] * 13 + [_p]
+    getattr(_lib, "dwconv2d_general_backward_" + _sfx).restype = _i
+    getattr(_lib, "dwconv2d_general_backward_" + _sfx).argtypes = [_p, _p, _p, _p, _p, _p, _z] + [_i] * 15 + [_p]
+
 ACTIVATIONS = {None: 0, "none": 0, "relu": 1, "relu6": 2, "silu": 3}
 
 _SUFFIX = {torch.float32: "f32", torch.float64: "f64", torch.float16: "f16", torch.bfloat16: "bf16"}
@@ -329,3 +337,64 @@ def dwconv2d_fused(input, kernel, scale, shift, activation, stride_h, stride_w, 
     if rc != 0:
         _raise(rc)
     return out
+
+
+# ---- dilation and depth multiplier -----------------------------------------------------------------------
+def _multiplier(input, kernel):
+    if input.dim() != 4 or kernel.dim() != 4 or kernel.shape[1] != 1 or input.shape[1] == 0 or \
+            kernel.shape[0] % input.shape[1] != 0 or kernel.shape[0] == 0:
+        raise RuntimeError(
+            f"kernel of shape {tuple(kernel.shape)} does not match an input of shape {tuple(input.shape)}: "
+            "expected (C*multiplier,1,KH,KW)"
+        )
+    return kernel.shape[0] // input.shape[1]
+
+
+def dwconv2d_general(input, kernel, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w):
+    """``F.conv2d(input, kernel, stride, padding, dilation, groups=C)`` for a kernel of shape (C*M,1,KH,KW)."""
+    _check_cuda(input, "input")
+    _check_cuda(kernel, "kernel")
+    m = _multiplier(input, kernel)
+    sfx = _suffix(input, kernel)
+    x, k = input.contiguous(), kernel.contiguous()
+    n, c, h, w = x.shape
+    kh, kw = k.shape[2], k.shape[3]
+    oh = max((h + 2 * pad_h - dil_h * (kh - 1) - 1) // stride_h + 1, 0) if h + 2 * pad_h - dil_h * (kh - 1) - 1 >= 0 else 0
+    ow = max((w + 2 * pad_w - dil_w * (kw - 1) - 1) // stride_w + 1, 0) if w + 2 * pad_w - dil_w * (kw - 1) - 1 >= 0 else 0
+    out = torch.empty((n, c * m, oh, ow), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = getattr(_lib, "dwconv2d_general_" + sfx)(
+            x.data_ptr(), k.data_ptr(), out.data_ptr(), n, c, h, w, m, kh, kw, stride_h, stride_w, pad_h, pad_w,
+            dil_h, dil_w, _stream(x),
+        )
+    if rc != 0:
+        _raise(rc)
+    return out
+
+
+def dwconv2d_general_backward(input, out_grad, kernel, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w):
+    """Both gradients of ``dwconv2d_general``; returns ``(grad_input, grad_kernel)``."""
+    _check_cuda(input, "input")
+    _check_cuda(out_grad, "out_grad")
+    _check_cuda(kernel, "kernel")
+    m = _multiplier(input, kernel)
+    sfx = _suffix(input, out_grad, kernel)
+    x, gy, k = input.contiguous(), out_grad.contiguous(), kernel.contiguous()
+    n, c, h, w = x.shape
+    if gy.dim() != 4 or gy.shape[0] != n or gy.shape[1] != c * m:
+        raise RuntimeError(f"out_grad of shape {tuple(gy.shape)} does not belong to input {tuple(x.shape)}")
+    oh, ow = gy.shape[2], gy.shape[3]
+    kh, kw = k.shape[2], k.shape[3]
+    gx = torch.empty_like(x)
+    gw = torch.empty_like(k)
+    ws_bytes = _lib.dwconv2d_general_backward_workspace_bytes(n, c, h, w, m, kh, kw, stride_h, stride_w, pad_h, pad_w,
+                                                              dil_h, dil_w, x.element_size())
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = getattr(_lib, "dwconv2d_general_backward_" + sfx)(
+            x.data_ptr(), gy.data_ptr(), k.data_ptr(), gx.data_ptr(), gw.data_ptr(), ws.data_ptr(), ws_bytes,
+            n, c, h, w, oh, ow, m, kh, kw, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, _stream(x),
+        )
+    if rc != 0:
+        _raise(rc)
+    return gx, gw

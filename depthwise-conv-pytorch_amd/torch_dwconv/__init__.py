@@ -2,4 +2,9 @@
 
 Public surface of the reference package (torch_dwconv/__init__.py:1).
 """
-from .dwconv import depthwise_conv2d, depthwise_conv2d_fused, DepthwiseConv2d  # noqa: F401
+from .dwconv import (  # noqa: F401
+    depthwise_conv2d,
+    depthwise_conv2d_fused,
+    depthwise_conv2d_general,
+    DepthwiseConv2d,
+)

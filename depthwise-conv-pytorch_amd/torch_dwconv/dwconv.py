@@ -140,6 +140,33 @@ def depthwise_conv2d(input, weight, bias=None, stride=1, padding=0, dilation=1, 
     return depthwise_conv2d_fn(input, weight, stride, padding, small)
 
 
+class DepthwiseConv2dGeneralFunction(Function):
+    """Autograd wrapper of the entry points with dilation and depth multiplier (not in the reference)."""
+
+    @staticmethod
+    def forward(ctx, input, kernel, stride, pad, dilation):
+        ctx.save_for_backward(input, kernel)
+        ctx.geometry = (stride[0], stride[1], pad[0], pad[1], dilation[0], dilation[1])
+        return _C.dwconv2d_general(input, kernel, *ctx.geometry)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, kernel = ctx.saved_tensors
+        grad_input, grad_kernel = _C.dwconv2d_general_backward(input, grad_output, kernel, *ctx.geometry)
+        return grad_input, grad_kernel, None, None, None
+
+
+def depthwise_conv2d_general(input, weight, stride=1, padding=0, dilation=1):
+    """``F.conv2d(input, weight, stride=stride, padding=padding, dilation=dilation, groups=C)`` for a ``weight`` of
+    shape ``(C*M, 1, KH, KW)``: the dilation and the depth multiplier ``M`` that ``depthwise_conv2d`` refuses, as the
+    reference does (torch_dwconv/dwconv.py:99-106).  With ``M == 1`` and no dilation it runs the same kernels as
+    ``depthwise_conv2d``; otherwise per-element kernels (correct for every geometry, not tuned)."""
+    stride = make_tuple(stride, 2)
+    padding = make_tuple(padding, 2)
+    dilation = make_tuple(dilation, 2)
+    return DepthwiseConv2dGeneralFunction.apply(input, weight, stride, padding, dilation)
+
+
 _TORCH_ACTIVATIONS = {None: None, "none": None, "relu": F.relu, "relu6": F.relu6, "silu": F.silu}
 
 

@@ -290,6 +290,52 @@ int dwconv2d_fused_nhwc_bf16(const unsigned short *input, const unsigned short *
     int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
     int activation, void *stream);
 
+/* ---- dilation and depth multiplier ------------------------------------------------------------------
+ * The two options the reference's check_options refuses (torch_dwconv/dwconv.py:99-106): a dilation
+ * above 1 and out_channels = multiplier * in_channels.  input (N,C,H,W); kernel and kernel_grad
+ * (C*multiplier,1,KH,KW); out and out_grad (N,C*multiplier,OH,OW) with
+ * OH = (H + 2*pad_h - dil_h*(KH-1) - 1) / stride_h + 1:
+ *   out[n, c*M+j, oy, ox] = sum_{ty,tx} input[n, c, oy*stride - pad + ty*dil, ox*stride - pad + tx*dil] * kernel[c*M+j, ty, tx]
+ * i.e. F.conv2d(groups=C, dilation=dil).  With multiplier 1 and dilation 1 the call is served by the tuned
+ * kernels behind dwconv2d_* / dwconv2d_backward_*; otherwise by per-element kernels (correct, not tuned).
+ * kernel_grad is bit-identical from run to run. */
+size_t dwconv2d_general_backward_workspace_bytes(int batch, int channel, int in_h, int in_w,
+                                                 int multiplier, int kernel_h, int kernel_w,
+                                                 int stride_h, int stride_w, int pad_h, int pad_w,
+                                                 int dil_h, int dil_w, int elem_size);
+int dwconv2d_general_f32(const float *input, const float *kernel, float *out,
+    int batch, int channel, int in_h, int in_w, int multiplier, int kernel_h, int kernel_w,
+    int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void *stream);
+int dwconv2d_general_backward_f32(const float *input, const float *out_grad, const float *kernel,
+    float *in_grad, float *kernel_grad, void *workspace, size_t workspace_bytes,
+    int batch, int channel, int in_h, int in_w, int out_h, int out_w, int multiplier,
+    int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+    int dil_h, int dil_w, void *stream);
+int dwconv2d_general_f64(const double *input, const double *kernel, double *out,
+    int batch, int channel, int in_h, int in_w, int multiplier, int kernel_h, int kernel_w,
+    int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void *stream);
+int dwconv2d_general_backward_f64(const double *input, const double *out_grad, const double *kernel,
+    double *in_grad, double *kernel_grad, void *workspace, size_t workspace_bytes,
+    int batch, int channel, int in_h, int in_w, int out_h, int out_w, int multiplier,
+    int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+    int dil_h, int dil_w, void *stream);
+int dwconv2d_general_f16(const unsigned short *input, const unsigned short *kernel, unsigned short *out,
+    int batch, int channel, int in_h, int in_w, int multiplier, int kernel_h, int kernel_w,
+    int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void *stream);
+int dwconv2d_general_backward_f16(const unsigned short *input, const unsigned short *out_grad, const unsigned short *kernel,
+    unsigned short *in_grad, unsigned short *kernel_grad, void *workspace, size_t workspace_bytes,
+    int batch, int channel, int in_h, int in_w, int out_h, int out_w, int multiplier,
+    int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+    int dil_h, int dil_w, void *stream);
+int dwconv2d_general_bf16(const unsigned short *input, const unsigned short *kernel, unsigned short *out,
+    int batch, int channel, int in_h, int in_w, int multiplier, int kernel_h, int kernel_w,
+    int stride_h, int stride_w, int pad_h, int pad_w, int dil_h, int dil_w, void *stream);
+int dwconv2d_general_backward_bf16(const unsigned short *input, const unsigned short *out_grad, const unsigned short *kernel,
+    unsigned short *in_grad, unsigned short *kernel_grad, void *workspace, size_t workspace_bytes,
+    int batch, int channel, int in_h, int in_w, int out_h, int out_w, int multiplier,
+    int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+    int dil_h, int dil_w, void *stream);
+
 /* Tuning/diagnostic hook: name of the kernel variant the last successful call
  * on this thread launched (e.g. "tile_f32<k3,s1,v4>"), for benchmarks and tests. */
 const char *dwconv_last_variant(void);

@@ -26,5 +26,10 @@ from .capi import (  # noqa: F401
     grad_input,
     grad_weight,
 )
-from .torch_reference import torch_reference, torch_reference_fused, torch_cpu_fp32_step  # noqa: F401
+from .torch_reference import (  # noqa: F401
+    torch_reference,
+    torch_reference_fused,
+    torch_reference_general,
+    torch_cpu_fp32_step,
+)
 from . import host_logic  # noqa: F401

@@ -21,6 +21,18 @@ def torch_reference(x, w, gy=None, stride=1, padding=0):
     return y.detach(), gx, gw
 
 
+def torch_reference_general(x, w, gy=None, stride=1, padding=0, dilation=1):
+    """fp64 CPU ``F.conv2d(x, w, stride, padding, dilation, groups=C)`` for a weight of shape (C*M,1,KH,KW) and, given
+    gy, both gradients: the options the reference's check_options refuses (torch_dwconv/dwconv.py:99-106)."""
+    xd = x.detach().to("cpu", torch.float64).requires_grad_(gy is not None)
+    wd = w.detach().to("cpu", torch.float64).requires_grad_(gy is not None)
+    y = F.conv2d(xd, wd, stride=stride, padding=padding, dilation=dilation, groups=xd.shape[1])
+    if gy is None:
+        return y.detach(), None, None
+    gx, gw = torch.autograd.grad(y, (xd, wd), gy.detach().to("cpu", torch.float64))
+    return y.detach(), gx, gw
+
+
 _ACTIVATIONS = {None: lambda v: v, "none": lambda v: v, "relu": F.relu, "relu6": F.relu6, "silu": F.silu}
 
 

@@ -746,3 +746,63 @@ def test_tensor_beyond_two_gib(dw, gpu, layout):
     assert abs(lhs - (wg.detach().double() * gw.double()).sum().item()) <= 1e-6 * abs(lhs) + 1e-2
     assert abs(lhs - (x.detach().double() * gx.double()).sum().item()) <= 1e-6 * abs(lhs) + 1e-2
 
+
+# ---- dilation and depth multiplier ---------------------------------------------------------------------------
+GENERAL_CASES = [
+    # (N, C, M, H, W, KH, KW, stride, pad, dilation)
+    (2, 4, 1, 14, 14, 3, 3, 1, 2, 2), (2, 3, 2, 9, 11, 3, 3, 1, 1, 1), (1, 5, 3, 13, 12, 5, 3, 2, 2, 2),
+    (2, 8, 1, 16, 16, 3, 3, 2, 3, 3), (2, 2, 4, 7, 7, 3, 3, 1, 0, 1), (1, 3, 2, 6, 6, 3, 3, 1, 1, 3),
+    (2, 6, 1, 20, 24, 3, 3, 1, 1, 1),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("case", GENERAL_CASES, ids=lambda c: "N%d_C%d_M%d_%dx%d_k%dx%d_s%d_p%d_d%d" % c)
+def test_dilation_and_depth_multiplier(dw, gpu, case, dtype):
+    from torch_dwconv import _C
+    from torch_dwconv.dwconv import depthwise_conv2d_general
+
+    n, c, m, h, w, kh, kw, s, p, d = case
+    g = torch.Generator("cpu").manual_seed(53)
+    x = torch.randn(n, c, h, w, generator=g).to(dtype)
+    wt = (torch.randn(c * m, 1, kh, kw, generator=g) / kh).to(dtype)
+    xg = x.to(gpu).requires_grad_(True)
+    wg = wt.to(gpu).requires_grad_(True)
+    y = depthwise_conv2d_general(xg, wg, stride=s, padding=p, dilation=d)
+    v_fwd = _C.last_variant()
+    gy = torch.randn(y.shape, generator=g).to(dtype)
+    gx, gw = torch.autograd.grad(y, (xg, wg), gy.to(gpu))
+    _announce(case, str(dtype), v_fwd, "|", _C.last_variant())
+    plain = m == 1 and d == 1
+    assert v_fwd.startswith("general_fwd") != plain, v_fwd  # the plain case runs the tuned kernels
+    y_ref, gx_ref, gw_ref = oracle.torch_reference_general(x, wt, gy, s, p, d)
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(_np(y.detach()).astype(np.float64), y_ref.numpy(), **tol)
+    np.testing.assert_allclose(_np(gx).astype(np.float64), gx_ref.numpy(), **tol)
+    gtol = 1e-4 if dtype == torch.float32 else 1e-12
+    np.testing.assert_allclose(_np(gw).astype(np.float64), gw_ref.numpy(), rtol=gtol, atol=gtol * float(gw_ref.abs().max()))
+    _, gw2 = torch.autograd.grad(depthwise_conv2d_general(xg, wg, stride=s, padding=p, dilation=d), (xg, wg), gy.to(gpu))
+    assert torch.equal(gw, gw2)
+
+
+def test_general_entry_point_errors(dw, gpu):
+    from torch_dwconv import _C
+    from torch_dwconv.dwconv import depthwise_conv2d_general
+
+    x = torch.randn(1, 4, 8, 8, device=gpu)
+    with pytest.raises(RuntimeError, match="multiplier"):
+        depthwise_conv2d_general(x, torch.randn(6, 1, 3, 3, device=gpu))
+    y = depthwise_conv2d_general(x.half(), torch.randn(8, 1, 3, 3, device=gpu).half(), padding=2, dilation=2)
+    assert y.shape == (1, 8, 8, 8) and y.dtype == torch.float16
+    ref = oracle.torch_reference_general(x.half(), torch.zeros(8, 1, 3, 3), None, 1, 2, 2)[0]
+    assert ref.shape == y.shape
+    lib = _C._lib
+    o = torch.empty(1, 8, 8, 8, device=gpu)
+    k = torch.randn(8, 1, 3, 3, device=gpu)
+    assert lib.dwconv2d_general_f32(x.data_ptr(), k.data_ptr(), o.data_ptr(), 1, 4, 8, 8, 0, 3, 3, 1, 1, 1, 1, 1, 1, None) == 1
+    assert b"multiplier" in lib.dwconv_last_error()
+    assert lib.dwconv2d_general_f32(x.data_ptr(), k.data_ptr(), o.data_ptr(), 1, 4, 8, 8, 2, 3, 3, 1, 1, 1, 1, 0, 1, None) == 1
+    # a dilated filter larger than the padded input gives an empty output, not an error
+    e = depthwise_conv2d_general(x, k, dilation=5)
+    assert e.shape == (1, 8, 0, 0)
+

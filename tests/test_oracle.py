@@ -305,3 +305,39 @@ def test_fused_reference_closed_forms():
                                rtol=1e-12, atol=1e-14)
     assert (z < 0).any() and (z > 6).any()  # every branch of the activations is exercised
 
+
+def test_general_reference_against_brute_force():
+    """torch_reference_general (torch's dilated, multiplied grouped conv) pinned by plain loops on a tiny case,
+    and its gradients by the adjoint identities."""
+    g = torch.Generator("cpu").manual_seed(47)
+    n, c, m, h, w, kh, kw, s, p, d = 2, 3, 2, 9, 8, 3, 2, 2, 2, 2
+    x = torch.randn(n, c, h, w, generator=g, dtype=torch.float64)
+    wt = torch.randn(c * m, 1, kh, kw, generator=g, dtype=torch.float64)
+    y, _, _ = oracle.torch_reference_general(x, wt, None, s, p, d)
+    oh = (h + 2 * p - d * (kh - 1) - 1) // s + 1
+    ow = (w + 2 * p - d * (kw - 1) - 1) // s + 1
+    assert tuple(y.shape) == (n, c * m, oh, ow)
+    ref = np.zeros((n, c * m, oh, ow))
+    xn, wn = x.numpy(), wt.numpy()
+    for b in range(n):
+        for oc in range(c * m):
+            for oy in range(oh):
+                for ox in range(ow):
+                    acc = 0.0
+                    for ty in range(kh):
+                        for tx in range(kw):
+                            iy, ix = oy * s - p + ty * d, ox * s - p + tx * d
+                            if 0 <= iy < h and 0 <= ix < w:
+                                acc += xn[b, oc // m, iy, ix] * wn[oc, 0, ty, tx]
+                    ref[b, oc, oy, ox] = acc
+    np.testing.assert_allclose(y.numpy(), ref, rtol=1e-12, atol=1e-12)
+    gy = torch.randn(y.shape, generator=g, dtype=torch.float64)
+    _, gx, gw = oracle.torch_reference_general(x, wt, gy, s, p, d)
+    lhs = float((y * gy).sum())
+    assert abs(lhs - float((x * gx).sum())) < 1e-9 * max(1.0, abs(lhs))
+    assert abs(lhs - float((wt * gw).sum())) < 1e-9 * max(1.0, abs(lhs))
+    # multiplier 1, dilation 1 is the plain depthwise convolution
+    w1 = torch.randn(c, 1, 3, 3, generator=g, dtype=torch.float64)
+    np.testing.assert_array_equal(oracle.torch_reference_general(x, w1, None, 1, 1, 1)[0].numpy(),
+                                  oracle.torch_reference(x, w1, None, 1, 1)[0].numpy())
+
