@@ -19,7 +19,6 @@ namespace dwconv {
 namespace {
 
 constexpr int kFusedLdsBudget = 36 * 1024;    // both images of a tile
-constexpr int kUx = 8, kUg = 2;               // float4 slots per lane that hold the next tile's x / gy band
 
 struct BwdS2Plan {
     StageLayout sx;   // x image: row r holds x row 2*q0 - pad + r, column c holds x column c - pad
@@ -41,7 +40,6 @@ struct BwdS2Plan {
     int n_items;
     int bq;
     int vec_gx;
-    int prefetch;     // the images of a tile fit the prefetch registers
 };
 
 template <int CTRL, int ROW_MASK, int BANK_MASK>
@@ -64,10 +62,8 @@ __device__ __forceinline__ float wave_sum_to_last_lane(float v)
 }
 
 // E = parity of the transposed problem's leading pad K - 1 - pad (the same on both axes).
-// PF: keep the next tile's bands in flight in registers (worth its ~50 registers for the 3x3 kernel only;
-// with more taps the lower occupancy costs more than the overlap brings).
 // BQ: half-resolution rows per lane (4; 2 for planes too low to give every lane a block of 4).
-template <typename IO, int K, int E, bool PF, int BQ>
+template <typename IO, int K, int E, int BQ>
 __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -98,47 +94,15 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
 #pragma unroll
     for (int t = 0; t < KK; ++t) wacc[t] = 0.f;
 
-    StagedTile<PF ? kUx : 1> tx;
-    StagedTile<PF ? kUg : 1> tg;
-    StageSlots<PF ? kUx : 1> qx;
-    StageSlots<PF ? kUg : 1> qg;
-    if constexpr (PF) {
-        stage_slots<kUx, IO>(p.sx, 1, qx);
-        stage_slots<kUg, IO>(p.sg, 1, qg);
-    }
-    if constexpr (PF) {
-        if (chunk < p.tiles_per_group) {
-        const int n = chunk / p.row_tiles, rt = chunk - n * p.row_tiles;
-        const long plane0 = static_cast<long>(n) * p.channel + c;
-        stage_fetch(p.sx, x, plane0, 1, 2 * rt * p.rows_per_tile - p.pad, qx, tx);
-        stage_fetch(p.sg, gy, plane0, 1, rt * p.rows_per_tile - p.m, qg, tg);
-        }
-    }
-
     for (int tile = chunk; tile < p.tiles_per_group; tile += p.chunks) {
         const int n = tile / p.row_tiles, rt = tile - n * p.row_tiles;
         const long plane0 = static_cast<long>(n) * p.channel + c;
         const int q0 = rt * p.rows_per_tile;
 
         if (tile != chunk) __syncthreads();  // the previous tile's window reads are done
-        if constexpr (PF) {
-            stage_commit(lds, qx, tx);
-            stage_commit(lds + p.g_base, qg, tg);
-        } else {
-            stage_tile(p.sx, x, lds, plane0, 1, 2 * q0 - p.pad);
-            stage_tile(p.sg, gy, lds + p.g_base, plane0, 1, q0 - p.m);
-        }
+        stage_tile(p.sx, x, lds, plane0, 1, 2 * q0 - p.pad);
+        stage_tile(p.sg, gy, lds + p.g_base, plane0, 1, q0 - p.m);
         __syncthreads();
-        if constexpr (PF) {
-          if (tile + p.chunks < p.tiles_per_group) {
-            // the next tile's bands travel while this one is computed
-            const int t1 = tile + p.chunks;
-            const int n1 = t1 / p.row_tiles, rt1 = t1 - n1 * p.row_tiles;
-            const long plane1 = static_cast<long>(n1) * p.channel + c;
-            stage_fetch(p.sx, x, plane1, 1, 2 * rt1 * p.rows_per_tile - p.pad, qx, tx);
-            stage_fetch(p.sg, gy, plane1, 1, rt1 * p.rows_per_tile - p.m, qg, tg);
-          }
-        }
 
         // ---- gy window: grad-input block, and this lane's gy elements from the window's centre
         float g[BQ][2];
@@ -335,26 +299,20 @@ long bwd_s2_case(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO
     if (p.sx.vec_in) p.sx.vec_in = stage_vector_mode(p.sx, 1, sizeof(IO));
     if (p.sg.vec_in) p.sg.vec_in = stage_vector_mode(p.sg, 1, sizeof(IO));
     if (p.vec_gx) p.vec_gx = vector_mode(1, p.sx.in_plane, sizeof(IO));
-    // all 256 lanes stage the images even when the tile has fewer items than that
-    const int threads = kThreads;
-    p.prefetch = bq == 4 && K == 3 && env_int("DWCONV_PREFETCH", 1) && p.sx.lds_rows * p.sx.spr <= kUx * threads &&
-                 p.sg.lds_rows * p.sg.spr <= kUg * threads;
     const size_t images = static_cast<size_t>(p.sx.plane_pitch + p.sg.plane_pitch) * 4;
     const size_t red = static_cast<size_t>(kThreads / 64) * K * K * 4;
     const size_t shmem = images > red ? images : red;
     const int E = (K - 1 - g.pad_h) & 1;
-    const dim3 grid(g.channel * p.chunks), block(threads);
+    const dim3 grid(g.channel * p.chunks), block(kThreads)  /* all 256 lanes stage the images even when the tile has fewer items */;
     if (bq == 2) {
-        if (E) hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 1, false, 2>), grid, block, shmem, stream, p);
-        else hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 0, false, 2>), grid, block, shmem, stream, p);
-    } else if (E && p.prefetch) hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 1, true, 4>), grid, block, shmem, stream, p);
-    else if (E) hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 1, false, 4>), grid, block, shmem, stream, p);
-    else if (p.prefetch) hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 0, true, 4>), grid, block, shmem, stream, p);
-    else hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 0, false, 4>), grid, block, shmem, stream, p);
+        if (E) hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 1, 2>), grid, block, shmem, stream, p);
+        else hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 0, 2>), grid, block, shmem, stream, p);
+    } else if (E) hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 1, 4>), grid, block, shmem, stream, p);
+    else hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 0, 4>), grid, block, shmem, stream, p);
     const int rc = check_launch("bwd_s2_kernel");
     if (rc != DWCONV_OK) return rc;
-    note_variant("bwd_tile_s2%s<k%d,e%d,bq%d> rows%d chunks%d vin%d vgy%d vgx%d pf%d", sizeof(IO) == 2 ? "16" : "", K, E, bq,
-                 p.rows_per_tile, p.chunks, p.sx.vec_in, p.sg.vec_in, p.vec_gx, p.prefetch);
+    note_variant("bwd_tile_s2%s<k%d,e%d,bq%d> rows%d chunks%d vin%d vgy%d vgx%d", sizeof(IO) == 2 ? "16" : "", K, E, bq,
+                 p.rows_per_tile, p.chunks, p.sx.vec_in, p.sg.vec_in, p.vec_gx);
     return launch_wgrad_final(p.partial, gw, g.channel, K * K, p.chunks, stream);
 }
 

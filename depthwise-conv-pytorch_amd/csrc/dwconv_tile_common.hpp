@@ -293,99 +293,6 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__res
     }
 }
 
-// The same staging in two halves, for kernels that walk several tiles: `stage_fetch` issues the global
-// loads of a tile into registers (U float4 slots per lane; the planner guarantees the tile has no more
-// than U * blockDim.x slots), `stage_commit` writes them to LDS.  Fetching tile t+1 right after
-// committing tile t keeps its loads in flight while tile t is being computed.
-template <int U>
-struct StagedTile {
-    float4 v[U];
-};
-
-// What does not change from tile to tile for the U slots of a lane: the row of the slot within the tile's
-// rows, its byte offset from the tile's first row, and its place in LDS.  Kernels that walk many tiles compute
-// this once, so that fetching a tile costs four instructions per slot.
-template <int U>
-struct StageSlots {
-    int r[U];          // row within the tile's rows; a hugely negative row for slots that always read zeros
-    unsigned off[U];   // ((plane * in_plane + r * in_w + column) * element size
-    int lds[U];        // float offset in the LDS image; slots past its end: the spare floats that end the image
-};
-
-template <int U, typename IO>
-__device__ __forceinline__ void stage_slots(const StageLayout &s, int nplanes, StageSlots<U> &q)
-{
-    const int total = nplanes * s.lds_rows * s.spr;
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-        const int slot = threadIdx.x + u * blockDim.x;
-        const int rowidx = fast_div(slot, s.spr_magic);
-        const int sc = slot - rowidx * s.spr;
-        const int pl = fast_div(rowidx, s.lds_rows_magic);
-        const int r = rowidx - pl * s.lds_rows;
-        const int ix = 4 * (s.g_lo + sc);
-        const bool reads = slot < total && static_cast<unsigned>(ix) < static_cast<unsigned>(s.in_w);
-        q.r[u] = reads ? r : -(1 << 30);
-        q.off[u] = (pl * s.in_plane + r * s.in_w + ix) * static_cast<unsigned>(sizeof(IO));
-        q.lds[u] = slot < total ? pl * s.plane_pitch + r * s.pitch + kSlack + ix + s.col_shift : nplanes * s.plane_pitch - 4;
-    }
-}
-
-template <int U, typename IO>
-__device__ __forceinline__ void stage_fetch(const StageLayout &s, const IO *__restrict__ in, long plane0,
-                                            int nplanes, int iy0, const StageSlots<U> &q, StagedTile<U> &t)
-{
-    const int total = nplanes * s.lds_rows * s.spr;
-    if (s.vec_in == 2) {
-        const __amdgpu_buffer_rsrc_t view = buffer_view(in + plane0 * s.in_plane);
-        const unsigned row_base = static_cast<unsigned>(iy0 * s.in_w) * static_cast<unsigned>(sizeof(IO));  // uniform
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const bool ok = static_cast<unsigned>(iy0 + q.r[u]) < static_cast<unsigned>(s.in_h);
-            t.v[u] = view_load4<IO>(view, ok ? q.off[u] + row_base : kOob);
-        }
-        return;
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-        const int slot = threadIdx.x + u * blockDim.x;
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (slot < total) {
-            const int rowidx = fast_div(slot, s.spr_magic);
-            const int sc = slot - rowidx * s.spr;
-            const int pl = fast_div(rowidx, s.lds_rows_magic);
-            const int r = rowidx - pl * s.lds_rows;
-            const int ix = 4 * (s.g_lo + sc);
-            const int iy = iy0 + r;
-            const bool row_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(s.in_h);
-            const IO *src = in + (plane0 + pl) * s.in_plane + static_cast<long>(iy) * s.in_w + ix;
-            if (s.vec_in) {
-                if (row_ok && ix >= 0 && ix < s.in_w) v = load4<IO>(src);
-            } else if (row_ok) {
-                if (static_cast<unsigned>(ix + 0) < static_cast<unsigned>(s.in_w)) v.x = Io<IO>::in(src[0]);
-                if (static_cast<unsigned>(ix + 1) < static_cast<unsigned>(s.in_w)) v.y = Io<IO>::in(src[1]);
-                if (static_cast<unsigned>(ix + 2) < static_cast<unsigned>(s.in_w)) v.z = Io<IO>::in(src[2]);
-                if (static_cast<unsigned>(ix + 3) < static_cast<unsigned>(s.in_w)) v.w = Io<IO>::in(src[3]);
-            }
-        }
-        t.v[u] = v;
-    }
-}
-
-template <int U>
-__device__ __forceinline__ void stage_commit(float *lds, const StageSlots<U> &q, const StagedTile<U> &t)
-{
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-        const float4 v = t.v[u];
-        float *dst = lds + q.lds[u];
-        dst[0] = v.x;
-        dst[1] = v.y;
-        dst[2] = v.z;
-        dst[3] = v.w;
-    }
-}
-
 // Pins an accumulator array at this point of a fully unrolled loop nest.  The empty asm makes every
 // element an input and an output, so all FMAs feeding it must be issued before, and its memory clobber
 // keeps later LDS reads after it.  Without such pins the compiler sinks every FMA of a window below

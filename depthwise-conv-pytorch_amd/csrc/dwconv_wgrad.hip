@@ -74,10 +74,8 @@ constexpr int kRedPitch = kThreads + 1;  // odd pitch: lanes of one wave reading
 // layout.  The lane first walks its gy window: that gives its block of grad-input (gy against the
 // rotated taps, stored straight to memory) and, from the window's centre, its block of gy for the
 // grad-weight sums.  gy is read from HBM once for both gradients.
-// PF: the band(s) of the next tile are fetched into registers while the current tile is computed.
-constexpr int kPrefetchSlots = 4;  // float4 slots per lane and image
 
-template <typename IO, int K, int S, int BH, bool GX, bool PF>
+template <typename IO, int K, int S, int BH, bool GX>
 __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -120,18 +118,6 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
         for (int t = 0; t < KK; ++t) rot[t] = Io<IO>::in(static_cast<const IO *>(p.taps)[(c0 + pl) * KK + KK - 1 - t]);
     }
 
-    StagedTile<PF ? kPrefetchSlots : 1> tx, tg;
-    StageSlots<PF ? kPrefetchSlots : 1> slots;  // x and gy bands share one layout
-    if constexpr (PF) stage_slots<kPrefetchSlots, IO>(p.st, nplanes, slots);
-    if constexpr (PF) {
-        if (t_begin < t_end) {
-            const int n = t_begin / p.row_tiles, rt = t_begin - n * p.row_tiles;
-            const long plane0 = static_cast<long>(n) * p.channel + c0;
-            stage_fetch(p.st, x, plane0, nplanes, rt * p.rows_per_tile * S - p.pad_h, slots, tx);
-            if constexpr (GX) stage_fetch(p.st, gy, plane0, nplanes, rt * p.rows_per_tile - p.pad_h, slots, tg);
-        }
-    }
-
     for (int tile = t_begin; tile < t_end; tile += t_step) {
         const int n = tile / p.row_tiles, rt = tile - n * p.row_tiles;
         const long plane0 = static_cast<long>(n) * p.channel + c0;
@@ -168,23 +154,9 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
         }
 
         if (tile != t_begin) __syncthreads();  // the previous tile's window reads are done
-        if constexpr (PF) {
-            stage_commit(lds, slots, tx);
-            if constexpr (GX) stage_commit(lds + p.g_base, slots, tg);
-        } else {
-            stage_tile(p.st, x, lds, plane0, nplanes, oy0 * S - p.pad_h);
-            if constexpr (GX) stage_tile(p.st, gy, lds + p.g_base, plane0, nplanes, oy0 - p.pad_h);
-        }
+        stage_tile(p.st, x, lds, plane0, nplanes, oy0 * S - p.pad_h);
+        if constexpr (GX) stage_tile(p.st, gy, lds + p.g_base, plane0, nplanes, oy0 - p.pad_h);
         __syncthreads();
-        if constexpr (PF) {
-            if (tile + t_step < t_end) {
-                const int t1 = tile + t_step;
-                const int n1 = t1 / p.row_tiles, rt1 = t1 - n1 * p.row_tiles;
-                const long plane1 = static_cast<long>(n1) * p.channel + c0;
-                stage_fetch(p.st, x, plane1, nplanes, rt1 * p.rows_per_tile * S - p.pad_h, slots, tx);
-                if constexpr (GX) stage_fetch(p.st, gy, plane1, nplanes, rt1 * p.rows_per_tile - p.pad_h, slots, tg);
-            }
-        }
 
         if constexpr (GX) {
             constexpr int PC = K / 2;  // the lane's own gy block sits PC rows and columns into its window
@@ -489,32 +461,18 @@ struct Launcher {
         p.vec_gx = (g.in_w % 4 == 0) && aligned4(gx);
         const size_t shmem = lds_bytes<K, S, BH>(p, fused);
         const dim3 grid(p.groups * p.chunks), block(kThreads);
-        // prefetching costs ~35 registers: worth it for the 3x3 kernels, whose tiles also fit the slots
-        const bool pf = K == 3 && env_int("DWCONV_PREFETCH", 1) &&
-                        p.planes_per_tile * p.st.lds_rows * p.st.spr <= kPrefetchSlots * kThreads;
         if (fused) p.st.vec_in = p.st.vec_in && aligned4(gy);  // gy is staged with the x image's layout
         if (p.st.vec_in) p.st.vec_in = stage_vector_mode(p.st, p.planes_per_tile, sizeof(IO));
         if (p.vec_gx) p.vec_gx = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
         if (p.vec_gy) p.vec_gy = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
         if constexpr (S == 1) {
-            if (fused) {
-                if constexpr (K == 3) {
-                    if (pf) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, true, true>), grid, block, shmem, stream, p);
-                }
-                if (!pf) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, true, false>), grid, block, shmem, stream, p);
-            }
+            if (fused) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, true>), grid, block, shmem, stream, p);
         }
-        if (!fused) {
-            if constexpr (K == 3 && S == 1) {
-                if (pf) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, false, true>), grid, block, shmem, stream, p);
-            }
-            if (!(pf && K == 3 && S == 1))
-                hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, false, false>), grid, block, shmem, stream, p);
-        }
+        if (!fused) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, false>), grid, block, shmem, stream, p);
         rc = check_launch("wgrad_tile_kernel");
         if (rc != DWCONV_OK) return;
-        note_variant("%s%s<k%d,s%d,bh%d> P%d rows%d chunks%d vin%d vgy%d pf%d", fused ? "bwd_tile" : "wgrad_tile",
-                     sizeof(IO) == 2 ? "16" : "", K, S, BH, p.planes_per_tile, p.rows_per_tile, p.chunks, p.st.vec_in, p.vec_gy, pf && S == 1 ? 1 : 0);
+        note_variant("%s%s<k%d,s%d,bh%d> P%d rows%d chunks%d vin%d vgy%d", fused ? "bwd_tile" : "wgrad_tile",
+                     sizeof(IO) == 2 ? "16" : "", K, S, BH, p.planes_per_tile, p.rows_per_tile, p.chunks, p.st.vec_in, p.vec_gy);
         rc = launch_wgrad_final(static_cast<const float *>(ws), gw, g.channel, K * K, p.chunks, stream);
     }
 };
