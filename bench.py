@@ -337,8 +337,17 @@ def main():
             traffic = json.load(f)["bytes_per_launch"].get(dom_name)
     except (OSError, ValueError, KeyError):
         traffic = None
+    # the device function behind the variant name, as rocprofv3 lists it (backward calls end with a ~4.5 us
+    # *_final_kernel that the per-call timing includes)
+    family = dom_name.split("<")[0].rstrip("16")
+    function = {"tile_down": "fir_down_kernel", "tile_up2": "fir_up2_kernel", "small_down": "small_down_kernel",
+                "small_up2": "small_up2_kernel", "small_bwd": "small_bwd_kernel + wgrad_tile_final_kernel",
+                "small_wgrad": "small_bwd_kernel + wgrad_tile_final_kernel",
+                "bwd_tile": "wgrad_tile_kernel + wgrad_tile_final_kernel",
+                "wgrad_tile": "wgrad_tile_kernel + wgrad_tile_final_kernel",
+                "bwd_tile_s2": "bwd_s2_kernel + wgrad_tile_final_kernel"}.get(family, family)
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": dom_name,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": dom_name, "kernel_function": function,
                 "launches_per_step": dom["launches"], "avg_launch_us": round(dom["ms"] * 1e3 / dom["launches"], 1),
                 "bytes_per_launch": dom["bytes"] // dom["launches"]}
 
