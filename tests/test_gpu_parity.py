@@ -806,100 +806,3 @@ def test_general_entry_point_errors(dw, gpu):
     e = depthwise_conv2d_general(x, k, dilation=5)
     assert e.shape == (1, 8, 0, 0)
 
-
-
-# ---- randomised geometry sweep --------------------------------------------------------------------
-def _draw_case(rng):
-    """One random problem: about two thirds in the geometry the tuned kernels take (square 3/5/7 filter, stride 1 or
-    2, mostly 'same' padding), the rest anything the operator accepts (rectangular filters up to 11, strides up to 3,
-    per-axis padding up to one more than the filter)."""
-    def extent():
-        r = rng.random()
-        if r < 0.35:
-            return rng.choice([7, 14, 28])
-        if r < 0.6:
-            return rng.randint(1, 33)
-        if r < 0.9:
-            return rng.randint(34, 130)
-        return rng.randint(131, 400)
-
-    if rng.random() < 0.65:
-        kh = kw = rng.choice([3, 3, 5, 5, 7])
-        sh = sw = rng.choice([1, 1, 2])
-        ph = pw = kh // 2 if rng.random() < 0.75 else rng.randint(0, kh - 1)
-        if rng.random() < 0.15:
-            ph = rng.randint(0, kh - 1)
-    else:
-        kh = rng.choice([1, 2, 3, 3, 3, 4, 5, 5, 7, 7, 9, 11])
-        kw = kh if rng.random() < 0.7 else rng.choice([1, 2, 3, 5, 7])
-        sh = rng.choice([1, 1, 1, 2, 2, 3])
-        sw = sh if rng.random() < 0.8 else rng.choice([1, 2, 3])
-        ph = rng.choice([0, kh // 2, kh // 2, kh - 1, rng.randint(0, kh + 1)])
-        pw = rng.choice([0, kw // 2, kw // 2, kw - 1, rng.randint(0, kw + 1)])
-    h = extent()
-    w = h if rng.random() < 0.5 else extent()
-    n = rng.choice([1, 2, 3, 5, 8])
-    c = rng.choice([1, 2, 3, 4, 5, 8, 12, 16, 24, 40, 64, 96])
-    while n * c * h * w > 3_000_000:  # keeps the fp64 CPU check of one case in the milliseconds
-        if c > 1:
-            c //= 2
-        else:
-            n, h = 1, max(1, h // 2)
-    dtype = rng.choice([torch.float32] * 4 + [torch.float16, torch.bfloat16, torch.float64])
-    layout = rng.choice(["nchw", "nchw", "nhwc"])
-    return n, c, h, w, kh, kw, sh, sw, ph, pw, dtype, layout
-
-
-@pytest.mark.parametrize("seed", [101, 102, 103])
-def test_randomised_geometry_sweep(dw, gpu, seed):
-    """300 seeded random problems per seed over filter extent, stride and padding per axis, plane size, element type
-    and layout, each checked in all three passes against PyTorch's fp64 CPU convolution (the oracle of the
-    reference's own tests, test/test_forward.py:14) to the bounds used elsewhere in this file.  Odd cases go through
-    autograd, even ones through the combined backward entry points directly."""
-    import random
-
-    from torch_dwconv import _C
-
-    rng = random.Random(seed)
-    families = set()
-    for it in range(300):
-        n, c, h, w, kh, kw, sh, sw, ph, pw, dtype, layout = _draw_case(rng)
-        oh, ow = (h + 2 * ph - kh) // sh + 1, (w + 2 * pw - kw) // sw + 1
-        if oh <= 0 or ow <= 0:
-            continue  # empty outputs: test_empty_and_degenerate_inputs
-        g = torch.Generator("cpu").manual_seed(seed * 100003 + it)
-        x = torch.randn(n, c, h, w, generator=g, dtype=torch.float64).to(dtype)
-        wt = (torch.randn(c, 1, kh, kw, generator=g, dtype=torch.float64) / (kh * kw) ** 0.5).to(dtype)
-        gy = torch.randn(n, c, oh, ow, generator=g, dtype=torch.float64).to(dtype)
-        case = f"seed{seed} it{it} N{n}C{c} {h}x{w} k{kh}x{kw} s{sh}x{sw} p{ph}x{pw} {dtype} {layout}"
-        _announce(case)
-        xg, gyg, wg = x.to(gpu), gy.to(gpu), wt.to(gpu)
-        if layout == "nhwc":
-            xg = xg.contiguous(memory_format=torch.channels_last)
-            gyg = gyg.contiguous(memory_format=torch.channels_last)
-        nhwc = _C.is_channels_last(xg)  # false for planes of one pixel or one channel, where the layouts coincide
-        xg.requires_grad_(True)
-        wg.requires_grad_(True)
-        y = dw.depthwise_conv2d(xg, wg, stride=(sh, sw), padding=(ph, pw))
-        families.add(_C.last_variant().split("<")[0].split(" ")[0])
-        if dtype == torch.float64 or it % 2:
-            gx, gw = torch.autograd.grad(y, (xg, wg), gyg)
-        elif nhwc:
-            gx, gw = _C.dwconv2d_backward_nhwc(xg.detach(), gyg, wg.detach(), sh, sw, ph, pw)
-        else:
-            gx, gw = _C.dwconv2d_backward(xg.detach(), gyg.contiguous(), wg.detach(), sh, sw, ph, pw)
-        assert y.dtype == dtype and gx.dtype == dtype and gw.dtype == dtype, case
-        if nhwc:
-            assert y.is_contiguous(memory_format=torch.channels_last), case
-            assert gx.is_contiguous(memory_format=torch.channels_last), case
-        y_ref, gx_ref, gw_ref = oracle.torch_reference(x, wt, gy, (sh, sw), (ph, pw))
-        step = {torch.float32: 0.0, torch.float64: 0.0, torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[dtype]
-        base, gw_base = (1e-11, 1e-11) if dtype == torch.float64 else (1e-5, 1e-4)
-        tol = dict(rtol=base + step, atol=base + step * 1e-2)
-        np.testing.assert_allclose(_np(y.double()), _np(y_ref), err_msg=case, **tol)
-        np.testing.assert_allclose(_np(gx.double()), _np(gx_ref), err_msg=case, **tol)
-        gw_tol = gw_base + step
-        np.testing.assert_allclose(_np(gw.double()), _np(gw_ref), rtol=gw_tol,
-                                   atol=gw_tol * max(float(gw_ref.abs().max()), 1e-30), err_msg=case)
-    # the sweep is only worth its name if it reaches every forward kernel family
-    assert {"tile_down", "small_down", "nhwc_down", "direct_f32", "direct_f64", "nhwc_fwd_direct"} <= families, families
