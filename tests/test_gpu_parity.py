@@ -438,6 +438,49 @@ def test_runs_on_the_current_stream(dw, gpu):
     assert torch.equal(out, ref)
 
 
+@pytest.mark.parametrize("layout", ["nchw", "nhwc"])
+def test_hip_graph_capture_and_replay(dw, gpu, layout):
+    """The entry points launch kernels only (no allocation, no synchronisation, no memset node), so a step made of
+    them can be captured into a HIP graph.  Every replay, with eager work and synchronisations in between and fresh
+    values in the static input buffers, must reproduce the eager results bit for bit (all three passes are
+    deterministic)."""
+    from torch_dwconv import _C
+
+    # a whole-plane kernel, the tiled ones at stride 1 and 2, and the per-element fallback (4x4 filter)
+    for shape in [(4, 16, 28, 28, 5, 1, 2), (2, 8, 56, 56, 3, 1, 1), (2, 8, 56, 60, 3, 2, 1), (2, 8, 9, 11, 4, 2, 1)]:
+        n, c, h, w, k, s, p = shape
+        x, wt, gy = (t.to(gpu) for t in make_inputs(shape, seed=23))
+        if layout == "nhwc":
+            x, gy = (t.contiguous(memory_format=torch.channels_last) for t in (x, gy))
+
+        def step():
+            if layout == "nhwc":
+                return (_C.dwconv2d_nhwc(x, wt, s, s, p, p), *_C.dwconv2d_backward_nhwc(x, gy, wt, s, s, p, p))
+            return (_C.dwconv2d(x, wt, 1, 1, s, s, p, p, p, p, True), *_C.dwconv2d_backward(x, gy, wt, s, s, p, p))
+
+        side = torch.cuda.Stream(device=gpu)
+        side.wait_stream(torch.cuda.current_stream(gpu))
+        with torch.cuda.stream(side):
+            step()  # warm-up outside the capture
+        torch.cuda.current_stream(gpu).wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            captured = step()
+        gen = torch.Generator("cpu").manual_seed(29)
+        for replay in range(4):
+            _announce(shape_id(shape), layout, "replay", replay)
+            x.copy_(torch.randn(x.shape, generator=gen))
+            gy.copy_(torch.randn(gy.shape, generator=gen))
+            graph.replay()
+            torch.cuda.synchronize(gpu)
+            eager = step()
+            torch.cuda.synchronize(gpu)
+            for name, a, b in zip(("out", "in_grad", "kernel_grad"), captured, eager):
+                assert torch.equal(a, b), (shape, layout, replay, name)
+        y_ref, gx_ref, gw_ref = oracle.torch_reference(x, wt, gy, s, p)
+        assert_parity(*captured, _np(y_ref), _np(gx_ref), _np(gw_ref), torch.float32)
+
+
 # ---- channels-last tensors ---------------------------------------------------------------------------------
 NHWC_SHAPES = [
     # (N, C, H, W, k, stride, pad): C % 4 == 0 and k in {3,5,7} take the vector kernels, the rest the per-element ones
