@@ -14,6 +14,8 @@
 // (torch_dwconv/dwconv.py:56-68) and x K*K times (torch_dwconv/dwconv_kernel.cu:260-306).
 #include "dwconv_tile_common.hpp"
 
+#include <type_traits>
+
 namespace dwconv {
 
 namespace {
@@ -63,7 +65,8 @@ __device__ __forceinline__ float wave_sum_to_last_lane(float v)
 
 // E = parity of the transposed problem's leading pad K - 1 - pad (the same on both axes).
 // BQ: half-resolution rows per lane (4; 2 for planes too low to give every lane a block of 4).
-template <typename IO, int K, int E, int BQ>
+// VIEWS: x, gy and gx all go through buffer views (sx.vec_in == sg.vec_in == vec_gx == 2), nothing else compiled in.
+template <typename IO, int K, int E, int BQ, bool VIEWS>
 __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -100,8 +103,8 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
         const int q0 = rt * p.rows_per_tile;
 
         if (tile != chunk) __syncthreads();  // the previous tile's window reads are done
-        stage_tile(p.sx, x, lds, plane0, 1, 2 * q0 - p.pad);
-        stage_tile(p.sg, gy, lds + p.g_base, plane0, 1, q0 - p.m);
+        stage_tile<IO, VIEWS>(p.sx, x, lds, plane0, 1, 2 * q0 - p.pad);
+        stage_tile<IO, VIEWS>(p.sg, gy, lds + p.g_base, plane0, 1, q0 - p.m);
         __syncthreads();
 
         // ---- gy window: grad-input block, and this lane's gy elements from the window's centre
@@ -150,7 +153,7 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
                 }
             pin_registers(xacc);
         }
-        if (p.vec_gx == 2) {
+        if (VIEWS || p.vec_gx == 2) {
             // branch-free: rows and column blocks past the end of the plane store out of range
             const int ox = 4 * cb;
             const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.gx) + plane0 * p.sx.in_plane);
@@ -162,7 +165,7 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
                 view_store4<IO>(view, ok ? (oy * p.sx.in_w + ox) * static_cast<unsigned>(sizeof(IO)) : kOob, xacc[b][0],
                                 xacc[b][1], xacc[b][2], xacc[b][3]);
             }
-        } else if (has_item) {
+        } else if (!VIEWS && has_item) {
             const int ox = 4 * cb;
             IO *dst = static_cast<IO *>(p.gx) + plane0 * p.sx.in_plane + ox;
 #pragma unroll
@@ -304,11 +307,19 @@ long bwd_s2_case(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO
     const size_t shmem = images > red ? images : red;
     const int E = (K - 1 - g.pad_h) & 1;
     const dim3 grid(g.channel * p.chunks), block(kThreads)  /* all 256 lanes stage the images even when the tile has fewer items */;
+    const bool views = p.sx.vec_in == 2 && p.sg.vec_in == 2 && p.vec_gx == 2 && !env_int("DWCONV_NO_VIEW_ONLY", 0);
+    auto launch = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, block, shmem, stream, p); };
+    auto pick = [&](auto e, auto b) {
+        constexpr int kE = decltype(e)::value, kB = decltype(b)::value;
+        if (views) launch(bwd_s2_kernel<IO, K, kE, kB, true>);
+        else launch(bwd_s2_kernel<IO, K, kE, kB, false>);
+    };
+    using std::integral_constant;
     if (bq == 2) {
-        if (E) hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 1, 2>), grid, block, shmem, stream, p);
-        else hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 0, 2>), grid, block, shmem, stream, p);
-    } else if (E) hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 1, 4>), grid, block, shmem, stream, p);
-    else hipLaunchKernelGGL((bwd_s2_kernel<IO, K, 0, 4>), grid, block, shmem, stream, p);
+        if (E) pick(integral_constant<int, 1>{}, integral_constant<int, 2>{});
+        else pick(integral_constant<int, 0>{}, integral_constant<int, 2>{});
+    } else if (E) pick(integral_constant<int, 1>{}, integral_constant<int, 4>{});
+    else pick(integral_constant<int, 0>{}, integral_constant<int, 4>{});
     const int rc = check_launch("bwd_s2_kernel");
     if (rc != DWCONV_OK) return rc;
     note_variant("bwd_tile_s2%s<k%d,e%d,bq%d> rows%d chunks%d vin%d vgy%d vgx%d", sizeof(IO) == 2 ? "16" : "", K, E, bq,

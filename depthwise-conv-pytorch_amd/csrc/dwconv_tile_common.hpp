@@ -209,12 +209,15 @@ __device__ __forceinline__ int xcd_contiguous_tile(int bid, int n_tiles)
 // their latencies overlap instead of adding up.
 constexpr int kStageBatch = 4;
 
-template <typename IO>
+// VIEW_ONLY: the caller guarantees s.vec_in == 2, and the other two ways of loading are not compiled in.  The
+// kernels keep an instance of each kind: with every alternative in one body, the values the unused ones need
+// stay live and push the scalar registers past what the hardware has.
+template <typename IO, bool VIEW_ONLY = false>
 __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__restrict__ in, float *lds,
                                            long plane0, int nplanes, int iy0)
 {
     const int total = nplanes * s.lds_rows * s.spr;
-    if (s.vec_in == 2) {
+    if (VIEW_ONLY || s.vec_in == 2) {
         // groups of four elements through a view of the tile's planes: slots outside the image read zeros
         const __amdgpu_buffer_rsrc_t view = buffer_view(in + plane0 * s.in_plane);
         for (int base = threadIdx.x; base < total; base += blockDim.x * kStageBatch) {
@@ -252,6 +255,7 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__res
         }
         return;
     }
+    if constexpr (VIEW_ONLY) return;
     for (int base = threadIdx.x; base < total; base += blockDim.x * kStageBatch) {
         float4 v[kStageBatch];
         int dst[kStageBatch];
