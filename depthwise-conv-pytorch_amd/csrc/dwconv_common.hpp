@@ -41,15 +41,37 @@ struct Io<bf16_t> {
         c.u = static_cast<uint32_t>(v.bits) << 16;
         return c.f;
     }
+    // Round to nearest even.  Device code uses the hardware conversion of gfx950 (v_cvt_pk_bf16_f32); the host
+    // version computes the same bits for every finite value and keeps a NaN a NaN.
     __host__ __device__ static bf16_t out(float v)
     {
+#if defined(__HIP_DEVICE_COMPILE__)
+        return bf16_t{__builtin_bit_cast(uint16_t, static_cast<__bf16>(v))};
+#else
         union { uint32_t u; float f; } c;
         c.f = v;
-        if ((c.u & 0x7fffffffu) > 0x7f800000u) return bf16_t{static_cast<uint16_t>((c.u >> 16) | 0x40u)};  // NaN stays NaN
-        c.u += 0x7fffu + ((c.u >> 16) & 1u);  // round to nearest even
+        if ((c.u & 0x7fffffffu) > 0x7f800000u) return bf16_t{static_cast<uint16_t>((c.u >> 16) | 0x40u)};
+        c.u += 0x7fffu + ((c.u >> 16) & 1u);
         return bf16_t{static_cast<uint16_t>(c.u >> 16)};
+#endif
     }
 };
+
+// Two sums as a pair of fp16 / bf16 in one register: a single conversion instruction each on gfx950.
+__device__ __forceinline__ uint32_t f16_pack2(float lo, float hi)
+{
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+}
+__device__ __forceinline__ uint32_t bf16_pack2(float lo, float hi)
+{
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
 
 // What a forward kernel applies to each sum before storing it: v * scale[c] + shift[c], then an activation.
 // scale / shift are per-channel arrays of the accumulation type (float; double for fp64 tensors) or null.

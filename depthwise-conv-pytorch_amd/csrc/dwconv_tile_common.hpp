@@ -5,6 +5,7 @@
 #include "dwconv_common.hpp"
 
 #include <cstdlib>
+#include <type_traits>
 
 namespace dwconv {
 
@@ -66,19 +67,12 @@ __device__ __forceinline__ void store4<float>(float *p, float a, float b, float 
 template <>
 __device__ __forceinline__ void store4<half_t>(half_t *p, float a, float b, float c, float d)
 {
-    union { uint32_t u; half_t h[2]; } lo, hi;
-    lo.h[0] = static_cast<half_t>(a);
-    lo.h[1] = static_cast<half_t>(b);
-    hi.h[0] = static_cast<half_t>(c);
-    hi.h[1] = static_cast<half_t>(d);
-    *reinterpret_cast<uint2 *>(p) = make_uint2(lo.u, hi.u);
+    *reinterpret_cast<uint2 *>(p) = make_uint2(f16_pack2(a, b), f16_pack2(c, d));
 }
 template <>
 __device__ __forceinline__ void store4<bf16_t>(bf16_t *p, float a, float b, float c, float d)
 {
-    const uint32_t lo = Io<bf16_t>::out(a).bits | (static_cast<uint32_t>(Io<bf16_t>::out(b).bits) << 16);
-    const uint32_t hi = Io<bf16_t>::out(c).bits | (static_cast<uint32_t>(Io<bf16_t>::out(d).bits) << 16);
-    *reinterpret_cast<uint2 *>(p) = make_uint2(lo, hi);
+    *reinterpret_cast<uint2 *>(p) = make_uint2(bf16_pack2(a, b), bf16_pack2(c, d));
 }
 
 // The same four elements as loaded, not yet widened: half the registers for the 16-bit types.
@@ -174,9 +168,13 @@ __device__ __forceinline__ void view_store4(__amdgpu_buffer_rsrc_t view, unsigne
         t.x = __float_as_uint(a); t.y = __float_as_uint(b); t.z = __float_as_uint(c); t.w = __float_as_uint(d);
         __builtin_amdgcn_raw_buffer_store_b128(t, view, off, 0, 0);
     } else {
-        union { IO e[4]; u32x2 u; } t;
-        t.e[0] = Io<IO>::out(a); t.e[1] = Io<IO>::out(b); t.e[2] = Io<IO>::out(c); t.e[3] = Io<IO>::out(d);
-        __builtin_amdgcn_raw_buffer_store_b64(t.u, view, off, 0, 0);
+        u32x2 t;
+        if constexpr (std::is_same<IO, bf16_t>::value) {
+            t.x = bf16_pack2(a, b); t.y = bf16_pack2(c, d);
+        } else {
+            t.x = f16_pack2(a, b); t.y = f16_pack2(c, d);
+        }
+        __builtin_amdgcn_raw_buffer_store_b64(t, view, off, 0, 0);
     }
 }
 
