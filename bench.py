@@ -332,9 +332,10 @@ def main():
     # measured HBM bytes per launch of that kernel, from the committed rocprofv3 --pmc summary (null if the
     # summary does not cover this variant)
     traffic = None
+    profiled = args.workload == "effnet_b0" and args.dtype == "f32" and args.batch == 128 and not args.only
     try:
         with open(os.path.join(ROOT, "profiles", "hbm_traffic.json" if args.layout == "nchw" else "hbm_traffic_nhwc.json")) as f:
-            traffic = json.load(f)["bytes_per_launch"].get(dom_name)
+            traffic = json.load(f)["bytes_per_launch"].get(dom_name) if profiled else None
     except (OSError, ValueError, KeyError):
         traffic = None
     # the device function behind the variant name, as rocprofv3 lists it (backward calls end with a ~4.5 us
