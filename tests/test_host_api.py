@@ -164,3 +164,29 @@ def test_package_exports():
 
     assert callable(torch_dwconv.depthwise_conv2d) and issubclass(torch_dwconv.DepthwiseConv2d, torch.nn.Module)
     from torch_dwconv.dwconv import DepthwiseConv2dFunction, depthwise_conv2d_fn, use_dwconv2d_small  # noqa: F401
+
+
+def test_product_code_never_reaches_for_the_oracle_or_working_files():
+    """The package under depthwise-conv-pytorch_amd/ is the product: it must not import the CPU oracle (test
+    infrastructure) or anything from the builder's working folder; bench.py may use the oracle only in its
+    cpu_baseline leg and the entry script only in smoke()."""
+    import re
+
+    pkg = os.path.join(ROOT, "depthwise-conv-pytorch_amd")
+    offenders = []
+    for folder, _, files in os.walk(pkg):
+        for name in files:
+            if not name.endswith((".py", ".hip", ".hpp", ".h", "Makefile")):
+                continue
+            text = open(os.path.join(folder, name), encoding="utf-8").read()
+            if re.search(r"^\s*(import|from)\s+oracle\b", text, re.M) or "_work/" in text or "oracle/" in text:
+                offenders.append(os.path.join(folder, name))
+    assert offenders == []
+    tracked = ["bench.py", "__graft_entry__.py", "include/dwconv_hip.h"]
+    for rel in tracked:
+        assert "_work/" not in open(os.path.join(ROOT, rel), encoding="utf-8").read(), rel
+    bench = open(os.path.join(ROOT, "bench.py"), encoding="utf-8").read()
+    uses = [m.start() for m in re.finditer(r"(import|from)\s+oracle\b", bench)]
+    start = bench.index("def cpu_baseline")
+    end = bench.index("\ndef ", start + 1)
+    assert uses and all(start < u < end for u in uses), "bench.py touches the oracle outside cpu_baseline()"
