@@ -131,11 +131,22 @@ class DepthwiseConv2dFunction(Function):
 depthwise_conv2d_fn = DepthwiseConv2dFunction.apply
 
 
+def _autocast(input, weight):
+    """Inside ``torch.autocast('cuda', dtype)`` both operands are cast to the autocast dtype, as PyTorch does for its own
+    convolutions (the casts are differentiable, so ``weight.grad`` keeps the parameter's dtype).  The reference has no
+    autocast rule: there a half-precision activation and an fp32 weight do not meet."""
+    if input.is_cuda and torch.is_autocast_enabled("cuda"):
+        dtype = torch.get_autocast_dtype("cuda")
+        return input.to(dtype), weight.to(dtype)
+    return input, weight
+
+
 def depthwise_conv2d(input, weight, bias=None, stride=1, padding=0, dilation=1, groups=None):
     """Reference: torch_dwconv/dwconv.py:115-130."""
     stride = make_tuple(stride, 2)
     padding = make_tuple(padding, 2)
     check_options(input.shape[1], weight.shape[0], dilation, groups, bias)
+    input, weight = _autocast(input, weight)
     small = use_dwconv2d_small(input, weight, (1, 1), stride, padding)
     return depthwise_conv2d_fn(input, weight, stride, padding, small)
 

@@ -14,7 +14,7 @@ from typing import List, Tuple
 import torch
 
 from . import _C
-from .dwconv import check_options, make_tuple
+from .dwconv import _autocast, check_options, make_tuple
 
 
 def _out_hw(h: int, w: int, kh: int, kw: int, stride: List[int], padding: List[int]) -> Tuple[int, int]:
@@ -71,4 +71,5 @@ def compiled_depthwise_conv2d(input, weight, bias=None, stride=1, padding=0, dil
     stride = list(make_tuple(stride, 2))
     padding = list(make_tuple(padding, 2))
     check_options(input.shape[1], weight.shape[0], dilation, groups, bias)
+    input, weight = _autocast(input, weight)
     return depthwise_conv2d_op(input, weight, stride, padding)

@@ -426,6 +426,29 @@ def test_module_matches_plain_conv(dw, gpu):
     torch.testing.assert_close(gw, m.weight.grad, rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+def test_autocast_casts_both_operands(dw, gpu, dtype):
+    """Under torch.autocast an fp32 activation and an fp32 parameter run in the autocast dtype, like F.conv2d; the
+    gradients come back in the dtypes of the leaves."""
+    shape = (2, 8, 28, 28, 3, 1, 1)
+    x, wt, gy = make_inputs(shape, seed=31)
+    xg = x.to(gpu).requires_grad_(True)
+    wg = wt.to(gpu).requires_grad_(True)
+    with torch.autocast("cuda", dtype=dtype):
+        y = dw.depthwise_conv2d(xg, wg, padding=1)
+        y_torch = torch.nn.functional.conv2d(xg, wg, padding=1, groups=8)
+    assert y.dtype == dtype == y_torch.dtype
+    gx, gw = torch.autograd.grad(y, (xg, wg), gy.to(gpu).to(dtype))
+    assert gx.dtype == torch.float32 and gw.dtype == torch.float32
+    y_ref, gx_ref, gw_ref = oracle.torch_reference(x.to(dtype), wt.to(dtype), gy.to(dtype), 1, 1)
+    step = 2.0 ** -11 if dtype == torch.float16 else 2.0 ** -8
+    np.testing.assert_allclose(_np(y.double()), _np(y_ref), rtol=step, atol=1e-5 + step * 1e-2)
+    np.testing.assert_allclose(_np(gx.double()), _np(gx_ref), rtol=step, atol=1e-5 + step * 1e-2)
+    np.testing.assert_allclose(_np(gw.double()), _np(gw_ref), rtol=step + 1e-4, atol=(step + 1e-4) * float(gw_ref.abs().max()))
+    # outside autocast nothing is cast
+    assert dw.depthwise_conv2d(xg, wg, padding=1).dtype == torch.float32
+
+
 def test_runs_on_the_current_stream(dw, gpu):
     x = torch.randn(4, 8, 64, 64, device=gpu)
     w = torch.randn(8, 1, 3, 3, device=gpu)
