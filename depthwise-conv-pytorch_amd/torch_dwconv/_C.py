@@ -268,8 +268,10 @@ def dwconv2d_nhwc(input, kernel, stride_h, stride_w, pad_h, pad_w):
     return out
 
 
-def dwconv2d_backward_nhwc(input, out_grad, kernel, stride_h, stride_w, pad_h, pad_w):
-    """Both gradients for channels-last ``input`` / ``out_grad``; ``grad_input`` comes back channels-last."""
+def dwconv2d_backward_nhwc(input, out_grad, kernel, stride_h, stride_w, pad_h, pad_w, need_input_grad=True,
+                           need_kernel_grad=True):
+    """Both gradients for channels-last ``input`` / ``out_grad``; ``grad_input`` comes back channels-last.  A gradient
+    that is not needed is not computed and comes back as ``None``."""
     _check_cuda(input, "input")
     _check_cuda(out_grad, "out_grad")
     _check_cuda(kernel, "kernel")
@@ -283,14 +285,17 @@ def dwconv2d_backward_nhwc(input, out_grad, kernel, stride_h, stride_w, pad_h, p
     n, c, h, w = x.shape
     oh, ow = gy.shape[2], gy.shape[3]
     kh, kw = k.shape[2], k.shape[3]
-    gx = torch.empty_like(x, memory_format=torch.channels_last)
-    gw = torch.empty_like(k)
+    if not (need_input_grad or need_kernel_grad):
+        return None, None
+    gx = torch.empty_like(x, memory_format=torch.channels_last) if need_input_grad else None
+    gw = torch.empty_like(k) if need_kernel_grad else None
     ws_bytes = _lib.dwconv2d_backward_nhwc_workspace_bytes(n, c, h, w, kh, kw, stride_h, stride_w, pad_h, pad_w,
                                                            x.element_size())
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):
         rc = getattr(_lib, "dwconv2d_backward_nhwc_" + sfx)(
-            x.data_ptr(), gy.data_ptr(), k.data_ptr(), gx.data_ptr(), gw.data_ptr(), ws.data_ptr(), ws_bytes,
+            x.data_ptr(), gy.data_ptr(), k.data_ptr(), gx.data_ptr() if need_input_grad else None,
+            gw.data_ptr() if need_kernel_grad else None, ws.data_ptr(), ws_bytes,
             n, c, h, w, oh, ow, kh, kw, stride_h, stride_w, pad_h, pad_w, _stream(x),
         )
     if rc != 0:

@@ -104,27 +104,31 @@ class DepthwiseConv2dFunction(Function):
     def backward(ctx, grad_output):
         input, kernel = ctx.saved_tensors
         stride, pad, g_pad = ctx.stride, ctx.pad, ctx.g_pad
-        # The reference always computes both gradients (:48-70).
+        # The reference always computes both gradients (:48-70).  Here a gradient nobody asked for (a frozen filter, the
+        # network's first layer) is skipped: autograd takes None for it.
+        need_input, need_kernel = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         if ctx.channels_last:
             grad_input, grad_kernel = _C.dwconv2d_backward_nhwc(
-                input, grad_output, kernel, stride[0], stride[1], pad[0], pad[1]
+                input, grad_output, kernel, stride[0], stride[1], pad[0], pad[1], need_input, need_kernel
             )
             return grad_input, grad_kernel, None, None, None, None
-        if input.dtype != torch.float64:
+        if input.dtype != torch.float64 and need_input and need_kernel:
             # one library call for the pair of calls below; same values, out_grad read once where fused
             grad_input, grad_kernel = _C.dwconv2d_backward(
                 input, grad_output, kernel, stride[0], stride[1], pad[0], pad[1]
             )
             return grad_input, grad_kernel, None, None, None, None
-        if ctx.use_small:
+        grad_input = grad_kernel = None
+        if need_input and ctx.use_small:
             grad_input = _C.dwconv2d_small(
                 grad_output, kernel, stride[0], stride[1], 1, 1, g_pad[0], g_pad[2], False
             )
-        else:
+        elif need_input:
             grad_input = _C.dwconv2d(grad_output, kernel, stride[0], stride[1], 1, 1, *g_pad, False)
-        grad_kernel = _C.dwconv2d_backward_kernel(
-            input, grad_output, kernel, 1, 1, stride[0], stride[1], pad[0], pad[1]
-        )
+        if need_kernel:
+            grad_kernel = _C.dwconv2d_backward_kernel(
+                input, grad_output, kernel, 1, 1, stride[0], stride[1], pad[0], pad[1]
+            )
         return grad_input, grad_kernel, None, None, None, None
 
 

@@ -449,6 +449,26 @@ def test_autocast_casts_both_operands(dw, gpu, dtype):
     assert dw.depthwise_conv2d(xg, wg, padding=1).dtype == torch.float32
 
 
+@pytest.mark.parametrize("layout", ["nchw", "nhwc"])
+def test_only_the_requested_gradients_are_computed(dw, gpu, layout):
+    """A leaf that does not require a gradient gets none (and costs no kernel); the other gradient is unchanged."""
+    shape = (3, 8, 28, 28, 5, 2, 2)
+    x, wt, gy = (t.to(gpu) for t in make_inputs(shape, seed=37))
+    if layout == "nhwc":
+        x, gy = (t.contiguous(memory_format=torch.channels_last) for t in (x, gy))
+    _, gx_both, gw_both, _ = run_three_passes(dw, x, wt, gy, 2, 2)
+    for need_x, need_w in [(True, False), (False, True)]:
+        xg = x.detach().clone().requires_grad_(need_x)
+        wg = wt.detach().clone().requires_grad_(need_w)
+        dw.depthwise_conv2d(xg, wg, stride=2, padding=2).backward(gy)
+        if need_x:
+            assert wg.grad is None
+            torch.testing.assert_close(xg.grad, gx_both, rtol=1e-6, atol=1e-6)
+        else:
+            assert xg.grad is None
+            torch.testing.assert_close(wg.grad, gw_both, rtol=1e-5, atol=1e-5)
+
+
 def test_runs_on_the_current_stream(dw, gpu):
     x = torch.randn(4, 8, 64, 64, device=gpu)
     w = torch.randn(8, 1, 3, 3, device=gpu)
