@@ -288,6 +288,9 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_wgrad_kernel(const NhwcPlan
     constexpr int KK = K * K;
     constexpr int ROWS = (BH - 1) * S + K, COLS = (TW - 1) * S + K;
     const int C = p.channel;
+    // (grid: chunk x channel group, dealt to the XCDs round-robin; giving every XCD a contiguous run of chunks,
+    // as the forward kernel does with its pixel groups, measured 2 % slower here)
+    const int chunk = blockIdx.x;
     const int c0 = blockIdx.y * p.lanes_c * CV;
     const int nch = min(p.lanes_c * CV, C - c0);
     const int pb_local = fast_div(threadIdx.x, p.lanes_c_magic);
@@ -302,7 +305,7 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_wgrad_kernel(const NhwcPlan
 #pragma unroll
         for (int v = 0; v < CV; ++v) acc[t][v] = 0.f;
 
-    for (long grp = blockIdx.x; grp * p.blocks_per_wg < p.blocks_total; grp += p.groups) {
+    for (long grp = chunk; grp * p.blocks_per_wg < p.blocks_total; grp += p.groups) {
         const long pb = grp * p.blocks_per_wg + pb_local;
         if (!lane_ok || pb >= p.blocks_total) continue;
         const int n = static_cast<int>(pb / per_image);
@@ -352,7 +355,7 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_wgrad_kernel(const NhwcPlan
 
     // Lanes that share channels (same lane_c, different pixel block) are added front to back, one tap row at a time.
     const int width = p.lanes_c * CV;  // floats per (pixel block, tap) line in LDS
-    float *out = p.partial + static_cast<long>(blockIdx.x) * KK * C;
+    float *out = p.partial + static_cast<long>(chunk) * KK * C;
 #pragma unroll
     for (int ty = 0; ty < K; ++ty) {
         if (ty) __syncthreads();
@@ -529,7 +532,7 @@ int pick_lanes_c(int lanes, int cap)
 }
 
 template <int K, int CV>
-bool plan_nhwc(NhwcPlan &p, const NhwcGeometry &g, int bh, int tw, int blocks_h, int blocks_w)
+bool plan_nhwc(NhwcPlan &p, const NhwcGeometry &g, int bh, int tw, int blocks_h, int blocks_w, int min_lanes = 1)
 {
     p.batch = g.batch;
     p.channel = g.channel;
@@ -537,7 +540,8 @@ bool plan_nhwc(NhwcPlan &p, const NhwcGeometry &g, int bh, int tw, int blocks_h,
     // images), so halo pixels are shared inside the workgroup's L1 instead of between workgroups.  Measured on
     // the EfficientNet-B0 layers: 8 lanes win on 7x7 and 14x14 maps, 16 on 28x28, 64 on larger ones.
     const long pixels = static_cast<long>(g.in_h) * g.in_w;
-    int cap = env_int("DWCONV_NHWC_LANES", pixels <= 256 ? 8 : pixels <= 1024 ? 16 : 64);
+    int cap = pixels <= 256 ? 8 : pixels <= 1024 ? 16 : 64;
+    cap = env_int("DWCONV_NHWC_LANES", std::max(cap, min_lanes));
     cap = std::max(1, std::min(cap, 64));
     while (cap > 1 && static_cast<size_t>(cap) * CV * K * K * 4 > static_cast<size_t>(kNhwcTapLds)) --cap;
     p.lanes_c = pick_lanes_c(g.channel / CV, cap);
@@ -638,7 +642,12 @@ long nhwc_wgrad_case(int mode, const IO *x, const IO *gy, IO *gw, void *ws, size
 {
     constexpr int CV = WgradShape<K>::CV, BH = WgradShape<K>::BH, TW = WgradShape<K>::TW;
     NhwcPlan p{};
-    if (!plan_nhwc<1, CV>(p, g, BH, TW, g.out_h, g.out_w)) return -1;
+    // At least a 128-byte line of every pixel per workgroup: with fewer channel lanes the other part of the line
+    // belongs to another workgroup, on another XCD as likely as not, and is fetched from HBM twice (measured on the
+    // 5x5 layers, which run two channels per lane: 2.2 x the bytes of x and gy).  The forward and grad-input
+    // kernels (four channels per lane) already cover a line in fp32 and did not gain from it with 16-bit elements.
+    const int line_lanes = env_int("DWCONV_NHWC_FULL_LINES", 1) ? static_cast<int>(128 / (CV * sizeof(IO))) : 1;
+    if (!plan_nhwc<1, CV>(p, g, BH, TW, g.out_h, g.out_w, line_lanes)) return -1;
     const int cgroups = p.cgroups;
     const long wg_iters = (p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg;
     long groups = env_int("DWCONV_NHWC_WGRAD_WGS", 1024) / cgroups;
