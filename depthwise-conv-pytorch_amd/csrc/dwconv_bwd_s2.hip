@@ -80,8 +80,11 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
     constexpr int XW_ROWS = (BQ - 1) * 2 + K;         // x window rows
     constexpr int NVX = (K + 2 + 3) / 4;              // x window columns, as float4s
 
-    const int c = blockIdx.x / p.chunks;
-    const int chunk = blockIdx.x - c * p.chunks;
+    // every XCD (own L2) gets a contiguous run of workgroups: chunks k and k + 1 of a channel walk neighbouring
+    // bands in step and share their halo rows (-2 % on the 112x112 layer)
+    const int wg = xcd_contiguous_tile(blockIdx.x, gridDim.x);
+    const int c = wg / p.chunks;
+    const int chunk = wg - c * p.chunks;
 
     const bool has_item = static_cast<int>(threadIdx.x) < p.n_items;
     const int item = has_item ? threadIdx.x : 0;
