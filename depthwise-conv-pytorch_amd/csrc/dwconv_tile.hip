@@ -47,6 +47,7 @@ struct TilePlan {
     unsigned ipp_magic;
     int tap_base;              // float offset of the tap table in LDS
     int vec_out;               // 128-bit global stores are legal
+    int lds_out;               // fir_down: results go back through LDS and out as one linear stream per plane
     Epilogue epi;              // forward kernels: applied to every sum before it is stored
 };
 
@@ -82,19 +83,13 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
     __syncthreads();
 
     const int n_items = nplanes * p.items_per_plane;
-    for (int item = threadIdx.x; item < n_items; item += blockDim.x) {
-        // (24-bit multiplies: full rate, and every operand here is an LDS-sized quantity)
-        const int pl = fast_div(item, p.ipp_magic);
-        const int rem = item - __mul24(pl, p.items_per_plane);
-        const int rb = fast_div(rem, p.ncb_magic);
-        const int cb = rem - __mul24(rb, p.ncb);
-
+    // the block of BH x 4 sums of one item
+    auto convolve = [&](int pl, int rb, int cb, float(&acc)[BH][4]) {
         float tapv[KK];
 #pragma unroll
         for (int t = 0; t < KK; ++t) tapv[t] = lds[p.tap_base + pl * KK + t];
 
         const float *base = lds + __mul24(pl, p.st.plane_pitch) + __mul24(rb * BH * S, p.st.pitch) + kSlack + 4 * cb * S;
-        float acc[BH][4];
 #pragma unroll
         for (int b = 0; b < BH; ++b)
 #pragma unroll
@@ -127,6 +122,51 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
                 epilogue_apply_block<1>(acc, p.epi, static_cast<int>((plane0 + pl) % p.channel));
             }
         }
+    };
+
+    if (p.lds_out) {
+        // One item per lane (the planner guarantees it).  The sums go back into LDS in the layout the band has in
+        // memory, over the input image, and leave as one linear stream per plane: every store instruction of a
+        // wavefront then covers 1 KiB of consecutive bytes, where lane-owned blocks write a row segment at a time
+        // and leave the 128-byte lines that straddle two rows to two partial writes.
+        const bool has_item = static_cast<int>(threadIdx.x) < n_items;
+        const int item = has_item ? threadIdx.x : 0;
+        const int pl = fast_div(item, p.ipp_magic);
+        const int rem = item - __mul24(pl, p.items_per_plane);
+        const int rb = fast_div(rem, p.ncb_magic);
+        const int cb = rem - __mul24(rb, p.ncb);
+        float acc[BH][4];
+        convolve(pl, rb, cb, acc);
+        const int rows_here = min(p.rows_per_tile, p.out_h - oy0);
+        const int run = rows_here * p.out_w;  // elements per plane, a multiple of four
+        __syncthreads();  // every window has been read: the image can be overwritten
+        if (has_item) {
+#pragma unroll
+            for (int b = 0; b < BH; ++b)
+                if (rb * BH + b < rows_here)
+                    *reinterpret_cast<float4 *>(lds + pl * run + (rb * BH + b) * p.out_w + 4 * cb) =
+                        make_float4(acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+        }
+        __syncthreads();
+        const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane);
+        const int run4 = run >> 2, total4 = nplanes * run4;
+        for (int i = threadIdx.x; i < total4; i += blockDim.x) {
+            const int q = nplanes == 1 ? 0 : i / run4;
+            const float4 v = reinterpret_cast<const float4 *>(lds)[i];
+            const unsigned off = (q * p.out_plane + oy0 * p.out_w + (i - q * run4) * 4) * static_cast<unsigned>(sizeof(IO));
+            view_store4<IO>(view, off, v.x, v.y, v.z, v.w);
+        }
+        return;
+    }
+
+    for (int item = threadIdx.x; item < n_items; item += blockDim.x) {
+        // (24-bit multiplies: full rate, and every operand here is an LDS-sized quantity)
+        const int pl = fast_div(item, p.ipp_magic);
+        const int rem = item - __mul24(pl, p.items_per_plane);
+        const int rb = fast_div(rem, p.ncb_magic);
+        const int cb = rem - __mul24(rb, p.ncb);
+        float acc[BH][4];
+        convolve(pl, rb, cb, acc);
         const int ox = 4 * cb;
         if (p.vec_out == 2) {
             // branch-free: rows past the end of the plane store out of range
@@ -333,10 +373,16 @@ int launch_down(TilePlan &p, hipStream_t stream)
     if (!plan_tiles(p, ceil_div(p.out_h, BH), BH, used_cols, K * K, rows_for)) return -1;
     if (p.st.vec_in) p.st.vec_in = stage_vector_mode(p.st, p.planes_per_tile, sizeof(IO));
     if (p.vec_out) p.vec_out = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
+    // Results through LDS: measured to pay where a workgroup owns a whole fp32 plane of a 3x3 stride-1 layer whose
+    // rows are not whole 128-byte lines (56x56: -10 %); neutral or worse elsewhere (+2 % with 16-bit elements, +9 %
+    // on a 5x5 stride-2 layer).
+    const bool lds_out_pays = sizeof(IO) == 4 && K == 3 && S == 1 && p.row_tiles == 1 && (p.out_w * sizeof(IO)) % 128 != 0;
+    p.lds_out = env_int("DWCONV_TILE_LDS_OUT", lds_out_pays) && p.vec_out == 2 &&
+                p.planes_per_tile * p.items_per_plane <= env_int("DWCONV_TILE_THREADS", kThreads);
     hipLaunchKernelGGL((fir_down_kernel<IO, K, S, FLIP, BH>), dim3(p.n_tiles), dim3(env_int("DWCONV_TILE_THREADS", kThreads)), lds_bytes(p, K * K),
                        stream, p);
-    note_variant("tile_down%s<k%d,s%d,%s,bh%d> P%d rows%d vin%d vout%d", sizeof(IO) == 2 ? "16" : "", K, S, FLIP ? "rot" : "fwd", BH,
-                 p.planes_per_tile, p.rows_per_tile, p.st.vec_in, p.vec_out);
+    note_variant("tile_down%s<k%d,s%d,%s,bh%d> P%d rows%d vin%d vout%d%s", sizeof(IO) == 2 ? "16" : "", K, S, FLIP ? "rot" : "fwd", BH,
+                 p.planes_per_tile, p.rows_per_tile, p.st.vec_in, p.vec_out, p.lds_out ? " ldsout" : "");
     return check_launch("fir_down_kernel");
 }
 
