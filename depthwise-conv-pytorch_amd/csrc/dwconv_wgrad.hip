@@ -328,6 +328,7 @@ bool make_plan(WgradPlan &p, const WgradGeometry &g, bool fused)
     auto tile_bytes = [&](int units, int planes) {
         return static_cast<long>(planes) * rows_for(units) * p.st.pitch * 4 * (fused ? 2 : 1);
     };
+    const int kLdsBudget = env_int("DWCONV_WGRAD_LDS", dwconv::kLdsBudget);
     const int row_units = ceil_div(g.out_h, BH);
     const int ipp_full = row_units * p.ncb;
     int units_per_tile, planes_per_tile;
