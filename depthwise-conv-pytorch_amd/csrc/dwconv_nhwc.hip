@@ -650,7 +650,9 @@ long nhwc_wgrad_case(int mode, const IO *x, const IO *gy, IO *gw, void *ws, size
     if (!plan_nhwc<1, CV>(p, g, BH, TW, g.out_h, g.out_w, line_lanes)) return -1;
     const int cgroups = p.cgroups;
     const long wg_iters = (p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg;
-    long groups = env_int("DWCONV_NHWC_WGRAD_WGS", 1024) / cgroups;
+    // One resident round of workgroups: the kernel's 170-250 registers leave two wavefronts per SIMD, i.e. two
+    // 256-lane workgroups on each of the 256 CUs (measured: 512 beats 256, 384, 640, 768 and 1024 by 3-10 %).
+    long groups = env_int("DWCONV_NHWC_WGRAD_WGS", 512) / cgroups;
     groups = std::max(1l, std::min(groups, wg_iters));
     p.groups = static_cast<int>(groups);
     const size_t need = static_cast<size_t>(groups) * K * K * g.channel * sizeof(float);
