@@ -216,10 +216,12 @@ constexpr int kStageBatch = 4;
 // VIEW_ONLY: the caller guarantees s.vec_in == 2, and the other two ways of loading are not compiled in.  The
 // kernels keep an instance of each kind: with every alternative in one body, the values the unused ones need
 // stay live and push the scalar registers past what the hardware has.
-template <typename IO, bool VIEW_ONLY = false>
+// BATCH: loads a lane has in flight at a time (kStageBatch unless a kernel measured better with another number).
+template <typename IO, bool VIEW_ONLY = false, int BATCH = kStageBatch>
 __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__restrict__ in, float *lds,
                                            long plane0, int nplanes, int iy0)
 {
+    constexpr int kStageBatch = BATCH;  // shadows the default within this function
     const int total = nplanes * s.lds_rows * s.spr;
     if (VIEW_ONLY || s.vec_in == 2) {
         // groups of four elements through a view of the tile's planes: slots outside the image read zeros
