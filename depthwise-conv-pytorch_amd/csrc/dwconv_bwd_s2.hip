@@ -224,7 +224,7 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
 }
 
 template <int K>
-bool plan_bwd_s2(BwdS2Plan &p, const WgradGeometry &g, int kBq)
+bool plan_bwd_s2(BwdS2Plan &p, const WgradGeometry &g, int kBq, size_t esize)
 {
     const int pad0 = K - 1 - g.pad_h;  // leading pad of the transposed problem
     const int E = pad0 & 1;
@@ -274,7 +274,11 @@ bool plan_bwd_s2(BwdS2Plan &p, const WgradGeometry &g, int kBq)
     const long tiles = static_cast<long>(g.batch) * bands;
     if (tiles > 0x7fffffffL) return false;
     p.tiles_per_group = static_cast<int>(tiles);
-    int chunks = ceil_div(env_int("DWCONV_WGRAD_WGS", 3072), g.channel);
+    // Workgroups in all.  The fp32 5x5 / 7x7 kernels gain from four times as many, shorter chunks (-7 % on a
+    // 56x56 layer, -4 % at 128x96); the 3x3 one does not, and with 16-bit elements, where the kernel is bound by
+    // instruction issue, the per-workgroup prologue and reduction make more chunks 8-15 % slower.
+    const int wgs = K >= 5 && esize == 4 ? 12288 : 3072;
+    int chunks = ceil_div(env_int("DWCONV_WGRAD_WGS", wgs), g.channel);
     if (chunks > p.tiles_per_group) chunks = p.tiles_per_group;
     if (chunks < 1) chunks = 1;
     p.chunks = chunks;
@@ -290,7 +294,7 @@ long bwd_s2_case(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO
     const int qrows = std::max((g.in_h + 1) / 2, g.out_h), pairs = ceil_div(std::max((g.in_w + 1) / 2, g.out_w), 2);
     const int bq = ceil_div(qrows, 4) * pairs * 2 <= kThreads ? 2 : 4;
     BwdS2Plan p{};
-    if (!plan_bwd_s2<K>(p, g, bq)) return -1;
+    if (!plan_bwd_s2<K>(p, g, bq, sizeof(IO))) return -1;
     const size_t need = static_cast<size_t>(g.channel) * p.chunks * K * K * sizeof(float);
     if (mode == 0) return static_cast<long>(need);
     if (ws == nullptr || ws_bytes < need)
