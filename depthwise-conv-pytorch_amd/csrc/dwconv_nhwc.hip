@@ -516,12 +516,20 @@ __global__ __launch_bounds__(256) void nhwc_gw_direct_final_kernel(const float *
 }
 
 // ---- planning -------------------------------------------------------------------------------------------
-// Channel lanes per workgroup: the largest divisor of `lanes` (= C / CV) that is at most `cap`, so that no
-// workgroup straddles the end of the channel axis; at least 8 (half a 128-byte line of fp32 float4 lanes)
-// or the cap itself when the divisors are all tiny.
-int pick_lanes_c(int lanes, int cap)
+// Channel lanes per workgroup, at most `cap`.  All of C when it fits (then the pixels of a row are one contiguous
+// run).  Otherwise a multiple of `line` lanes (= one 128-byte line of fp32 channels), so that every pixel's
+// segment starts and ends on a line: the largest such divisor of `lanes` (= C / CV), else the largest such
+// count below the cap, whose last channel group is then partly idle.  A segment that is not whole lines makes
+// every load fetch the lines at its ends in full (C = 240 in groups of 60 channels: 240-byte segments cost
+// 384 bytes of L1-to-L2 requests each, and the 28x28 layers ran 1.3-1.6 x slower than with 128-byte ones).
+int pick_lanes_c(int lanes, int cap, int line)
 {
     if (lanes <= cap) return lanes;
+    if (line > 1 && cap >= line) {
+        for (int d = cap / line * line; d >= line; d -= line)
+            if (lanes % d == 0) return d;
+        return cap / line * line;
+    }
     int best = 1;
     for (int d = cap; d >= 1; --d)
         if (lanes % d == 0) {
@@ -532,7 +540,8 @@ int pick_lanes_c(int lanes, int cap)
 }
 
 template <int K, int CV>
-bool plan_nhwc(NhwcPlan &p, const NhwcGeometry &g, int bh, int tw, int blocks_h, int blocks_w, int min_lanes = 1)
+bool plan_nhwc(NhwcPlan &p, const NhwcGeometry &g, int bh, int tw, int blocks_h, int blocks_w, int min_lanes = 1,
+               const char *lanes_env = "DWCONV_NHWC_LANES")
 {
     p.batch = g.batch;
     p.channel = g.channel;
@@ -541,10 +550,10 @@ bool plan_nhwc(NhwcPlan &p, const NhwcGeometry &g, int bh, int tw, int blocks_h,
     // the EfficientNet-B0 layers: 8 lanes win on 7x7 and 14x14 maps, 16 on 28x28, 64 on larger ones.
     const long pixels = static_cast<long>(g.in_h) * g.in_w;
     int cap = pixels <= 256 ? 8 : pixels <= 1024 ? 16 : 64;
-    cap = env_int("DWCONV_NHWC_LANES", std::max(cap, min_lanes));
+    cap = env_int(lanes_env, std::max(cap, min_lanes));
     cap = std::max(1, std::min(cap, 64));
     while (cap > 1 && static_cast<size_t>(cap) * CV * K * K * 4 > static_cast<size_t>(kNhwcTapLds)) --cap;
-    p.lanes_c = pick_lanes_c(g.channel / CV, cap);
+    p.lanes_c = pick_lanes_c(g.channel / CV, cap, env_int("DWCONV_NHWC_ALIGN", 1) ? 32 / CV : 1);
     p.lanes_c_magic = magic_u16(p.lanes_c);
     p.blocks_per_wg = kNhwcThreads / p.lanes_c;
     p.blocks_y = ceil_div(blocks_h, bh);
@@ -647,7 +656,7 @@ long nhwc_wgrad_case(int mode, const IO *x, const IO *gy, IO *gw, void *ws, size
     // 5x5 layers, which run two channels per lane: 2.2 x the bytes of x and gy).  The forward and grad-input
     // kernels (four channels per lane) already cover a line in fp32 and did not gain from it with 16-bit elements.
     const int line_lanes = env_int("DWCONV_NHWC_FULL_LINES", 1) ? static_cast<int>(128 / (CV * sizeof(IO))) : 1;
-    if (!plan_nhwc<1, CV>(p, g, BH, TW, g.out_h, g.out_w, line_lanes)) return -1;
+    if (!plan_nhwc<1, CV>(p, g, BH, TW, g.out_h, g.out_w, line_lanes, "DWCONV_NHWC_WGRAD_LANES")) return -1;
     const int cgroups = p.cgroups;
     const long wg_iters = (p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg;
     // One resident round of workgroups: the kernel's 170-250 registers leave two wavefronts per SIMD, i.e. two
