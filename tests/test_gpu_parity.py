@@ -532,6 +532,8 @@ NHWC_SHAPES = [
     (2, 8, 12, 12, 5, 2, 0), (1, 4, 10, 9, 3, 2, 2), (2, 20, 6, 5, 5, 1, 4), (1, 260, 5, 5, 3, 1, 1),
     (3, 1152, 7, 7, 3, 1, 1), (2, 8, 1, 9, 3, 1, 1), (2, 8, 9, 1, 3, 2, 1), (2, 4, 33, 35, 5, 2, 1),
     (2, 3, 9, 11, 3, 1, 1), (1, 6, 8, 8, 4, 2, 1), (2, 5, 7, 7, 1, 1, 0), (1, 2, 12, 10, 9, 1, 4),
+    # channel groups of whole 128-byte lines whose last group is partly idle (C / 4 = 60 lanes in groups of 16, 18 in groups of 8)
+    (2, 240, 28, 28, 5, 1, 2), (2, 240, 28, 28, 3, 2, 1), (1, 72, 14, 14, 3, 1, 1),
 ]
 
 
@@ -567,6 +569,15 @@ def test_channels_last_matches_oracle(dw, gpu, shape):
     np.testing.assert_allclose(_np(gw).astype(np.float64), gw_ref, rtol=1e-4, atol=1e-4 * np.abs(gw_ref).max())
     _, gw2 = torch.autograd.grad(dw.depthwise_conv2d(xg, wg, stride=s, padding=p), (xg, wg), _channels_last(gy, gpu))
     assert torch.equal(gw, gw2)
+
+
+def test_channels_last_channel_groups_are_whole_lines(dw, gpu):
+    """C = 240 on a 28x28 map: the workgroups take 16 channel lanes (256 bytes per pixel), not the 15 that divide C / 4."""
+    from torch_dwconv import _C
+
+    x = _channels_last(torch.randn(2, 240, 28, 28), gpu)
+    dw.depthwise_conv2d(x, torch.randn(240, 1, 5, 5, device=gpu), padding=2)
+    assert _C.last_variant().endswith("lanes_c16"), _C.last_variant()
 
 
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float16, torch.bfloat16], ids=["f64", "f16", "bf16"])
