@@ -322,13 +322,13 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_wgrad_kernel(const NhwcPlan
             buffer_view(static_cast<const IO *>(p.in2) + static_cast<long>(n0) * p.out_h * p.out_w * C);
         const unsigned chan_off = c * static_cast<unsigned>(sizeof(IO));
 
+        // out_grad rows are fetched one window row before their first use (row b meets window rows b*S ... b*S+K-1),
+        // so a tall block keeps only the rows in use in registers (the loop is unrolled: a row's registers are
+        // free again after its last use)
         float g[BH][TW * CV];
-        {
-            NhwcCols<TW> gcols;
-            nhwc_cols<TW>(ox0, p.out_w, pixel_bytes, (n - n0) * (p.out_h * grow_bytes) + chan_off, gcols);
-#pragma unroll
-            for (int b = 0; b < BH; ++b) nhwc_load_row<IO, TW, CV>(gview, oy0 + b, p.out_h, grow_bytes, gcols, g[b]);
-        }
+        NhwcCols<TW> gcols;
+        nhwc_cols<TW>(ox0, p.out_w, pixel_bytes, (n - n0) * (p.out_h * grow_bytes) + chan_off, gcols);
+        nhwc_load_row<IO, TW, CV>(gview, oy0, p.out_h, grow_bytes, gcols, g[0]);
         float rows[2][COLS * CV];
         NhwcCols<COLS> cols;
         nhwc_cols<COLS>(ix0, p.in_w, pixel_bytes, (n - n0) * (p.in_h * row_bytes) + chan_off, cols);
@@ -337,10 +337,15 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_wgrad_kernel(const NhwcPlan
         for (int r = 0; r < ROWS; ++r) {
             float(&cur)[COLS * CV] = rows[r & 1];
             if (r + 1 < ROWS) nhwc_load_row<IO, COLS, CV>(xview, iy0 + r + 1, p.in_h, row_bytes, cols, rows[(r + 1) & 1]);
+            if ((r + 1) % S == 0 && (r + 1) / S < BH)
+                nhwc_load_row<IO, TW, CV>(gview, oy0 + (r + 1) / S, p.out_h, grow_bytes, gcols, g[(r + 1) / S]);
+            // window row r meets out_grad row b in tap row ty = r - b*S (looping over ty keeps the body small
+            // enough for the unroller whatever BH is)
 #pragma unroll
-            for (int b = 0; b < BH; ++b) {
-                const int ty = r - b * S;
-                if (ty < 0 || ty >= K) continue;
+            for (int ty = 0; ty < K; ++ty) {
+                const int bs = r - ty;
+                if (bs < 0 || bs % S != 0 || bs / S >= BH) continue;
+                const int b = bs / S;
 #pragma unroll
                 for (int tx = 0; tx < K; ++tx)
 #pragma unroll
@@ -640,7 +645,11 @@ template <int K>
 struct WgradShape {
     // K*K*CV sums live in registers: 36 for 3x3 with four channels per lane, 50 / 98 with two for 5x5 / 7x7
     static constexpr int CV = K == 3 ? 4 : 2;
-    static constexpr int BH = K == 7 ? 2 : 4;
+    // Seven output rows per block for 3x3 and 5x5: the K - 1 halo rows of x are fetched for seven rows instead of
+    // four (fewer L1-to-L2 requests, which is what bounds these kernels; -2 % on the EfficientNet-B0 step), and 7
+    // divides the map heights of the usual networks.  Only the rows of out_grad in use are live, so the block
+    // height costs no registers.  The 7x7 kernel is bound by its arithmetic and runs faster with two rows.
+    static constexpr int BH = K == 7 ? 2 : 7;
     static constexpr int TW = 4;
 };
 
