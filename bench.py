@@ -370,7 +370,8 @@ def main():
                 "small_wgrad": "small_bwd_kernel + wgrad_tile_final_kernel",
                 "bwd_tile": "wgrad_tile_kernel + wgrad_tile_final_kernel",
                 "wgrad_tile": "wgrad_tile_kernel + wgrad_tile_final_kernel",
-                "bwd_tile_s2": "bwd_s2_kernel + wgrad_tile_final_kernel"}.get(family, family)
+                "bwd_tile_s2": "bwd_s2_kernel + wgrad_tile_final_kernel",
+                "nhwc_bwd": "nhwc_bwd_fused_kernel + nhwc_wgrad_final_kernel"}.get(family, family)
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": dom_name, "kernel_function": function,
                 "launches_per_step": dom["launches"], "avg_launch_us": round(dom["ms"] * 1e3 / dom["launches"], 1),

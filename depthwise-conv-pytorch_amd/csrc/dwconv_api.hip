@@ -314,6 +314,10 @@ int nhwc_backward_any(const T *in, const T *gy, const T *taps, T *gx, T *gw, voi
     if (has_out && gy == nullptr) return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     char first[sizeof(g_variant)] = "";
+    if (gx != nullptr && gw != nullptr && has_out && in != nullptr && taps != nullptr) {
+        rc = nhwc_backward_fused<T>(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+        if (rc >= 0) return rc;
+    }
     if (gx != nullptr) {
         if (has_out && taps == nullptr) return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");
         rc = nhwc_grad_input<T>(gy, taps, gx, g, stream);

@@ -255,6 +255,9 @@ int nhwc_forward(const T *in, const T *taps, T *out, const NhwcGeometry &g, hipS
 template <typename T>
 int nhwc_grad_input(const T *gy, const T *taps, T *gx, const NhwcGeometry &g, hipStream_t stream);
 template <typename T>
+int nhwc_backward_fused(const T *x, const T *gy, const T *taps, T *gx, T *gw, void *ws, size_t ws_bytes,
+                        const NhwcGeometry &g, hipStream_t stream);
+template <typename T>
 size_t nhwc_grad_weight_workspace(const NhwcGeometry &g);
 template <typename T>
 int nhwc_grad_weight(const T *x, const T *gy, T *gw, void *ws, size_t ws_bytes, const NhwcGeometry &g,

@@ -380,6 +380,151 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_wgrad_kernel(const NhwcPlan
     }
 }
 
+// Grad-input and grad-weight of a stride-1 layer whose output has the extent of its input (pad = K / 2) in one
+// sweep: in = x, in2 = out_grad, out = in_grad, all H x W.  The lane owns a BH x TW block of pixels and CV channels.
+// It walks the window rows of out_grad (block + K/2 halo either side, fetched once) and, K/2 rows behind, those of
+// x.  A row of out_grad feeds the K rows of in_grad it touches (rotated taps from LDS; a row of in_grad is stored
+// as soon as its last window row has passed) and its centre pixels are kept for the K rows of x they meet in the
+// grad-weight sums.  The loop is unrolled, so only the rows in use are live.  out_grad is read once instead of
+// twice and the separate grad-input kernel goes away.  The end of the kernel is that of nhwc_wgrad_kernel.
+template <typename IO, int K, int CV, int BH, int TW>
+__global__ __launch_bounds__(kNhwcThreads) void nhwc_bwd_fused_kernel(const NhwcPlan p)
+{
+    extern __shared__ float4 lds_raw[];
+    float *lds = reinterpret_cast<float *>(lds_raw);
+    constexpr int KK = K * K, P = K / 2;
+    constexpr int ROWS = BH + K - 1, COLS = TW + K - 1;
+    const int C = p.channel;
+    const int chunk = blockIdx.x;
+    const int c0 = blockIdx.y * p.lanes_c * CV;
+    const int nch = min(p.lanes_c * CV, C - c0);
+    const int pb_local = fast_div(threadIdx.x, p.lanes_c_magic);
+    const int lane_c = threadIdx.x - pb_local * p.lanes_c;
+    const bool lane_ok = pb_local < p.blocks_per_wg && CV * lane_c < nch;
+    const int c = c0 + (lane_ok ? CV * lane_c : 0);
+    const int per_image = p.blocks_x * p.blocks_y;
+    nhwc_stage_taps<IO, KK, true>(static_cast<const IO *>(p.taps), lds, c0, nch);
+    __syncthreads();
+    const float *wl = lds + (lane_ok ? CV * lane_c : 0);
+
+    float acc[KK][CV];
+#pragma unroll
+    for (int t = 0; t < KK; ++t)
+#pragma unroll
+        for (int v = 0; v < CV; ++v) acc[t][v] = 0.f;
+
+    for (long grp = chunk; grp * p.blocks_per_wg < p.blocks_total; grp += p.groups) {
+        const long pb = grp * p.blocks_per_wg + pb_local;
+        if (!lane_ok || pb >= p.blocks_total) continue;
+        const int n = static_cast<int>(pb / per_image);
+        const int rem = static_cast<int>(pb - static_cast<long>(n) * per_image);
+        const int by = rem / p.blocks_x, bx = rem - by * p.blocks_x;
+        const int oy0 = by * BH, ox0 = bx * TW;
+        const int iy0 = oy0 - P, ix0 = ox0 - P;
+        // views of x, out_grad and in_grad from the first image of this group of pixel blocks (uniform); the three
+        // tensors have the same extent, so one set of column offsets serves all of them
+        const int n0 = static_cast<int>(grp * p.blocks_per_wg / per_image);
+        const unsigned pixel_bytes = C * sizeof(IO), row_bytes = p.in_w * pixel_bytes;
+        const long image0 = static_cast<long>(n0) * p.in_h * p.in_w * C;
+        const __amdgpu_buffer_rsrc_t xview = buffer_view(static_cast<const IO *>(p.in) + image0);
+        const __amdgpu_buffer_rsrc_t gview = buffer_view(static_cast<const IO *>(p.in2) + image0);
+        const __amdgpu_buffer_rsrc_t oview = buffer_view(static_cast<IO *>(p.out) + image0);
+        const unsigned lane_off = (n - n0) * (p.in_h * row_bytes) + c * static_cast<unsigned>(sizeof(IO));
+        NhwcCols<COLS> cols;
+        nhwc_cols<COLS>(ix0, p.in_w, pixel_bytes, lane_off, cols);
+
+        float gxs[BH][TW * CV];  // in_grad sums
+        float gb[BH][TW * CV];   // centre pixels of the out_grad rows (the block itself)
+#pragma unroll
+        for (int b = 0; b < BH; ++b)
+#pragma unroll
+            for (int o = 0; o < TW * CV; ++o) gxs[b][o] = 0.f;
+        float xr[2][COLS * CV], gr[2][COLS * CV];
+        nhwc_load_row<IO, COLS, CV>(gview, iy0, p.in_h, row_bytes, cols, gr[0]);
+#pragma unroll
+        for (int t = 0; t < ROWS + P; ++t) {
+            const int r = t - P;  // window row of x in this step (out_grad runs P rows ahead)
+            if (t + 1 < ROWS) nhwc_load_row<IO, COLS, CV>(gview, iy0 + t + 1, p.in_h, row_bytes, cols, gr[(t + 1) & 1]);
+            if (r + 1 >= 0 && r + 1 < ROWS)
+                nhwc_load_row<IO, COLS, CV>(xview, iy0 + r + 1, p.in_h, row_bytes, cols, xr[(r + 1) & 1]);
+            if (t < ROWS) {
+                float(&gcur)[COLS * CV] = gr[t & 1];
+                // in_grad row b meets this row in rotated tap row u = t - b
+#pragma unroll
+                for (int u = 0; u < K; ++u) {
+                    const int b = t - u;
+                    if (b < 0 || b >= BH) continue;
+#pragma unroll
+                    for (int v = 0; v < K; ++v) {
+                        float w[CV];
+#pragma unroll
+                        for (int q = 0; q < CV; ++q) w[q] = wl[(u * K + v) * nch + q];
+#pragma unroll
+                        for (int o = 0; o < TW; ++o)
+#pragma unroll
+                            for (int q = 0; q < CV; ++q)
+                                gxs[b][CV * o + q] = fmaf(gcur[CV * (o + v) + q], w[q], gxs[b][CV * o + q]);
+                    }
+                }
+                if (t - P >= 0 && t - P < BH) {
+#pragma unroll
+                    for (int o = 0; o < TW * CV; ++o) gb[t - P][o] = gcur[CV * P + o];
+                }
+                if (t - (K - 1) >= 0 && t - (K - 1) < BH) {
+                    const int b = t - (K - 1);
+                    const unsigned roff = oy0 + b < p.in_h ? (oy0 + b) * row_bytes : kOob;
+#pragma unroll
+                    for (int o = 0; o < TW; ++o) {
+                        const unsigned off = __builtin_elementwise_add_sat(roff, cols.off[o + P]);
+                        if constexpr (CV == 4)
+                            view_store4<IO>(oview, off, gxs[b][4 * o], gxs[b][4 * o + 1], gxs[b][4 * o + 2], gxs[b][4 * o + 3]);
+                        else
+                            view_store2<IO>(oview, off, gxs[b][2 * o], gxs[b][2 * o + 1]);
+                    }
+                }
+            }
+            if (r >= 0 && r < ROWS) {
+                float(&xcur)[COLS * CV] = xr[r & 1];
+                // window row r of x meets out_grad row b in tap row ty = r - b
+#pragma unroll
+                for (int ty = 0; ty < K; ++ty) {
+                    const int b = r - ty;
+                    if (b < 0 || b >= BH) continue;
+#pragma unroll
+                    for (int tx = 0; tx < K; ++tx)
+#pragma unroll
+                        for (int o = 0; o < TW; ++o)
+#pragma unroll
+                            for (int q = 0; q < CV; ++q)
+                                acc[ty * K + tx][q] = fmaf(gb[b][CV * o + q], xcur[CV * (o + tx) + q], acc[ty * K + tx][q]);
+                }
+            }
+            pin_registers(acc);
+        }
+    }
+    __syncthreads();  // the taps in LDS are done with: the sums of the lanes go through the same memory
+
+    const int width = p.lanes_c * CV;
+    float *out = p.partial + static_cast<long>(chunk) * KK * C;
+#pragma unroll
+    for (int ty = 0; ty < K; ++ty) {
+        if (ty) __syncthreads();
+        if (pb_local < p.blocks_per_wg) {
+#pragma unroll
+            for (int tx = 0; tx < K; ++tx)
+#pragma unroll
+                for (int v = 0; v < CV; ++v) lds[(pb_local * K + tx) * width + CV * lane_c + v] = lane_ok ? acc[ty * K + tx][v] : 0.f;
+        }
+        __syncthreads();
+        for (int e = threadIdx.x; e < K * nch; e += blockDim.x) {
+            const int tx = e / nch, cl = e - tx * nch;
+            float s = 0.f;
+            for (int q = 0; q < p.blocks_per_wg; ++q) s += lds[(q * K + tx) * width + cl];
+            out[static_cast<long>(ty * K + tx) * C + c0 + cl] = s;
+        }
+    }
+}
+
 // Grad-weight, pass 2: gw[c][t] = sum over chunks of partial[chunk][t][c].  16 lanes per output add contiguous
 // sixteenths of the chunks in fp64; the sixteen sums are then added in order: bit-identical from run to run.
 constexpr int kNhwcFinalParts = 16;
@@ -523,17 +668,24 @@ __global__ __launch_bounds__(256) void nhwc_gw_direct_final_kernel(const float *
 // ---- planning -------------------------------------------------------------------------------------------
 // Channel lanes per workgroup, at most `cap`.  All of C when it fits (then the pixels of a row are one contiguous
 // run).  Otherwise a multiple of `line` lanes (= one 128-byte line of fp32 channels), so that every pixel's
-// segment starts and ends on a line: the largest such divisor of `lanes` (= C / CV), else the largest such
-// count below the cap, whose last channel group is then partly idle.  A segment that is not whole lines makes
+// segment starts and ends on a line: the count under the cap that leaves the fewest lanes of the last channel
+// group idle (none when it divides `lanes` = C / CV).  A segment that is not whole lines makes
 // every load fetch the lines at its ends in full (C = 240 in groups of 60 channels: 240-byte segments cost
 // 384 bytes of L1-to-L2 requests each, and the 28x28 layers ran 1.3-1.6 x slower than with 128-byte ones).
 int pick_lanes_c(int lanes, int cap, int line)
 {
     if (lanes <= cap) return lanes;
     if (line > 1 && cap >= line) {
-        for (int d = cap / line * line; d >= line; d -= line)
-            if (lanes % d == 0) return d;
-        return cap / line * line;
+        // the count that leaves the fewest idle lanes in the last group; the larger one on a tie
+        int best = line, best_padded = (lanes + line - 1) / line * line;
+        for (int d = 2 * line; d <= cap; d += line) {
+            const int padded = (lanes + d - 1) / d * d;
+            if (padded <= best_padded) {
+                best = d;
+                best_padded = padded;
+            }
+        }
+        return best;
     }
     int best = 1;
     for (int d = cap; d >= 1; --d)
@@ -554,9 +706,11 @@ bool plan_nhwc(NhwcPlan &p, const NhwcGeometry &g, int bh, int tw, int blocks_h,
     // images), so halo pixels are shared inside the workgroup's L1 instead of between workgroups.  Measured on
     // the EfficientNet-B0 layers: 8 lanes win on 7x7 and 14x14 maps, 16 on 28x28, 64 on larger ones.
     const long pixels = static_cast<long>(g.in_h) * g.in_w;
-    int cap = pixels <= 256 ? 8 : pixels <= 1024 ? 16 : 64;
+    // (large maps: all of C when a workgroup still holds two pixel blocks of it, e.g. C = 144 with two channels
+    // per lane: whole-C workgroups of 72 lanes beat 16-lane groups by 8-15 % on the 56x56 grad-weight kernels)
+    int cap = pixels <= 256 ? 8 : pixels <= 1024 ? 16 : 256 / CV;
     cap = env_int(lanes_env, std::max(cap, min_lanes));
-    cap = std::max(1, std::min(cap, 64));
+    cap = std::max(1, std::min(cap, 128));
     while (cap > 1 && static_cast<size_t>(cap) * CV * K * K * 4 > static_cast<size_t>(kNhwcTapLds)) --cap;
     p.lanes_c = pick_lanes_c(g.channel / CV, cap, env_int("DWCONV_NHWC_ALIGN", 1) ? 32 / CV : 1);
     p.lanes_c_magic = magic_u16(p.lanes_c);
@@ -715,6 +869,63 @@ long nhwc_wgrad_fast(int mode, const IO *x, const IO *gy, IO *gw, void *ws, size
     return -1;
 }
 
+// Fused backward of 3x3 stride-1 layers with pad 1 (the 5x5 instance needs 256 registers, one wavefront per SIMD,
+// and lost to the two separate kernels on every layer measured).  mode 0: workspace bytes; mode 1: launch.
+// -1 when the kernel does not cover g.
+template <typename IO, int K>
+long nhwc_bwd_fused_case(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
+                         const NhwcGeometry &g, hipStream_t stream)
+{
+    constexpr int CV = 2, BH = 7, TW = 4;
+    NhwcPlan p{};
+    const int line_lanes = static_cast<int>(128 / (CV * sizeof(IO)));
+    if (!plan_nhwc<K, CV>(p, g, BH, TW, g.out_h, g.out_w, line_lanes, "DWCONV_NHWC_WGRAD_LANES")) return -1;
+    const int cgroups = p.cgroups;
+    const long wg_iters = (p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg;
+    long groups = env_int("DWCONV_NHWC_WGRAD_WGS", 512) / cgroups;
+    groups = std::max(1l, std::min(groups, wg_iters));
+    p.groups = static_cast<int>(groups);
+    const size_t need = static_cast<size_t>(groups) * K * K * g.channel * sizeof(float);
+    if (mode == 0) return static_cast<long>(need);
+    if (ws == nullptr || ws_bytes < need)
+        return fail(DWCONV_ERR_WORKSPACE, "backward needs a workspace of %zu bytes, got %zu", need, ws_bytes);
+    p.in = x;
+    p.in2 = gy;
+    p.taps = taps;
+    p.out = gx;
+    p.partial = static_cast<float *>(ws);
+    p.in_h = g.in_h;
+    p.in_w = g.in_w;
+    p.out_h = g.out_h;
+    p.out_w = g.out_w;
+    p.pad_h = g.pad_h;
+    p.pad_w = g.pad_w;
+    const size_t shmem = static_cast<size_t>(p.lanes_c) * CV * 4 * std::max(K * K, p.blocks_per_wg * K);
+    hipLaunchKernelGGL((nhwc_bwd_fused_kernel<IO, K, CV, BH, TW>), dim3(p.groups, cgroups), dim3(kNhwcThreads), shmem, stream, p);
+    int rc = check_launch("nhwc_bwd_fused_kernel");
+    if (rc != DWCONV_OK) return rc;
+    note_variant("nhwc_bwd%s<k%d,s1,cv%d,%dx%d> lanes_c%d chunks%d", sizeof(IO) == 2 ? "16" : "", K, CV, BH, TW, p.lanes_c, p.groups);
+    hipLaunchKernelGGL(nhwc_wgrad_final_kernel<IO>, dim3(ceil_div(g.channel * K * K, 16)), dim3(256), 0, stream,
+                       p.partial, gw, g.channel, K * K, p.groups);
+    return check_launch("nhwc_wgrad_final_kernel");
+}
+
+bool nhwc_fused_ok(const NhwcGeometry &g)
+{
+    if (!env_int("DWCONV_NHWC_FUSED_BWD", 1) || !nhwc_fast_ok(g)) return false;
+    const int K = g.kernel_h;
+    return K == 3 && g.stride_h == 1 && g.pad_h == K / 2 && g.pad_w == K / 2 && g.out_h == g.in_h &&
+           g.out_w == g.in_w;
+}
+
+template <typename IO>
+long nhwc_bwd_fused(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
+                    const NhwcGeometry &g, hipStream_t stream)
+{
+    if (!nhwc_fused_ok(g)) return -1;
+    return nhwc_bwd_fused_case<IO, 3>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+}
+
 template <typename T>
 int direct_chunks(const NhwcGeometry &g)
 {
@@ -814,6 +1025,8 @@ size_t nhwc_grad_weight_workspace(const NhwcGeometry &g)
     if constexpr (!std::is_same<T, double>::value) {
         const long fast = nhwc_wgrad_fast<T>(0, nullptr, nullptr, nullptr, nullptr, 0, g, nullptr);
         if (fast > 0 && static_cast<size_t>(fast) > need) need = static_cast<size_t>(fast);
+        const long fused = nhwc_bwd_fused<T>(0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, g, nullptr);
+        if (fused > 0 && static_cast<size_t>(fused) > need) need = static_cast<size_t>(fused);
     }
     return need;
 }
@@ -851,7 +1064,21 @@ int nhwc_grad_weight(const T *x, const T *gy, T *gw, void *ws, size_t ws_bytes, 
     return check_launch("nhwc_gw_direct_final_kernel");
 }
 
+// Both gradients of one layer in one sweep where nhwc_bwd_fused_kernel covers the geometry; -1 otherwise.
+template <typename T>
+int nhwc_backward_fused(const T *x, const T *gy, const T *taps, T *gx, T *gw, void *ws, size_t ws_bytes,
+                        const NhwcGeometry &g, hipStream_t stream)
+{
+    if constexpr (!std::is_same<T, double>::value) {
+        if (static_cast<long>(g.batch) * g.out_h * g.out_w * g.channel > 0 && aligned4(x) && aligned4(gy) && aligned4(gx))
+            return static_cast<int>(nhwc_bwd_fused<T>(1, x, gy, taps, gx, gw, ws, ws_bytes, g, stream));
+    }
+    return -1;
+}
+
 #define DWCONV_INSTANTIATE(T)                                                                                          \
+    template int nhwc_backward_fused<T>(const T *, const T *, const T *, T *, T *, void *, size_t, const NhwcGeometry &,    \
+                                        hipStream_t);                                                                  \
     template int nhwc_forward<T>(const T *, const T *, T *, const NhwcGeometry &, hipStream_t);                        \
     template int nhwc_grad_input<T>(const T *, const T *, T *, const NhwcGeometry &, hipStream_t);                     \
     template size_t nhwc_grad_weight_workspace<T>(const NhwcGeometry &);                                               \

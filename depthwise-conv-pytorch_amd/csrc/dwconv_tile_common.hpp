@@ -184,6 +184,22 @@ __device__ __forceinline__ void view_store4(__amdgpu_buffer_rsrc_t view, unsigne
     }
 }
 
+// Two results as elements at byte offset `off` of the view; dropped when `off` is at or beyond kOob.
+template <typename IO, int POLICY = kStoreStreaming>
+__device__ __forceinline__ void view_store2(__amdgpu_buffer_rsrc_t view, unsigned off, float a, float b)
+{
+    if constexpr (sizeof(IO) == 4) {
+        u32x2 t;
+        t.x = __float_as_uint(a); t.y = __float_as_uint(b);
+        __builtin_amdgcn_raw_buffer_store_b64(t, view, off, 0, POLICY);
+    } else {
+        unsigned t;
+        if constexpr (std::is_same<IO, bf16_t>::value) t = bf16_pack2(a, b);
+        else t = f16_pack2(a, b);
+        __builtin_amdgcn_raw_buffer_store_b32(t, view, off, 0, POLICY);
+    }
+}
+
 // True when groups of four elements starting at `p` may be moved with one vector access.
 template <typename IO>
 inline bool aligned4(const IO *p)
