@@ -571,6 +571,52 @@ def test_channels_last_matches_oracle(dw, gpu, shape):
     assert torch.equal(gw, gw2)
 
 
+FUSED_NHWC_SHAPES = [(2, 8, 14, 14, 3, 1, 1), (3, 32, 9, 11, 3, 1, 1), (1, 72, 15, 6, 3, 1, 1), (2, 144, 56, 56, 3, 1, 1),
+                     (5, 260, 7, 7, 3, 1, 1), (2, 4, 1, 5, 3, 1, 1), (1, 12, 29, 30, 3, 1, 1)]
+
+
+@pytest.mark.parametrize("shape", FUSED_NHWC_SHAPES, ids=shape_id)
+def test_channels_last_fused_backward(dw, gpu, shape, monkeypatch):
+    """3x3 stride-1 'same' layers, channels-last: one kernel makes both gradients.  Against the oracle, against the two
+    separate kernels, bit-identical from run to run; one gradient alone still takes the separate kernels; the autograd
+    route returns the same bits as the direct entry point."""
+    from torch_dwconv import _C
+
+    n, c, h, w, k, s, p = shape
+    x, wt, gy = make_inputs(shape, seed=41)
+    xg, wg, gyg = _channels_last(x, gpu), wt.to(gpu), _channels_last(gy, gpu)
+    gx, gw = _C.dwconv2d_backward_nhwc(xg, gyg, wg, s, s, p, p)
+    _announce(shape_id(shape), _C.last_variant())
+    assert _C.last_variant().startswith("nhwc_bwd<k3,s1"), _C.last_variant()
+    assert gx.is_contiguous(memory_format=torch.channels_last) or c == 1 or h * w == 1
+    gx_ref = oracle.grad_input(_np(gy), _np(wt), (h, w), s, p)
+    gw_ref = oracle.grad_weight(_np(x), _np(gy), wt.shape, s, p)
+    np.testing.assert_allclose(_np(gx).astype(np.float64), gx_ref, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(_np(gw).astype(np.float64), gw_ref, rtol=1e-4, atol=1e-4 * np.abs(gw_ref).max())
+    gx2, gw2 = _C.dwconv2d_backward_nhwc(xg, gyg, wg, s, s, p, p)
+    assert torch.equal(gw, gw2) and torch.equal(gx, gx2)
+    xa, wa = xg.clone().requires_grad_(True), wg.clone().requires_grad_(True)
+    gxa, gwa = torch.autograd.grad(dw.depthwise_conv2d(xa, wa, stride=s, padding=p), (xa, wa), gyg)
+    assert torch.equal(gxa, gx) and torch.equal(gwa, gw)
+    gx_only, none = _C.dwconv2d_backward_nhwc(xg, gyg, wg, s, s, p, p, need_kernel_grad=False)
+    assert none is None and not _C.last_variant().startswith("nhwc_bwd"), _C.last_variant()
+    np.testing.assert_allclose(_np(gx_only), _np(gx), rtol=1e-6, atol=1e-6)
+    monkeypatch.setenv("DWCONV_NHWC_FUSED_BWD", "0")
+    gx3, gw3 = _C.dwconv2d_backward_nhwc(xg, gyg, wg, s, s, p, p)
+    assert "nhwc_wgrad" in _C.last_variant(), _C.last_variant()
+    np.testing.assert_allclose(_np(gx3), _np(gx), rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(_np(gw3), _np(gw), rtol=1e-5, atol=1e-5 * float(gw.abs().max()))
+    monkeypatch.delenv("DWCONV_NHWC_FUSED_BWD")
+    for dtype, tol in ((torch.float16, 4e-3), (torch.bfloat16, 3e-2)):
+        xh, wh, gh = xg.to(dtype), wg.to(dtype), gyg.to(dtype)
+        gxh, gwh = _C.dwconv2d_backward_nhwc(xh, gh, wh, s, s, p, p)
+        assert _C.last_variant().startswith("nhwc_bwd16<k3,s1"), _C.last_variant()
+        _, gx_r, gw_r = oracle.torch_reference(xh.cpu(), wh.cpu(), gh.cpu(), s, p)
+        np.testing.assert_allclose(_np(gxh.float()).astype(np.float64), _np(gx_r), rtol=tol, atol=tol)
+        np.testing.assert_allclose(_np(gwh.float()).astype(np.float64), _np(gw_r), rtol=tol,
+                                   atol=tol * max(1.0, float(np.abs(_np(gw_r)).max())))
+
+
 def test_channels_last_channel_groups_are_whole_lines(dw, gpu):
     """C = 240 on a 28x28 map: the workgroups take 16 channel lanes (256 bytes per pixel), not the 15 that divide C / 4."""
     from torch_dwconv import _C
