@@ -3,6 +3,7 @@
 #include "dwconv_common.hpp"
 
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 #include <cstdarg>
@@ -435,6 +436,42 @@ int general_backward_any(const T *in, const T *gy, const T *taps, T *gx, T *gw, 
 }  // namespace
 }  // namespace dwconv
 
+// ---- scratch memory of the entry point that allocates nothing -------------------------------------------
+// Partial grad-weight sums of dwconv2d_backward_noalloc_f32 live in this array instead of a caller's
+// workspace.  Every device the library runs on holds its own copy, at its own address, until the process
+// ends.  In host code the name is only a handle for hipGetSymbolAddress: kernels and copies get the
+// per-device address that call returns, never the name itself.
+static __device__ __align__(256) unsigned char scratch[DWCONV_NOALLOC_SCRATCH_BYTES];
+
+namespace dwconv {
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+// Address of `scratch` on the current device (looked up once per device).
+int scratch_of_current_device(void **ptr)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(DWCONV_ERR_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(DWCONV_ERR_UNSUPPORTED, "device ordinal %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || p == nullptr)
+            return fail(DWCONV_ERR_LAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return DWCONV_OK;
+}
+
+}  // namespace
+}  // namespace dwconv
+
 using namespace dwconv;
 
 extern "C" {
@@ -581,6 +618,28 @@ int dwconv2d_backward_f32(const float *input, const float *out_grad, const float
     return backward_any<float>(input, out_grad, kernel, in_grad, kernel_grad, workspace, workspace_bytes, batch,
                                channel, in_h, in_w, out_h, out_w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w,
                                stream);
+}
+
+int dwconv2d_backward_noalloc_f32(const float *input, const float *out_grad, const float *kernel, float *in_grad,
+                                  float *kernel_grad, int batch, int channel, int in_h, int in_w, int out_h,
+                                  int out_w, int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h,
+                                  int pad_w, void *stream)
+{
+    WgradGeometry g;
+    const int rc = make_wgrad_geometry(g, input, out_grad, kernel_grad, batch, channel, in_h, in_w, out_h, out_w,
+                                       kernel_h, kernel_w, 1, 1, stride_h, stride_w, pad_h, pad_w);
+    if (rc != DWCONV_OK) return rc;
+    const size_t need = (batch > 0 && channel > 0) ? wgrad_workspace<float>(g) : 0;
+    if (need > sizeof(scratch))
+        return fail(DWCONV_ERR_WORKSPACE,
+                    "dwconv2d_backward_noalloc_f32: this geometry needs %zu bytes of scratch memory, the built-in "
+                    "buffer holds %zu; call dwconv2d_backward_f32 with a workspace of your own",
+                    need, sizeof(scratch));
+    void *ws = nullptr;
+    const int rs = scratch_of_current_device(&ws);
+    if (rs != DWCONV_OK) return rs;
+    return backward_any<float>(input, out_grad, kernel, in_grad, kernel_grad, ws, sizeof(scratch), batch, channel, in_h,
+                               in_w, out_h, out_w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, stream);
 }
 
 // ---- channels-last tensors ----

@@ -51,6 +51,11 @@ for _name in ("dwconv2d_backward_f32", "dwconv2d_backward_f16", "dwconv2d_backwa
     getattr(_lib, _name).restype = _i
     getattr(_lib, _name).argtypes = [_p, _p, _p, _p, _p, _p, _z] + [_i] * 12 + [_p]
 
+# the entry point that allocates nothing: no workspace argument (include/dwconv_hip.h)
+NOALLOC_SCRATCH_BYTES = 32 << 20
+_lib.dwconv2d_backward_noalloc_f32.restype = _i
+_lib.dwconv2d_backward_noalloc_f32.argtypes = [_p] * 5 + [_i] * 12 + [_p]
+
 for _name in ("dwconv2d_nhwc_f32", "dwconv2d_nhwc_f64", "dwconv2d_nhwc_f16", "dwconv2d_nhwc_bf16"):
     getattr(_lib, _name).restype = _i
     getattr(_lib, _name).argtypes = [_p, _p, _p] + [_i] * 10 + [_p]
@@ -236,6 +241,31 @@ def dwconv2d_backward(input, out_grad, kernel, stride_h, stride_w, pad_h, pad_w)
     if rc != 0:
         _raise(rc)
     return gx, gw
+
+
+def dwconv2d_backward_noalloc(input, out_grad, kernel, in_grad, kernel_grad, stride_h, stride_w, pad_h, pad_w):
+    """``dwconv2d_backward`` into tensors the caller already owns, with no allocation anywhere: float32, dense NCHW
+    tensors only; the library's built-in scratch buffer (``NOALLOC_SCRATCH_BYTES`` per device) stands for the
+    workspace.  Calls on one device share that buffer: keep them on one stream.  No counterpart in the reference."""
+    for name, t in (("input", input), ("out_grad", out_grad), ("kernel", kernel), ("in_grad", in_grad),
+                    ("kernel_grad", kernel_grad)):
+        _check_cuda(t, name)
+        if t.dtype != torch.float32 or not t.is_contiguous():
+            raise RuntimeError(f"{name} must be a contiguous float32 tensor")
+    _check_shapes(input, kernel)
+    if out_grad.dim() != 4 or out_grad.shape[:2] != input.shape[:2]:
+        raise RuntimeError(f"out_grad of shape {tuple(out_grad.shape)} does not belong to input {tuple(input.shape)}")
+    if in_grad.shape != input.shape or kernel_grad.shape != kernel.shape:
+        raise RuntimeError("in_grad / kernel_grad must have the shapes of input / kernel")
+    n, c, h, w = input.shape
+    with torch.cuda.device(input.device):
+        rc = _lib.dwconv2d_backward_noalloc_f32(
+            input.data_ptr(), out_grad.data_ptr(), kernel.data_ptr(), in_grad.data_ptr(), kernel_grad.data_ptr(),
+            n, c, h, w, out_grad.shape[2], out_grad.shape[3], kernel.shape[2], kernel.shape[3],
+            stride_h, stride_w, pad_h, pad_w, _stream(input),
+        )
+    if rc != 0:
+        _raise(rc)
 
 
 # ---- channels-last tensors -----------------------------------------------------------------------------

@@ -199,6 +199,23 @@ int dwconv2d_backward_bf16(const unsigned short *input, const unsigned short *ou
                            int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
                            void *stream);
 
+/* dwconv2d_backward_f32 for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): the same kernels and the same results, bit for
+ * bit, but the partial grad-weight sums go to a buffer of DWCONV_NOALLOC_SCRATCH_BYTES that is part of
+ * the library's device image, so there is no workspace argument and the call allocates nothing.  It has no
+ * counterpart in the reference (whose backward allocates its results, torch_dwconv/dwconv_kernel.cu:782,
+ * :1026).  A geometry whose dwconv2d_backward_kernel_workspace_bytes(..., elem_size = 4) exceeds
+ * DWCONV_NOALLOC_SCRATCH_BYTES is refused with DWCONV_ERR_WORKSPACE before anything is launched.  Every
+ * device holds one such buffer, shared by all calls on it: the kernels overwrite what they read from it,
+ * so nothing needs clearing between calls, but two calls that overlap in time on one device (different
+ * streams or threads) race on it -- run them on one stream or order them yourself.  The buffer's address
+ * is looked up on the first call on each device; make that call outside stream capture. */
+#define DWCONV_NOALLOC_SCRATCH_BYTES (32u << 20)
+int dwconv2d_backward_noalloc_f32(const float *input, const float *out_grad, const float *kernel,
+                                  float *in_grad, float *kernel_grad, int batch, int channel,
+                                  int in_h, int in_w, int out_h, int out_w, int kernel_h, int kernel_w,
+                                  int stride_h, int stride_w, int pad_h, int pad_w, void *stream);
+
 /* ---- channels-last (NHWC) tensors -------------------------------------------------------------
  * No counterpart in the reference, which makes every tensor NCHW-contiguous before its kernels run
  * (torch_dwconv/dwconv_kernel.cu:741, :855, :1023): these entry points serve callers whose activations are

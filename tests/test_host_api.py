@@ -88,6 +88,18 @@ def test_argument_errors_come_back_as_status_codes(lib):
 
 
 # ---- python surface ------------------------------------------------------------
+def test_noalloc_entry_point_refuses_oversized_geometry_without_a_gpu(lib):
+    # the size check comes before anything touches a device, so it can be exercised here
+    n, c, h, k = 2, 65536, 16, 15
+    need = lib.dwconv2d_backward_kernel_workspace_bytes(n, c, h, h, h, h, k, k, 1, 1, 7, 7, 4)
+    assert need > 32 << 20
+    lib.dwconv2d_backward_noalloc_f32.restype = ctypes.c_int
+    lib.dwconv2d_backward_noalloc_f32.argtypes = [ctypes.c_void_p] * 5 + [ctypes.c_int] * 12 + [ctypes.c_void_p]
+    rc = lib.dwconv2d_backward_noalloc_f32(8, 8, 8, 8, 8, n, c, h, h, h, h, k, k, 1, 1, 7, 7, None)
+    assert rc == 3  # DWCONV_ERR_WORKSPACE
+    assert b"scratch" in lib.dwconv_last_error()
+
+
 def test_make_tuple_matches_restatement(dw):
     for v in (1, 3, (1, 2), [2, 1], [4], (5,), []):
         assert dw.make_tuple(v, 2) == oracle.host_logic.expand(v, 2)

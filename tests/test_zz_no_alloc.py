@@ -1,0 +1,102 @@
+"""The entry point that allocates nothing (dwconv2d_backward_noalloc_f32) against dwconv2d_backward_f32.
+
+Both run the same kernels with the same plan, so the results must be equal bit for bit.  Two calls in a row on one
+device, the second on a smaller problem: the built-in scratch buffer keeps the first call's partial sums, and the
+second call must not see them."""
+import ctypes
+
+import pytest
+import torch
+
+import shapes
+from torch_dwconv import _C
+
+pytestmark = pytest.mark.gpu
+
+# every kernel family behind dwconv2d_backward_f32: fused tiled stride 1, fused stride 2, fused whole-plane,
+# the two separate passes (pad 0), the per-element kernels (rectangular filter)
+PAIRS = [
+    ((16, 48, 56, 56, 3, 1, 1), (4, 24, 28, 28, 5, 2, 2)),
+    ((32, 96, 14, 14, 5, 1, 2), (3, 10, 7, 7, 3, 1, 1)),
+    ((8, 32, 64, 64, 5, 2, 2), (8, 32, 33, 35, 3, 1, 0)),
+    ((64, 128, 7, 7, 7, 1, 3), (2, 5, 19, 23, 7, 1, 3)),
+]
+
+
+def _reference(x, gy, w, s, p):
+    """dwconv2d_backward_f32 through the C ABI with a workspace from torch."""
+    n, c, h, wd = x.shape
+    oh, ow = gy.shape[2:]
+    kh, kw = w.shape[2:]
+    need = _C._lib.dwconv2d_backward_kernel_workspace_bytes(n, c, h, wd, oh, ow, kh, kw, s, s, p, p, 4)
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=x.device)
+    gx = torch.full_like(x, float("nan"))
+    gw = torch.full_like(w, float("nan"))
+    rc = _C._lib.dwconv2d_backward_f32(x.data_ptr(), gy.data_ptr(), w.data_ptr(), gx.data_ptr(), gw.data_ptr(),
+                                       ws.data_ptr(), need, n, c, h, wd, oh, ow, kh, kw, s, s, p, p,
+                                       ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, _C._lib.dwconv_last_error().decode()
+    return gx, gw, need, _C.last_variant()
+
+
+def _noalloc(x, gy, w, s, p):
+    n, c, h, wd = x.shape
+    oh, ow = gy.shape[2:]
+    kh, kw = w.shape[2:]
+    gx = torch.full_like(x, float("nan"))
+    gw = torch.full_like(w, float("nan"))
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    rc = _C._lib.dwconv2d_backward_noalloc_f32(x.data_ptr(), gy.data_ptr(), w.data_ptr(), gx.data_ptr(),
+                                               gw.data_ptr(), n, c, h, wd, oh, ow, kh, kw, s, s, p, p,
+                                               ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, _C._lib.dwconv_last_error().decode()
+    assert torch.cuda.memory_allocated() == before
+    return gx, gw, _C.last_variant()
+
+
+@pytest.mark.parametrize("first,second", PAIRS, ids=lambda s: shapes.shape_id(s))
+def test_noalloc_matches_backward_two_calls_in_a_row(first, second):
+    dev = torch.device("cuda:0")
+    for shape in (first, second):  # second call: smaller problem, same scratch buffer
+        x, w, gy = (t.to(dev) for t in shapes.make_inputs(shape, seed=7))
+        s, p = shape[5], shape[6]
+        gx, gw, variant = _noalloc(x, gy, w, s, p)
+        gx_ref, gw_ref, need, variant_ref = _reference(x, gy, w, s, p)
+        torch.cuda.synchronize()
+        assert need <= _C.NOALLOC_SCRATCH_BYTES
+        assert variant == variant_ref
+        assert not torch.isnan(gx).any() and not torch.isnan(gw).any()
+        assert torch.equal(gx, gx_ref), f"{shapes.shape_id(shape)} [{variant}] in_grad differs"
+        assert torch.equal(gw, gw_ref), f"{shapes.shape_id(shape)} [{variant}] kernel_grad differs"
+
+
+def test_noalloc_wrapper_and_oracle():
+    """The Python wrapper, checked against the CPU oracle as well (1e-5 / 1e-4 bounds as everywhere)."""
+    import numpy as np
+
+    import oracle
+
+    dev = torch.device("cuda:0")
+    shape = (6, 40, 28, 28, 3, 2, 1)
+    x, w, gy = shapes.make_inputs(shape, seed=3)
+    xg, wg, gyg = x.to(dev), w.to(dev), gy.to(dev)
+    gx = torch.full_like(xg, float("nan"))
+    gw = torch.full_like(wg, float("nan"))
+    _C.dwconv2d_backward_noalloc(xg, gyg, wg, gx, gw, 2, 2, 1, 1)
+    gx_ref = oracle.grad_input(gy.numpy(), w.numpy(), (28, 28), 2, 1)
+    gw_ref = oracle.grad_weight(x.numpy(), gy.numpy(), w.shape, 2, 1)
+    np.testing.assert_allclose(gx.cpu().numpy(), gx_ref, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(gw.cpu().numpy(), gw_ref, rtol=1e-4, atol=1e-4 * np.abs(gw_ref).max())
+
+
+def test_noalloc_rejects_oversized_geometry():
+    """Beyond the built-in buffer the call is refused before anything is launched."""
+    n, c, h, k = 2, 65536, 16, 15
+    need = _C._lib.dwconv2d_backward_kernel_workspace_bytes(n, c, h, h, h, h, k, k, 1, 1, 7, 7, 4)
+    assert need > _C.NOALLOC_SCRATCH_BYTES
+    one = torch.zeros(1, device="cuda:0")
+    rc = _C._lib.dwconv2d_backward_noalloc_f32(one.data_ptr(), one.data_ptr(), one.data_ptr(), one.data_ptr(),
+                                               one.data_ptr(), n, c, h, h, h, h, k, k, 1, 1, 7, 7, None)
+    assert rc == 3  # DWCONV_ERR_WORKSPACE
+    assert "scratch" in _C._lib.dwconv_last_error().decode()
