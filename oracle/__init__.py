@@ -31,5 +31,6 @@ from .torch_reference import (  # noqa: F401
     torch_reference_fused,
     torch_reference_general,
     torch_cpu_fp32_step,
+    shift_add_reference,
 )
 from . import host_logic  # noqa: F401

@@ -33,6 +33,38 @@ def torch_reference_general(x, w, gy=None, stride=1, padding=0, dilation=1):
     return y.detach(), gx, gw
 
 
+def shift_add_reference(x, w, gy, stride, padding):
+    """(y, gx, gw) in fp64 on whatever device ``x`` lives on, from the closed forms alone: one strided slice of the
+    zero-padded input per tap, multiplied and added (no convolution routine of any library is involved).
+
+        y [n,c,oy,ox] = sum_{i,j} xpad[n,c, oy*s+i, ox*s+j] * w[c,i,j]
+        gxpad[n,c, oy*s+i, ox*s+j] += gy[n,c,oy,ox] * w[c,i,j]          (then the padding is cut off)
+        gw[c,i,j]     = sum_{n,oy,ox} gy[n,c,oy,ox] * xpad[n,c, oy*s+i, ox*s+j]
+
+    which is what torch_dwconv/dwconv_kernel.cu:148-178 and :269-297 evaluate per output.  Used for whole-tensor
+    checks at sizes where the C oracle would take minutes; pinned against it in tests/test_oracle.py."""
+    sh, sw = (stride, stride) if isinstance(stride, int) else stride
+    ph, pw = (padding, padding) if isinstance(padding, int) else padding
+    xd, wd, gd = x.detach().double(), w.detach().double(), gy.detach().double()
+    n, c, h, wid = xd.shape
+    kh, kw = wd.shape[2:]
+    oh, ow = gd.shape[2:]
+    xpad = F.pad(xd, (pw, pw, ph, ph))
+    y = torch.zeros_like(gd)
+    gxpad = torch.zeros_like(xpad)
+    gw = torch.zeros_like(wd)
+    for i in range(kh):
+        for j in range(kw):
+            # rows i, i+s, ... (oh of them) and columns j, j+s, ... (ow of them) of the padded plane
+            window = xpad[:, :, i:i + (oh - 1) * sh + 1:sh, j:j + (ow - 1) * sw + 1:sw]
+            tap = wd[:, 0, i, j].view(1, c, 1, 1)
+            y += window * tap
+            gxpad[:, :, i:i + (oh - 1) * sh + 1:sh, j:j + (ow - 1) * sw + 1:sw] += gd * tap
+            gw[:, 0, i, j] = (gd * window).sum(dim=(0, 2, 3))
+    gx = gxpad[:, :, ph:ph + h, pw:pw + wid].contiguous()
+    return y, gx, gw
+
+
 _ACTIVATIONS = {None: lambda v: v, "none": lambda v: v, "relu": F.relu, "relu6": F.relu6, "silu": F.silu}
 
 

@@ -341,3 +341,58 @@ def test_general_reference_against_brute_force():
     np.testing.assert_array_equal(oracle.torch_reference_general(x, w1, None, 1, 1, 1)[0].numpy(),
                                   oracle.torch_reference(x, w1, None, 1, 1)[0].numpy())
 
+
+
+# --------------------------------------------------------------------------
+# the whole-tensor reference of the full-size GPU tests, and the routing restatement
+# --------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [(2, 3, 9, 8, 3, 1, 1), (2, 3, 9, 8, 3, 2, 1), (1, 4, 13, 11, 5, 2, 2),
+                                   (2, 2, 7, 7, 7, 1, 3), (1, 2, 12, 15, 5, 1, 0), (2, 2, 11, 10, 4, 3, 1),
+                                   (1, 3, 10, 9, 3, 2, 0)], ids=shape_id)
+def test_shift_add_reference_equals_c_oracle(shape):
+    n, c, h, w, k, s, p = shape
+    x, wt, gy = make_inputs(shape, seed=41, dtype=torch.float64)
+    y, gx, gw = oracle.shift_add_reference(x, wt, gy, s, p)
+    np.testing.assert_allclose(y.numpy(), oracle.forward(x.numpy(), wt.numpy(), s, p), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(gx.numpy(), oracle.grad_input(gy.numpy(), wt.numpy(), (h, w), s, p), rtol=1e-12,
+                               atol=1e-12)
+    np.testing.assert_allclose(gw.numpy(), oracle.grad_weight(x.numpy(), gy.numpy(), wt.shape, s, p), rtol=1e-12,
+                               atol=1e-12)
+    # rectangular filter, stride and padding as well
+    g = torch.Generator("cpu").manual_seed(43)
+    x = torch.randn(2, 3, 12, 10, generator=g, dtype=torch.float64)
+    wt = torch.randn(3, 1, 5, 2, generator=g, dtype=torch.float64)
+    gy = torch.randn(2, 3, 5, 9, generator=g, dtype=torch.float64)
+    y, gx, gw = oracle.shift_add_reference(x, wt, gy, (2, 1), (1, 0))
+    np.testing.assert_allclose(y.numpy(), oracle.forward(x.numpy(), wt.numpy(), (2, 1), (1, 0)), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(gx.numpy(), oracle.grad_input(gy.numpy(), wt.numpy(), (12, 10), (2, 1), (1, 0)),
+                               rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(gw.numpy(), oracle.grad_weight(x.numpy(), gy.numpy(), wt.shape, (2, 1), (1, 0)),
+                               rtol=1e-12, atol=1e-12)
+
+
+# Which of its three paths the reference takes for every benchmark layer, read off torch_dwconv/dwconv.py:123-130
+# and dwconv_kernel.cu:652-662 by hand: (H, k, stride) -> path ("native_conv2d" = the F.conv2d hand-off).
+ROUTING_TABLE = [
+    ((56, 3, 1), "large"), ((256, 5, 1), "large"), ((112, 3, 1), "large"), ((112, 3, 2), "large"),
+    ((56, 5, 2), "large"), ((28, 5, 1), "small"), ((28, 3, 2), "native_conv2d"), ((14, 3, 1), "small"),
+    ((14, 5, 1), "small"), ((14, 5, 2), "native_conv2d"), ((7, 5, 1), "small"), ((7, 3, 1), "small"),
+    ((7, 7, 1), "native_conv2d"),    # 49 taps > ceil(7/2)*7 = 28 lanes
+    ((14, 7, 1), "small"), ((56, 7, 1), "large"), ((28, 7, 1), "small"),
+    ((33, 3, 1), "large"), ((32, 3, 1), "small"), ((4, 3, 1), "native_conv2d"),
+]
+
+
+@pytest.mark.parametrize("geom,expected", ROUTING_TABLE)
+def test_route_matches_the_reference_routing_table(geom, expected):
+    h, k, s = geom
+    p = k // 2
+    small = oracle.use_dwconv2d_small(h, h, k, k, 1, 1, s, s, p, p)
+    assert oracle.host_logic.route((h, h), (k, k), (s, s), (p, p), small) == expected
+
+
+def test_route_rectangular_planes():
+    # one axis above 32 is enough for the large path (dwconv.py:125: `and`)
+    assert oracle.host_logic.route((40, 8), (3, 3), (2, 2), (1, 1), False) == "large"
+    assert oracle.host_logic.route((8, 40), (3, 3), (2, 2), (1, 1), False) == "large"
+    assert oracle.host_logic.route((32, 32), (3, 3), (2, 2), (1, 1), False) == "native_conv2d"
