@@ -128,35 +128,33 @@ def schedule(layers, separate_backward):
     return calls
 
 
-def cpu_baseline(layers_shapes, torch, budget_s=20.0):
-    """fp32 F.conv2d(groups=C) forward + both gradients on the host cores, on a batch
-    slice of every layer of the workload; scaled to the full batch."""
+def cpu_baseline(layers, torch, iters=5, budget_s=30.0):
+    """fp32 F.conv2d(groups=C) forward + both gradients on the host cores, every layer of the workload at its full
+    batch (the same tensors the GPU step runs on, copied to the host).  A step is the sum over the layers; the step is
+    repeated `iters` times after one untimed pass and min / median / max are reported.  Layers are dropped from the
+    end only if the time budget runs out (said in `sample`)."""
     from oracle import torch_cpu_fp32_step
 
     cores = os.cpu_count() or 1
     threads = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
-    full_batch = layers_shapes[0][0]
-    sample_batch = max(1, min(full_batch, 8))
-    g = torch.Generator("cpu").manual_seed(0)
-    t_total, bytes_total = 0.0, 0
     t_start = time.perf_counter()
-    done = 0
-    for (n, c, h, w, k, s, p) in layers_shapes:
-        nb = max(1, min(n, sample_batch))
-        oh, ow = (h + 2 * p - k) // s + 1, (w + 2 * p - k) // s + 1
-        x = torch.randn(nb, c, h, w, generator=g)
-        wt = torch.randn(c, 1, k, k, generator=g) / k
-        gy = torch.randn(nb, c, oh, ow, generator=g)
-        t, threads = torch_cpu_fp32_step(x, wt, gy, s, p, iters=3, threads=threads)
-        t_total += t * (n / nb)
+    per_layer, bytes_total, done = [], 0, 0
+    for l in layers:
+        n, c, h, w, oh, ow, k, s, p = l.geom
+        x, wt, gy = l.x.float().cpu(), l.w.float().cpu(), l.gy.float().cpu()
+        times, threads = torch_cpu_fp32_step(x, wt, gy, s, p, iters=iters, threads=threads, all_times=True)
+        per_layer.append(times)
         bytes_total += 12 * (n * c * h * w + n * c * oh * ow + c * k * k)
         done += 1
         if time.perf_counter() - t_start > budget_s:
             break
-    sample = (f"torch {torch.__version__} F.conv2d(groups=C) fp32 fwd + autograd.grad(x,w), median of 3, "
-              f"batch slice {sample_batch} of {full_batch} on {done} of {len(layers_shapes)} layers, time scaled to the full batch")
-    return {"value": round(bytes_total / t_total / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
-            "sample": sample, "ms_per_step_scaled": round(t_total * 1e3, 1)}
+    steps = sorted(sum(t[i] for t in per_layer) for i in range(iters))
+    med = steps[len(steps) // 2]
+    sample = (f"torch {torch.__version__} F.conv2d(groups=C) fp32 fwd + autograd.grad(x,w) at the full batch of "
+              f"{layers[0].geom[0]} on {done} of {len(layers)} layers, {iters} timed steps after one warm-up; value = median")
+    return {"value": round(bytes_total / med / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": sample, "ms_per_step": {"min": round(steps[0] * 1e3, 1), "median": round(med * 1e3, 1),
+                                              "max": round(steps[-1] * 1e3, 1)}}
 
 
 def miopen_native(layers, torch, iters=3):
@@ -184,7 +182,9 @@ def miopen_native(layers, torch, iters=3):
 
 def epilogue_comparison(layers, lib, torch, stream, dtype, layout, iters=10):
     """Forward + folded batch-norm + SiLU over the workload: one fused C-ABI call per layer against the plain forward
-    call followed by PyTorch's elementwise ops on its output.  Returns (fused ms, unfused ms, convolution-only ms) per pass over the layers."""
+    call followed by PyTorch's elementwise ops on its output, and the same block in training (forward + all four
+    gradients through autograd).  Returns (fused ms, unfused ms, convolution-only ms, training fused ms, training
+    composed ms) per pass over the layers."""
     import torch.nn.functional as F
 
     fn = getattr(lib, ("dwconv2d_fused_nhwc_" if layout == "nhwc" else "dwconv2d_fused_") + dtype)
@@ -214,8 +214,32 @@ def epilogue_comparison(layers, lib, torch, stream, dtype, layout, iters=10):
         for l, _, _, _, _, _ in prepared:
             call(l, None, None, 0)
 
+    # the same block in training: forward + backward through the fused autograd Function (recompute, one
+    # epilogue-backward sweep) against depthwise_conv2d followed by PyTorch's differentiable elementwise ops
+    from torch_dwconv.dwconv import depthwise_conv2d, depthwise_conv2d_fused
+
+    train = []
+    for l, scale, shift, _, _, _ in prepared:
+        n, c, h, w, oh, ow, k, s, p = l.geom
+        fmt = torch.channels_last if layout == "nhwc" else torch.contiguous_format
+        x = (l.x.view(n, h, w, c).permute(0, 3, 1, 2) if layout == "nhwc" else l.x).detach().requires_grad_(True)
+        gy = l.gy.view(n, oh, ow, c).permute(0, 3, 1, 2) if layout == "nhwc" else l.gy
+        assert x.is_contiguous(memory_format=fmt)
+        train.append((x, l.w.detach().requires_grad_(True), scale.detach().requires_grad_(True),
+                      shift.detach().requires_grad_(True), gy, s, p))
+
+    def train_fused():
+        for x, w, scale, shift, gy, s, p in train:
+            y = depthwise_conv2d_fused(x, w, shift, scale, "silu", s, p)
+            torch.autograd.grad(y, (x, w, scale, shift), gy)
+
+    def train_composed():
+        for x, w, scale, shift, gy, s, p in train:
+            y = F.silu(depthwise_conv2d(x, w, stride=s, padding=p) * scale.view(1, -1, 1, 1) + shift.view(1, -1, 1, 1))
+            torch.autograd.grad(y, (x, w, scale, shift), gy)
+
     out = []
-    for run in (fused, unfused, conv_only):
+    for run in (fused, unfused, conv_only, train_fused, train_composed):
         run()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -424,12 +448,15 @@ def main():
         except Exception as e:  # the comparison is informative only
             result["miopen_native_ms_per_step"] = f"failed: {type(e).__name__}"
     if args.epilogue:
-        fused_ms, unfused_ms, conv_ms = epilogue_comparison(layers, lib, torch, stream, args.dtype, args.layout)
+        fused_ms, unfused_ms, conv_ms, train_fused_ms, train_composed_ms = epilogue_comparison(
+            layers, lib, torch, stream, args.dtype, args.layout)
         result["fused_epilogue"] = {"what": "forward + per-channel scale/shift + SiLU over the workload's layers",
                                     "fused_ms": round(fused_ms, 4), "conv_then_torch_elementwise_ms": round(unfused_ms, 4),
-                                    "conv_only_ms": round(conv_ms, 4)}
+                                    "conv_only_ms": round(conv_ms, 4),
+                                    "training_fwd_bwd_fused_ms": round(train_fused_ms, 4),
+                                    "training_fwd_bwd_conv_then_torch_elementwise_ms": round(train_composed_ms, 4)}
     if not args.no_cpu_baseline and args.dtype == "f32" and args.layout == "nchw":
-        result["cpu_baseline"] = cpu_baseline(shapes, torch)
+        result["cpu_baseline"] = cpu_baseline(layers, torch)
     print(json.dumps(result))
 
 

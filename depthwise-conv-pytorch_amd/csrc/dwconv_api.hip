@@ -716,6 +716,39 @@ DWCONV_FUSED_ENTRY_POINTS(f16, unsigned short, half_t, float)
 DWCONV_FUSED_ENTRY_POINTS(bf16, unsigned short, bf16_t, float)
 #undef DWCONV_FUSED_ENTRY_POINTS
 
+// ---- backward of the fused epilogue ----
+size_t dwconv2d_epilogue_backward_workspace_bytes(int batch, int channel, int out_h, int out_w, int channels_last)
+{
+    return epilogue_backward_workspace(batch, channel, out_h, out_w, channels_last != 0);
+}
+
+#define DWCONV_EPILOGUE_BACKWARD(SUFFIX, CTYPE, TYPE)                                                                  \
+    int dwconv2d_epilogue_backward_##SUFFIX(const CTYPE *conv_out, const CTYPE *out_grad, const float *scale,           \
+                                            const float *shift, CTYPE *conv_out_grad, float *scale_shift_grad,          \
+                                            void *workspace, size_t workspace_bytes, int batch, int channel, int out_h, \
+                                            int out_w, int activation, int channels_last, void *stream)                 \
+    {                                                                                                                  \
+        if (check_activation(activation) != DWCONV_OK) return DWCONV_ERR_INVALID_ARGUMENT;                             \
+        if (batch < 0 || channel < 0 || out_h < 0 || out_w < 0)                                                        \
+            return fail(DWCONV_ERR_INVALID_ARGUMENT, "negative tensor extent");                                        \
+        if (channel > 0 && scale_shift_grad == nullptr) return fail(DWCONV_ERR_INVALID_ARGUMENT, "null gradient pointer"); \
+        if (1ll * batch * channel * out_h * out_w == 0) {                                                              \
+            note_variant("zero");                                                                                      \
+            return launch_fill_zero(scale_shift_grad, static_cast<size_t>(channel) * 2 * sizeof(float),                \
+                                    static_cast<hipStream_t>(stream));                                                 \
+        }                                                                                                              \
+        if (conv_out == nullptr || out_grad == nullptr || conv_out_grad == nullptr)                                    \
+            return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");                                           \
+        return epilogue_backward<TYPE>(reinterpret_cast<const TYPE *>(conv_out), reinterpret_cast<const TYPE *>(out_grad), \
+                                       scale, shift, reinterpret_cast<TYPE *>(conv_out_grad), scale_shift_grad, workspace, \
+                                       workspace_bytes, batch, channel, out_h, out_w, activation, channels_last != 0,  \
+                                       static_cast<hipStream_t>(stream));                                              \
+    }
+DWCONV_EPILOGUE_BACKWARD(f32, float, float)
+DWCONV_EPILOGUE_BACKWARD(f16, unsigned short, half_t)
+DWCONV_EPILOGUE_BACKWARD(bf16, unsigned short, bf16_t)
+#undef DWCONV_EPILOGUE_BACKWARD
+
 // ---- dilation and depth multiplier ----
 size_t dwconv2d_general_backward_workspace_bytes(int batch, int channel, int in_h, int in_w, int multiplier,
                                                  int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h,

@@ -263,6 +263,13 @@ template <typename T>
 int nhwc_grad_weight(const T *x, const T *gy, T *gw, void *ws, size_t ws_bytes, const NhwcGeometry &g,
                      hipStream_t stream);
 
+// ---- backward of the fused forward epilogue: dwconv_epilogue_bwd.hip (IO = float, half_t or bf16_t) ----
+size_t epilogue_backward_workspace(int batch, int channel, int out_h, int out_w, bool channels_last);
+template <typename IO>
+int epilogue_backward(const IO *conv, const IO *out_grad, const float *scale, const float *shift, IO *conv_grad,
+                      float *param_grad, void *ws, size_t ws_bytes, int batch, int channel, int out_h, int out_w, int act,
+                      bool channels_last, hipStream_t stream);
+
 // ---- dilation and depth multiplier: dwconv_general.hip (T = float, double, half_t or bf16_t) ----
 template <typename T>
 int general_forward(const T *in, const T *taps, T *out, const GeneralGeometry &g, hipStream_t stream);

@@ -541,15 +541,14 @@ __global__ __launch_bounds__(256) void nhwc_wgrad_final_kernel(const float *__re
     const int k0 = part * per, k1 = min(chunks, k0 + per);
     const float *src = partial + (live ? e : 0);
     double s = 0.0;
-    int k = k0;
-    for (; k + 8 <= k1; k += 8) {
+    // eight loads at a time, the ones past this lane's share replaced by zero (never a one-by-one tail)
+    for (int k = k0; k < k1; k += 8) {
         float v[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = src[(k + j) * stride];
+        for (int j = 0; j < 8; ++j) v[j] = src[min(k + j, k1 - 1) * stride];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) s += static_cast<double>(v[j]);
+        for (int j = 0; j < 8; ++j) s += static_cast<double>(k + j < k1 ? v[j] : 0.f);
     }
-    for (; k < k1; ++k) s += static_cast<double>(src[k * stride]);
     red[part][el] = s;
     __syncthreads();
     if (part == 0 && live) {

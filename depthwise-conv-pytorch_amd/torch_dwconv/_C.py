@@ -71,6 +71,12 @@ for _sfx in ("f32", "f64", "f16", "bf16"):
         getattr(_lib, _name).restype = _i
         getattr(_lib, _name).argtypes = [_p, _p, _p, _p, _p] + [_i] * 11 + [_p]
 
+_lib.dwconv2d_epilogue_backward_workspace_bytes.restype = _z
+_lib.dwconv2d_epilogue_backward_workspace_bytes.argtypes = [_i] * 5
+for _sfx in ("f32", "f16", "bf16"):
+    getattr(_lib, "dwconv2d_epilogue_backward_" + _sfx).restype = _i
+    getattr(_lib, "dwconv2d_epilogue_backward_" + _sfx).argtypes = [_p] * 7 + [_z] + [_i] * 6 + [_p]
+
 _lib.dwconv2d_general_backward_workspace_bytes.restype = _z
 _lib.dwconv2d_general_backward_workspace_bytes.argtypes = [_i] * 14
 for _sfx in ("f32", "f64", "f16", "bf16"):
@@ -372,6 +378,49 @@ def dwconv2d_fused(input, kernel, scale, shift, activation, stride_h, stride_w, 
     if rc != 0:
         _raise(rc)
     return out
+
+
+def dwconv2d_epilogue_backward(conv_out, out_grad, scale, shift, activation):
+    """Backward of ``act(conv_out * scale[c] + shift[c])`` in one sweep (float32, float16 or bfloat16; NCHW or
+    channels-last, taken from ``conv_out``): returns ``(conv_out_grad, scale_grad, shift_grad)``.  ``conv_out`` is
+    overwritten with ``conv_out_grad`` (the same tensor comes back); the two parameter gradients are float32
+    vectors of ``C`` entries.  No counterpart in the reference."""
+    _check_cuda(conv_out, "conv_out")
+    _check_cuda(out_grad, "out_grad")
+    sfx = _suffix(conv_out, out_grad)
+    if sfx == "f64":
+        raise RuntimeError("dwconv2d_epilogue_backward has no float64 entry point")
+    if activation not in ACTIVATIONS:
+        raise ValueError(f"unknown activation {activation!r}; expected one of None, 'relu', 'relu6', 'silu'")
+    if conv_out.dim() != 4 or out_grad.shape != conv_out.shape:
+        raise RuntimeError(f"out_grad of shape {tuple(out_grad.shape)} does not belong to conv_out {tuple(conv_out.shape)}")
+    nhwc = is_channels_last(conv_out)
+    fmt = torch.channels_last if nhwc else torch.contiguous_format
+    if not conv_out.is_contiguous(memory_format=fmt):
+        raise RuntimeError("conv_out must be dense (NCHW or channels-last): it is overwritten in place")
+    gy = out_grad.contiguous(memory_format=fmt)
+    n, c, oh, ow = conv_out.shape
+    params = []
+    for name, t in (("scale", scale), ("shift", shift)):
+        if t is None:
+            params.append(None)
+            continue
+        _check_cuda(t, name)
+        if t.numel() != c:
+            raise RuntimeError(f"{name} must have one entry per channel ({c}), got {tuple(t.shape)}")
+        params.append(t.detach().reshape(-1).to(device=conv_out.device, dtype=torch.float32).contiguous())
+    grads = torch.empty((c, 2), dtype=torch.float32, device=conv_out.device)
+    ws_bytes = _lib.dwconv2d_epilogue_backward_workspace_bytes(n, c, oh, ow, int(nhwc))
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=conv_out.device)
+    with torch.cuda.device(conv_out.device):
+        rc = getattr(_lib, "dwconv2d_epilogue_backward_" + sfx)(
+            conv_out.data_ptr(), gy.data_ptr(), params[0].data_ptr() if params[0] is not None else None,
+            params[1].data_ptr() if params[1] is not None else None, conv_out.data_ptr(), grads.data_ptr(),
+            ws.data_ptr(), ws_bytes, n, c, oh, ow, ACTIVATIONS[activation], int(nhwc), _stream(conv_out),
+        )
+    if rc != 0:
+        _raise(rc)
+    return conv_out, grads[:, 0], grads[:, 1]
 
 
 # ---- dilation and depth multiplier -----------------------------------------------------------------------

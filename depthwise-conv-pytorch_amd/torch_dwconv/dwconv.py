@@ -185,13 +185,55 @@ def depthwise_conv2d_general(input, weight, stride=1, padding=0, dilation=1):
 _TORCH_ACTIVATIONS = {None: None, "none": None, "relu": F.relu, "relu6": F.relu6, "silu": F.silu}
 
 
+class DepthwiseConv2dFusedFunction(Function):
+    """Autograd wrapper of the fused forward ``act(conv(x, w) * scale + shift)`` (not in the reference).
+
+    Forward: one kernel; only the inputs are kept for the backward pass (no pre-activation tensor).  Backward:
+    the convolution result is recomputed with the plain forward kernel, one sweep turns it and ``grad_output``
+    into the gradient of the convolution result plus the gradients of ``scale`` and ``shift``
+    (``_C.dwconv2d_epilogue_backward``), and that goes through the ordinary backward kernels."""
+
+    @staticmethod
+    def forward(ctx, input, kernel, scale, shift, activation, stride, pad):
+        ctx.save_for_backward(input, kernel, scale, shift)
+        ctx.activation, ctx.stride, ctx.pad = activation, stride, pad
+        return _C.dwconv2d_fused(input, kernel, scale, shift, activation, stride[0], stride[1], pad[0], pad[1])
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, kernel, scale, shift = ctx.saved_tensors
+        stride, pad = ctx.stride, ctx.pad
+        need_input, need_kernel, need_scale, need_shift = ctx.needs_input_grad[:4]
+        if _C.is_channels_last(input):
+            conv = _C.dwconv2d_nhwc(input, kernel, stride[0], stride[1], pad[0], pad[1])
+        else:
+            conv = _C.dwconv2d(input, kernel, 1, 1, stride[0], stride[1], pad[0], pad[0], pad[1], pad[1], True)
+        conv_grad, scale_grad, shift_grad = _C.dwconv2d_epilogue_backward(conv, grad_output, scale, shift, ctx.activation)
+        grad_input = grad_kernel = None
+        if _C.is_channels_last(input):
+            grad_input, grad_kernel = _C.dwconv2d_backward_nhwc(input, conv_grad, kernel, stride[0], stride[1], pad[0],
+                                                                pad[1], need_input, need_kernel)
+        elif need_input and need_kernel:
+            grad_input, grad_kernel = _C.dwconv2d_backward(input, conv_grad, kernel, stride[0], stride[1], pad[0], pad[1])
+        elif need_input:
+            g_pad = tuple(v for a in (0, 1) for v in (kernel.shape[2 + a] - pad[a] - 1,
+                                                      input.shape[2 + a] - conv.shape[2 + a] * stride[a] + pad[a]))
+            grad_input = _C.dwconv2d(conv_grad, kernel, stride[0], stride[1], 1, 1, *g_pad, False)
+        elif need_kernel:
+            grad_kernel = _C.dwconv2d_backward_kernel(input, conv_grad, kernel, 1, 1, stride[0], stride[1], pad[0], pad[1])
+        scale_grad = scale_grad.to(scale.dtype).view_as(scale) if need_scale and scale is not None else None
+        shift_grad = shift_grad.to(shift.dtype).view_as(shift) if need_shift and shift is not None else None
+        return grad_input, grad_kernel, scale_grad, shift_grad, None, None, None
+
+
 def depthwise_conv2d_fused(input, weight, bias=None, scale=None, activation=None, stride=1, padding=0):
     """``act(depthwise_conv2d(input, weight) * scale[c] + bias[c])``: the convolution together with the step that
     follows it in EfficientNet / MobileNet blocks (bias or folded batch-norm, then ReLU / ReLU6 / SiLU).
 
-    Not in the reference, whose ``check_options`` rejects a bias (torch_dwconv/dwconv.py:108-109).  Without
-    gradients (inference) this is one kernel; when a gradient is needed the same value is composed from
-    ``depthwise_conv2d`` and PyTorch's elementwise ops, so that autograd differentiates it.
+    Not in the reference, whose ``check_options`` rejects a bias (torch_dwconv/dwconv.py:108-109).  One kernel in the
+    forward pass, with or without gradients.  In training the backward pass recomputes the convolution result instead of
+    keeping it (``DepthwiseConv2dFusedFunction``); float64 tensors, which have no such kernels, are composed from
+    ``depthwise_conv2d`` and PyTorch's elementwise ops when a gradient is needed.
     """
     if activation not in _TORCH_ACTIVATIONS:
         raise ValueError(f"unknown activation {activation!r}; expected one of None, 'relu', 'relu6', 'silu'")
@@ -203,6 +245,8 @@ def depthwise_conv2d_fused(input, weight, bias=None, scale=None, activation=None
     )
     if not needs_grad:
         return _C.dwconv2d_fused(input, weight, scale, bias, activation, stride[0], stride[1], padding[0], padding[1])
+    if input.dtype != torch.float64:
+        return DepthwiseConv2dFusedFunction.apply(input, weight, scale, bias, activation, stride, padding)
     out = depthwise_conv2d(input, weight, None, stride, padding)
     if scale is not None:
         out = out * scale.view(1, -1, 1, 1).to(out.dtype)

@@ -308,6 +308,26 @@ int dwconv2d_fused_nhwc_bf16(const unsigned short *input, const unsigned short *
     int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
     int activation, void *stream);
 
+/* Backward of that epilogue, for training through the fused forward (no counterpart in the reference).  The fused
+ * forward keeps nothing but its inputs; in the backward pass the caller recomputes conv_out = conv(input, kernel)
+ * with dwconv2d_* / dwconv2d_nhwc_* and calls this entry point, which makes in one sweep
+ *   conv_out_grad       = out_grad * act'(z) * scale[c],   z = conv_out * scale[c] + shift[c]
+ *   scale_shift_grad[c][0] = sum over (n,y,x) of out_grad * act'(z) * conv_out      (gradient of scale)
+ *   scale_shift_grad[c][1] = sum over (n,y,x) of out_grad * act'(z)                 (gradient of shift)
+ * conv_out_grad (it may alias conv_out) is then the out_grad of dwconv2d_backward_*.  Tensors are
+ * (N,C,OH,OW) or, with channels_last != 0, (N,OH,OW,C); scale / shift may be NULL as in the forward;
+ * scale_shift_grad holds 2 * channel floats and is bit-identical from run to run.  fp32 arithmetic. */
+size_t dwconv2d_epilogue_backward_workspace_bytes(int batch, int channel, int out_h, int out_w, int channels_last);
+int dwconv2d_epilogue_backward_f32(const float *conv_out, const float *out_grad, const float *scale, const float *shift,
+    float *conv_out_grad, float *scale_shift_grad, void *workspace, size_t workspace_bytes, int batch, int channel,
+    int out_h, int out_w, int activation, int channels_last, void *stream);
+int dwconv2d_epilogue_backward_f16(const unsigned short *conv_out, const unsigned short *out_grad, const float *scale,
+    const float *shift, unsigned short *conv_out_grad, float *scale_shift_grad, void *workspace, size_t workspace_bytes,
+    int batch, int channel, int out_h, int out_w, int activation, int channels_last, void *stream);
+int dwconv2d_epilogue_backward_bf16(const unsigned short *conv_out, const unsigned short *out_grad, const float *scale,
+    const float *shift, unsigned short *conv_out_grad, float *scale_shift_grad, void *workspace, size_t workspace_bytes,
+    int batch, int channel, int out_h, int out_w, int activation, int channels_last, void *stream);
+
 /* ---- dilation and depth multiplier ------------------------------------------------------------------
  * The two options the reference's check_options refuses (torch_dwconv/dwconv.py:99-106): a dilation
  * above 1 and out_channels = multiplier * in_channels.  input (N,C,H,W); kernel and kernel_grad

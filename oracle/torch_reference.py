@@ -79,10 +79,11 @@ def torch_reference_fused(x, w, scale=None, shift=None, activation=None, stride=
     return _ACTIVATIONS[activation](y)
 
 
-def torch_cpu_fp32_step(x, w, gy, stride, padding, iters=3, threads=None):
+def torch_cpu_fp32_step(x, w, gy, stride, padding, iters=3, threads=None, all_times=False):
     """Time fp32 ``F.conv2d(groups=C)`` forward + both gradients on the host cores.
 
-    Baseline only (never the correctness oracle).  Returns (median seconds, threads).
+    Baseline only (never the correctness oracle).  Returns (median seconds, threads), or with ``all_times`` the list
+    of the ``iters`` timings in run order (after one untimed warm-up pass) instead of their median.
     """
     if threads:
         torch.set_num_threads(threads)
@@ -95,5 +96,7 @@ def torch_cpu_fp32_step(x, w, gy, stride, padding, iters=3, threads=None):
         y = F.conv2d(x, w, stride=stride, padding=padding, groups=x.shape[1])
         torch.autograd.grad(y, (x, w), gy)
         times.append(time.perf_counter() - t0)
+    if all_times:
+        return times[1:], torch.get_num_threads()
     times = sorted(times[1:])
     return times[len(times) // 2], torch.get_num_threads()

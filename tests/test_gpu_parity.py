@@ -839,7 +839,7 @@ def test_fused_epilogue_other_dtypes_and_autograd(dw, gpu):
         assert y.dtype == dtype
         ref = oracle.torch_reference_fused(xs, ws, scale, shift, "relu6", s, p)
         np.testing.assert_allclose(_np(y.double()), ref.numpy(), rtol=step, atol=1e-5 + step * 1e-2)
-    # with gradients the value is composed from differentiable pieces: same value, gradients as torch's
+    # with gradients: the same fused forward kernel, gradients as torch's
     xg = x.to(gpu).requires_grad_(True)
     wg = wt.to(gpu).requires_grad_(True)
     bg = shift.to(gpu).requires_grad_(True)
@@ -865,6 +865,116 @@ def test_fused_epilogue_other_dtypes_and_autograd(dw, gpu):
     rc = _C._lib.dwconv2d_fused_f32(xg.data_ptr(), wg.data_ptr(), None, None, y_fused.data_ptr(), n, c, h, w, k, k,
                                     s, s, p, p, 9, None)
     assert rc == 1 and b"activation" in _C._lib.dwconv_last_error()
+
+
+def _fused_reference_grads(x, wt, scale, shift, gy, activation, s, p):
+    """fp64 CPU autograd of PyTorch's own composition conv -> * scale -> + shift -> activation."""
+    import torch.nn.functional as F
+
+    act = {None: lambda v: v, "relu": F.relu, "relu6": F.relu6, "silu": F.silu}[activation]
+    leaves = [t.double().requires_grad_(True) if t is not None else None for t in (x, wt, scale, shift)]
+    xr, wr, sr, br = leaves
+    y = F.conv2d(xr, wr, stride=s, padding=p, groups=x.shape[1])
+    if sr is not None:
+        y = y * sr.view(1, -1, 1, 1)
+    if br is not None:
+        y = y + br.view(1, -1, 1, 1)
+    y = act(y)
+    wanted = [t for t in leaves if t is not None]
+    grads = iter(torch.autograd.grad(y, wanted, gy.double()))
+    return y.detach(), [next(grads) if t is not None else None for t in leaves]
+
+
+FUSED_TRAIN_CASES = [
+    # shape, channels_last: every backward kernel family behind the fused training path
+    ((3, 8, 56, 56, 3, 1, 1), False), ((2, 6, 30, 33, 5, 2, 2), False), ((4, 12, 14, 14, 5, 1, 2), False),
+    ((3, 8, 7, 7, 3, 1, 1), False), ((2, 5, 9, 11, 4, 2, 1), False), ((2, 16, 20, 24, 3, 1, 1), True),
+    ((2, 8, 15, 13, 5, 2, 2), True), ((2, 5, 9, 9, 3, 1, 1), True),
+]
+
+
+@pytest.mark.parametrize("activation", [None, "relu", "relu6", "silu"])
+@pytest.mark.parametrize("case", FUSED_TRAIN_CASES, ids=lambda c: shape_id(c[0]) + ("_nhwc" if c[1] else ""))
+def test_fused_epilogue_training_path(dw, gpu, case, activation):
+    """Training through the fused forward: one forward kernel (no saved pre-activation), and a backward that
+    recomputes the convolution and runs the epilogue-backward sweep; all four gradients against fp64 autograd of
+    PyTorch's own composition, layouts preserved, parameter gradients bit-identical from run to run."""
+    from torch_dwconv import _C
+    from torch_dwconv.dwconv import depthwise_conv2d_fused
+
+    shape, nhwc = case
+    n, c, h, w, k, s, p = shape
+    x, wt, gy = make_inputs(shape, seed=47)
+    x = x * 2
+    g = torch.Generator("cpu").manual_seed(48)
+    scale = torch.randn(c, generator=g) + 1.5
+    shift = torch.randn(c, generator=g)
+    fmt = torch.channels_last if nhwc else torch.contiguous_format
+    for sc, sh in [(scale, shift), (None, shift), (scale, None)]:
+        leaves = [x.to(gpu).contiguous(memory_format=fmt).requires_grad_(True), wt.to(gpu).requires_grad_(True),
+                  sc.to(gpu).requires_grad_(True) if sc is not None else None,
+                  sh.to(gpu).requires_grad_(True) if sh is not None else None]
+        xg, wg, sg, bg = leaves
+        y = depthwise_conv2d_fused(xg, wg, bg, sg, activation, s, p)
+        assert y.grad_fn is not None and "Fused" in type(y.grad_fn).__name__
+        assert y.is_contiguous(memory_format=fmt)
+        wanted = [t for t in leaves if t is not None]
+        got = iter(torch.autograd.grad(y, wanted, gy.to(gpu).contiguous(memory_format=fmt), retain_graph=True))
+        got = [next(got) if t is not None else None for t in leaves]
+        _announce(shape_id(shape), "nhwc" if nhwc else "nchw", activation, _C.last_variant())
+        y_ref, ref = _fused_reference_grads(x, wt, sc, sh, gy, activation, s, p)
+        np.testing.assert_allclose(_np(y).astype(np.float64), y_ref.numpy(), rtol=1e-5, atol=1e-5)
+        assert got[0].is_contiguous(memory_format=fmt)
+        np.testing.assert_allclose(_np(got[0]).astype(np.float64), ref[0].numpy(), rtol=1e-4, atol=2e-5)
+        for a, b in zip(got[1:], ref[1:]):
+            if b is None:
+                assert a is None
+                continue
+            assert a.shape == b.shape and a.dtype == torch.float32
+            np.testing.assert_allclose(_np(a).astype(np.float64), b.numpy(), rtol=1e-4, atol=1e-4 * float(b.abs().max()))
+        again = iter(torch.autograd.grad(y, wanted, gy.to(gpu).contiguous(memory_format=fmt)))
+        again = [next(again) if t is not None else None for t in leaves]
+        for a, b in zip(got, again):
+            assert (a is None and b is None) or torch.equal(a, b)
+
+
+def test_fused_epilogue_training_partial_gradients_and_dtypes(dw, gpu):
+    """Only the gradients that are asked for come back; 16-bit tensors train through the same path."""
+    from torch_dwconv.dwconv import depthwise_conv2d_fused
+
+    shape = (3, 8, 28, 28, 5, 2, 2)
+    n, c, h, w, k, s, p = shape
+    x, wt, gy = make_inputs(shape, seed=49)
+    scale, shift = torch.linspace(0.5, 2.0, c), torch.linspace(-1.0, 1.0, c)
+    _, ref = _fused_reference_grads(x, wt, scale, shift, gy, "silu", s, p)
+    # frozen filter and scale: gradients of the input and the bias only
+    xg = x.to(gpu).requires_grad_(True)
+    bg = shift.to(gpu).requires_grad_(True)
+    y = depthwise_conv2d_fused(xg, wt.to(gpu), bg, scale.to(gpu), "silu", s, p)
+    y.backward(gy.to(gpu))
+    np.testing.assert_allclose(_np(xg.grad).astype(np.float64), ref[0].numpy(), rtol=1e-4, atol=2e-5)
+    np.testing.assert_allclose(_np(bg.grad).astype(np.float64), ref[3].numpy(), rtol=1e-4, atol=1e-4 * float(ref[3].abs().max()))
+    # frozen input: gradients of the filter and the scale
+    wg = wt.to(gpu).requires_grad_(True)
+    sg = scale.to(gpu).requires_grad_(True)
+    depthwise_conv2d_fused(x.to(gpu), wg, shift.to(gpu), sg, "silu", s, p).backward(gy.to(gpu))
+    np.testing.assert_allclose(_np(wg.grad).astype(np.float64), ref[1].numpy(), rtol=1e-4, atol=1e-4 * float(ref[1].abs().max()))
+    np.testing.assert_allclose(_np(sg.grad).astype(np.float64), ref[2].numpy(), rtol=1e-4, atol=1e-4 * float(ref[2].abs().max()))
+    for dtype, step in [(torch.float16, 2.0 ** -11), (torch.bfloat16, 2.0 ** -8)]:
+        xs, ws, gs = x.to(dtype), wt.to(dtype), gy.to(dtype)
+        # a smooth activation: with ReLU6 an element whose pre-activation sits within a rounding step of a corner
+        # can land on the other side when the recomputed convolution result is rounded to 16 bits
+        _, refh = _fused_reference_grads(xs, ws, scale, shift, gs, "silu", s, p)
+        leaves = [xs.to(gpu).requires_grad_(True), ws.to(gpu).requires_grad_(True), scale.to(gpu).requires_grad_(True),
+                  shift.to(gpu).requires_grad_(True)]
+        y = depthwise_conv2d_fused(leaves[0], leaves[1], leaves[3], leaves[2], "silu", s, p)
+        got = torch.autograd.grad(y, leaves, gs.to(gpu))
+        assert got[0].dtype == dtype and got[1].dtype == dtype and got[2].dtype == torch.float32
+        # the recomputed convolution result and its gradient are rounded to the 16-bit format on the way (as the
+        # intermediate tensors of PyTorch's own composition would be): a few rounding steps of tolerance
+        np.testing.assert_allclose(_np(got[0].double()), refh[0].numpy(), rtol=4 * step, atol=4 * step * float(refh[0].abs().max()))
+        for a, b in zip(got[1:], refh[1:]):
+            np.testing.assert_allclose(_np(a.double()), b.numpy(), rtol=4 * step + 1e-3, atol=(4 * step + 1e-3) * float(b.abs().max()))
 
 
 def test_plane_beyond_two_gib(dw, gpu):

@@ -45,8 +45,21 @@ def test_registered_ops_have_fake_implementations():
         x, w = torch.empty(2, 8, 17, 19), torch.empty(8, 1, 5, 5)
         y = torch.ops.torch_dwconv.depthwise_conv2d(x, w, [2, 2], [2, 2])
         assert tuple(y.shape) == (2, 8, 9, 10)
-        gx, gw = torch.ops.torch_dwconv.depthwise_conv2d_backward(x, y, w, [2, 2], [2, 2])
-        assert gx.shape == x.shape and gw.shape == w.shape
+        assert y.is_contiguous()
+        gx, gw = torch.ops.torch_dwconv.depthwise_conv2d_backward(x, y, w, [2, 2], [2, 2], [True, True])
+        assert gx.shape == x.shape and gw.shape == w.shape and gx.is_contiguous()
+        gx, gw = torch.ops.torch_dwconv.depthwise_conv2d_backward(x, y, w, [2, 2], [2, 2], [False, True])
+        assert gx.numel() == 0 and gw.shape == w.shape
+        # channels-last in, channels-last out (strides as the real kernels produce them)
+        xc = x.contiguous(memory_format=torch.channels_last)
+        yc = torch.ops.torch_dwconv.depthwise_conv2d(xc, w, [2, 2], [2, 2])
+        assert yc.is_contiguous(memory_format=torch.channels_last) and not yc.is_contiguous()
+        gx, _ = torch.ops.torch_dwconv.depthwise_conv2d_backward(xc, yc, w, [2, 2], [2, 2], [True, False])
+        assert gx.stride() == xc.stride()
+        # an input that is neither dense NCHW nor channels-last is computed (and returned) dense NCHW
+        xs = torch.empty(2, 8, 17, 38)[:, :, :, ::2]
+        gx, _ = torch.ops.torch_dwconv.depthwise_conv2d_backward(xs, y, w, [2, 2], [2, 2], [True, True])
+        assert gx.is_contiguous()
 
 
 def test_compiled_entry_keeps_the_option_checks():
@@ -77,6 +90,53 @@ def test_registered_op_values_gradients_and_compile(gpu):
         # through torch.compile without a code generator: the op stays one opaque node
         fn = torch.compile(lambda a, b: compiled_depthwise_conv2d(a, b, stride=s, padding=k // 2) * 2.0, backend="aot_eager")
         torch.testing.assert_close(fn(x, w), y_ref * 2.0)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("layout", ["nchw", "nhwc"])
+def test_registered_op_backward_through_compile(gpu, layout):
+    """Forward and backward traced by torch.compile (AOT autograd, fake tensors first): values, memory layouts and the
+    skipping of a gradient nobody wants, for dense NCHW and channels-last inputs, against the eager autograd Function
+    and against the fp64 oracle."""
+    import numpy as np
+
+    import oracle
+    from torch_dwconv import _C, depthwise_conv2d
+    from torch_dwconv.ops import compiled_depthwise_conv2d
+
+    fmt = torch.channels_last if layout == "nhwc" else torch.contiguous_format
+    g = torch.Generator("cpu").manual_seed(5)
+    for (c, h, k, s) in [(8, 28, 3, 1), (12, 30, 5, 2)]:
+        p = k // 2
+        x0 = torch.randn(3, c, h, h, generator=g)
+        w0 = torch.randn(c, 1, k, k, generator=g) / k
+        x = x0.to(gpu).contiguous(memory_format=fmt).requires_grad_(True)
+        w = w0.to(gpu).requires_grad_(True)
+        fn = torch.compile(lambda a, b: compiled_depthwise_conv2d(a, b, stride=s, padding=p), backend="aot_eager")
+        y = fn(x, w)
+        assert y.is_contiguous(memory_format=fmt)
+        gy0 = torch.randn(y.shape, generator=g)
+        gy = gy0.to(gpu).contiguous(memory_format=fmt)
+        gx, gw = torch.autograd.grad(y, (x, w), gy)
+        assert gx.is_contiguous(memory_format=fmt) and gw.is_contiguous()
+        variant = _C.last_variant()
+        assert variant.startswith("nhwc_") == (layout == "nhwc"), variant
+        y_e = depthwise_conv2d(x, w, stride=s, padding=p)
+        gx_e, gw_e = torch.autograd.grad(y_e, (x, w), gy)
+        assert torch.equal(y, y_e) and torch.equal(gx, gx_e) and torch.equal(gw, gw_e)
+        np.testing.assert_allclose(y.detach().cpu().numpy(), oracle.forward(x0.numpy(), w0.numpy(), s, p), rtol=1e-5, atol=1e-5)
+        np.testing.assert_allclose(gx.cpu().numpy(), oracle.grad_input(gy0.numpy(), w0.numpy(), (h, h), s, p), rtol=1e-5, atol=1e-5)
+        gw_ref = oracle.grad_weight(x0.numpy(), gy0.numpy(), w0.shape, s, p)
+        np.testing.assert_allclose(gw.cpu().numpy(), gw_ref, rtol=1e-4, atol=1e-4 * np.abs(gw_ref).max())
+        # a frozen filter: only grad-input is computed (one kernel, no grad-weight variant in the name)
+        xf = x.detach().clone().requires_grad_(True)
+        fn(xf, w.detach()).backward(gy)
+        assert torch.equal(xf.grad, gx_e)
+        assert "wgrad" not in _C.last_variant() and "bwd" not in _C.last_variant(), _C.last_variant()
+        # a frozen input: only grad-weight
+        wf = w.detach().clone().requires_grad_(True)
+        fn(x.detach(), wf).backward(gy)
+        torch.testing.assert_close(wf.grad, gw_e, rtol=1e-5, atol=1e-5)
 
 
 @pytest.mark.gpu
