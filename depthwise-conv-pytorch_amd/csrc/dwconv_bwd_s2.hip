@@ -160,7 +160,7 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
         if (VIEWS || p.vec_gx == 2) {
             // branch-free: rows and column blocks past the end of the plane store out of range
             const int ox = 4 * cb;
-            const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.gx) + plane0 * p.sx.in_plane);
+            const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.gx) + plane0 * p.sx.in_plane, static_cast<long>(p.sx.in_plane) * sizeof(IO));  // this plane only
             const bool col_ok = has_item && ox < p.sx.in_w;
 #pragma unroll
             for (int b = 0; b < 2 * BQ; ++b) {

@@ -126,7 +126,8 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_down_kernel(const NhwcPlan 
     const int n0 = static_cast<int>(static_cast<long>(pg) * p.blocks_per_wg / per_image);
     const unsigned pixel_bytes = C * sizeof(IO), row_bytes = p.in_w * pixel_bytes;
     const __amdgpu_buffer_rsrc_t view =
-        buffer_view(static_cast<const IO *>(p.in) + static_cast<long>(n0) * p.in_h * p.in_w * C);
+        buffer_view(static_cast<const IO *>(p.in) + static_cast<long>(n0) * p.in_h * p.in_w * C,
+                    static_cast<long>(p.batch - n0) * p.in_h * row_bytes);
     const unsigned lane_off = (n - n0) * (p.in_h * row_bytes) + c * static_cast<unsigned>(sizeof(IO));
 
     float acc[BH][TW * 4];
@@ -170,7 +171,8 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_down_kernel(const NhwcPlan 
     // branch-free stores through a view of the output: pixels past the edge of the image store out of range
     const unsigned out_row_bytes = p.out_w * pixel_bytes;
     const __amdgpu_buffer_rsrc_t out_view =
-        buffer_view(static_cast<IO *>(p.out) + static_cast<long>(n0) * p.out_h * p.out_w * C);
+        buffer_view(static_cast<IO *>(p.out) + static_cast<long>(n0) * p.out_h * p.out_w * C,
+                    static_cast<long>(p.batch - n0) * p.out_h * out_row_bytes);
     NhwcCols<TW> ocols;
     nhwc_cols<TW>(ox0, p.out_w, pixel_bytes, (n - n0) * (p.out_h * out_row_bytes) + c * static_cast<unsigned>(sizeof(IO)), ocols);
 #pragma unroll
@@ -224,7 +226,8 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_up2_kernel(const NhwcPlan p
     const int n0 = static_cast<int>(static_cast<long>(pg) * p.blocks_per_wg / per_image);
     const unsigned pixel_bytes = C * sizeof(IO), row_bytes = p.in_w * pixel_bytes;
     const __amdgpu_buffer_rsrc_t view =
-        buffer_view(static_cast<const IO *>(p.in) + static_cast<long>(n0) * p.in_h * p.in_w * C);
+        buffer_view(static_cast<const IO *>(p.in) + static_cast<long>(n0) * p.in_h * p.in_w * C,
+                    static_cast<long>(p.batch - n0) * p.in_h * row_bytes);
     const unsigned lane_off = (n - n0) * (p.in_h * row_bytes) + c * static_cast<unsigned>(sizeof(IO));
 
     float acc[BH][TW * 4];
@@ -264,7 +267,8 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_up2_kernel(const NhwcPlan p
 
     const unsigned out_row_bytes = p.out_w * pixel_bytes;
     const __amdgpu_buffer_rsrc_t out_view =
-        buffer_view(static_cast<IO *>(p.out) + static_cast<long>(n0) * p.out_h * p.out_w * C);
+        buffer_view(static_cast<IO *>(p.out) + static_cast<long>(n0) * p.out_h * p.out_w * C,
+                    static_cast<long>(p.batch - n0) * p.out_h * out_row_bytes);
     NhwcCols<TW> ocols;
     nhwc_cols<TW>(ix0, p.out_w, pixel_bytes, (n - n0) * (p.out_h * out_row_bytes) + c * static_cast<unsigned>(sizeof(IO)), ocols);
 #pragma unroll
@@ -317,9 +321,11 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_wgrad_kernel(const NhwcPlan
         const int n0 = static_cast<int>(grp * p.blocks_per_wg / per_image);
         const unsigned pixel_bytes = C * sizeof(IO), row_bytes = p.in_w * pixel_bytes, grow_bytes = p.out_w * pixel_bytes;
         const __amdgpu_buffer_rsrc_t xview =
-            buffer_view(static_cast<const IO *>(p.in) + static_cast<long>(n0) * p.in_h * p.in_w * C);
+            buffer_view(static_cast<const IO *>(p.in) + static_cast<long>(n0) * p.in_h * p.in_w * C,
+                    static_cast<long>(p.batch - n0) * p.in_h * row_bytes);
         const __amdgpu_buffer_rsrc_t gview =
-            buffer_view(static_cast<const IO *>(p.in2) + static_cast<long>(n0) * p.out_h * p.out_w * C);
+            buffer_view(static_cast<const IO *>(p.in2) + static_cast<long>(n0) * p.out_h * p.out_w * C,
+                    static_cast<long>(p.batch - n0) * p.out_h * grow_bytes);
         const unsigned chan_off = c * static_cast<unsigned>(sizeof(IO));
 
         // out_grad rows are fetched one window row before their first use (row b meets window rows b*S ... b*S+K-1),
@@ -426,9 +432,10 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_bwd_fused_kernel(const Nhwc
         const int n0 = static_cast<int>(grp * p.blocks_per_wg / per_image);
         const unsigned pixel_bytes = C * sizeof(IO), row_bytes = p.in_w * pixel_bytes;
         const long image0 = static_cast<long>(n0) * p.in_h * p.in_w * C;
-        const __amdgpu_buffer_rsrc_t xview = buffer_view(static_cast<const IO *>(p.in) + image0);
-        const __amdgpu_buffer_rsrc_t gview = buffer_view(static_cast<const IO *>(p.in2) + image0);
-        const __amdgpu_buffer_rsrc_t oview = buffer_view(static_cast<IO *>(p.out) + image0);
+        const long span = static_cast<long>(p.batch - n0) * p.in_h * row_bytes;  // to the end of the tensor
+        const __amdgpu_buffer_rsrc_t xview = buffer_view(static_cast<const IO *>(p.in) + image0, span);
+        const __amdgpu_buffer_rsrc_t gview = buffer_view(static_cast<const IO *>(p.in2) + image0, span);
+        const __amdgpu_buffer_rsrc_t oview = buffer_view(static_cast<IO *>(p.out) + image0, span);
         const unsigned lane_off = (n - n0) * (p.in_h * row_bytes) + c * static_cast<unsigned>(sizeof(IO));
         NhwcCols<COLS> cols;
         nhwc_cols<COLS>(ix0, p.in_w, pixel_bytes, lane_off, cols);

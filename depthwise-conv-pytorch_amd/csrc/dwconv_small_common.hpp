@@ -101,7 +101,7 @@ __device__ __forceinline__ void lds_to_run(IO *__restrict__ g, const float *lds,
 {
     const int n4 = n >> 2;
     constexpr int U = 4;
-    const __amdgpu_buffer_rsrc_t view = buffer_view(g);  // g is uniform: one run per wavefront
+    const __amdgpu_buffer_rsrc_t view = buffer_view(g, static_cast<long>(n) * sizeof(IO));  // g is uniform: one run per wavefront
     for (int base = threadIdx.x; base < n4; base += kWave * U) {
         float4 v[U];
 #pragma unroll

@@ -148,7 +148,7 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
                         make_float4(acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
         }
         __syncthreads();
-        const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane);
+        const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO));
         const int run4 = run >> 2, total4 = nplanes * run4;
         for (int i = threadIdx.x; i < total4; i += blockDim.x) {
             const int q = nplanes == 1 ? 0 : i / run4;
@@ -170,7 +170,7 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
         const int ox = 4 * cb;
         if (p.vec_out == 2) {
             // branch-free: rows past the end of the plane store out of range
-            const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane);
+            const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO));
             const unsigned o0 = (pl * p.out_plane + ox) * static_cast<unsigned>(sizeof(IO));
 #pragma unroll
             for (int b = 0; b < BH; ++b) {
@@ -275,7 +275,7 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
         const int ox = 4 * cb;
         if (p.vec_out == 2) {
             // branch-free: rows past the end of the plane store out of range
-            const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane);
+            const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO));
             const unsigned o0 = (pl * p.out_plane + ox) * static_cast<unsigned>(sizeof(IO));
 #pragma unroll
             for (int b = 0; b < 2 * BQ; ++b) {

@@ -117,16 +117,19 @@ __device__ __forceinline__ float4 widen4<bf16_t>(const uint2 &raw)
 }
 
 // ---- loads through a buffer view ------------------------------------------------------------------------------
-// A raw buffer view of kOob bytes from `base` (uniform).  A load whose byte offset is at or beyond kOob returns
-// zeros, so an element outside the image needs no branch and no select: its offset is replaced by kOob.  The
-// planners keep every real offset below kOob.
+// A raw buffer view of `bytes` bytes from `base` (both uniform): what the workgroup may really touch there.  A load
+// whose byte offset is at or beyond the extent returns zeros and a store there is dropped, so an element outside the
+// image needs no branch and no select: its offset is replaced by kOob, which is beyond every extent (extents are
+// clamped to kOob; the planners keep every real offset below it).  Because the extent is the real span and not a
+// blanket 2 GiB, an index slip in a kernel reads zeros or writes nothing instead of touching a neighbouring allocation.
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 constexpr unsigned kOob = 0x80000000u;
 
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_view(const void *base)
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_view(const void *base, long bytes)
 {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, kOob, 0x00020000);
+    const unsigned extent = bytes < static_cast<long>(kOob) ? static_cast<unsigned>(bytes) : kOob;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, extent, 0x00020000);
 }
 
 // CV consecutive elements at byte offset `off` of the view, widened to fp32.
@@ -241,7 +244,7 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__res
     const int total = nplanes * s.lds_rows * s.spr;
     if (VIEW_ONLY || s.vec_in == 2) {
         // groups of four elements through a view of the tile's planes: slots outside the image read zeros
-        const __amdgpu_buffer_rsrc_t view = buffer_view(in + plane0 * s.in_plane);
+        const __amdgpu_buffer_rsrc_t view = buffer_view(in + plane0 * s.in_plane, static_cast<long>(nplanes) * s.in_plane * sizeof(IO));
         for (int base = threadIdx.x; base < total; base += blockDim.x * kStageBatch) {
             float4 v[kStageBatch];
             int dst[kStageBatch];

@@ -136,7 +136,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
             if (p.vec_gy == 2) {
                 // branch-free: rows past the plane (and lanes without an item) read zeros through the view
                 const unsigned off = ((pl * p.out_plane + ox) + oy * p.out_w) * static_cast<unsigned>(sizeof(IO));
-                v = view_load4<IO>(buffer_view(gy + plane0 * p.out_plane), has_item && oy < p.out_h ? off : kOob);
+                v = view_load4<IO>(buffer_view(gy + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO)), has_item && oy < p.out_h ? off : kOob);
             } else if (has_item && oy < p.out_h) {
                 if (p.vec_gy) {
                     v = load4<IO>(row);
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
             }
             if (p.vec_gx == 2) {
                 // branch-free: rows past the end of the plane (and lanes without an item) store out of range
-                const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.gx) + plane0 * p.st.in_plane);
+                const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.gx) + plane0 * p.st.in_plane, static_cast<long>(nplanes) * p.st.in_plane * sizeof(IO));
                 const unsigned o0 = (pl * p.st.in_plane + ox) * static_cast<unsigned>(sizeof(IO));
 #pragma unroll
                 for (int b = 0; b < BH; ++b) {
