@@ -100,3 +100,37 @@ def test_noalloc_rejects_oversized_geometry():
                                                one.data_ptr(), n, c, h, h, h, h, k, k, 1, 1, 7, 7, None)
     assert rc == 3  # DWCONV_ERR_WORKSPACE
     assert "scratch" in _C._lib.dwconv_last_error().decode()
+
+
+def test_noalloc_inside_a_hip_graph():
+    """What the entry point is for: a backward step captured into a HIP graph (no allocation may happen during
+    capture).  Every replay, with fresh input values and eager work in between, must equal the eager call bit for bit."""
+    dev = torch.device("cuda:0")
+    shape = (8, 32, 28, 28, 5, 1, 2)
+    n, c, h, wd, k, s, p = shape
+    x, w, gy = (t.to(dev) for t in shapes.make_inputs(shape, seed=11))
+    gx = torch.empty_like(x)
+    gw = torch.empty_like(w)
+
+    def call(stream):
+        rc = _C._lib.dwconv2d_backward_noalloc_f32(x.data_ptr(), gy.data_ptr(), w.data_ptr(), gx.data_ptr(), gw.data_ptr(),
+                                                   n, c, h, wd, gy.shape[2], gy.shape[3], k, k, s, s, p, p,
+                                                   ctypes.c_void_p(stream.cuda_stream))
+        assert rc == 0, _C._lib.dwconv_last_error().decode()
+
+    call(torch.cuda.current_stream())  # first call on the device: looks up the scratch buffer, outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(torch.cuda.current_stream())
+    gen = torch.Generator("cpu").manual_seed(13)
+    for replay in range(3):
+        x.copy_(torch.randn(x.shape, generator=gen))
+        gy.copy_(torch.randn(gy.shape, generator=gen))
+        gx.fill_(float("nan"))
+        gw.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        gx_ref, gw_ref, _, _ = _reference(x, gy, w, s, p)
+        torch.cuda.synchronize()
+        assert torch.equal(gx, gx_ref) and torch.equal(gw, gw_ref), replay
