@@ -485,8 +485,10 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_bwd_fused_kernel(const Nhwc
                         const unsigned off = __builtin_elementwise_add_sat(roff, cols.off[o + P]);
                         if constexpr (CV == 4)
                             view_store4<IO>(oview, off, gxs[b][4 * o], gxs[b][4 * o + 1], gxs[b][4 * o + 2], gxs[b][4 * o + 3]);
-                        else
+                        else if constexpr (CV == 2)
                             view_store2<IO>(oview, off, gxs[b][2 * o], gxs[b][2 * o + 1]);
+                        else
+                            view_store1<IO>(oview, off, gxs[b][o]);
                     }
                 }
             }
@@ -875,14 +877,12 @@ long nhwc_wgrad_fast(int mode, const IO *x, const IO *gy, IO *gw, void *ws, size
     return -1;
 }
 
-// Fused backward of 3x3 stride-1 layers with pad 1 (the 5x5 instance needs 256 registers, one wavefront per SIMD,
-// and lost to the two separate kernels on every layer measured).  mode 0: workspace bytes; mode 1: launch.
-// -1 when the kernel does not cover g.
-template <typename IO, int K>
+// Fused backward of K x K stride-1 layers with pad K/2: CV channels per lane, BH x TW results per lane.
+// mode 0: workspace bytes; mode 1: launch.  -1 when the kernel does not cover g.
+template <typename IO, int K, int CV = 2, int BH = 7, int TW = 4>
 long nhwc_bwd_fused_case(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
                          const NhwcGeometry &g, hipStream_t stream)
 {
-    constexpr int CV = 2, BH = 7, TW = 4;
     NhwcPlan p{};
     const int line_lanes = static_cast<int>(128 / (CV * sizeof(IO)));
     if (!plan_nhwc<K, CV>(p, g, BH, TW, g.out_h, g.out_w, line_lanes, "DWCONV_NHWC_WGRAD_LANES")) return -1;
@@ -920,7 +920,7 @@ bool nhwc_fused_ok(const NhwcGeometry &g)
 {
     if (!env_int("DWCONV_NHWC_FUSED_BWD", 1) || !nhwc_fast_ok(g)) return false;
     const int K = g.kernel_h;
-    return K == 3 && g.stride_h == 1 && g.pad_h == K / 2 && g.pad_w == K / 2 && g.out_h == g.in_h &&
+    return (K == 3 || K == 5) && g.stride_h == 1 && g.pad_h == K / 2 && g.pad_w == K / 2 && g.out_h == g.in_h &&
            g.out_w == g.in_w;
 }
 
@@ -929,6 +929,18 @@ long nhwc_bwd_fused(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx,
                     const NhwcGeometry &g, hipStream_t stream)
 {
     if (!nhwc_fused_ok(g)) return -1;
+    if (g.kernel_h == 5) {
+        // 25 sums per channel: with two channels per lane the kernel needs 228 registers (7 x 2 blocks) to 262 (4 x 4)
+        // and loses to the two separate kernels; with ONE fp32 channel per lane (dword accesses, 32 lanes per
+        // 128-byte line) it fits 167 registers with 7 x 4 blocks, three wavefronts per SIMD, and wins on every 5x5
+        // layer of the stack (28x28 C=240: 112 -> 91 us, 14x14 C=672: 75 -> 68, C=480: 59 -> 50, 7x7 C=1152: 42 -> 39).
+        // 16-bit elements (two channels per 4-byte access) stay on the separate kernels.
+        if constexpr (sizeof(IO) == 4) {
+            if (env_int("DWCONV_NHWC_FUSED5", 1))
+                return nhwc_bwd_fused_case<IO, 5, 1, 7, 4>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+        }
+        return -1;
+    }
     return nhwc_bwd_fused_case<IO, 3>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
 }
 

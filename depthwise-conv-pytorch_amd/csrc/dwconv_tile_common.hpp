@@ -147,6 +147,9 @@ __device__ __forceinline__ void view_load(__amdgpu_buffer_rsrc_t view, unsigned 
             const float4 w = widen4<IO>(make_uint2(t.x, t.y));
             v[0] = w.x; v[1] = w.y; v[2] = w.z; v[3] = w.w;
         }
+    } else if constexpr (CV == 1) {
+        static_assert(sizeof(IO) == 4, "a single element per lane is an fp32 one");
+        v[0] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(view, off, 0, 0));
     } else {
         static_assert(CV == 2 && sizeof(IO) == 2, "two 16-bit elements");
         const unsigned t = __builtin_amdgcn_raw_buffer_load_b32(view, off, 0, 0);
@@ -201,6 +204,14 @@ __device__ __forceinline__ void view_store2(__amdgpu_buffer_rsrc_t view, unsigne
         else t = f16_pack2(a, b);
         __builtin_amdgcn_raw_buffer_store_b32(t, view, off, 0, POLICY);
     }
+}
+
+// One fp32 result at byte offset `off` of the view; dropped when `off` is at or beyond the extent.
+template <typename IO, int POLICY = kStoreStreaming>
+__device__ __forceinline__ void view_store1(__amdgpu_buffer_rsrc_t view, unsigned off, float a)
+{
+    static_assert(sizeof(IO) == 4, "a single element per lane is an fp32 one");
+    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(a), view, off, 0, POLICY);
 }
 
 // True when groups of four elements starting at `p` may be moved with one vector access.
