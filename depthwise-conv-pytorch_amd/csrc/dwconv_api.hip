@@ -94,6 +94,10 @@ int run_fir(const T *in, const T *taps, T *out, const Geometry &g, hipStream_t s
         if (!force_generic()) {
             int rc = try_launch_fir_small<T>(in, taps, out, g, stream);
             if (rc >= 0) return rc;
+            if constexpr (sizeof(T) == 2) {
+                rc = try_launch_fir_tiled16<T>(in, taps, out, g, stream);
+                if (rc >= 0) return rc;
+            }
             rc = try_launch_fir_tiled<T>(in, taps, out, g, stream);
             if (rc >= 0) return rc;
         }

@@ -214,6 +214,10 @@ int launch_wgrad_direct(const T *in, const T *gy, T *gw, void *ws, size_t ws_byt
 // or a positive dwconv_status on a launch error.
 template <typename IO>  // float, half_t or bf16_t
 int try_launch_fir_tiled(const IO *in, const IO *taps, IO *out, const Geometry &g, hipStream_t stream);
+// The same for 16-bit tensors whose rows are whole groups of eight elements: raw 16-bit LDS image and two-element
+// dot products (dwconv_tile16.hip).  -1 when it does not cover g.
+template <typename IO>
+int try_launch_fir_tiled16(const IO *in, const IO *taps, IO *out, const Geometry &g, hipStream_t stream);
 
 // ---- whole-plane kernels for maps 7, 14 or 28 wide: dwconv_small.hip (same return convention) ----
 template <typename IO>  // float, half_t or bf16_t

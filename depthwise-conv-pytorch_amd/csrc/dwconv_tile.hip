@@ -79,7 +79,7 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
     const int oy0 = rt * p.rows_per_tile;
 
     stage_taps<IO, KK, FLIP>(p, lds, plane0, nplanes);
-    stage_tile(p.st, static_cast<const IO *>(p.in), lds, plane0, nplanes, oy0 * S - p.row_shift);
+    stage_tile<IO, false, kStageBatch, true>(p.st, static_cast<const IO *>(p.in), lds, plane0, nplanes, oy0 * S - p.row_shift);
     __syncthreads();
 
     const int n_items = nplanes * p.items_per_plane;
@@ -220,7 +220,7 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
     const int qy0 = rt * p.rows_per_tile;
 
     stage_taps<IO, KK, true>(p, lds, plane0, nplanes);
-    stage_tile(p.st, static_cast<const IO *>(p.in), lds, plane0, nplanes, qy0 - p.row_shift);
+    stage_tile<IO, false, kStageBatch, true>(p.st, static_cast<const IO *>(p.in), lds, plane0, nplanes, qy0 - p.row_shift);
     __syncthreads();
 
     const int n_items = nplanes * p.items_per_plane;
@@ -373,7 +373,9 @@ int launch_down(TilePlan &p, hipStream_t stream)
     auto rows_for = [](int units) { return (units * BH - 1) * S + K; };
     // A stride-2 layer reads four times what it writes: smaller tiles (more workgroups per CU, more loads in flight)
     // beat the halo rows they add: -17 % on a 56x56 5x5 layer, -3 % on a 112x112 3x3 one, -6 % on 128x96 5x5.
-    constexpr int kBudget = S == 2 ? 20 * 1024 : dwconv::kLdsBudget;
+    // (16-bit elements land in an fp32 image, so the same bytes in flight need twice the LDS: 28 KiB measured best
+    // on the 112x112 3x3 layer, -12 %.)
+    constexpr int kBudget = S == 2 ? (sizeof(IO) == 2 ? 28 : 20) * 1024 : dwconv::kLdsBudget;
     if (!plan_tiles(p, ceil_div(p.out_h, BH), BH, used_cols, K * K, rows_for, kBudget)) return -1;
     if (p.st.vec_in) p.st.vec_in = stage_vector_mode(p.st, p.planes_per_tile, sizeof(IO));
     if (p.vec_out) p.vec_out = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
