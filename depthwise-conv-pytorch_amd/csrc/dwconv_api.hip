@@ -186,6 +186,10 @@ size_t wgrad_workspace(const WgradGeometry &g)
         if (sm > need) need = sm;
         const size_t s2 = bwd_s2_workspace(g);
         if (s2 > need) need = s2;
+        if constexpr (sizeof(T) == 2) {
+            const size_t t16 = bwd_tiled16_workspace(g);
+            if (t16 > need) need = t16;
+        }
     }
     return need;
 }
@@ -246,6 +250,10 @@ int backward_any(const T *in, const T *gy, const T *taps, T *gx, T *gw, void *ws
         if (taps == nullptr || gx == nullptr) return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");
         rc = try_launch_bwd_small<T>(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
         if (rc >= 0) return rc;
+        if constexpr (sizeof(T) == 2) {
+            rc = try_launch_bwd_tiled16<T>(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+            if (rc >= 0) return rc;
+        }
         rc = try_launch_bwd_tiled<T>(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
         if (rc >= 0) return rc;
         rc = try_launch_bwd_s2<T>(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);

@@ -44,24 +44,6 @@ struct BwdS2Plan {
     int vec_gx;
 };
 
-template <int CTRL, int ROW_MASK, int BANK_MASK>
-__device__ __forceinline__ float dpp_add(float v)
-{
-    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, BANK_MASK, true);
-    return v + __int_as_float(moved);
-}
-
-// Sum of the 64 lanes, delivered in lane 63; fixed association order.
-__device__ __forceinline__ float wave_sum_to_last_lane(float v)
-{
-    v = dpp_add<0x111, 0xf, 0xf>(v);  // row_shr:1
-    v = dpp_add<0x112, 0xf, 0xf>(v);  // row_shr:2
-    v = dpp_add<0x114, 0xf, 0xf>(v);  // row_shr:4
-    v = dpp_add<0x118, 0xf, 0xf>(v);  // row_shr:8
-    v = dpp_add<0x142, 0xa, 0xf>(v);  // row_bcast:15 into rows 1 and 3
-    v = dpp_add<0x143, 0xc, 0xf>(v);  // row_bcast:31 into rows 2 and 3
-    return v;
-}
 
 // E = parity of the transposed problem's leading pad K - 1 - pad (the same on both axes).
 // BQ: half-resolution rows per lane (4; 2 for planes too low to give every lane a block of 4).

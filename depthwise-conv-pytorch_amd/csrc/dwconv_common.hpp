@@ -246,6 +246,12 @@ int try_launch_wgrad_tiled(const IO *in, const IO *gy, IO *gw, void *ws, size_t 
 template <typename IO>
 int try_launch_bwd_tiled(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
                          const WgradGeometry &g, hipStream_t stream);
+// The same for 16-bit tensors whose rows are whole groups of eight elements: raw 16-bit LDS images and two-element
+// dot products (dwconv_bwd16.hip).  bwd_tiled16_workspace is 0 where the kernel does not cover g.
+size_t bwd_tiled16_workspace(const WgradGeometry &g);
+template <typename IO>
+int try_launch_bwd_tiled16(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
+                           const WgradGeometry &g, hipStream_t stream);
 
 // The same for stride-2 layers: dwconv_bwd_s2.hip.
 size_t bwd_s2_workspace(const WgradGeometry &g);  // 0 when that kernel does not cover g

@@ -14,13 +14,11 @@
 //           with a mask (a garbage partner times a zero tap would turn an Inf next to the window into a NaN).
 // Same results as the fp32-image kernel up to the order of the fp32 additions.
 // Replaces, for these tensors, what torch_dwconv/dwconv_kernel.cu:69-181 computes with `scalar_t` = half.
-#include "dwconv_tile_common.hpp"
+#include "dwconv_tile16_common.hpp"
 
 namespace dwconv {
 
 namespace {
-
-constexpr int kPadL = 8;  // element j of an image row holds input column j - kPadL
 
 struct Tile16Plan {
     const void *in;
@@ -28,40 +26,22 @@ struct Tile16Plan {
     void *out;
     long planes;
     int channel;
-    int in_h, in_w, in_plane;
+    Image16 im;
     int out_h, out_w, out_plane;
     int pad_h, pad_w;
     int rows_per_tile;     // output rows per tile, a multiple of BH
     int row_tiles;         // tiles per plane
     int planes_per_tile;
     int n_tiles;
-    int lds_rows;          // input rows per plane image
-    unsigned lds_rows_magic;
-    int spr;               // 8-element slots per image row
-    unsigned spr_magic;
-    int pitch;             // elements per image row (a multiple of 8)
-    int plane_pitch;       // elements per plane image
     int ncb;               // column blocks per row
     unsigned ncb_magic;
     int items_per_plane;
     unsigned ipp_magic;
     int tap_base;          // dword offset of the tap tables in LDS
-    int dump;              // element offset of eight spare elements
+    int dump;              // slot index of a spare slot
     int lout;              // results leave through LDS as one linear stream per plane (one item per lane)
     Epilogue epi;
 };
-
-template <typename IO>
-__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c)
-{
-    if constexpr (std::is_same<IO, bf16_t>::value) {
-        typedef __bf16 v2 __attribute__((ext_vector_type(2)));
-        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2, a), __builtin_bit_cast(v2, b), c, false);
-    } else {
-        typedef _Float16 v2 __attribute__((ext_vector_type(2)));
-        return __builtin_amdgcn_fdot2(__builtin_bit_cast(v2, a), __builtin_bit_cast(v2, b), c, false);
-    }
-}
 
 // PW1: parity of the left padding (the first element of a lane's window is the high half of a dword when odd).
 // EPI: the epilogue of the fused forward entry points is compiled in (its temporaries cost 12 registers, a wavefront
@@ -76,7 +56,6 @@ __global__ __launch_bounds__(kThreads) void fir_down16_kernel(const Tile16Plan p
     constexpr int TPP = K * (KP + 1);        // dwords of a plane's tap table: KP pairs and the last tap as (0, t)
     constexpr int WIN_ROWS = (BH - 1) * S + K;
     constexpr int NDW = (PW1 + (OWI - 1) * S + K - 1) / 2 + 1;  // dwords of a window row
-    constexpr int kBatch = 4;
 
     const int tile = xcd_contiguous_tile(blockIdx.x, p.n_tiles);
     const int pg = tile / p.row_tiles, rt = tile - pg * p.row_tiles;
@@ -98,81 +77,7 @@ __global__ __launch_bounds__(kThreads) void fir_down16_kernel(const Tile16Plan p
         lds32[p.tap_base + i] = j < KP ? (tap(2 * j) | (tap(2 * j + 1) << 16)) : (tap(K - 1) << 16);
     }
 
-    // image: every 8-element slot of every row, zeros (loads beyond the view) outside the plane
-    {
-        const __amdgpu_buffer_rsrc_t view =
-            buffer_view(static_cast<const IO *>(p.in) + plane0 * p.in_plane, static_cast<long>(nplanes) * p.in_plane * sizeof(IO));
-        u32x4 *image = reinterpret_cast<u32x4 *>(lds_raw);  // one slot per element
-        const int nthreads = blockDim.x;
-        const int rpp_raw = fast_div(nthreads, p.spr_magic);
-        const int rpp = max(rpp_raw, 1);                    // rows per pass of the workgroup
-        const int col_step = rpp_raw ? p.spr : nthreads;    // one trip unless a row has more slots than lanes
-        const int rl = fast_div(threadIdx.x, p.spr_magic);
-        const int spitch = p.pitch >> 3, dump = p.dump >> 3;  // in slots
-        if (rl < rpp) {
-            for (int sc = threadIdx.x - __mul24(rl, p.spr); sc < p.spr; sc += col_step) {
-                const int ix = 8 * sc - kPadL;
-                const bool col_ok = static_cast<unsigned>(ix) < static_cast<unsigned>(p.in_w);
-                if (nplanes == 1) {
-                    const int lo = max(iy0, 0);
-                    const unsigned span = static_cast<unsigned>(max(min(p.in_h, iy0 + p.lds_rows) - lo, 0));
-                    const unsigned off_step = __mul24(rpp, p.in_w) * 2u;
-                    const int dst_step = __mul24(rpp, spitch);
-                    int iy = iy0 + rl;
-                    unsigned off = (__mul24(iy, p.in_w) + ix) * 2u;
-                    int dst = __mul24(rl, spitch) + sc;
-                    int rb = 0;
-                    // whole batches (uniform bound, unconditional stores), then one batch whose rows past the image
-                    // go to the spare slot
-                    for (; rb + rpp * kBatch <= p.lds_rows; rb += rpp * kBatch) {
-                        u32x4 v[kBatch];
-#pragma unroll
-                        for (int u = 0; u < kBatch; ++u) {
-                            const bool ok = col_ok && static_cast<unsigned>(iy + u * rpp - lo) < span;
-                            v[u] = __builtin_amdgcn_raw_buffer_load_b128(view, ok ? off + u * off_step : kOob, 0, 0);
-                        }
-#pragma unroll
-                        for (int u = 0; u < kBatch; ++u) image[dst + u * dst_step] = v[u];
-                        iy += rpp * kBatch;
-                        off += off_step * kBatch;
-                        dst += dst_step * kBatch;
-                    }
-                    if (rb < p.lds_rows) {
-                        u32x4 v[kBatch];
-#pragma unroll
-                        for (int u = 0; u < kBatch; ++u) {
-                            const bool ok = col_ok && static_cast<unsigned>(iy + u * rpp - lo) < span;
-                            v[u] = __builtin_amdgcn_raw_buffer_load_b128(view, ok ? off + u * off_step : kOob, 0, 0);
-                        }
-#pragma unroll
-                        for (int u = 0; u < kBatch; ++u)
-                            image[rb + rl + u * rpp < p.lds_rows ? dst + u * dst_step : dump] = v[u];
-                    }
-                } else {
-                    const int total_rows = nplanes * p.lds_rows;
-                    const int pslots = p.plane_pitch >> 3;
-                    for (int ra = rl; ra < total_rows; ra += rpp * kBatch) {
-                        u32x4 v[kBatch];
-                        int dst[kBatch];
-#pragma unroll
-                        for (int u = 0; u < kBatch; ++u) {
-                            const bool live = ra + u * rpp < total_rows;
-                            const int rc = min(ra + u * rpp, total_rows - 1);
-                            const int pl = fast_div(rc, p.lds_rows_magic);
-                            const int r = rc - __mul24(pl, p.lds_rows);
-                            const int iy = iy0 + r;
-                            const bool ok = live && col_ok && static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
-                            const unsigned off = (__mul24(pl, p.in_plane) + __mul24(iy, p.in_w) + ix) * 2u;
-                            v[u] = __builtin_amdgcn_raw_buffer_load_b128(view, ok ? off : kOob, 0, 0);
-                            dst[u] = live ? __mul24(pl, pslots) + __mul24(r, spitch) + sc : dump;
-                        }
-#pragma unroll
-                        for (int u = 0; u < kBatch; ++u) image[dst[u]] = v[u];
-                    }
-                }
-            }
-        }
-    }
+    stage_image16(p.im, static_cast<const IO *>(p.in) + plane0 * p.im.in_plane, lds32, p.dump, nplanes, iy0);
     __syncthreads();
 
     const int n_items = nplanes * p.items_per_plane;
@@ -189,22 +94,24 @@ __global__ __launch_bounds__(kThreads) void fir_down16_kernel(const Tile16Plan p
         // the first filter row's last tap as fp32: its product starts every sum (a plain multiply needs no zeroed
         // accumulator, which the accumulating dot product would)
         const float t0_last = Io<IO>::in(__builtin_bit_cast(IO, static_cast<uint16_t>(tp[0][KP] >> 16)));
-        // first dword of the lane's window in image row rb * BH * S
-        const uint32_t *base = lds32 + ((__mul24(pl, p.plane_pitch) + __mul24(rb * BH * S, p.pitch) + kPadL + cb * (OWI * S) - p.pad_w - PW1) >> 1);
-        const int rpitch = p.pitch >> 1;  // dwords per image row
-
+        // The lane's window starts at logical dword 4 * cb + PH of image row rb * BH * S (pad_w = K / 2 puts its first
+        // element (K/2 + PW1) / 2 dwords left of the lane's block, which starts at dword 4 + 4 * cb); window dword i is
+        // LDS dword base[swz(PH + i)].
+        constexpr int PH = 4 - (K / 2 + PW1) / 2;
+        const uint32_t *base = lds32 + __mul24(pl, p.im.pp) + __mul24(rb * BH * S, p.im.rp) + 5 * cb;
+        const int rpitch = p.im.rp;  // dwords per image row
         // (no zero fill: the first product of every sum starts from the constant, see below)
         // window rows are read one ahead of their use, into alternating registers, and the sums pinned after every
         // row (see pin_registers)
         uint32_t win[2][NDW];
 #pragma unroll
-        for (int i = 0; i < NDW; ++i) win[0][i] = base[i];
+        for (int i = 0; i < NDW; ++i) win[0][i] = base[swz(PH + i)];
 #pragma unroll
         for (int wr = 0; wr < WIN_ROWS; ++wr) {
             const uint32_t(&d)[NDW] = win[wr & 1];
             if (wr + 1 < WIN_ROWS) {
 #pragma unroll
-                for (int i = 0; i < NDW; ++i) win[(wr + 1) & 1][i] = base[(wr + 1) * rpitch + i];
+                for (int i = 0; i < NDW; ++i) win[(wr + 1) & 1][i] = base[(wr + 1) * rpitch + swz(PH + i)];
             }
             // pairs that start at an odd element
             uint32_t q[NDW];
@@ -279,9 +186,17 @@ __global__ __launch_bounds__(kThreads) void fir_down16_kernel(const Tile16Plan p
                     if (rb * BH + b < rows_here) {
                         uint32_t t[OWI / 2];
                         pack_row(acc[b], t);
+                        // (one 128- or 64-bit write per lane at a multiple of its size: conflict-free)
                         uint32_t *d = lds32 + ((__mul24(pl, run) + __mul24(rb * BH + b, p.out_w) + cb * OWI) >> 1);
-#pragma unroll
-                        for (int i = 0; i < OWI / 2; ++i) d[i] = t[i];
+                        if constexpr (OWI == 8) {
+                            u32x4 v;
+                            v.x = t[0]; v.y = t[1]; v.z = t[2]; v.w = t[3];
+                            *reinterpret_cast<u32x4 *>(d) = v;
+                        } else {
+                            u32x2 v;
+                            v.x = t[0]; v.y = t[1];
+                            *reinterpret_cast<u32x2 *>(d) = v;
+                        }
                     }
                 }
             }
@@ -340,12 +255,10 @@ int launch_down16(Tile16Plan &p, hipStream_t stream)
     p.ncb = p.out_w / OWI;
     // elements of a row the windows touch: up to input column (out_w - 1) * S - pad_w + K - 1, and its pair partner
     const int last_col = (p.out_w - 1) * S - p.pad_w + K;
-    p.spr = ceil_div(kPadL + max(last_col + 1, p.in_w), 8);
-    // eight spare elements per row keep the rows of consecutive row blocks off the same banks
-    p.pitch = 8 * p.spr + 8;
+    layout_image16(p.im, last_col);
     auto rows_for = [](int units) { return (units * BH - 1) * S + K; };
     auto bytes = [&](int units, int planes) {
-        return static_cast<long>(planes) * (static_cast<long>(rows_for(units)) * p.pitch * 2 + TPP * 4) + 16;
+        return static_cast<long>(planes) * (static_cast<long>(rows_for(units)) * p.im.rp * 4 + TPP * 4) + 20;
     };
 
     const int row_units = ceil_div(p.out_h, BH);
@@ -368,22 +281,14 @@ int launch_down16(Tile16Plan &p, hipStream_t stream)
     p.planes_per_tile = planes_per_tile;
     p.rows_per_tile = units_per_tile * BH;
     p.row_tiles = ceil_div(row_units, units_per_tile);
-    p.lds_rows = rows_for(units_per_tile);
-    p.plane_pitch = p.lds_rows * p.pitch;
+    if (!finish_image16(p.im, rows_for(units_per_tile), planes_per_tile)) return -1;
     p.items_per_plane = units_per_tile * p.ncb;
-    const long slots = static_cast<long>(planes_per_tile) * p.lds_rows * p.spr;
-    if (slots >= 65536 || planes_per_tile * p.items_per_plane >= 65536) return -1;  // 16-bit reciprocals
-    // 24-bit multiplies of the staging loop
-    if (p.in_h >= (1 << 23) || p.in_w >= (1 << 23) || (planes_per_tile > 1 && p.in_plane >= (1 << 23))) return -1;
-    if (static_cast<long>(planes_per_tile) * p.in_plane * 2 >= static_cast<long>(kOob) ||
-        static_cast<long>(planes_per_tile) * p.out_plane * 2 >= static_cast<long>(kOob))
-        return -1;
-    p.spr_magic = magic_u16(p.spr);
-    p.lds_rows_magic = magic_u16(p.lds_rows);
+    if (planes_per_tile * p.items_per_plane >= 65536) return -1;  // 16-bit reciprocals
+    if (static_cast<long>(planes_per_tile) * p.out_plane * 2 >= static_cast<long>(kOob)) return -1;
     p.ncb_magic = magic_u16(p.ncb);
     p.ipp_magic = magic_u16(p.items_per_plane);
-    p.dump = planes_per_tile * p.plane_pitch;
-    p.tap_base = (p.dump + 8) / 2;
+    p.dump = planes_per_tile * p.im.lds_rows * (p.im.pitch / 8);
+    p.tap_base = 5 * (p.dump + 1);
     const long tiles = ceil_div(p.planes, static_cast<long>(planes_per_tile)) * p.row_tiles;
     if (tiles > 0x7fffffffL) return -1;
     p.n_tiles = static_cast<int>(tiles);
@@ -403,10 +308,10 @@ int launch_down16(Tile16Plan &p, hipStream_t stream)
 template <typename IO, int K, int S, bool FLIP>
 int launch_down16_parity(Tile16Plan &p, hipStream_t stream)
 {
-    const bool seven = (p.out_h % 7 == 0 || p.out_h > 64) && p.out_h % 4 != 0;
-    if (p.pad_w & 1)
-        return seven ? launch_down16<IO, K, S, 1, FLIP, 7>(p, stream) : launch_down16<IO, K, S, 1, FLIP, 4>(p, stream);
-    return seven ? launch_down16<IO, K, S, 0, FLIP, 7>(p, stream) : launch_down16<IO, K, S, 0, FLIP, 4>(p, stream);
+    const int forced = env_int("DWCONV_TILE_BH", 0);
+    const bool seven = forced ? forced == 7 : (p.out_h % 7 == 0 || p.out_h > 64) && p.out_h % 4 != 0;
+    constexpr int PW1 = (K / 2) & 1;  // the left padding is K / 2
+    return seven ? launch_down16<IO, K, S, PW1, FLIP, 7>(p, stream) : launch_down16<IO, K, S, PW1, FLIP, 4>(p, stream);
 }
 
 }  // namespace
@@ -421,8 +326,12 @@ int try_launch_fir_tiled16(const IO *in, const IO *taps, IO *out, const Geometry
     if (g.kernel_w != K || (K != 3 && K != 5 && K != 7)) return -1;
     if (g.up_h != 1 || g.up_w != 1 || g.down_w != S || (S != 1 && S != 2)) return -1;
     if (S == 2 && !g.forward) return -1;
-    if (g.pad_h0 < 0 || g.pad_w0 < 0 || g.pad_h0 > 7 || g.pad_w0 > 7) return -1;
+    // (the window's place within its LDS slots is a compile-time constant: left padding K/2 only)
+    if (g.pad_h0 < 0 || g.pad_h0 > 7 || g.pad_w0 != K / 2) return -1;
     if (g.in_w % 8 != 0 || g.out_w % (S == 1 ? 8 : 4) != 0 || g.in_h < 1) return -1;
+    // Input rows of at least 96 elements: narrower planes have too few 8-wide blocks to occupy the lanes, and the
+    // fp32-image kernel with its 4-wide blocks is as fast there (56 x 56: 57-58 us either way).
+    if (g.in_w < env_int("DWCONV_T16_MIN_W", 96)) return -1;
     if (reinterpret_cast<uintptr_t>(in) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 16 != 0) return -1;
     if (static_cast<long>(g.in_h) * g.in_w >= (1l << 30) || static_cast<long>(g.out_h) * g.out_w >= (1l << 30)) return -1;
 
@@ -433,9 +342,9 @@ int try_launch_fir_tiled16(const IO *in, const IO *taps, IO *out, const Geometry
     p.planes = g.planes();
     p.channel = g.channel;
     p.epi = g.epi;
-    p.in_h = g.in_h;
-    p.in_w = g.in_w;
-    p.in_plane = g.in_h * g.in_w;
+    p.im.in_h = g.in_h;
+    p.im.in_w = g.in_w;
+    p.im.in_plane = g.in_h * g.in_w;
     p.out_h = g.out_h;
     p.out_w = g.out_w;
     p.out_plane = g.out_h * g.out_w;

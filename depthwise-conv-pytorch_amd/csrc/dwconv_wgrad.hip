@@ -49,27 +49,6 @@ struct WgradPlan {
     int strided;           // chunk k takes tiles k, k+chunks, ... instead of a contiguous range
 };
 
-template <int CTRL, int ROW_MASK, int BANK_MASK>
-__device__ __forceinline__ float dpp_add(float v)
-{
-    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, BANK_MASK, true);
-    return v + __int_as_float(moved);
-}
-
-// Sum of the 64 lanes, delivered in lane 63; fixed association order.
-__device__ __forceinline__ float wave_sum_to_last_lane(float v)
-{
-    v = dpp_add<0x111, 0xf, 0xf>(v);  // row_shr:1
-    v = dpp_add<0x112, 0xf, 0xf>(v);  // row_shr:2
-    v = dpp_add<0x114, 0xf, 0xf>(v);  // row_shr:4
-    v = dpp_add<0x118, 0xf, 0xf>(v);  // row_shr:8  -> lane 15 of each row of 16 holds the row sum
-    v = dpp_add<0x142, 0xa, 0xf>(v);  // row_bcast:15 into rows 1 and 3
-    v = dpp_add<0x143, 0xc, 0xf>(v);  // row_bcast:31 into rows 2 and 3
-    return v;
-}
-
-constexpr int kRedPitch = kThreads + 1;  // odd pitch: lanes of one wave reading one column spread over the banks
-
 // GX (stride 1, pad = K/2 only): the band of gy is staged in LDS next to the band of x, with the same
 // layout.  The lane first walks its gy window: that gives its block of grad-input (gy against the
 // rotated taps, stored straight to memory) and, from the window's centre, its block of gy for the
