@@ -534,6 +534,173 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_bwd_fused_kernel(const Nhwc
     }
 }
 
+// Grad-input and grad-weight of a stride-2 layer with pad K / 2 and even input extents (out = in / 2) in one sweep:
+// in = x (in_h x in_w), in2 = out_grad (out_h x out_w), out = in_grad.  The lane owns a BQH x BQW block of out_grad
+// pixels and CV channels, i.e. a 2 BQH x 2 BQW block of in_grad and the (2 BQH + K - 2) x (2 BQW + K - 2) window of
+// x its sums need.  With q0 the block's first out_grad row and d = q - q0:
+//   in_grad row 2 q0 + b   += out_grad row q0 + d  *  tap row ty = b + P - 2 d        (P = K / 2; 0 <= ty < K)
+//   sum[ty][tx]            += out_grad row q0 + j  *  x window row r = 2 j + ty        (x row 2 q0 - P + r)
+// and the same along columns.  The lane walks the P/2 + BQH + (P + 1)/2 window rows of out_grad once: each feeds the
+// rows of in_grad it touches (a row is stored as soon as no later out_grad row reaches it) and, where it belongs to
+// the lane's own block, is kept for the x rows it meets; two x rows are consumed per out_grad row, right behind it.
+// The loop is unrolled, so only the rows in use are live.  out_grad is read once instead of twice and the separate
+// grad-input kernel (nhwc_up2_kernel) goes away.  The end of the kernel is that of nhwc_wgrad_kernel.
+template <typename IO, int K, int CV, int BQH, int BQW>
+__global__ __launch_bounds__(kNhwcThreads) void nhwc_bwd_s2_fused_kernel(const NhwcPlan p)
+{
+    extern __shared__ float4 lds_raw[];
+    float *lds = reinterpret_cast<float *>(lds_raw);
+    constexpr int KK = K * K, P = K / 2;
+    constexpr int DMIN = -(P / 2);                        // first out_grad row / column of the window, relative to the block
+    constexpr int GROWS = BQH + P, GCOLS = BQW + P;       // out_grad window
+    constexpr int XROWS = 2 * (BQH - 1) + K, XCOLS = 2 * (BQW - 1) + K;  // x window
+    constexpr int GXH = 2 * BQH, GXW = 2 * BQW;           // in_grad block
+    constexpr int STEPS = GROWS + P / 2;                  // x rows 2 (t - P/2), 2 (t - P/2) + 1 are consumed in step t
+    static_assert(2 * (STEPS - 1 - P / 2) + 1 >= XROWS - 1, "every x row has its step");
+    const int C = p.channel;
+    const int chunk = blockIdx.x;
+    const int c0 = blockIdx.y * p.lanes_c * CV;
+    const int nch = min(p.lanes_c * CV, C - c0);
+    const int pb_local = fast_div(threadIdx.x, p.lanes_c_magic);
+    const int lane_c = threadIdx.x - pb_local * p.lanes_c;
+    const bool lane_ok = pb_local < p.blocks_per_wg && CV * lane_c < nch;
+    const int c = c0 + (lane_ok ? CV * lane_c : 0);
+    const int per_image = p.blocks_x * p.blocks_y;
+    nhwc_stage_taps<IO, KK, false>(static_cast<const IO *>(p.taps), lds, c0, nch);
+    __syncthreads();
+    const float *wl = lds + (lane_ok ? CV * lane_c : 0);
+
+    float acc[KK][CV];
+#pragma unroll
+    for (int t = 0; t < KK; ++t)
+#pragma unroll
+        for (int v = 0; v < CV; ++v) acc[t][v] = 0.f;
+
+    for (long grp = chunk; grp * p.blocks_per_wg < p.blocks_total; grp += p.groups) {
+        const long pb = grp * p.blocks_per_wg + pb_local;
+        if (!lane_ok || pb >= p.blocks_total) continue;
+        const int n = static_cast<int>(pb / per_image);
+        const int rem = static_cast<int>(pb - static_cast<long>(n) * per_image);
+        const int by = rem / p.blocks_x, bx = rem - by * p.blocks_x;
+        const int q0 = by * BQH, qx0 = bx * BQW;          // the block in out_grad
+        const int xr0 = 2 * q0 - P, xc0 = 2 * qx0 - P;    // first row / column of the x window
+        // views from the first image of this group of pixel blocks (uniform): x and in_grad share an extent
+        const int n0 = static_cast<int>(grp * p.blocks_per_wg / per_image);
+        const unsigned pixel_bytes = C * sizeof(IO);
+        const unsigned xrow_bytes = p.in_w * pixel_bytes, grow_bytes = p.out_w * pixel_bytes;
+        const long ximage0 = static_cast<long>(n0) * p.in_h * p.in_w * C, gimage0 = static_cast<long>(n0) * p.out_h * p.out_w * C;
+        const long xspan = static_cast<long>(p.batch - n0) * p.in_h * xrow_bytes;
+        const long gspan = static_cast<long>(p.batch - n0) * p.out_h * grow_bytes;
+        const __amdgpu_buffer_rsrc_t xview = buffer_view(static_cast<const IO *>(p.in) + ximage0, xspan);
+        const __amdgpu_buffer_rsrc_t gview = buffer_view(static_cast<const IO *>(p.in2) + gimage0, gspan);
+        const __amdgpu_buffer_rsrc_t oview = buffer_view(static_cast<IO *>(p.out) + ximage0, xspan);
+        NhwcCols<XCOLS> xcols;
+        nhwc_cols<XCOLS>(xc0, p.in_w, pixel_bytes, (n - n0) * (p.in_h * xrow_bytes) + c * static_cast<unsigned>(sizeof(IO)), xcols);
+        NhwcCols<GCOLS> gcols;
+        nhwc_cols<GCOLS>(qx0 + DMIN, p.out_w, pixel_bytes, (n - n0) * (p.out_h * grow_bytes) + c * static_cast<unsigned>(sizeof(IO)), gcols);
+
+        float gxs[GXH][GXW * CV];   // in_grad sums
+        float gb[BQH][BQW * CV];    // the lane's own rows of out_grad
+#pragma unroll
+        for (int b = 0; b < GXH; ++b)
+#pragma unroll
+            for (int o = 0; o < GXW * CV; ++o) gxs[b][o] = 0.f;
+        float gr[2][GCOLS * CV], xr[2][XCOLS * CV];
+        nhwc_load_row<IO, GCOLS, CV>(gview, q0 + DMIN, p.out_h, grow_bytes, gcols, gr[0]);
+        nhwc_load_row<IO, XCOLS, CV>(xview, xr0, p.in_h, xrow_bytes, xcols, xr[0]);
+#pragma unroll
+        for (int t = 0; t < STEPS; ++t) {
+            if (t + 1 < GROWS) nhwc_load_row<IO, GCOLS, CV>(gview, q0 + DMIN + t + 1, p.out_h, grow_bytes, gcols, gr[(t + 1) & 1]);
+            if (t < GROWS) {
+                float(&gcur)[GCOLS * CV] = gr[t & 1];
+                const int d = DMIN + t;
+                // in_grad row b meets this row in tap row ty = b + P - 2 d, in_grad column o meets window column j
+                // in tap column tx = o + P - 2 (DMIN + j)
+#pragma unroll
+                for (int b = 0; b < GXH; ++b) {
+                    const int ty = b + P - 2 * d;
+                    if (ty < 0 || ty >= K) continue;
+#pragma unroll
+                    for (int o = 0; o < GXW; ++o)
+#pragma unroll
+                        for (int j = 0; j < GCOLS; ++j) {
+                            const int tx = o + P - 2 * (DMIN + j);
+                            if (tx < 0 || tx >= K) continue;
+#pragma unroll
+                            for (int q = 0; q < CV; ++q)
+                                gxs[b][CV * o + q] = fmaf(gcur[CV * j + q], wl[(ty * K + tx) * nch + q], gxs[b][CV * o + q]);
+                        }
+                }
+                if (d >= 0 && d < BQH) {
+#pragma unroll
+                    for (int o = 0; o < BQW * CV; ++o) gb[d >= 0 && d < BQH ? d : 0][o] = gcur[CV * (-DMIN) + o];
+                }
+                // rows no later out_grad row reaches: b < 2 (d + 1) - P; those finished before this step were stored then
+#pragma unroll
+                for (int b = 0; b < GXH; ++b) {
+                    const bool done_now = b < 2 * (d + 1) - P || t == GROWS - 1;
+                    const bool done_before = t > 0 && b < 2 * d - P;
+                    if (!done_now || done_before) continue;
+                    const unsigned roff = 2 * q0 + b < p.in_h ? (2 * q0 + b) * xrow_bytes : kOob;
+#pragma unroll
+                    for (int o = 0; o < GXW; ++o) {
+                        const unsigned off = __builtin_elementwise_add_sat(roff, xcols.off[o + P]);
+                        if constexpr (CV == 4)
+                            view_store4<IO>(oview, off, gxs[b][4 * o], gxs[b][4 * o + 1], gxs[b][4 * o + 2], gxs[b][4 * o + 3]);
+                        else if constexpr (CV == 2)
+                            view_store2<IO>(oview, off, gxs[b][2 * o], gxs[b][2 * o + 1]);
+                        else
+                            view_store1<IO>(oview, off, gxs[b][o]);
+                    }
+                }
+            }
+            // the x rows whose out_grad rows (own rows up to t - P/2) have all passed
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int r = 2 * (t - P / 2) + h;
+                if (r < 0 || r >= XROWS) continue;
+                if (r + 1 < XROWS) nhwc_load_row<IO, XCOLS, CV>(xview, xr0 + r + 1, p.in_h, xrow_bytes, xcols, xr[(r + 1) & 1]);
+                float(&xcur)[XCOLS * CV] = xr[r & 1];
+#pragma unroll
+                for (int ty = 0; ty < K; ++ty) {
+                    if ((r - ty) % 2 != 0) continue;
+                    const int j = (r - ty) / 2;
+                    if (r - ty < 0 || j >= BQH) continue;
+#pragma unroll
+                    for (int tx = 0; tx < K; ++tx)
+#pragma unroll
+                        for (int i = 0; i < BQW; ++i)
+#pragma unroll
+                            for (int q = 0; q < CV; ++q)
+                                acc[ty * K + tx][q] = fmaf(gb[j][CV * i + q], xcur[CV * (2 * i + tx) + q], acc[ty * K + tx][q]);
+                }
+            }
+            pin_registers(acc);
+        }
+    }
+    __syncthreads();  // the taps in LDS are done with: the sums of the lanes go through the same memory
+
+    const int width = p.lanes_c * CV;
+    float *out = p.partial + static_cast<long>(chunk) * KK * C;
+#pragma unroll
+    for (int ty = 0; ty < K; ++ty) {
+        if (ty) __syncthreads();
+        if (pb_local < p.blocks_per_wg) {
+#pragma unroll
+            for (int tx = 0; tx < K; ++tx)
+#pragma unroll
+                for (int v = 0; v < CV; ++v) lds[(pb_local * K + tx) * width + CV * lane_c + v] = lane_ok ? acc[ty * K + tx][v] : 0.f;
+        }
+        __syncthreads();
+        for (int e = threadIdx.x; e < K * nch; e += blockDim.x) {
+            const int tx = e / nch, cl = e - tx * nch;
+            float sum = 0.f;
+            for (int q = 0; q < p.blocks_per_wg; ++q) sum += lds[(q * K + tx) * width + cl];
+            out[static_cast<long>(ty * K + tx) * C + c0 + cl] = sum;
+        }
+    }
+}
+
 // Grad-weight, pass 2: gw[c][t] = sum over chunks of partial[chunk][t][c].  16 lanes per output add contiguous
 // sixteenths of the chunks in fp64; the sixteen sums are then added in order: bit-identical from run to run.
 constexpr int kNhwcFinalParts = 16;
@@ -916,6 +1083,53 @@ long nhwc_bwd_fused_case(int mode, const IO *x, const IO *gy, const IO *taps, IO
     return check_launch("nhwc_wgrad_final_kernel");
 }
 
+// Fused backward of K x K stride-2 layers with pad K/2 and even input extents.  mode 0: workspace bytes; mode 1:
+// launch.  -1 when the kernel does not cover g.
+template <typename IO, int K, int CV, int BQH, int BQW>
+long nhwc_bwd_s2_fused_case(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
+                            const NhwcGeometry &g, hipStream_t stream)
+{
+    NhwcPlan p{};
+    const int line_lanes = static_cast<int>(128 / (CV * sizeof(IO)));
+    if (!plan_nhwc<K, CV>(p, g, BQH, BQW, g.out_h, g.out_w, line_lanes, "DWCONV_NHWC_WGRAD_LANES")) return -1;
+    const int cgroups = p.cgroups;
+    const long wg_iters = (p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg;
+    long groups = env_int("DWCONV_NHWC_WGRAD_WGS", 512) / cgroups;
+    groups = std::max(1l, std::min(groups, wg_iters));
+    p.groups = static_cast<int>(groups);
+    const size_t need = static_cast<size_t>(groups) * K * K * g.channel * sizeof(float);
+    if (mode == 0) return static_cast<long>(need);
+    if (ws == nullptr || ws_bytes < need)
+        return fail(DWCONV_ERR_WORKSPACE, "backward needs a workspace of %zu bytes, got %zu", need, ws_bytes);
+    p.in = x;
+    p.in2 = gy;
+    p.taps = taps;
+    p.out = gx;
+    p.partial = static_cast<float *>(ws);
+    p.in_h = g.in_h;
+    p.in_w = g.in_w;
+    p.out_h = g.out_h;
+    p.out_w = g.out_w;
+    p.pad_h = g.pad_h;
+    p.pad_w = g.pad_w;
+    const size_t shmem = static_cast<size_t>(p.lanes_c) * CV * 4 * std::max(K * K, p.blocks_per_wg * K);
+    hipLaunchKernelGGL((nhwc_bwd_s2_fused_kernel<IO, K, CV, BQH, BQW>), dim3(p.groups, cgroups), dim3(kNhwcThreads), shmem, stream, p);
+    int rc = check_launch("nhwc_bwd_s2_fused_kernel");
+    if (rc != DWCONV_OK) return rc;
+    note_variant("nhwc_bwd%s<k%d,s2,cv%d,%dx%d> lanes_c%d chunks%d", sizeof(IO) == 2 ? "16" : "", K, CV, BQH, BQW, p.lanes_c, p.groups);
+    hipLaunchKernelGGL(nhwc_wgrad_final_kernel<IO>, dim3(ceil_div(g.channel * K * K, 16)), dim3(256), 0, stream,
+                       p.partial, gw, g.channel, K * K, p.groups);
+    return check_launch("nhwc_wgrad_final_kernel");
+}
+
+bool nhwc_fused_s2_ok(const NhwcGeometry &g)
+{
+    if (!env_int("DWCONV_NHWC_FUSED_S2", 1) || !env_int("DWCONV_NHWC_FUSED_BWD", 1) || !nhwc_fast_ok(g)) return false;
+    const int K = g.kernel_h;
+    return (K == 3 || K == 5) && g.stride_h == 2 && g.pad_h == K / 2 && g.pad_w == K / 2 && g.in_h % 2 == 0 &&
+           g.in_w % 2 == 0 && g.out_h == g.in_h / 2 && g.out_w == g.in_w / 2;
+}
+
 bool nhwc_fused_ok(const NhwcGeometry &g)
 {
     if (!env_int("DWCONV_NHWC_FUSED_BWD", 1) || !nhwc_fast_ok(g)) return false;
@@ -928,6 +1142,19 @@ template <typename IO>
 long nhwc_bwd_fused(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
                     const NhwcGeometry &g, hipStream_t stream)
 {
+    if (nhwc_fused_s2_ok(g)) {
+        // One fp32 channel per lane, as for the 5x5 stride-1 kernel: blocks of 7 x 4 out_grad pixels for 3x3 filters
+        // (95 registers; 112x112 C=96: 274 -> 257 us against the two separate kernels, 28x28 C=240: 56 -> 56), 4 x 2 for
+        // 5x5 (157 registers; 56x56 C=144: 147 -> 137 us, 14x14 C=672: 49 -> 48).  Measured and left out: two channels
+        // per lane with 4 x 2 or 7 x 2 blocks (3x3: 260-268 and 63 us; 5x5: 251 registers, 141 and 53 us), four channels
+        // with 2 x 2 blocks (186 registers, 260 and 64 us), 7 x 4 blocks for 5x5 (256 registers: twice the time).
+        // 16-bit elements (two channels per 4-byte access) stay on the separate kernels.
+        if constexpr (sizeof(IO) == 4) {
+            if (g.kernel_h == 3) return nhwc_bwd_s2_fused_case<IO, 3, 1, 7, 4>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+            return nhwc_bwd_s2_fused_case<IO, 5, 1, 4, 2>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+        }
+        return -1;
+    }
     if (!nhwc_fused_ok(g)) return -1;
     if (g.kernel_h == 5) {
         // 25 sums per channel: with two channels per lane the kernel needs 228 registers (7 x 2 blocks) to 262 (4 x 4)

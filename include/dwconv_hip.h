@@ -242,9 +242,9 @@ size_t dwconv2d_backward_nhwc_workspace_bytes(int batch, int channel, int in_h, 
                                               int pad_h, int pad_w, int elem_size);
 
 /* Both gradients (either of in_grad, kernel_grad may be NULL to skip it).  kernel_grad is overwritten
- * and bit-identical from run to run.  With both asked for, stride-1 layers with a 3x3 filter and pad 1
- * (any element type) or a 5x5 filter and pad 2 (fp32) are served by one kernel that reads out_grad once;
- * the workspace is needed even then. */
+ * and bit-identical from run to run.  With both asked for, layers with a 3x3 filter and pad 1 or a 5x5
+ * filter and pad 2 are served by one kernel that reads out_grad once: stride 1 (3x3: any element type,
+ * 5x5: fp32) and stride 2 on even extents (fp32); the workspace is needed even then. */
 int dwconv2d_backward_nhwc_f32(const float *input, const float *out_grad, const float *kernel,
                                float *in_grad, float *kernel_grad, void *workspace,
                                size_t workspace_bytes, int batch, int channel, int in_h, int in_w,

@@ -711,6 +711,45 @@ def test_channels_last_fused_backward(dw, gpu, shape, monkeypatch):
                                    atol=tol * max(1.0, float(np.abs(_np(gw_r)).max())))
 
 
+FUSED_NHWC_OTHER = [
+    # (shape, variant prefix): 5x5 stride 1, and stride 2 on even extents (3x3 in 7 x 4 blocks, 5x5 in 4 x 2 blocks)
+    ((2, 8, 14, 14, 5, 1, 2), "nhwc_bwd<k5,s1"), ((1, 36, 9, 11, 5, 1, 2), "nhwc_bwd<k5,s1"),
+    ((2, 8, 14, 14, 3, 2, 1), "nhwc_bwd<k3,s2"), ((1, 24, 30, 18, 3, 2, 1), "nhwc_bwd<k3,s2"),
+    ((3, 4, 2, 2, 3, 2, 1), "nhwc_bwd<k3,s2"), ((1, 96, 112, 112, 3, 2, 1), "nhwc_bwd<k3,s2"),
+    ((2, 8, 14, 14, 5, 2, 2), "nhwc_bwd<k5,s2"), ((1, 40, 22, 10, 5, 2, 2), "nhwc_bwd<k5,s2"),
+    ((2, 144, 56, 56, 5, 2, 2), "nhwc_bwd<k5,s2"), ((5, 260, 2, 6, 5, 2, 2), "nhwc_bwd<k5,s2"),
+    # odd extents are not covered by the fused stride-2 kernel
+    ((2, 8, 15, 14, 3, 2, 1), "nhwc_up2"),
+]
+
+
+@pytest.mark.parametrize("case", FUSED_NHWC_OTHER, ids=lambda c: shape_id(c[0]))
+def test_channels_last_fused_backward_other_layers(dw, gpu, case, monkeypatch):
+    """The one-kernel backward for 5x5 stride-1 and for stride-2 layers, channels-last fp32: against the oracle,
+    against the two separate kernels, bit-identical from run to run (outputs start as NaN)."""
+    from torch_dwconv import _C
+
+    shape, prefix = case
+    n, c, h, w, k, s, p = shape
+    x, wt, gy = make_inputs(shape, seed=53)
+    xg, wg, gyg = _channels_last(x, gpu), wt.to(gpu), _channels_last(gy, gpu)
+    with poisoned_allocations():
+        gx, gw = _C.dwconv2d_backward_nhwc(xg, gyg, wg, s, s, p, p)
+    _announce(shape_id(shape), _C.last_variant())
+    assert _C.last_variant().startswith(prefix), _C.last_variant()
+    gx_ref = oracle.grad_input(_np(gy), _np(wt), (h, w), s, p)
+    gw_ref = oracle.grad_weight(_np(x), _np(gy), wt.shape, s, p)
+    np.testing.assert_allclose(_np(gx).astype(np.float64), gx_ref, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(_np(gw).astype(np.float64), gw_ref, rtol=1e-4, atol=1e-4 * np.abs(gw_ref).max())
+    gx2, gw2 = _C.dwconv2d_backward_nhwc(xg, gyg, wg, s, s, p, p)
+    assert torch.equal(gw, gw2) and torch.equal(gx, gx2)
+    monkeypatch.setenv("DWCONV_NHWC_FUSED_BWD", "0")
+    gx3, gw3 = _C.dwconv2d_backward_nhwc(xg, gyg, wg, s, s, p, p)
+    assert "nhwc_wgrad" in _C.last_variant() and not _C.last_variant().startswith("nhwc_bwd"), _C.last_variant()
+    np.testing.assert_allclose(_np(gx3), _np(gx), rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(_np(gw3), _np(gw), rtol=1e-5, atol=1e-5 * float(gw.abs().max()))
+
+
 def test_channels_last_channel_groups_are_whole_lines(dw, gpu):
     """C = 240 on a 28x28 map: the workgroups take 16 channel lanes (256 bytes per pixel), not the 15 that divide C / 4."""
     from torch_dwconv import _C

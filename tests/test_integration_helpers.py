@@ -131,12 +131,14 @@ def test_registered_op_backward_through_compile(gpu, layout):
         # a frozen filter: only grad-input is computed (one kernel, no grad-weight variant in the name)
         xf = x.detach().clone().requires_grad_(True)
         fn(xf, w.detach()).backward(gy)
-        assert torch.equal(xf.grad, gx_e)
+        # (a single gradient takes the separate kernels, which add in another order than the fused one: same bounds
+        # as against the oracle, not the same bits)
+        torch.testing.assert_close(xf.grad, gx_e, rtol=1e-5, atol=1e-5)
         assert "wgrad" not in _C.last_variant() and "bwd" not in _C.last_variant(), _C.last_variant()
         # a frozen input: only grad-weight
         wf = w.detach().clone().requires_grad_(True)
         fn(x.detach(), wf).backward(gy)
-        torch.testing.assert_close(wf.grad, gw_e, rtol=1e-5, atol=1e-5)
+        torch.testing.assert_close(wf.grad, gw_e, rtol=1e-4, atol=1e-4 * float(gw_e.abs().max()))
 
 
 @pytest.mark.gpu
