@@ -1168,6 +1168,17 @@ long nhwc_bwd_fused(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx,
         }
         return -1;
     }
+    if constexpr (sizeof(IO) == 4) {
+        // fp32, 3x3: one channel per lane and 7 x 8 pixel blocks where C is whole groups of 32 lanes (a 128-byte line
+        // of every pixel per group), four channels per lane and 7 x 2 blocks otherwise (C = 144: 36 lanes).  Against
+        // two channels per lane and 7 x 4 blocks: 112x112 C=32 125.5 -> 120.6 us, 14x14 C=480 40.0 -> 35.8, 7x7 C=1152
+        // 29.7 -> 27.1, 56x56 C=144 155.7 -> 149.8 (one channel per lane there: 171-173, its fifth group is half empty).
+        if (env_int("DWCONV_NHWC_F3_SHAPE", 1)) {
+            if (g.channel % 32 == 0)
+                return nhwc_bwd_fused_case<IO, 3, 1, 7, 8>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+            return nhwc_bwd_fused_case<IO, 3, 4, 7, 2>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+        }
+    }
     return nhwc_bwd_fused_case<IO, 3>(mode, x, gy, taps, gx, gw, ws, ws_bytes, g, stream);
 }
 
