@@ -92,7 +92,8 @@ __device__ __forceinline__ void nhwc_stage_taps(const IO *__restrict__ taps, flo
 }
 
 // out[n,oy,ox,c] = sum_{ty,tx} in[n, oy*S - pad_h + ty, ox*S - pad_w + tx, c] * f[c,ty,tx]
-template <typename IO, int K, int S, bool FLIP, int BH, int TW>
+// CV channels per lane (4: one 128-bit access per pixel for fp32; 1: 32 lanes per 128-byte line of a pixel).
+template <typename IO, int K, int S, bool FLIP, int BH, int TW, int CV = 4>
 __global__ __launch_bounds__(kNhwcThreads) void nhwc_down_kernel(const NhwcPlan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -104,23 +105,23 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_down_kernel(const NhwcPlan 
     // groups that share halo rows, and the channel groups of one pixel group (neighbouring addresses), meet there
     const int wg = xcd_contiguous_tile(blockIdx.x, p.wgs);
     const int pg = wg / p.cgroups;
-    const int c0 = (wg - pg * p.cgroups) * p.lanes_c * 4;
-    const int nch = min(p.lanes_c * 4, C - c0);
+    const int c0 = (wg - pg * p.cgroups) * p.lanes_c * CV;
+    const int nch = min(p.lanes_c * CV, C - c0);
     nhwc_stage_taps<IO, KK, FLIP>(static_cast<const IO *>(p.taps), lds, c0, nch);
     __syncthreads();
 
     const int pb_local = fast_div(threadIdx.x, p.lanes_c_magic);
     const int lane_c = threadIdx.x - pb_local * p.lanes_c;
     const long pb = static_cast<long>(pg) * p.blocks_per_wg + pb_local;
-    if (pb_local >= p.blocks_per_wg || pb >= p.blocks_total || 4 * lane_c >= nch) return;
+    if (pb_local >= p.blocks_per_wg || pb >= p.blocks_total || CV * lane_c >= nch) return;
     const int per_image = p.blocks_x * p.blocks_y;
     const int n = static_cast<int>(pb / per_image);
     const int rem = static_cast<int>(pb - static_cast<long>(n) * per_image);
     const int by = rem / p.blocks_x, bx = rem - by * p.blocks_x;
     const int oy0 = by * BH, ox0 = bx * TW;
     const int iy0 = oy0 * S - p.pad_h, ix0 = ox0 * S - p.pad_w;
-    const int c = c0 + 4 * lane_c;
-    const float *wl = lds + 4 * lane_c;
+    const int c = c0 + CV * lane_c;
+    const float *wl = lds + CV * lane_c;
     // view of the input from the first image this workgroup touches (uniform); this lane's image and channels
     // are part of its column offsets
     const int n0 = static_cast<int>(static_cast<long>(pg) * p.blocks_per_wg / per_image);
@@ -130,43 +131,43 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_down_kernel(const NhwcPlan 
                     static_cast<long>(p.batch - n0) * p.in_h * row_bytes);
     const unsigned lane_off = (n - n0) * (p.in_h * row_bytes) + c * static_cast<unsigned>(sizeof(IO));
 
-    float acc[BH][TW * 4];
+    float acc[BH][TW * CV];
 #pragma unroll
     for (int b = 0; b < BH; ++b)
 #pragma unroll
-        for (int o = 0; o < TW * 4; ++o) acc[b][o] = 0.f;
+        for (int o = 0; o < TW * CV; ++o) acc[b][o] = 0.f;
 
     // Rows are loaded one ahead of their use (two row buffers, alternating) and the sums pinned after every
     // row: otherwise the compiler hoists the loads of the whole window to the top and keeps all of it in registers.
-    float rows[2][COLS * 4];
+    float rows[2][COLS * CV];
     NhwcCols<COLS> cols;
     nhwc_cols<COLS>(ix0, p.in_w, pixel_bytes, lane_off, cols);
-    nhwc_load_row<IO, COLS>(view, iy0, p.in_h, row_bytes, cols, rows[0]);
+    nhwc_load_row<IO, COLS, CV>(view, iy0, p.in_h, row_bytes, cols, rows[0]);
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
-        float(&cur)[COLS * 4] = rows[r & 1];
-        if (r + 1 < ROWS) nhwc_load_row<IO, COLS>(view, iy0 + r + 1, p.in_h, row_bytes, cols, rows[(r + 1) & 1]);
+        float(&cur)[COLS * CV] = rows[r & 1];
+        if (r + 1 < ROWS) nhwc_load_row<IO, COLS, CV>(view, iy0 + r + 1, p.in_h, row_bytes, cols, rows[(r + 1) & 1]);
 #pragma unroll
         for (int b = 0; b < BH; ++b) {
             const int ty = r - b * S;
             if (ty < 0 || ty >= K) continue;
 #pragma unroll
             for (int tx = 0; tx < K; ++tx) {
-                const float4 w = *reinterpret_cast<const float4 *>(wl + (ty * K + tx) * nch);
+                float w[CV];
 #pragma unroll
-                for (int o = 0; o < TW; ++o) {
-                    acc[b][4 * o + 0] = fmaf(cur[4 * (o * S + tx) + 0], w.x, acc[b][4 * o + 0]);
-                    acc[b][4 * o + 1] = fmaf(cur[4 * (o * S + tx) + 1], w.y, acc[b][4 * o + 1]);
-                    acc[b][4 * o + 2] = fmaf(cur[4 * (o * S + tx) + 2], w.z, acc[b][4 * o + 2]);
-                    acc[b][4 * o + 3] = fmaf(cur[4 * (o * S + tx) + 3], w.w, acc[b][4 * o + 3]);
-                }
+                for (int q = 0; q < CV; ++q) w[q] = wl[(ty * K + tx) * nch + q];
+#pragma unroll
+                for (int o = 0; o < TW; ++o)
+#pragma unroll
+                    for (int q = 0; q < CV; ++q)
+                        acc[b][CV * o + q] = fmaf(cur[CV * (o * S + tx) + q], w[q], acc[b][CV * o + q]);
             }
         }
         pin_registers(acc);
     }
 
     if constexpr (!FLIP) {
-        if (p.epi.enabled()) epilogue_apply_block<4>(acc, p.epi, c);
+        if (p.epi.enabled()) epilogue_apply_block<CV>(acc, p.epi, c);
     }
     // branch-free stores through a view of the output: pixels past the edge of the image store out of range
     const unsigned out_row_bytes = p.out_w * pixel_bytes;
@@ -180,9 +181,15 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_down_kernel(const NhwcPlan 
         const int oy = oy0 + b;
         const unsigned roff = oy < p.out_h ? oy * out_row_bytes : kOob;
 #pragma unroll
-        for (int o = 0; o < TW; ++o)
-            view_store4<IO>(out_view, __builtin_elementwise_add_sat(roff, ocols.off[o]), acc[b][4 * o], acc[b][4 * o + 1],
-                            acc[b][4 * o + 2], acc[b][4 * o + 3]);
+        for (int o = 0; o < TW; ++o) {
+            const unsigned off = __builtin_elementwise_add_sat(roff, ocols.off[o]);
+            if constexpr (CV == 4)
+                view_store4<IO>(out_view, off, acc[b][4 * o], acc[b][4 * o + 1], acc[b][4 * o + 2], acc[b][4 * o + 3]);
+            else if constexpr (CV == 2)
+                view_store2<IO>(out_view, off, acc[b][2 * o], acc[b][2 * o + 1]);
+            else
+                view_store1<IO>(out_view, off, acc[b][o]);
+        }
     }
 }
 
@@ -919,17 +926,29 @@ bool nhwc_fast_ok(const NhwcGeometry &g)
     return true;
 }
 
-template <typename IO, int K, int S, bool FLIP, int TW = 4>
+template <typename IO, int K, int S, bool FLIP, int BH = 4, int TW = 4, int CV = 4>
 int launch_nhwc_down(const IO *in, const IO *taps, IO *out, const NhwcGeometry &g, int in_h, int in_w, int out_h,
                      int out_w, int pad_h, int pad_w, hipStream_t stream)
 {
-    constexpr int BH = 4;
-    if constexpr (K > 3 && TW == 4) {
-        if (env_int("DWCONV_NHWC_TW", 4) == 2)
-            return launch_nhwc_down<IO, K, S, FLIP, 2>(in, taps, out, g, in_h, in_w, out_h, out_w, pad_h, pad_w, stream);
+    if constexpr (BH == 4 && TW == 4 && CV == 4) {
+        if constexpr (K > 3) {
+            if (env_int("DWCONV_NHWC_TW", 4) == 2)
+                return launch_nhwc_down<IO, K, S, FLIP, 4, 2, 4>(in, taps, out, g, in_h, in_w, out_h, out_w, pad_h, pad_w, stream);
+        }
+        // Blocks of 7 x 2 pixels (the registers of 4 x 4) halve the halo rows a lane fetches per output row.  Forward
+        // fp32, where seven rows divide the map or it is large: 3x3 stride 1 (112x112 C=32 83.0 -> 80.4 us, 14x14 C=480
+        // 23.7 -> 21.2, 56x56 C=144 and 7x7 C=1152 unchanged) and 5x5 stride 2 on maps of 28 rows and more (56x56
+        // C=144 72.2 -> 66.5; 14x14 C=672 is 2 us slower with them).  One or two channels per lane with 7 x 8, 7 x 4,
+        // 4 x 8 or 4 x 4 blocks won on single layers and lost on others (1.68-1.74 ms per step against 1.67).
+        if constexpr (sizeof(IO) == 4 && !FLIP && ((K == 3 && S == 1) || (K == 5 && S == 2))) {
+            const bool tall = (out_h % 7 == 0 || out_h >= 56) && (K == 3 || out_h >= 28);
+            if (env_int("DWCONV_NHWC_DOWN_7X2", tall))
+                return launch_nhwc_down<IO, K, S, FLIP, 7, 2, 4>(in, taps, out, g, in_h, in_w, out_h, out_w, pad_h, pad_w, stream);
+        }
     }
     NhwcPlan p{};
-    if (!plan_nhwc<K, 4>(p, g, BH, TW, out_h, out_w)) return -1;
+    const int line_lanes = CV == 4 ? 1 : static_cast<int>(128 / (CV * sizeof(IO)));
+    if (!plan_nhwc<K, CV>(p, g, BH, TW, out_h, out_w, line_lanes)) return -1;
     p.in = in;
     p.taps = taps;
     p.out = out;
@@ -941,10 +960,10 @@ int launch_nhwc_down(const IO *in, const IO *taps, IO *out, const NhwcGeometry &
     p.pad_h = pad_h;
     p.pad_w = pad_w;
     const dim3 grid(p.wgs);
-    const size_t shmem = static_cast<size_t>(p.lanes_c) * 4 * K * K * 4;
-    hipLaunchKernelGGL((nhwc_down_kernel<IO, K, S, FLIP, BH, TW>), grid, dim3(kNhwcThreads), shmem, stream, p);
-    note_variant("nhwc_down%s<k%d,s%d,%s,%dx%d> lanes_c%d", sizeof(IO) == 2 ? "16" : "", K, S, FLIP ? "rot" : "fwd", BH, TW,
-                 p.lanes_c);
+    const size_t shmem = static_cast<size_t>(p.lanes_c) * CV * K * K * 4;
+    hipLaunchKernelGGL((nhwc_down_kernel<IO, K, S, FLIP, BH, TW, CV>), grid, dim3(kNhwcThreads), shmem, stream, p);
+    note_variant("nhwc_down%s<k%d,s%d,%s,%dx%d%s> lanes_c%d", sizeof(IO) == 2 ? "16" : "", K, S, FLIP ? "rot" : "fwd", BH, TW,
+                 CV == 4 ? "" : (CV == 2 ? ",cv2" : ",cv1"), p.lanes_c);
     return check_launch("nhwc_down_kernel");
 }
 
