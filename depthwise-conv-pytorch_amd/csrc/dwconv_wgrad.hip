@@ -47,6 +47,7 @@ struct WgradPlan {
     int g_base;            // float offset of the gy image (same layout as the x image)
     int vec_gx;
     int strided;           // chunk k takes tiles k, k+chunks, ... instead of a contiguous range
+    int lds_gx;            // fused: grad-input goes back through LDS and leaves as one linear stream (one plane per tile)
 };
 
 // GX (stride 1, pad = K/2 only): the band of gy is staged in LDS next to the band of x, with the same
@@ -137,9 +138,9 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
         if constexpr (GX) stage_tile(p.st, gy, lds + p.g_base, plane0, nplanes, oy0 - p.pad_h);
         __syncthreads();
 
+        float xacc[GX ? BH : 1][4];  // grad-input block (kept until the tile's window reads are over when it leaves through LDS)
         if constexpr (GX) {
             constexpr int PC = K / 2;  // the lane's own gy block sits PC rows and columns into its window
-            float xacc[BH][4];
 #pragma unroll
             for (int b = 0; b < BH; ++b)
 #pragma unroll
@@ -168,7 +169,9 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
                 }
                 pin_registers(xacc);
             }
-            if (p.vec_gx == 2) {
+            if (p.lds_gx) {
+                // stored after the grad-weight sums, below
+            } else if (p.vec_gx == 2) {
                 // branch-free: rows past the end of the plane (and lanes without an item) store out of range
                 const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.gx) + plane0 * p.st.in_plane, static_cast<long>(nplanes) * p.st.in_plane * sizeof(IO));
                 const unsigned o0 = (pl * p.st.in_plane + ox) * static_cast<unsigned>(sizeof(IO));
@@ -216,6 +219,32 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
                         acc[ty * K + tx] = fmaf(g[b][o], win[o * S + tx], acc[ty * K + tx]);
             }
             pin_registers(acc);
+        }
+
+        if constexpr (GX) {
+            if (p.lds_gx) {
+                // One plane per tile (the planner guarantees it).  The grad-input block goes into LDS in the layout the
+                // band has in memory, over the x image, and leaves as one linear stream: every store of a wavefront
+                // covers 1 KiB of consecutive bytes.  Lane-owned blocks write a row segment per instruction, and rows
+                // that are not whole 64-byte bursts (56 floats) leave the bursts that straddle two rows to two writes.
+                const int rows_here = min(p.rows_per_tile, p.st.in_h - oy0);
+                const int run = rows_here * p.st.in_w;  // floats, a multiple of four
+                __syncthreads();                        // every window has been read
+                if (has_item) {
+#pragma unroll
+                    for (int b = 0; b < BH; ++b)
+                        if (rb * BH + b < rows_here)
+                            *reinterpret_cast<float4 *>(lds + (rb * BH + b) * p.st.in_w + ox) =
+                                make_float4(xacc[b][0], xacc[b][1], xacc[b][2], xacc[b][3]);
+                }
+                __syncthreads();
+                const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.gx) + plane0 * p.st.in_plane, static_cast<long>(p.st.in_plane) * sizeof(IO));
+                const unsigned o0 = oy0 * p.st.in_w * static_cast<unsigned>(sizeof(IO));
+                for (int i = threadIdx.x; i < (run >> 2); i += blockDim.x) {
+                    const float4 v = reinterpret_cast<const float4 *>(lds)[i];
+                    view_store4<IO>(view, o0 + i * 4 * static_cast<unsigned>(sizeof(IO)), v.x, v.y, v.z, v.w);
+                }
+            }
         }
     }
 
@@ -447,14 +476,20 @@ struct Launcher {
         if (p.st.vec_in) p.st.vec_in = stage_vector_mode(p.st, p.planes_per_tile, sizeof(IO));
         if (p.vec_gx) p.vec_gx = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
         if (p.vec_gy) p.vec_gy = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
+        // grad-input through LDS: 3x3 filters on fp32 rows that are not whole 64-byte bursts, one plane per tile
+        // (56x56: 148 -> 143 us; rows of 112 or 256 floats: unchanged or 1.5 % slower; 7x7 filters, which are bound
+        // by arithmetic, 3 % slower; 16-bit elements 2 % slower)
+        const bool lds_gx_pays = sizeof(IO) == 4 && K == 3 && (g.in_w * sizeof(IO)) % 64 != 0;
+        p.lds_gx = fused && p.planes_per_tile == 1 && p.vec_gx == 2 && env_int("DWCONV_WGRAD_LDS_GX", lds_gx_pays);
         if constexpr (S == 1) {
             if (fused) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, true>), grid, block, shmem, stream, p);
         }
         if (!fused) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, false>), grid, block, shmem, stream, p);
         rc = check_launch("wgrad_tile_kernel");
         if (rc != DWCONV_OK) return;
-        note_variant("%s%s<k%d,s%d,bh%d> P%d rows%d chunks%d vin%d vgy%d", fused ? "bwd_tile" : "wgrad_tile",
-                     sizeof(IO) == 2 ? "16" : "", K, S, BH, p.planes_per_tile, p.rows_per_tile, p.chunks, p.st.vec_in, p.vec_gy);
+        note_variant("%s%s<k%d,s%d,bh%d> P%d rows%d chunks%d vin%d vgy%d%s", fused ? "bwd_tile" : "wgrad_tile",
+                     sizeof(IO) == 2 ? "16" : "", K, S, BH, p.planes_per_tile, p.rows_per_tile, p.chunks, p.st.vec_in, p.vec_gy,
+                     p.lds_gx ? " ldsgx" : "");
         rc = launch_wgrad_final(static_cast<const float *>(ws), gw, g.channel, K * K, p.chunks, stream);
     }
 };
