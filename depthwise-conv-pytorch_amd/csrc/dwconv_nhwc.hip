@@ -932,7 +932,8 @@ int launch_nhwc_down(const IO *in, const IO *taps, IO *out, const NhwcGeometry &
 {
     if constexpr (BH == 4 && TW == 4 && CV == 4) {
         if constexpr (K > 3) {
-            if (env_int("DWCONV_NHWC_TW", 4) == 2)
+            // 5x5 stride 2 onto maps of fewer than 28 rows: twice the lanes with 4 x 2 blocks (14x14 C=672 25.7 -> 21.7 us)
+            if (env_int("DWCONV_NHWC_TW", sizeof(IO) == 4 && !FLIP && K == 5 && S == 2 && out_h < 28 ? 2 : 4) == 2)
                 return launch_nhwc_down<IO, K, S, FLIP, 4, 2, 4>(in, taps, out, g, in_h, in_w, out_h, out_w, pad_h, pad_w, stream);
         }
         // Blocks of 7 x 2 pixels (the registers of 4 x 4) halve the halo rows a lane fetches per output row.  Forward
@@ -1074,7 +1075,11 @@ long nhwc_bwd_fused_case(int mode, const IO *x, const IO *gy, const IO *taps, IO
     if (!plan_nhwc<K, CV>(p, g, BH, TW, g.out_h, g.out_w, line_lanes, "DWCONV_NHWC_WGRAD_LANES")) return -1;
     const int cgroups = p.cgroups;
     const long wg_iters = (p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg;
-    long groups = env_int("DWCONV_NHWC_WGRAD_WGS", 512) / cgroups;
+    // Workgroups per chip: a multiple of the 256 compute units (576-704 and 800-896 are 5-25 % slower than 512 or
+    // 768).  The 5x5 kernel holds three workgroups per unit and is bound by its own arithmetic, so a third
+    // resident workgroup hides more latency (7x7 C=1152 40.4 -> 36.1 us, 14x14 C=672 69.6 -> 61.0, C=480 51.2 ->
+    // 49.0, 28x28 C=240 91.9 -> 90.1); the 3x3 kernels wait for memory and lose 3-20 % with more than two.
+    long groups = env_int("DWCONV_NHWC_WGRAD_WGS", K == 5 ? 768 : 512) / cgroups;
     groups = std::max(1l, std::min(groups, wg_iters));
     p.groups = static_cast<int>(groups);
     const size_t need = static_cast<size_t>(groups) * K * K * g.channel * sizeof(float);
@@ -1113,7 +1118,10 @@ long nhwc_bwd_s2_fused_case(int mode, const IO *x, const IO *gy, const IO *taps,
     if (!plan_nhwc<K, CV>(p, g, BQH, BQW, g.out_h, g.out_w, line_lanes, "DWCONV_NHWC_WGRAD_LANES")) return -1;
     const int cgroups = p.cgroups;
     const long wg_iters = (p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg;
-    long groups = env_int("DWCONV_NHWC_WGRAD_WGS", 512) / cgroups;
+    // three workgroups per compute unit for the 5x5 kernel on small maps (14x14 C=672 48.8 -> 43.8 us), two
+    // elsewhere (56x56 C=144 is 5 % slower with three)
+    const bool small_map = K == 5 && static_cast<long>(g.out_h) * g.out_w <= 196;
+    long groups = env_int("DWCONV_NHWC_WGRAD_WGS", small_map ? 768 : 512) / cgroups;
     groups = std::max(1l, std::min(groups, wg_iters));
     p.groups = static_cast<int>(groups);
     const size_t need = static_cast<size_t>(groups) * K * K * g.channel * sizeof(float);
