@@ -931,6 +931,14 @@ int launch_nhwc_down(const IO *in, const IO *taps, IO *out, const NhwcGeometry &
                      int out_w, int pad_h, int pad_w, hipStream_t stream)
 {
     if constexpr (BH == 4 && TW == 4 && CV == 4) {
+        if constexpr (K == 5 && S == 1 && sizeof(IO) == 4 && !FLIP) {
+            // 5x5 stride 1 on maps of 14 or 28 rows: one channel per lane and 7 x 8 blocks fetch 2.4 input pixels per
+            // result instead of 4 (14x14 C=480 31.5 -> 27.1 us, 28x28 C=240 60.5 -> 59.2, 14x14 C=672 unchanged; 7x7
+            // maps lose 1.5 us, and 7 x 4 or 4 x 8 blocks with one or two channels per lane lose 3-10 us everywhere)
+            const bool fits = out_h % 7 == 0 && out_h >= 14 && g.channel % 32 == 0;
+            if (env_int("DWCONV_NHWC_K5_7X8", fits))
+                return launch_nhwc_down<IO, K, S, FLIP, 7, 8, 1>(in, taps, out, g, in_h, in_w, out_h, out_w, pad_h, pad_w, stream);
+        }
         if constexpr (K > 3) {
             // 5x5 stride 2 onto maps of fewer than 28 rows: twice the lanes with 4 x 2 blocks (14x14 C=672 25.7 -> 21.7 us)
             if (env_int("DWCONV_NHWC_TW", sizeof(IO) == 4 && !FLIP && K == 5 && S == 2 && out_h < 28 ? 2 : 4) == 2)

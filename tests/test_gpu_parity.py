@@ -628,6 +628,9 @@ NHWC_SHAPES = [
     (2, 3, 9, 11, 3, 1, 1), (1, 6, 8, 8, 4, 2, 1), (2, 5, 7, 7, 1, 1, 0), (1, 2, 12, 10, 9, 1, 4),
     # channel groups of whole 128-byte lines whose last group is partly idle (C / 4 = 60 lanes in groups of 16, 18 in groups of 8)
     (2, 240, 28, 28, 5, 1, 2), (2, 240, 28, 28, 3, 2, 1), (1, 72, 14, 14, 3, 1, 1),
+    # 5x5 forward lane shapes: one channel per lane with 7 x 8 pixel blocks (C % 32 == 0, 14 or 28 rows; a width that is
+    # not a multiple of 8), 4 x 2 blocks for stride 2 onto small maps
+    (2, 96, 14, 14, 5, 1, 2), (1, 64, 28, 20, 5, 1, 2), (2, 672, 14, 14, 5, 2, 2),
 ]
 
 
@@ -748,6 +751,18 @@ def test_channels_last_fused_backward_other_layers(dw, gpu, case, monkeypatch):
     assert "nhwc_wgrad" in _C.last_variant() and not _C.last_variant().startswith("nhwc_bwd"), _C.last_variant()
     np.testing.assert_allclose(_np(gx3), _np(gx), rtol=1e-6, atol=1e-6)
     np.testing.assert_allclose(_np(gw3), _np(gw), rtol=1e-5, atol=1e-5 * float(gw.abs().max()))
+
+
+def test_channels_last_forward_lane_shapes(dw, gpu):
+    """5x5 forward: one channel per lane and 7 x 8 blocks on 14-row maps with C % 32 == 0, 4 x 2 blocks for stride 2
+    onto a 7x7 map, four channels per lane and 4 x 4 blocks otherwise."""
+    from torch_dwconv import _C
+
+    for (c, hw, s, want) in [(96, 14, 1, "nhwc_down<k5,s1,fwd,7x8,cv1>"), (672, 14, 2, "nhwc_down<k5,s2,fwd,4x2>"),
+                             (240, 28, 1, "nhwc_down<k5,s1,fwd,4x4>"), (96, 12, 1, "nhwc_down<k5,s1,fwd,4x4>")]:
+        x = _channels_last(torch.randn(2, c, hw, hw), gpu)
+        dw.depthwise_conv2d(x, torch.randn(c, 1, 5, 5, device=gpu), stride=s, padding=2)
+        assert _C.last_variant().startswith(want), (_C.last_variant(), want)
 
 
 def test_channels_last_channel_groups_are_whole_lines(dw, gpu):
