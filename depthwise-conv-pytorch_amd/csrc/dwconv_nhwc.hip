@@ -43,6 +43,7 @@ struct NhwcPlan {
     Epilogue epi;            // forward kernel: applied to every sum before it is stored
     int cgroups;             // workgroups along the channel axis
     int wgs;                 // forward / grad-input: workgroups in all (1-D grid)
+    int xcd_chunks;          // backward: chunks are dealt to the XCDs in contiguous runs
 };
 
 // ---- window loads through a buffer view (nhwc_view / view_load, dwconv_tile_common.hpp) -----------------------
@@ -301,8 +302,10 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_wgrad_kernel(const NhwcPlan
     const int C = p.channel;
     // (grid: chunk x channel group, dealt to the XCDs round-robin; giving every XCD a contiguous run of chunks,
     // as the forward kernel does with its pixel groups, measured 2 % slower here)
-    const int chunk = blockIdx.x;
-    const int c0 = blockIdx.y * p.lanes_c * CV;
+    // 1-D grid, channel group fastest; with xcd_chunks every XCD (own L2) takes a contiguous run of chunks
+    const int wg = p.xcd_chunks ? xcd_contiguous_tile(blockIdx.x, p.groups * p.cgroups) : static_cast<int>(blockIdx.x);
+    const int chunk = wg / p.cgroups;
+    const int c0 = (wg - chunk * p.cgroups) * p.lanes_c * CV;
     const int nch = min(p.lanes_c * CV, C - c0);
     const int pb_local = fast_div(threadIdx.x, p.lanes_c_magic);
     const int lane_c = threadIdx.x - pb_local * p.lanes_c;
@@ -408,8 +411,10 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_bwd_fused_kernel(const Nhwc
     constexpr int KK = K * K, P = K / 2;
     constexpr int ROWS = BH + K - 1, COLS = TW + K - 1;
     const int C = p.channel;
-    const int chunk = blockIdx.x;
-    const int c0 = blockIdx.y * p.lanes_c * CV;
+    // 1-D grid, channel group fastest; with xcd_chunks every XCD (own L2) takes a contiguous run of chunks
+    const int wg = p.xcd_chunks ? xcd_contiguous_tile(blockIdx.x, p.groups * p.cgroups) : static_cast<int>(blockIdx.x);
+    const int chunk = wg / p.cgroups;
+    const int c0 = (wg - chunk * p.cgroups) * p.lanes_c * CV;
     const int nch = min(p.lanes_c * CV, C - c0);
     const int pb_local = fast_div(threadIdx.x, p.lanes_c_magic);
     const int lane_c = threadIdx.x - pb_local * p.lanes_c;
@@ -565,8 +570,10 @@ __global__ __launch_bounds__(kNhwcThreads) void nhwc_bwd_s2_fused_kernel(const N
     constexpr int STEPS = GROWS + P / 2;                  // x rows 2 (t - P/2), 2 (t - P/2) + 1 are consumed in step t
     static_assert(2 * (STEPS - 1 - P / 2) + 1 >= XROWS - 1, "every x row has its step");
     const int C = p.channel;
-    const int chunk = blockIdx.x;
-    const int c0 = blockIdx.y * p.lanes_c * CV;
+    // 1-D grid, channel group fastest; with xcd_chunks every XCD (own L2) takes a contiguous run of chunks
+    const int wg = p.xcd_chunks ? xcd_contiguous_tile(blockIdx.x, p.groups * p.cgroups) : static_cast<int>(blockIdx.x);
+    const int chunk = wg / p.cgroups;
+    const int c0 = (wg - chunk * p.cgroups) * p.lanes_c * CV;
     const int nch = min(p.lanes_c * CV, C - c0);
     const int pb_local = fast_div(threadIdx.x, p.lanes_c_magic);
     const int lane_c = threadIdx.x - pb_local * p.lanes_c;
@@ -1030,6 +1037,7 @@ long nhwc_wgrad_case(int mode, const IO *x, const IO *gy, IO *gw, void *ws, size
     long groups = env_int("DWCONV_NHWC_WGRAD_WGS", 512) / cgroups;
     groups = std::max(1l, std::min(groups, wg_iters));
     p.groups = static_cast<int>(groups);
+    p.xcd_chunks = env_int("DWCONV_NHWC_XCD_CHUNKS", 0);
     const size_t need = static_cast<size_t>(groups) * K * K * g.channel * sizeof(float);
     if (mode == 0) return static_cast<long>(need);
     if (ws == nullptr || ws_bytes < need)
@@ -1044,7 +1052,7 @@ long nhwc_wgrad_case(int mode, const IO *x, const IO *gy, IO *gw, void *ws, size
     p.pad_h = g.pad_h;
     p.pad_w = g.pad_w;
     const size_t shmem = static_cast<size_t>(p.blocks_per_wg) * K * p.lanes_c * CV * 4;
-    hipLaunchKernelGGL((nhwc_wgrad_kernel<IO, K, S, CV, BH, TW>), dim3(p.groups, cgroups), dim3(kNhwcThreads), shmem, stream, p);
+    hipLaunchKernelGGL((nhwc_wgrad_kernel<IO, K, S, CV, BH, TW>), dim3(p.groups * cgroups), dim3(kNhwcThreads), shmem, stream, p);
     int rc = check_launch("nhwc_wgrad_kernel");
     if (rc != DWCONV_OK) return rc;
     note_variant("nhwc_wgrad%s<k%d,s%d,cv%d,%dx%d> lanes_c%d chunks%d", sizeof(IO) == 2 ? "16" : "", K, S, CV, BH, TW,
@@ -1090,6 +1098,7 @@ long nhwc_bwd_fused_case(int mode, const IO *x, const IO *gy, const IO *taps, IO
     long groups = env_int("DWCONV_NHWC_WGRAD_WGS", K == 5 ? 768 : 512) / cgroups;
     groups = std::max(1l, std::min(groups, wg_iters));
     p.groups = static_cast<int>(groups);
+    p.xcd_chunks = env_int("DWCONV_NHWC_XCD_CHUNKS", 0);
     const size_t need = static_cast<size_t>(groups) * K * K * g.channel * sizeof(float);
     if (mode == 0) return static_cast<long>(need);
     if (ws == nullptr || ws_bytes < need)
@@ -1106,7 +1115,7 @@ long nhwc_bwd_fused_case(int mode, const IO *x, const IO *gy, const IO *taps, IO
     p.pad_h = g.pad_h;
     p.pad_w = g.pad_w;
     const size_t shmem = static_cast<size_t>(p.lanes_c) * CV * 4 * std::max(K * K, p.blocks_per_wg * K);
-    hipLaunchKernelGGL((nhwc_bwd_fused_kernel<IO, K, CV, BH, TW>), dim3(p.groups, cgroups), dim3(kNhwcThreads), shmem, stream, p);
+    hipLaunchKernelGGL((nhwc_bwd_fused_kernel<IO, K, CV, BH, TW>), dim3(p.groups * cgroups), dim3(kNhwcThreads), shmem, stream, p);
     int rc = check_launch("nhwc_bwd_fused_kernel");
     if (rc != DWCONV_OK) return rc;
     note_variant("nhwc_bwd%s<k%d,s1,cv%d,%dx%d> lanes_c%d chunks%d", sizeof(IO) == 2 ? "16" : "", K, CV, BH, TW, p.lanes_c, p.groups);
@@ -1132,6 +1141,10 @@ long nhwc_bwd_s2_fused_case(int mode, const IO *x, const IO *gy, const IO *taps,
     long groups = env_int("DWCONV_NHWC_WGRAD_WGS", small_map ? 768 : 512) / cgroups;
     groups = std::max(1l, std::min(groups, wg_iters));
     p.groups = static_cast<int>(groups);
+    // Workgroups whose pixel blocks share halo rows run at the same time.  Dealt round-robin to the XCDs, they fetch
+    // those rows into several L2s; in contiguous runs per XCD the 5x5 kernel on large maps fetches less (56x56 C=144
+    // 139.3 -> 135.7 us).  Every other backward kernel is 1-4 us slower that way.
+    p.xcd_chunks = env_int("DWCONV_NHWC_XCD_CHUNKS", K == 5 && !small_map);
     const size_t need = static_cast<size_t>(groups) * K * K * g.channel * sizeof(float);
     if (mode == 0) return static_cast<long>(need);
     if (ws == nullptr || ws_bytes < need)
@@ -1148,7 +1161,7 @@ long nhwc_bwd_s2_fused_case(int mode, const IO *x, const IO *gy, const IO *taps,
     p.pad_h = g.pad_h;
     p.pad_w = g.pad_w;
     const size_t shmem = static_cast<size_t>(p.lanes_c) * CV * 4 * std::max(K * K, p.blocks_per_wg * K);
-    hipLaunchKernelGGL((nhwc_bwd_s2_fused_kernel<IO, K, CV, BQH, BQW>), dim3(p.groups, cgroups), dim3(kNhwcThreads), shmem, stream, p);
+    hipLaunchKernelGGL((nhwc_bwd_s2_fused_kernel<IO, K, CV, BQH, BQW>), dim3(p.groups * cgroups), dim3(kNhwcThreads), shmem, stream, p);
     int rc = check_launch("nhwc_bwd_s2_fused_kernel");
     if (rc != DWCONV_OK) return rc;
     note_variant("nhwc_bwd%s<k%d,s2,cv%d,%dx%d> lanes_c%d chunks%d", sizeof(IO) == 2 ? "16" : "", K, CV, BQH, BQW, p.lanes_c, p.groups);
