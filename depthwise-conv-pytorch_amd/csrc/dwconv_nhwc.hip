@@ -887,7 +887,7 @@ int pick_lanes_c(int lanes, int cap, int line)
 
 template <int K, int CV>
 bool plan_nhwc(NhwcPlan &p, const NhwcGeometry &g, int bh, int tw, int blocks_h, int blocks_w, int min_lanes = 1,
-               const char *lanes_env = "DWCONV_NHWC_LANES")
+               const char *lanes_env = "DWCONV_NHWC_LANES", int exact_lanes = 0)
 {
     p.batch = g.batch;
     p.channel = g.channel;
@@ -902,6 +902,7 @@ bool plan_nhwc(NhwcPlan &p, const NhwcGeometry &g, int bh, int tw, int blocks_h,
     cap = std::max(1, std::min(cap, 128));
     while (cap > 1 && static_cast<size_t>(cap) * CV * K * K * 4 > static_cast<size_t>(kNhwcTapLds)) --cap;
     p.lanes_c = pick_lanes_c(g.channel / CV, cap, env_int("DWCONV_NHWC_ALIGN", 1) ? 32 / CV : 1);
+    if (exact_lanes > 0 && getenv(lanes_env) == nullptr && (g.channel / CV) % exact_lanes == 0) p.lanes_c = exact_lanes;
     p.lanes_c_magic = magic_u16(p.lanes_c);
     p.blocks_per_wg = kNhwcThreads / p.lanes_c;
     p.blocks_y = ceil_div(blocks_h, bh);
@@ -1132,7 +1133,11 @@ long nhwc_bwd_s2_fused_case(int mode, const IO *x, const IO *gy, const IO *taps,
 {
     NhwcPlan p{};
     const int line_lanes = static_cast<int>(128 / (CV * sizeof(IO)));
-    if (!plan_nhwc<K, CV>(p, g, BQH, BQW, g.out_h, g.out_w, line_lanes, "DWCONV_NHWC_WGRAD_LANES")) return -1;
+    // C = 144 (4.5 lines per pixel) with the 5x5 kernel: three groups of 48 channels, 192-byte segments that start on
+    // 64-byte boundaries, instead of five groups of 32 whose last is half idle (56x56: 135.8 -> 129.5 us).  The other
+    // kernels, and C = 240 in groups of 48 or 80, are 1-4 us slower than with 32.
+    const int lanes48 = K == 5 && CV == 1 && g.channel % 32 != 0 && g.channel % 48 == 0 ? 48 : 0;
+    if (!plan_nhwc<K, CV>(p, g, BQH, BQW, g.out_h, g.out_w, line_lanes, "DWCONV_NHWC_WGRAD_LANES", lanes48)) return -1;
     const int cgroups = p.cgroups;
     const long wg_iters = (p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg;
     // three workgroups per compute unit for the 5x5 kernel on small maps (14x14 C=672 48.8 -> 43.8 us), two
