@@ -88,9 +88,11 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
         const int q0 = rt * p.rows_per_tile;
 
         if (tile != chunk) __syncthreads();  // the previous tile's window reads are done
-        // two loads in flight per lane and image (not four): -3 % on the 112x112 layer, the two images' loads overlap
-        stage_tile<IO, VIEWS, 2>(p.sx, x, lds, plane0, 1, 2 * q0 - p.pad);
-        stage_tile<IO, VIEWS, 2>(p.sg, gy, lds + p.g_base, plane0, 1, q0 - p.m);
+        // fp32: two 16-byte loads in flight per lane and image (not four): -3 % on the 112x112 layer, the two images'
+        // loads overlap.  16-bit elements: four 8-byte loads, the same bytes in flight (112x112 C=96 176 -> 166 us).
+        constexpr int kInFlight = sizeof(IO) == 2 ? 4 : 2;
+        stage_tile<IO, VIEWS, kInFlight>(p.sx, x, lds, plane0, 1, 2 * q0 - p.pad);
+        stage_tile<IO, VIEWS, kInFlight>(p.sg, gy, lds + p.g_base, plane0, 1, q0 - p.m);
         __syncthreads();
 
         // ---- gy window: grad-input block, and this lane's gy elements from the window's centre
