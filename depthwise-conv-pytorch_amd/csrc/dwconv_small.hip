@@ -269,6 +269,15 @@ int launch_small_down_any(SmallPlan &p, int S, bool rot, hipStream_t stream)
             if (p.planes < 64l * 2048)
                 return rot ? launch_small_down<IO, W, K, 1, true, 2>(p, stream) : launch_small_down<IO, W, K, 1, false, 2>(p, stream);
         }
+        if constexpr (W != 7) {
+            // One output row per lane (twice the lanes per plane, half the planes per wavefront, 80 instead of 140
+            // registers) against two: 28x28 maps gain with every filter and element type (fp32 5x5 C=240 43.3 -> 39.0 us,
+            // 7x7 C=192 27.8 -> 20.4, bf16 5x5 30.7 -> 28.4); 14x14 maps gain 1-2 us in fp32 with 3x3 and 5x5 filters
+            // and lose 1-3 us with 7x7 filters or 16-bit elements.
+            const bool one_row = W == 28 || (sizeof(IO) == 4 && K <= 5);
+            if (env_int("DWCONV_SMALL_BH", one_row ? 1 : 2) == 1)
+                return rot ? launch_small_down<IO, W, K, 1, true, 1>(p, stream) : launch_small_down<IO, W, K, 1, false, 1>(p, stream);
+        }
         return rot ? launch_small_down<IO, W, K, 1, true, BH1>(p, stream) : launch_small_down<IO, W, K, 1, false, BH1>(p, stream);
     }
     if constexpr (W % 2 == 0) {
