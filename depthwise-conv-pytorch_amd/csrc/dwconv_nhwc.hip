@@ -949,7 +949,7 @@ int launch_nhwc_down(const IO *in, const IO *taps, IO *out, const NhwcGeometry &
         }
         if constexpr (K > 3) {
             // 5x5 stride 2 onto maps of fewer than 28 rows: twice the lanes with 4 x 2 blocks (14x14 C=672 25.7 -> 21.7 us)
-            if (env_int("DWCONV_NHWC_TW", sizeof(IO) == 4 && !FLIP && K == 5 && S == 2 && out_h < 28 ? 2 : 4) == 2)
+            if (env_int("DWCONV_NHWC_TW", !FLIP && K == 5 && S == 2 && out_h < 28 ? 2 : 4) == 2)
                 return launch_nhwc_down<IO, K, S, FLIP, 4, 2, 4>(in, taps, out, g, in_h, in_w, out_h, out_w, pad_h, pad_w, stream);
         }
         // Blocks of 7 x 2 pixels (the registers of 4 x 4) halve the halo rows a lane fetches per output row.  Forward
@@ -957,8 +957,11 @@ int launch_nhwc_down(const IO *in, const IO *taps, IO *out, const NhwcGeometry &
         // 23.7 -> 21.2, 56x56 C=144 and 7x7 C=1152 unchanged) and 5x5 stride 2 on maps of 28 rows and more (56x56
         // C=144 72.2 -> 66.5; 14x14 C=672 is 2 us slower with them).  One or two channels per lane with 7 x 8, 7 x 4,
         // 4 x 8 or 4 x 4 blocks won on single layers and lost on others (1.68-1.74 ms per step against 1.67).
-        if constexpr (sizeof(IO) == 4 && !FLIP && ((K == 3 && S == 1) || (K == 5 && S == 2))) {
-            const bool tall = (out_h % 7 == 0 || out_h >= 56) && (K == 3 || out_h >= 28);
+        if constexpr (!FLIP && ((K == 3 && S == 1) || (K == 5 && S == 2))) {
+            // (16-bit elements: 5x5 stride 2 alike, 56x56 C=144 54.2 -> 48.1 us; 3x3 stride 1 only on maps of 14 to 28 rows,
+            // 14x14 C=480 19.9 -> 17.1, while 56x56 C=144 and 7x7 C=1152 lose 6 and 1.5 us with them)
+            const bool tall = sizeof(IO) == 4 ? (out_h % 7 == 0 || out_h >= 56) && (K == 3 || out_h >= 28)
+                                              : (K == 5 ? out_h >= 28 : out_h % 7 == 0 && out_h >= 14 && out_h <= 28);
             if (env_int("DWCONV_NHWC_DOWN_7X2", tall))
                 return launch_nhwc_down<IO, K, S, FLIP, 7, 2, 4>(in, taps, out, g, in_h, in_w, out_h, out_w, pad_h, pad_w, stream);
         }
