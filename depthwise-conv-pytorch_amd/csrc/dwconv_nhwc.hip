@@ -1038,7 +1038,9 @@ long nhwc_wgrad_case(int mode, const IO *x, const IO *gy, IO *gw, void *ws, size
     const long wg_iters = (p.blocks_total + p.blocks_per_wg - 1) / p.blocks_per_wg;
     // One resident round of workgroups: the kernel's 170-250 registers leave two wavefronts per SIMD, i.e. two
     // 256-lane workgroups on each of the 256 CUs (measured: 512 beats 256, 384, 640, 768 and 1024 by 3-10 %).
-    long groups = env_int("DWCONV_NHWC_WGRAD_WGS", 512) / cgroups;
+    // (16-bit elements, 5x5 stride 2: 768 take the 56x56 C=144 backward from 113.6 to 105.8 us and leave 14x14 C=672 alone;
+    // every other instance of this kernel loses 3-7 us with 768)
+    long groups = env_int("DWCONV_NHWC_WGRAD_WGS", sizeof(IO) == 2 && K == 5 && S == 2 ? 768 : 512) / cgroups;
     groups = std::max(1l, std::min(groups, wg_iters));
     p.groups = static_cast<int>(groups);
     p.xcd_chunks = env_int("DWCONV_NHWC_XCD_CHUNKS", 0);
@@ -1099,7 +1101,9 @@ long nhwc_bwd_fused_case(int mode, const IO *x, const IO *gy, const IO *taps, IO
     // 768).  The 5x5 kernel holds three workgroups per unit and is bound by its own arithmetic, so a third
     // resident workgroup hides more latency (7x7 C=1152 40.4 -> 36.1 us, 14x14 C=672 69.6 -> 61.0, C=480 51.2 ->
     // 49.0, 28x28 C=240 91.9 -> 90.1); the 3x3 kernels wait for memory and lose 3-20 % with more than two.
-    long groups = env_int("DWCONV_NHWC_WGRAD_WGS", K == 5 ? 768 : 512) / cgroups;
+    // The two-channel 3x3 instance (168 registers, three workgroups per unit; what 16-bit tensors run) takes 768 as well:
+    // bf16 7x7 C=1152 23.7 -> 18.6 us, 56x56 C=144 94.2 -> 90.6, 112x112 C=32 72.6 -> 70.3, 14x14 C=480 30.0 -> 31.4.
+    long groups = env_int("DWCONV_NHWC_WGRAD_WGS", K == 5 || CV == 2 ? 768 : 512) / cgroups;
     groups = std::max(1l, std::min(groups, wg_iters));
     p.groups = static_cast<int>(groups);
     p.xcd_chunks = env_int("DWCONV_NHWC_XCD_CHUNKS", 0);
