@@ -224,62 +224,81 @@ def boundary_planes(n, c, rng, extra=4):
 def full_size_references(shape, x, wt, gy, gpu):
     """fp64 references for whole tensors: the C oracle where it finishes in seconds, otherwise the shift-and-add
     closed form on the device (pinned against the C oracle in tests/test_oracle.py) with the C oracle on boundary
-    and random planes on top."""
+    and random planes on top.  16-bit inputs are widened exactly: the references see the rounded values."""
     n, c, h, w, k, s, p = shape
     if x.numel() <= C_ORACLE_WHOLE_LIMIT:
-        xn, wn, gn = _np(x), _np(wt), _np(gy)
+        xn, wn, gn = _np(x.double()), _np(wt.double()), _np(gy.double())
         return (oracle.forward(xn, wn, s, p), oracle.grad_input(gn, wn, (h, w), s, p),
                 oracle.grad_weight(xn, gn, wt.shape, s, p), "c-oracle")
     y, gx, gw = oracle.shift_add_reference(x.to(gpu), wt.to(gpu), gy.to(gpu), s, p)
     return y, gx, gw, "shift-add"
 
 
-def check_full_size(dw, gpu, shape, seed=0, layouts=("nchw",), n_planes=4):
+def full_size_tolerances(dtype):
+    """(rtol, atol) of y / gx and the relative bound of gw: the fp32 bounds of this file, plus one rounding step of
+    the element type for 16-bit tensors (2^-11 for fp16, 2^-8 for bf16; the sums are fp32 and rounded once)."""
+    if dtype == torch.float32:
+        return 1e-5, 1e-5, 1e-4
+    step = 2.0 ** -11 if dtype == torch.float16 else 2.0 ** -8
+    return step, 1e-5 + step * 1e-2, step + 1e-4
+
+
+def check_full_size(dw, gpu, shape, seed=0, layouts=("nchw",), n_planes=4, dtype=torch.float32, expect=None):
     """Full-size run with the planner decisions of the real configuration.  Every element of y, gx and gw is
     compared with an fp64 reference (outputs start as NaN); boundary and random planes are checked against the C
-    oracle as well; adjoint identities; grad-weight bit-identical from run to run; both backward routes."""
+    oracle as well; adjoint identities; grad-weight bit-identical from run to run; both backward routes.
+    `expect` = (forward, backward) prefixes the kernel variant strings must start with."""
+    from torch_dwconv import _C
+
     n, c, h, w, k, s, p = shape
-    x, wt, gy = make_inputs(shape, seed=seed)
+    x, wt, gy = (t.to(dtype) for t in make_inputs(shape, seed=seed))
+    rtol, atol, gw_rtol = full_size_tolerances(dtype)
     y_ref, gx_ref, gw_ref, how = full_size_references(shape, x, wt, gy, gpu)
     gw_ref_np = gw_ref if isinstance(gw_ref, np.ndarray) else _np(gw_ref)
-    gw_atol = 1e-4 * float(np.abs(gw_ref_np).max())
+    gw_atol = gw_rtol * float(np.abs(gw_ref_np).max())
     rng = np.random.default_rng(seed + 1)
     planes = boundary_planes(n, c, rng, extra=n_planes) if how != "c-oracle" else []
     plane_refs = {}
     for b, ch in planes:
-        xs, ws, gs = _np(x[b:b + 1, ch:ch + 1]), _np(wt[ch:ch + 1]), _np(gy[b:b + 1, ch:ch + 1])
+        xs, ws, gs = (_np(t.double()) for t in (x[b:b + 1, ch:ch + 1], wt[ch:ch + 1], gy[b:b + 1, ch:ch + 1]))
         plane_refs[(b, ch)] = (oracle.forward(xs, ws, s, p)[0, 0], oracle.grad_input(gs, ws, (h, w), s, p)[0, 0])
     chans = sorted({0, 1, c // 2, c - 2, c - 1} & set(range(c))) if how != "c-oracle" else []
     if chans:
-        gw_c = oracle.grad_weight(_np(x[:, chans]), _np(gy[:, chans]), (len(chans), 1, k, k), s, p)
+        gw_c = oracle.grad_weight(_np(x[:, chans].double()), _np(gy[:, chans].double()), (len(chans), 1, k, k), s, p)
 
     def check(tag, y, gx, gw):
         if y is not None:
-            assert_close_on_device(y, y_ref, 1e-5, 1e-5, f"{tag} y")
-        assert_close_on_device(gx, gx_ref, 1e-5, 1e-5, f"{tag} gx")
-        assert_close_on_device(gw, gw_ref, 1e-4, gw_atol, f"{tag} gw")
+            assert_close_on_device(y, y_ref, rtol, atol, f"{tag} y")
+        assert_close_on_device(gx, gx_ref, rtol, atol, f"{tag} gx")
+        assert_close_on_device(gw, gw_ref, gw_rtol, gw_atol, f"{tag} gw")
         for (b, ch), (yp, gxp) in plane_refs.items():
             if y is not None:
-                np.testing.assert_allclose(_np(y[b, ch]).astype(np.float64), yp, rtol=1e-5, atol=1e-5)
-            np.testing.assert_allclose(_np(gx[b, ch]).astype(np.float64), gxp, rtol=1e-5, atol=1e-5)
+                np.testing.assert_allclose(_np(y[b, ch].double()), yp, rtol=rtol, atol=atol)
+            np.testing.assert_allclose(_np(gx[b, ch].double()), gxp, rtol=rtol, atol=atol)
         if chans:
-            np.testing.assert_allclose(_np(gw[chans]).astype(np.float64), gw_c, rtol=1e-4, atol=gw_atol)
+            np.testing.assert_allclose(_np(gw[chans].double()), gw_c, rtol=gw_rtol, atol=gw_atol)
 
+    # the inner products below see every rounding of a 16-bit result once
+    adj_tol = 1e-6 if dtype == torch.float32 else 1e-2 * rtol
     for layout in layouts:
         fmt = torch.channels_last if layout == "nhwc" else torch.contiguous_format
         xg, wg, gg = x.to(gpu).contiguous(memory_format=fmt), wt.to(gpu), gy.to(gpu).contiguous(memory_format=fmt)
         with poisoned_allocations():
             y, gx, gw, variant = run_three_passes(dw, xg, wg, gg, s, p)
-        _announce(shape_id(shape), layout, how, variant)
+        v_bwd = _C.last_variant()
+        _announce(shape_id(shape), str(dtype), layout, how, variant, "|", v_bwd)
+        if expect is not None:
+            assert variant.startswith(expect[0]) and v_bwd.startswith(expect[1]), (variant, v_bwd, expect)
+        assert y.dtype == dtype and gx.dtype == dtype and gw.dtype == dtype
         if layout == "nhwc":
             assert y.is_contiguous(memory_format=torch.channels_last) and gx.is_contiguous(memory_format=torch.channels_last)
-        check(f"{shape_id(shape)} {layout} [{variant}]", y, gx, gw)
+        check(f"{shape_id(shape)} {layout} [{variant} | {v_bwd}]", y, gx, gw)
         # size-independent property: <y, gy> == <x, gx> == <w, gw>, accumulated in fp64 on the device
         lhs = (y.double() * gg.double()).sum().item()
         mid = (xg.double() * gx.double()).sum().item()
         rhs = (wg.double() * gw.double()).sum().item()
         scale = (y.double().abs() * gg.double().abs()).sum().item()
-        assert abs(lhs - mid) <= 1e-6 * scale and abs(lhs - rhs) <= 1e-6 * scale
+        assert abs(lhs - mid) <= adj_tol * scale and abs(lhs - rhs) <= adj_tol * scale
         # bit-identical grad-weight on a second run
         with poisoned_allocations():
             _, _, gw2, _ = run_three_passes(dw, xg, wg, gg, s, p)
@@ -323,6 +342,45 @@ def test_stress_grad_weight_determinism(dw, gpu):
     torch.cuda.synchronize()
     for r in runs[1:]:
         assert torch.equal(runs[0], r)
+
+
+# 16-bit tensors at the batch the benchmark runs: chunk counts, planes per tile, the XCD mapping and the remainder
+# paths are functions of the tensor sizes, so the small shapes of test_half_precision_io never reach them.
+HALF_FULL_SIZE = {
+    0: ("tile_down16_dot2", "bwd_tile16_dot2"),    # 112x112 C32 3x3: 16-bit LDS images, fused backward
+    1: ("tile_down16_dot2", "bwd_tile_s216"),      # 112x112 C96 3x3 stride 2
+    2: ("tile_down16<", "bwd_tile16<"),            # 56x56 C144 3x3
+    3: ("tile_down16<", "bwd_tile_s216"),          # 56x56 C144 5x5 stride 2
+    4: ("small_down16", "small_bwd16"),            # 28x28 C240 5x5
+    5: ("small_down16", "small_bwd16"),            # 28x28 C240 3x3 stride 2
+    8: ("small_down16", "small_bwd16"),            # 14x14 C672 5x5
+    9: ("small_down16", "small_bwd16"),            # 14x14 C672 5x5 stride 2
+    10: ("small_down16", "small_bwd16"),           # 7x7 C1152 5x5
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("layer", sorted(HALF_FULL_SIZE), ids=lambda i: shape_id(effnet_layers()[i]))
+def test_half_precision_full_batch(dw, gpu, layer, dtype):
+    """EfficientNet-B0 layers at batch 128 with 16-bit tensors: whole tensors against the fp64 reference on the
+    rounded inputs (outputs start as NaN), one rounding step of tolerance, bit-identical grad-weight."""
+    check_full_size(dw, gpu, effnet_layers()[layer], seed=41, dtype=dtype, expect=HALF_FULL_SIZE[layer])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+def test_half_precision_large_maps_full_size(dw, gpu, dtype):
+    check_full_size(dw, gpu, CFG2, seed=43, dtype=dtype)
+    check_full_size(dw, gpu, CONVNEXT_T[0], seed=44, dtype=dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+def test_half_precision_several_tiles_per_workgroup(dw, gpu, dtype, monkeypatch):
+    """A workgroup of the fused 16-bit backward that walks three or more tiles (sums carried over tiles, strided
+    chunk walk, grad-input streamed out of LDS between tiles), forced on a small tensor by capping the grid."""
+    monkeypatch.setenv("DWCONV_WGRAD_WGS", "8")
+    shape = (9, 4, 40, 104, 3, 1, 1)
+    check_full_size(dw, gpu, shape, seed=45, dtype=dtype, expect=("tile_down16_dot2", "bwd_tile16_dot2"))
+    check_full_size(dw, gpu, (13, 3, 37, 96, 5, 1, 2), seed=46, dtype=dtype, expect=("tile_down16_dot2", "bwd_tile16_dot2"))
 
 
 # ---- closed forms on the device ----------------------------------------------------------
@@ -848,6 +906,18 @@ def test_channels_last_full_size_layers(dw, gpu, shape):
     """Every EfficientNet-B0 layer at batch 128, channels-last: whole tensors against the fp64 reference (outputs
     start as NaN), adjoint identities, bit-identical grad-weight."""
     check_full_size(dw, gpu, shape, seed=37, layouts=("nhwc",))
+
+
+@pytest.mark.parametrize("shape", CFG4 + CONVNEXT_T + [STRESS], ids=shape_id)
+def test_channels_last_full_size_large_filters(dw, gpu, shape):
+    """The 7x7 workloads and the grad-weight stress case in channels-last at full size."""
+    check_full_size(dw, gpu, shape, seed=38, layouts=("nhwc",))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("layer", [0, 1, 3, 4, 7, 9, 10], ids=lambda i: shape_id(effnet_layers()[i]))
+def test_channels_last_half_precision_full_batch(dw, gpu, layer, dtype):
+    check_full_size(dw, gpu, effnet_layers()[layer], seed=39, layouts=("nhwc",), dtype=dtype)
 
 
 # ---- forward with a fused per-channel scale / shift and activation -------------------------------------------

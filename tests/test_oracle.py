@@ -163,6 +163,44 @@ def test_backward_direction_is_conv_transpose(k, s, p):
     np.testing.assert_allclose(got2, _np(ref2), rtol=1e-12, atol=1e-12)
 
 
+RAW_MODES = [
+    # (kh, kw, up_h, up_w, down_h, down_w, pad_h0, pad_h1, pad_w0, pad_w1, forward)
+    (3, 3, 2, 2, 2, 2, 1, 1, 1, 1, True),       # up and down together
+    (5, 5, 2, 2, 2, 2, 2, 1, 3, 0, True),
+    (4, 3, 3, 2, 2, 3, 0, 0, 1, 1, False),      # rectangular everything, rotated taps
+    (3, 3, 2, 2, 1, 1, 1, 2, 0, 3, True),       # forward direction with up > 1 (taps not rotated)
+    (5, 4, 1, 3, 2, 1, 4, 0, 0, 5, True),
+    (3, 3, 1, 1, 1, 1, -1, 2, 1, -2, True),     # negative pads crop the input
+    (5, 5, 2, 2, 1, 1, -2, 3, -1, -1, False),
+    (4, 4, 2, 2, 3, 3, -1, -1, 2, 2, False),
+    (1, 1, 3, 3, 2, 2, 0, 0, 0, 0, True),
+    (7, 7, 2, 1, 1, 2, 3, 3, 3, 3, False),
+]
+
+
+@pytest.mark.parametrize("mode", RAW_MODES, ids=lambda m: "k%dx%d_u%d%d_d%d%d_p%d.%d.%d.%d_%s" % (m[:10] + ("fwd" if m[10] else "rot",)))
+def test_raw_operator_modes_equal_zero_stuffing_plus_strided_conv(mode):
+    """The raw operator of dwconv_kernel.cu:69-181 in the modes the autograd path never uses (up and down
+    together, forward with up > 1, negative pads), against PyTorch: zero-stuff the input by hand (up - 1 zeros after
+    every sample: mid = out*down + up - 1 - pad0, in = floor(mid / up), tap = (in + 1)*up - mid - 1 at :122-178
+    places sample i at position i*up), pad (crop for negative pads), then a strided grouped correlation with the
+    taps as given (forward) or rotated by 180 degrees (backward, :108-113)."""
+    kh, kw, uh, uw, dh, dw_, ph0, ph1, pw0, pw1, fwd = mode
+    g = torch.Generator("cpu").manual_seed(kh * 100 + kw * 10 + uh + dh)
+    n, c, h, w = 2, 3, 9, 11
+    x = torch.randn(n, c, h, w, generator=g, dtype=torch.float64)
+    k = torch.randn(c, 1, kh, kw, generator=g, dtype=torch.float64)
+    stuffed = torch.zeros(n, c, h * uh, w * uw, dtype=torch.float64)
+    stuffed[:, :, ::uh, ::uw] = x
+    padded = F.pad(stuffed, (pw0, pw1, ph0, ph1))
+    taps = k if fwd else torch.flip(k, dims=(2, 3))
+    want = F.conv2d(padded, taps, stride=(dh, dw_), groups=c)
+    got = oracle.dwconv2d(x.numpy(), k.numpy(), uh, uw, dh, dw_, ph0, ph1, pw0, pw1, fwd)
+    assert got.shape == tuple(want.shape)
+    assert got.size > 0
+    np.testing.assert_allclose(got, want.numpy(), rtol=1e-12, atol=1e-12)
+
+
 def test_small_operator_equals_large_operator():
     g = torch.Generator().manual_seed(2)
     x = _np(torch.randn(2, 3, 9, 11, generator=g, dtype=torch.float64))
