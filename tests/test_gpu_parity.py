@@ -285,7 +285,11 @@ def check_full_size(dw, gpu, shape, seed=0, layouts=("nchw",), n_planes=4, dtype
         xg, wg, gg = x.to(gpu).contiguous(memory_format=fmt), wt.to(gpu), gy.to(gpu).contiguous(memory_format=fmt)
         with poisoned_allocations():
             y, gx, gw, variant = run_three_passes(dw, xg, wg, gg, s, p)
-        v_bwd = _C.last_variant()
+        v_bwd = ""
+        if layout == "nchw":
+            # (autograd runs the backward on its own thread; the variant note is per thread)
+            _C.dwconv2d_backward(xg, gg, wg, s, s, p, p)
+            v_bwd = _C.last_variant()
         _announce(shape_id(shape), str(dtype), layout, how, variant, "|", v_bwd)
         if expect is not None:
             assert variant.startswith(expect[0]) and v_bwd.startswith(expect[1]), (variant, v_bwd, expect)
