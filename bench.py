@@ -34,8 +34,22 @@ EFFNET_B0 = [
     (240, 28, 5, 1), (240, 28, 3, 2), (480, 14, 3, 1), (480, 14, 5, 1),
     (672, 14, 5, 1), (672, 14, 5, 2), (1152, 7, 5, 1), (1152, 7, 3, 1),
 ]
+
+
+def effnet_at(batch, res):
+    """The same 12 layers for a res x res network input (224 gives EFFNET_B0's maps: 112, 56, 28, 14, 7)."""
+    shapes, h = [], res // 2
+    for (c, _, k, s) in EFFNET_B0:
+        shapes.append((batch, c, h, h, k, s, k // 2))
+        h = (h + 2 * (k // 2) - k) // s + 1
+    return shapes
+
+
 WORKLOADS = {
     "effnet_b0": lambda batch: [(batch, c, h, h, k, s, k // 2) for (c, h, k, s) in EFFNET_B0],
+    # other input resolutions: 256 -> maps 128, 64, 32, 16, 8; 240 (EfficientNet-B1's) -> 120, 60, 30, 15, 8
+    "effnet_b0_256": lambda batch: effnet_at(batch, 256),
+    "effnet_b0_240": lambda batch: effnet_at(batch, 240),
     "cfg1": lambda batch: [(8, 32, 56, 56, 3, 1, 1)],
     "cfg2": lambda batch: [(16, 64, 256, 256, 5, 1, 2)],
     "cfg4": lambda batch: [(256, 1024, 7, 7, 7, 1, 3), (128, 512, 14, 14, 7, 1, 3)],

@@ -1,5 +1,5 @@
 // Helpers shared by the whole-plane kernels for small feature maps: LDS rows of a
-// compile-time width and flat runs of planes between global memory and LDS.
+// compile-time width (or capacity) and flat runs of planes between global memory and LDS.
 #pragma once
 
 #include "dwconv_tile_common.hpp"
@@ -7,6 +7,53 @@
 namespace dwconv {
 
 constexpr int kWave = 64;
+
+// ---- plans and per-width entry points ---------------------------------------------------------------------
+// Width instances of the whole-plane kernels: exact widths, and ragged capacity classes for every other width.
+// Each instance is its own translation unit (dwconv_small_width.hip); the dispatchers call them through the
+// function templates declared below.
+#define DWCONV_SMALL_EXACT_WIDTHS(X) X(7) X(8) X(14) X(16) X(28) X(32)
+#define DWCONV_SMALL_RAGGED_WIDTHS(X) X(8) X(16) X(24) X(32)
+
+inline bool small_width_is_exact(int w) { return w == 7 || w == 8 || w == 14 || w == 16 || w == 28 || w == 32; }
+// capacity class of a width that has no exact instance; 0 when it is too wide for this family
+inline int small_ragged_class(int w) { return w < 1 || w > 32 ? 0 : (w + 7) / 8 * 8; }
+
+struct SmallPlan {
+    const void *in;    // element type IO of the kernel template
+    const void *taps;
+    void *out;
+    long planes;
+    int channel;
+    int in_h, out_h;
+    int in_w, out_w;       // real widths (the kernels of an exact instance use their template constant)
+    int pad_h;             // leading zero rows (down) or m = (pad0 + E) / 2 (up2)
+    int planes_per_run;    // P
+    int lanes_per_plane;   // LPP
+    unsigned lpp_magic;
+    Epilogue epi;          // forward kernels: applied to every sum before it is stored
+};
+
+// Launches the forward / grad-input kernel of width instance (W, RAG) for p: K in {3,5,7}; up2 = false: decimation
+// S in {1,2}, taps rotated if `rot`; up2 = true: the transposed stride-2 problem.  -1 when the instance does not
+// cover the case.
+template <int W, bool RAG, typename IO>
+int small_fir_width(SmallPlan &p, int K, int S, bool rot, bool up2, hipStream_t stream);
+
+struct SmallBwdArgs {
+    const void *x;    // element type IO
+    const void *gy;
+    const void *taps;
+    void *gx;
+    void *gw;
+    void *ws;
+    size_t ws_bytes;
+};
+
+// mode 0: workspace bytes of the grad-weight partial sums; mode 1: grad-weight; mode 2: grad-weight + grad-input.
+// Returns -1 when the instance does not cover g, a dwconv_status otherwise (mode 0: the byte count).
+template <int W, bool RAG, typename IO>
+long small_bwd_width(int mode, const SmallBwdArgs &a, const WgradGeometry &g, hipStream_t stream);
 
 // ---- LDS rows -----------------------------------------------------------------------------
 template <int N>
@@ -43,6 +90,41 @@ __device__ __forceinline__ void lds_store_row(float *p, const float *r)
     } else {
 #pragma unroll
         for (int i = 0; i < N; ++i) p[i] = r[i];
+    }
+}
+
+// Width-aware forms.  RAG = false: the row is exactly N elements.  RAG = true: N is a capacity and the real width
+// (1..N, uniform) comes at run time: a row starts anywhere, so it is read element by element, up to N - 1 floats past
+// its end (the LDS allocation of a ragged kernel ends with N spare floats), and what was read past the real width is
+// dropped by mask_row.
+template <int N, bool RAG>
+__device__ __forceinline__ void lds_load_row_w(const float *p, float (&r)[N])
+{
+    if constexpr (RAG) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) r[i] = p[i];
+    } else {
+        lds_load_row<N>(p, r);
+    }
+}
+
+// dst = src where the lane's row exists (`ok`) and, for ragged widths, the column does (i < w); zero elsewhere.
+template <int N, bool RAG>
+__device__ __forceinline__ void mask_row(const float (&src)[N], float (&dst)[N], bool ok, int w)
+{
+#pragma unroll
+    for (int i = 0; i < N; ++i) dst[i] = (ok && (!RAG || i < w)) ? src[i] : 0.f;
+}
+
+template <int N, bool RAG>
+__device__ __forceinline__ void lds_store_row_w(float *p, const float *r, int w)
+{
+    if constexpr (RAG) {
+#pragma unroll
+        for (int i = 0; i < N; ++i)
+            if (i < w) p[i] = r[i];
+    } else {
+        lds_store_row<N>(p, r);
     }
 }
 
@@ -96,8 +178,12 @@ __device__ __forceinline__ void runs_to_lds(const IO *__restrict__ ga, float *la
     if (tb < nb) lb[tb] = Io<IO>::in(gb[tb]);
 }
 
+// A run that starts `head` elements (1..3) past a 4-element boundary is moved as the aligned span that contains it:
+// `g` points at that boundary, `n` counts the head too, and the run's first element sits at lds[head].  Loading such a
+// span reads up to three elements of the neighbouring run (harmless); storing it must not write them: the first
+// group of four goes out element by element, from `head` on.
 template <typename IO>
-__device__ __forceinline__ void lds_to_run(IO *__restrict__ g, const float *lds, int n)
+__device__ __forceinline__ void lds_to_run(IO *__restrict__ g, const float *lds, int n, int head = 0)
 {
     const int n4 = n >> 2;
     constexpr int U = 4;
@@ -110,11 +196,14 @@ __device__ __forceinline__ void lds_to_run(IO *__restrict__ g, const float *lds,
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int i = base + u * kWave;
-            view_store4<IO>(view, i < n4 ? i * 4u * static_cast<unsigned>(sizeof(IO)) : kOob, v[u].x, v[u].y, v[u].z, v[u].w);
+            const bool whole = i < n4 && (i > 0 || head == 0);
+            view_store4<IO>(view, whole ? i * 4u * static_cast<unsigned>(sizeof(IO)) : kOob, v[u].x, v[u].y, v[u].z, v[u].w);
         }
     }
-    const int tail = n4 * 4 + threadIdx.x;
-    if (tail < n) g[tail] = Io<IO>::out(lds[tail]);
+    const int t = threadIdx.x;
+    if (head != 0 && n4 > 0 && t >= head && t < 4) g[t] = Io<IO>::out(lds[t]);
+    const int tail = n4 * 4 + t;
+    if (tail < n && tail >= head) g[tail] = Io<IO>::out(lds[tail]);
 }
 
 // This lane's K*K taps straight from global memory (the lanes of one plane read the same addresses).

@@ -1,0 +1,321 @@
+// Whole-plane kernels for small feature maps (up to 32 elements wide, "same" column padding); element type fp32,
+// fp16 or bf16, LDS and arithmetic fp32.
+//
+// Planes of a small map are tiny (196 B to 4 KiB) and sit back to back in memory,
+// so the only way to move them at HBM speed is to treat a run of P planes as one
+// flat stream: 128-bit loads of the run into LDS (same layout as in memory, no
+// index arithmetic), arithmetic out of LDS, results back into LDS in their
+// memory layout, 128-bit stores of the run.  One wavefront (a 64-lane workgroup,
+// so no cross-wave barrier exists) owns a run; a CU holds about ten such
+// wavefronts, each with several loads in flight.
+//
+// A lane owns BH full-width output rows of one plane.  Because it holds whole
+// rows, which taps fall off the left/right edge is known at compile time (they
+// are simply not emitted); rows above/below the plane are replaced by zeros
+// with a select.  The reference's counterpart (torch_dwconv/dwconv_kernel.cu:308-442,
+// :444-588) keeps a zero-filled padded tile in shared memory and re-reads every
+// tap for every output; it takes any plane up to 32 x 32 (:652-671), and so does this family.
+//
+// The plane width is a template parameter in one of two ways.  Exact (RAG = false): rows are W elements and are
+// read with vector reads where W allows.  Ragged (RAG = true): W is a capacity and the real width (1..W) arrives
+// at run time; rows are read element by element, columns past the real width are zeroed by a wavefront-uniform
+// select and their sums are never stored.  One translation unit per instance (dwconv_small_width.hip).
+//
+//   small_down_kernel : up = 1, decimation S; forward, and grad-input of stride-1 layers (FLIP)
+//   small_up2_kernel  : up = 2, taps rotated; grad-input of stride-2 layers
+// (grad-weight and the fused backward of these maps: dwconv_small_bwd.hpp)
+#pragma once
+
+#include "dwconv_small_common.hpp"
+
+namespace dwconv {
+
+namespace {
+
+// out[oy,ox] = sum_{ty,tx} in[oy*S - pad_h + ty, ox*S - K/2 + tx] * f[ty,tx]
+template <typename IO, int W, bool RAG, int K, int S, bool FLIP, int BH>
+__global__ __launch_bounds__(kWave) void small_down_kernel(const SmallPlan p)
+{
+    extern __shared__ float4 lds_raw[];
+    float *lds = reinterpret_cast<float *>(lds_raw);
+    constexpr int OW = (W - 1) / S + 1;  // output columns a lane computes (the real count when exact)
+    constexpr int PW = K / 2;
+    constexpr int WIN_ROWS = (BH - 1) * S + K;
+    const int w_in = RAG ? p.in_w : W, w_out = RAG ? p.out_w : OW;
+
+    const long plane0 = static_cast<long>(blockIdx.x) * p.planes_per_run;
+    const int nplanes = static_cast<int>(min(static_cast<long>(p.planes_per_run), p.planes - plane0));
+    const int in_plane = p.in_h * w_in, out_plane = p.out_h * w_out;
+
+    const int pl_raw = fast_div(threadIdx.x, p.lpp_magic);
+    const int rb = threadIdx.x - pl_raw * p.lanes_per_plane;
+    const bool active = pl_raw < nplanes;
+    const int pl = active ? pl_raw : 0;
+
+    // runs that start off a 4-element boundary are moved as the aligned span around them (see lds_to_run)
+    const long in0 = plane0 * in_plane, out0 = plane0 * out_plane;
+    const int hin = static_cast<int>(in0 & 3), hout = static_cast<int>(out0 & 3);
+
+    float tapv[K * K];
+    load_taps<K * K, FLIP>(static_cast<const IO *>(p.taps), static_cast<int>((plane0 + pl) % p.channel), tapv);
+    run_to_lds(static_cast<const IO *>(p.in) + (in0 - hin), lds, nplanes * in_plane + hin);
+    __syncthreads();
+
+    float acc[BH][OW];
+#pragma unroll
+    for (int b = 0; b < BH; ++b)
+#pragma unroll
+        for (int o = 0; o < OW; ++o) acc[b][o] = 0.f;
+
+    const int oy0 = rb * BH;
+    const float *plane = lds + hin + pl * in_plane;
+    // rows are read one ahead of their use and the sums pinned after every row (see pin_registers)
+    float nxt[W];
+    bool nxt_ok;
+    {
+        const int iy = oy0 * S - p.pad_h;
+        nxt_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
+        lds_load_row_w<W, RAG>(plane + (nxt_ok ? iy : 0) * w_in, nxt);
+    }
+#pragma unroll
+    for (int wr = 0; wr < WIN_ROWS; ++wr) {
+        float row[W];
+        mask_row<W, RAG>(nxt, row, nxt_ok, w_in);
+        if (wr + 1 < WIN_ROWS) {
+            const int iy = oy0 * S - p.pad_h + wr + 1;
+            nxt_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
+            lds_load_row_w<W, RAG>(plane + (nxt_ok ? iy : 0) * w_in, nxt);
+        }
+#pragma unroll
+        for (int b = 0; b < BH; ++b) {
+            const int ty = wr - b * S;
+            if (ty < 0 || ty >= K) continue;
+#pragma unroll
+            for (int tx = 0; tx < K; ++tx)
+#pragma unroll
+                for (int o = 0; o < OW; ++o) {
+                    const int ix = o * S - PW + tx;
+                    if (ix < 0 || ix >= W) continue;
+                    acc[b][o] = fmaf(row[ix], tapv[ty * K + tx], acc[b][o]);
+                }
+        }
+        pin_registers(acc);
+    }
+    if constexpr (!FLIP) {
+        if (p.epi.enabled()) {
+            epilogue_apply_block<1>(acc, p.epi, static_cast<int>((plane0 + pl) % p.channel));
+        }
+    }
+    __syncthreads();  // every lane has read its input rows: the run can be overwritten in place
+
+    if (active) {
+        float *dst = lds + hout + pl * out_plane;
+#pragma unroll
+        for (int b = 0; b < BH; ++b)
+            if (oy0 + b < p.out_h) lds_store_row_w<OW, RAG>(dst + (oy0 + b) * w_out, acc[b], w_out);
+    }
+    __syncthreads();
+    lds_to_run(static_cast<IO *>(p.out) + (out0 - hout), lds, nplanes * out_plane + hout, hout);
+}
+
+// up = 2, taps rotated, "same" padding of the forward conv (leading pad of the transposed problem = K/2):
+//   out[2q + r] = sum_a in[q - m + r + a] * g'[r + 2a],  g'[t] = g[t - E],  E = (K/2) & 1,  m = (K/2 + E) / 2.
+// Input planes are W wide (or up to W, ragged), output planes 2W or 2W - 1 (the forward input had an odd extent);
+// a lane owns output rows 2q, 2q+1.
+template <typename IO, int W, bool RAG, int K>
+__global__ __launch_bounds__(kWave) void small_up2_kernel(const SmallPlan p)
+{
+    extern __shared__ float4 lds_raw[];
+    float *lds = reinterpret_cast<float *>(lds_raw);
+    constexpr int OW = 2 * W;
+    constexpr int E = (K / 2) & 1;
+    constexpr int M = (K / 2 + E) / 2;
+    constexpr int KA = (K + E + 1) / 2;
+    constexpr int WIN_ROWS = KA + 1;
+    const int w_in = RAG ? p.in_w : W, w_out = RAG ? p.out_w : OW;
+
+    const long plane0 = static_cast<long>(blockIdx.x) * p.planes_per_run;
+    const int nplanes = static_cast<int>(min(static_cast<long>(p.planes_per_run), p.planes - plane0));
+    const int in_plane = p.in_h * w_in, out_plane = p.out_h * w_out;
+
+    const int pl_raw = fast_div(threadIdx.x, p.lpp_magic);
+    const int q = threadIdx.x - pl_raw * p.lanes_per_plane;
+    const bool active = pl_raw < nplanes;
+    const int pl = active ? pl_raw : 0;
+
+    const long in0 = plane0 * in_plane, out0 = plane0 * out_plane;
+    const int hin = static_cast<int>(in0 & 3), hout = static_cast<int>(out0 & 3);
+
+    float tapv[K * K];
+    load_taps<K * K, true>(static_cast<const IO *>(p.taps), static_cast<int>((plane0 + pl) % p.channel), tapv);
+    run_to_lds(static_cast<const IO *>(p.in) + (in0 - hin), lds, nplanes * in_plane + hin);
+    __syncthreads();
+
+    float acc[2][OW];
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int o = 0; o < OW; ++o) acc[r][o] = 0.f;
+
+    const float *plane = lds + hin + pl * in_plane;
+    float nxt[W];
+    bool nxt_ok;
+    {
+        const int iy = q - p.pad_h;
+        nxt_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
+        lds_load_row_w<W, RAG>(plane + (nxt_ok ? iy : 0) * w_in, nxt);
+    }
+#pragma unroll
+    for (int wr = 0; wr < WIN_ROWS; ++wr) {
+        float row[W];
+        mask_row<W, RAG>(nxt, row, nxt_ok, w_in);
+        if (wr + 1 < WIN_ROWS) {
+            const int iy = q - p.pad_h + wr + 1;
+            nxt_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
+            lds_load_row_w<W, RAG>(plane + (nxt_ok ? iy : 0) * w_in, nxt);
+        }
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const int a = wr - r;
+            if (a < 0 || a >= KA) continue;
+            const int fy = r + 2 * a - E;
+            if (fy < 0 || fy >= K) continue;
+#pragma unroll
+            for (int o = 0; o < OW; ++o) {
+                const int xq = o / 2, rx = o % 2;
+#pragma unroll
+                for (int ax = 0; ax < KA; ++ax) {
+                    const int fx = rx + 2 * ax - E;
+                    const int ix = xq - M + rx + ax;
+                    if (fx < 0 || fx >= K || ix < 0 || ix >= W) continue;
+                    acc[r][o] = fmaf(row[ix], tapv[fy * K + fx], acc[r][o]);
+                }
+            }
+        }
+        pin_registers(acc);
+    }
+    __syncthreads();
+
+    if (active) {
+        float *dst = lds + hout + pl * out_plane;
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+            if (2 * q + r < p.out_h) lds_store_row_w<OW, RAG>(dst + (2 * q + r) * w_out, acc[r], w_out);
+    }
+    __syncthreads();
+    lds_to_run(static_cast<IO *>(p.out) + (out0 - hout), lds, nplanes * out_plane + hout, hout);
+}
+
+// LDS of a run of `planes` planes (the larger of its input and output image, plus the up to three elements in front
+// of a run that starts off a 4-element boundary) plus, for ragged widths, the spare floats that reads past the last
+// row land in.
+size_t small_lds_bytes(int planes, int in_plane, int out_plane, int spare)
+{
+    return (static_cast<size_t>(planes) * (in_plane > out_plane ? in_plane : out_plane) + 4 + spare) * 4;
+}
+
+// Planes per wavefront: as many as there are lane slots within the LDS budget; when a plane is not a multiple of 4
+// elements a multiple of 4 of them if that costs less than half (every run then starts on a 4-element boundary).
+int planes_per_run(int lanes_per_plane, int in_plane, int out_plane, long planes)
+{
+    int P = kWave / lanes_per_plane;
+    while (P > 0 && small_lds_bytes(P, in_plane, out_plane, 0) > 16 * 1024) --P;
+    if ((in_plane % 4 != 0 || out_plane % 4 != 0) && P >= 4) P -= P % 4;
+    if (static_cast<long>(P) > planes && in_plane % 4 == 0 && out_plane % 4 == 0) P = static_cast<int>(planes);
+    return P;
+}
+
+// Fills in the run shape of p (lanes_per_plane set); false when the geometry does not fit a wavefront.
+bool finish_plan(SmallPlan &p, size_t &shmem, long &runs, int spare)
+{
+    if (p.lanes_per_plane < 1 || p.lanes_per_plane > kWave) return false;
+    const int in_plane = p.in_h * p.in_w, out_plane = p.out_h * p.out_w;
+    p.planes_per_run = planes_per_run(p.lanes_per_plane, in_plane, out_plane, p.planes);
+    if (p.planes_per_run < 1) return false;
+    p.lpp_magic = magic_u16(p.lanes_per_plane);
+    runs = (p.planes + p.planes_per_run - 1) / p.planes_per_run;
+    if (runs > 0x7fffffffL) return false;
+    shmem = small_lds_bytes(p.planes_per_run, in_plane, out_plane, spare);
+    return true;
+}
+
+template <typename IO, int W, bool RAG, int K, int S, bool FLIP, int BH>
+int launch_small_down(SmallPlan &p, hipStream_t stream)
+{
+    p.lanes_per_plane = ceil_div(p.out_h, BH);
+    size_t shmem;
+    long runs;
+    if (!finish_plan(p, shmem, runs, RAG ? W : 0)) return -1;
+    hipLaunchKernelGGL((small_down_kernel<IO, W, RAG, K, S, FLIP, BH>), dim3(static_cast<unsigned>(runs)), dim3(kWave),
+                       shmem, stream, p);
+    note_variant("small_down%s<%s%d,k%d,s%d,%s,bh%d> P%d", sizeof(IO) == 2 ? "16" : "", RAG ? "r" : "w", W, K, S,
+                 FLIP ? "rot" : "fwd", BH, p.planes_per_run);
+    return check_launch("small_down_kernel");
+}
+
+template <typename IO, int W, bool RAG, int K>
+int launch_small_up2(SmallPlan &p, hipStream_t stream)
+{
+    p.lanes_per_plane = ceil_div(p.out_h, 2);
+    size_t shmem;
+    long runs;
+    if (!finish_plan(p, shmem, runs, RAG ? W : 0)) return -1;
+    hipLaunchKernelGGL((small_up2_kernel<IO, W, RAG, K>), dim3(static_cast<unsigned>(runs)), dim3(kWave), shmem, stream, p);
+    note_variant("small_up2%s<%s%d,k%d> P%d", sizeof(IO) == 2 ? "16" : "", RAG ? "r" : "w", W, K, p.planes_per_run);
+    return check_launch("small_up2_kernel");
+}
+
+// Rows per lane.  Measured on the 7-, 14- and 28-wide maps and carried over to their neighbours:
+//  * up to 8 wide: a lane takes a whole plane (64 planes per wavefront) when there are enough planes to fill the
+//    device that way, otherwise two rows (four lanes per plane);
+//  * up to 16 wide: one row per lane (twice the lanes per plane, half the planes per wavefront, 80 instead of 140
+//    registers) for fp32 with 3x3 and 5x5 filters (1-2 us per layer), two rows with 7x7 filters or 16-bit
+//    elements (one row loses 1-3 us there);
+//  * wider: one row (28x28 fp32 5x5 C=240 43.3 -> 39.0 us, 7x7 C=192 27.8 -> 20.4, bf16 5x5 30.7 -> 28.4);
+//  * stride 2: one row.
+// Ragged instances come with one choice each (two for the 16-wide class).
+template <typename IO, int W, bool RAG, int K>
+int launch_small_down_any(SmallPlan &p, int S, bool rot, hipStream_t stream)
+{
+#define DWCONV_DOWN(BHV)                                                                    \
+    return rot ? launch_small_down<IO, W, RAG, K, 1, true, BHV>(p, stream)                  \
+               : launch_small_down<IO, W, RAG, K, 1, false, BHV>(p, stream)
+    if (S == 1) {
+        if constexpr (W <= 8) {
+            if constexpr (!RAG) {
+                if (p.planes >= 64l * 2048) { DWCONV_DOWN(W); }
+            }
+            DWCONV_DOWN(2);
+        } else if constexpr (W <= 16) {
+            const bool one_row = sizeof(IO) == 4 && K <= 5;
+            if (env_int("DWCONV_SMALL_BH", one_row ? 1 : 2) == 1) { DWCONV_DOWN(1); }
+            DWCONV_DOWN(2);
+        } else {
+            DWCONV_DOWN(1);
+        }
+    }
+#undef DWCONV_DOWN
+    if (S == 2 && !rot) return launch_small_down<IO, W, RAG, K, 2, false, 1>(p, stream);
+    return -1;
+}
+
+}  // namespace
+
+template <int W, bool RAG, typename IO>
+int small_fir_width(SmallPlan &p, int K, int S, bool rot, bool up2, hipStream_t stream)
+{
+    if (up2) {
+        if constexpr (W <= 16) {
+            if (K == 3) return launch_small_up2<IO, W, RAG, 3>(p, stream);
+            if (K == 5) return launch_small_up2<IO, W, RAG, 5>(p, stream);
+            if (K == 7) return launch_small_up2<IO, W, RAG, 7>(p, stream);
+        }
+        return -1;
+    }
+    if (K == 3) return launch_small_down_any<IO, W, RAG, 3>(p, S, rot, stream);
+    if (K == 5) return launch_small_down_any<IO, W, RAG, 5>(p, S, rot, stream);
+    if (K == 7) return launch_small_down_any<IO, W, RAG, 7>(p, S, rot, stream);
+    return -1;
+}
+
+}  // namespace dwconv

@@ -105,6 +105,20 @@ SMALL = [
     (3, 12, 7, 7, 5, 1, 2), (5, 20, 7, 7, 3, 1, 1), (3, 8, 7, 7, 7, 1, 3), (2, 13, 14, 14, 3, 1, 1),
     (3, 10, 14, 14, 5, 2, 2), (5, 11, 28, 28, 3, 2, 1), (3, 6, 28, 28, 5, 1, 2), (2, 4, 28, 28, 7, 2, 3),
     (2, 70, 14, 14, 7, 1, 3), (2, 68, 7, 7, 5, 1, 2), (2, 3, 20, 14, 3, 1, 1), (2, 4, 10, 7, 5, 1, 2),
+    # whole-plane kernels at the other widths up to 32: exact instances (8, 16, 32) and ragged classes (any other
+    # width), both strides, odd extents (stride 2 of an odd plane: gx is 2*gy - 1 wide), planes that are not a
+    # multiple of four elements
+    (3, 8, 8, 8, 3, 1, 1), (2, 12, 8, 8, 5, 1, 2), (2, 8, 8, 8, 7, 1, 3), (3, 8, 8, 8, 5, 2, 2),
+    (2, 6, 16, 16, 3, 1, 1), (2, 5, 16, 16, 5, 1, 2), (2, 4, 16, 16, 7, 1, 3), (3, 6, 16, 16, 5, 2, 2), (2, 4, 16, 16, 3, 2, 1),
+    (2, 3, 32, 32, 3, 1, 1), (2, 4, 32, 32, 5, 1, 2), (1, 3, 32, 32, 7, 1, 3), (2, 3, 32, 32, 3, 2, 1), (2, 2, 32, 32, 7, 2, 3),
+    (2, 8, 15, 15, 3, 1, 1), (2, 8, 15, 15, 5, 1, 2), (1, 4, 15, 15, 7, 1, 3), (3, 8, 15, 15, 5, 2, 2), (2, 12, 15, 15, 3, 2, 1),
+    (2, 3, 30, 30, 5, 1, 2), (2, 2, 30, 30, 3, 2, 1), (1, 3, 30, 30, 7, 1, 3), (2, 3, 30, 30, 7, 2, 3),
+    (2, 4, 12, 12, 5, 1, 2), (2, 3, 24, 24, 3, 1, 1), (2, 5, 20, 20, 5, 2, 2), (2, 4, 9, 9, 3, 1, 1), (3, 8, 9, 9, 5, 2, 2),
+    (2, 4, 5, 5, 3, 1, 1), (2, 4, 6, 4, 5, 1, 2), (2, 3, 40, 10, 3, 1, 1), (2, 4, 7, 22, 5, 1, 2), (2, 4, 13, 26, 7, 1, 3),
+    (2, 8, 7, 7, 3, 2, 1), (2, 4, 11, 7, 5, 2, 2), (2, 4, 31, 31, 3, 1, 1), (4, 4, 17, 17, 5, 1, 2), (2, 16, 3, 3, 3, 1, 1),
+    # runs of planes that start off a 4-element boundary (odd planes, channel groups that are not multiples of four)
+    (3, 5, 15, 15, 3, 1, 1), (3, 7, 9, 9, 5, 2, 2), (2, 3, 31, 29, 7, 1, 3), (3, 5, 30, 30, 3, 2, 1), (5, 3, 7, 7, 5, 1, 2),
+    (3, 6, 13, 13, 3, 2, 1), (2, 9, 5, 7, 3, 1, 1),
 ]
 
 
@@ -335,6 +349,30 @@ def test_large_kernel_small_map_layers(dw, gpu, shape):
     check_full_size(dw, gpu, shape)
 
 
+def effnet_layers_at(res, batch=128):
+    """The 12 layers for a res x res network input (224: the BASELINE maps; 256: 128/64/32/16/8; 240: 120/60/30/15/8)."""
+    from shapes import EFFNET_B0
+
+    shapes, h = [], res // 2
+    for (c, _, k, s) in EFFNET_B0:
+        shapes.append((batch, c, h, h, k, s, k // 2))
+        h = (h + 2 * (k // 2) - k) // s + 1
+    return shapes
+
+
+@pytest.mark.parametrize("shape", effnet_layers_at(256)[4:] + effnet_layers_at(240)[4:10], ids=shape_id)
+def test_small_maps_of_other_resolutions_full_batch(dw, gpu, shape):
+    """Maps 32, 16, 8, 30 and 15 wide at batch 128 (the whole-plane kernels' exact and ragged width instances):
+    whole tensors against the fp64 reference, outputs start as NaN."""
+    check_full_size(dw, gpu, shape, seed=51, expect=("small_down", "small_bwd"))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("shape", [effnet_layers_at(256)[i] for i in (4, 5, 7, 10)] + [effnet_layers_at(240)[i] for i in (4, 5, 8, 9)], ids=shape_id)
+def test_small_maps_of_other_resolutions_half_precision(dw, gpu, shape, dtype):
+    check_full_size(dw, gpu, shape, seed=52, dtype=dtype, expect=("small_down16", "small_bwd16"))
+
+
 def test_stress_grad_weight_determinism(dw, gpu):
     n, c, h, w, k, s, p = STRESS
     check_full_size(dw, gpu, STRESS)
@@ -472,6 +510,10 @@ HALF_SHAPES = [(2, 6, 14, 14, 3, 1, 1), (2, 5, 28, 28, 5, 2, 2), (2, 4, 56, 56, 
                (1, 8, 7, 7, 5, 1, 2), (2, 4, 112, 112, 3, 2, 1), (1, 2, 33, 35, 7, 1, 3), (2, 8, 14, 14, 5, 2, 2),
                (3, 4, 28, 28, 7, 1, 3), (2, 8, 7, 7, 7, 1, 3), (2, 3, 64, 64, 5, 2, 2), (2, 3, 40, 44, 7, 2, 3),
                (3, 5, 14, 14, 7, 1, 3), (1, 3, 9, 11, 4, 2, 1),
+               # whole-plane kernels, other widths (exact 8/16/32, ragged classes)
+               (2, 8, 8, 8, 5, 1, 2), (2, 6, 16, 16, 3, 1, 1), (2, 4, 32, 32, 5, 2, 2), (2, 8, 15, 15, 5, 1, 2),
+               (2, 8, 15, 15, 3, 2, 1), (2, 4, 30, 30, 7, 1, 3), (2, 4, 20, 12, 3, 1, 1), (3, 5, 15, 15, 5, 1, 2),
+               (3, 3, 31, 31, 3, 2, 1),
                # rows of at least 96 elements in whole groups of eight: the kernels with 16-bit LDS images and
                # two-element dot products (7-row and 4-row blocks, several planes per workgroup, odd heights)
                (1, 3, 96, 104, 3, 1, 1), (1, 2, 100, 96, 5, 1, 2), (1, 2, 98, 112, 7, 1, 3), (1, 2, 97, 120, 5, 2, 2),
