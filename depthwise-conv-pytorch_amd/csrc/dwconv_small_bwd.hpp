@@ -20,9 +20,10 @@ namespace dwconv {
 
 namespace {
 
-// float4s per lane that hold one run (the planes of a wavefront's channels in one image): 1792 floats up to 28
-// columns (two 28 x 28 planes), 2048 beyond (two 32 x 32 planes)
-constexpr int run_regs(int w) { return w > 28 ? 8 : 7; }
+// float4s per lane that hold one run (the planes of a wavefront's channels in one image): 1792 floats for the
+// 7-, 14- and 28-wide instances (nine 14 x 14 planes, two 28 x 28 ones), 2048 for the others (eight 16 x 16 or
+// 15 x 15 planes, two 32 x 32 ones)
+constexpr int run_regs(int w) { return (w == 7 || w == 14 || w == 28) ? 7 : 8; }
 constexpr int run_floats(int w) { return run_regs(w) * kWave * 4; }
 constexpr int kSmallRedPitch = kWave + 1;
 
@@ -38,6 +39,7 @@ struct SmallBwdPlan {
     int pad_h;
     int planes_per_run;  // channels per wavefront
     int g_off;           // float offset of the gy run's span in LDS (a multiple of four)
+    int zero_off;        // float offset of the row of zeros in LDS (a multiple of four)
     int lanes_per_plane;
     unsigned lpp_magic;
     int chunks, images_per_chunk;
@@ -68,8 +70,11 @@ __device__ __forceinline__ void run_commit(const IO *__restrict__ g, float *lds,
 }
 
 // PF: the runs of the next image are fetched into registers while the current image is processed
-// (56 registers in fp32, 28 for 16-bit elements; dropped for the fp32 7x7 filter, whose sums and taps already take 98).
-template <typename IO, int W, bool RAG, int K, int S, int BH, bool GX, bool PF = (K < 7 || sizeof(IO) == 2)>
+// (56-64 registers in fp32, half for 16-bit elements; dropped for the fp32 7x7 filter, whose sums and taps already
+// take 98, and for fp32 rows beyond 28 elements, whose row registers do: with it the 32-wide 5x5 instance needs 280
+// registers, one wavefront per SIMD).
+template <typename IO, int W, bool RAG, int K, int S, int BH, bool GX,
+          bool PF = (sizeof(IO) == 2 || (K < 7 && W <= 28))>
 __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -92,6 +97,8 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
     const int nx = nplanes * in_plane, ng = nplanes * out_plane;
     float *lds_x = lds;
     float *lds_g = lds + p.g_off;
+    const float *zrow = lds + p.zero_off;  // stands in for the rows above and below a plane (cleared before the first barrier)
+    clear_zero_row<W>(lds + p.zero_off);
 
     const int pl_raw = fast_div(threadIdx.x, p.lpp_magic);
     const int rb = threadIdx.x - pl_raw * p.lanes_per_plane;
@@ -141,28 +148,19 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
 #pragma unroll
             for (int b = 0; b < BH; ++b) {
                 const bool ok = active && oy0 + b < p.out_h;
-                float raw[OW];
-                lds_load_row_w<OW, RAG>(lds_g + hg + pl * out_plane + (ok ? oy0 + b : 0) * w_out, raw);
-                mask_row<OW, RAG>(raw, g[b], ok, w_out);
+                lds_load_row_w<OW, RAG>(ok ? lds_g + hg + pl * out_plane + (oy0 + b) * w_out : zrow, g[b], w_out);
             }
             const float *plane = lds_x + hx + pl * in_plane;
             // rows are read one ahead of their use and the sums pinned after every row (see pin_registers)
+            auto row_at = [&](int iy) { return static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h) ? plane + iy * w_in : zrow; };
             float nxt[W];
-            bool nxt_ok;
-            {
-                const int iy = oy0 * S - p.pad_h;
-                nxt_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
-                lds_load_row_w<W, RAG>(plane + (nxt_ok ? iy : 0) * w_in, nxt);
-            }
+            lds_load_row_w<W, RAG>(row_at(oy0 * S - p.pad_h), nxt, w_in);
 #pragma unroll
             for (int wr = 0; wr < WIN_ROWS; ++wr) {
                 float row[W];
-                mask_row<W, RAG>(nxt, row, nxt_ok, w_in);
-                if (wr + 1 < WIN_ROWS) {
-                    const int iy = oy0 * S - p.pad_h + wr + 1;
-                    nxt_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
-                    lds_load_row_w<W, RAG>(plane + (nxt_ok ? iy : 0) * w_in, nxt);
-                }
+#pragma unroll
+                for (int i = 0; i < W; ++i) row[i] = nxt[i];
+                if (wr + 1 < WIN_ROWS) lds_load_row_w<W, RAG>(row_at(oy0 * S - p.pad_h + wr + 1), nxt, w_in);
 #pragma unroll
                 for (int b = 0; b < BH; ++b) {
                     const int ty = wr - b * S;
@@ -189,24 +187,17 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
 #pragma unroll
                 for (int o = 0; o < W; ++o) xacc[b][o] = 0.f;
             const float *gplane = lds_g + hg + pl * out_plane;
+            auto grow_at = [&](int gyr) { return static_cast<unsigned>(gyr) < static_cast<unsigned>(p.out_h) ? gplane + gyr * w_out : zrow; };
             if constexpr (S == 1) {
                 // gx[iy,ix] = sum_{ty,tx} gy[iy - PW + ty, ix - PW + tx] * rot[ty,tx]   (out extent == in extent)
                 float nxt[OW];
-                bool nxt_ok;
-                {
-                    const int gyr = oy0 - PW;
-                    nxt_ok = static_cast<unsigned>(gyr) < static_cast<unsigned>(p.out_h);
-                    lds_load_row_w<OW, RAG>(gplane + (nxt_ok ? gyr : 0) * w_out, nxt);
-                }
+                lds_load_row_w<OW, RAG>(grow_at(oy0 - PW), nxt, w_out);
 #pragma unroll
                 for (int wr = 0; wr < BH - 1 + K; ++wr) {
                     float row[OW];
-                    mask_row<OW, RAG>(nxt, row, nxt_ok, w_out);
-                    if (wr + 1 < BH - 1 + K) {
-                        const int gyr = oy0 - PW + wr + 1;
-                        nxt_ok = static_cast<unsigned>(gyr) < static_cast<unsigned>(p.out_h);
-                        lds_load_row_w<OW, RAG>(gplane + (nxt_ok ? gyr : 0) * w_out, nxt);
-                    }
+#pragma unroll
+                    for (int i = 0; i < OW; ++i) row[i] = nxt[i];
+                    if (wr + 1 < BH - 1 + K) lds_load_row_w<OW, RAG>(grow_at(oy0 - PW + wr + 1), nxt, w_out);
 #pragma unroll
                     for (int b = 0; b < BH; ++b) {
                         const int ty = wr - b;
@@ -228,21 +219,13 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
                 constexpr int M = (PW + E) / 2;
                 constexpr int KA = (K + E + 1) / 2;
                 float nxt[OW];
-                bool nxt_ok;
-                {
-                    const int gyr = rb - M;
-                    nxt_ok = static_cast<unsigned>(gyr) < static_cast<unsigned>(p.out_h);
-                    lds_load_row_w<OW, RAG>(gplane + (nxt_ok ? gyr : 0) * w_out, nxt);
-                }
+                lds_load_row_w<OW, RAG>(grow_at(rb - M), nxt, w_out);
 #pragma unroll
                 for (int wr = 0; wr < KA + 1; ++wr) {
                     float row[OW];
-                    mask_row<OW, RAG>(nxt, row, nxt_ok, w_out);
-                    if (wr + 1 < KA + 1) {
-                        const int gyr = rb - M + wr + 1;
-                        nxt_ok = static_cast<unsigned>(gyr) < static_cast<unsigned>(p.out_h);
-                        lds_load_row_w<OW, RAG>(gplane + (nxt_ok ? gyr : 0) * w_out, nxt);
-                    }
+#pragma unroll
+                    for (int i = 0; i < OW; ++i) row[i] = nxt[i];
+                    if (wr + 1 < KA + 1) lds_load_row_w<OW, RAG>(grow_at(rb - M + wr + 1), nxt, w_out);
 #pragma unroll
                     for (int r = 0; r < 2; ++r) {
                         const int a = wr - r;
@@ -344,7 +327,8 @@ long small_bwd_case(int mode, const SmallBwdArgs &a, const WgradGeometry &g, hip
     p.gx = a.gx;
     p.partial = static_cast<float *>(a.ws);
     // (ragged rows are read up to W - 1 floats past their end: spare floats behind the gy run)
-    const size_t runs = (static_cast<size_t>(p.g_off) + p.planes_per_run * g.out_h * g.out_w + 4 + (RAG ? W : 0)) * 4;
+    p.zero_off = round_up(p.g_off + p.planes_per_run * g.out_h * g.out_w + 4 + (RAG ? W : 0), 4);
+    const size_t runs = static_cast<size_t>(p.zero_off + zero_row_floats(W)) * 4;
     const size_t red = static_cast<size_t>(K) * K * kSmallRedPitch * 4;
     const size_t shmem = runs > red ? runs : red;
     const int groups = ceil_div(g.channel, p.planes_per_run);

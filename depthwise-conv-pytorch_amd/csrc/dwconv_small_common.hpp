@@ -31,6 +31,7 @@ struct SmallPlan {
     int planes_per_run;    // P
     int lanes_per_plane;   // LPP
     unsigned lpp_magic;
+    int zero_off;          // float offset of the row of zeros in LDS (a multiple of four)
     Epilogue epi;          // forward kernels: applied to every sum before it is stored
 };
 
@@ -94,26 +95,33 @@ __device__ __forceinline__ void lds_store_row(float *p, const float *r)
 }
 
 // Width-aware forms.  RAG = false: the row is exactly N elements.  RAG = true: N is a capacity and the real width
-// (1..N, uniform) comes at run time: a row starts anywhere, so it is read element by element, up to N - 1 floats past
-// its end (the LDS allocation of a ragged kernel ends with N spare floats), and what was read past the real width is
-// dropped by mask_row.
+// (N - 7 .. N, uniform) comes at run time: a row starts anywhere, so it is read element by element, up to N - 1 floats
+// past its end (the LDS allocation of a ragged kernel ends with N spare floats), and what was read past the real
+// width is replaced by zero (a select under a wavefront-uniform condition, and only for the last seven columns:
+// a capacity class spans eight widths).
+//
+// Rows above or below the plane are not masked element by element: every kernel keeps a row of zeros in LDS
+// (zero_row_floats(W) floats, cleared by clear_zero_row) and points the read at it instead, one select on the address.
 template <int N, bool RAG>
-__device__ __forceinline__ void lds_load_row_w(const float *p, float (&r)[N])
+__device__ __forceinline__ void lds_load_row_w(const float *p, float (&r)[N], int w)
 {
     if constexpr (RAG) {
 #pragma unroll
         for (int i = 0; i < N; ++i) r[i] = p[i];
+#pragma unroll
+        for (int i = (N > 7 ? N - 7 : 0); i < N; ++i) r[i] = i < w ? r[i] : 0.f;
     } else {
         lds_load_row<N>(p, r);
     }
 }
 
-// dst = src where the lane's row exists (`ok`) and, for ragged widths, the column does (i < w); zero elsewhere.
-template <int N, bool RAG>
-__device__ __forceinline__ void mask_row(const float (&src)[N], float (&dst)[N], bool ok, int w)
+constexpr int zero_row_floats(int w) { return (w + 3) / 4 * 4 + 4; }
+
+template <int W>
+__device__ __forceinline__ void clear_zero_row(float *zrow)
 {
-#pragma unroll
-    for (int i = 0; i < N; ++i) dst[i] = (ok && (!RAG || i < w)) ? src[i] : 0.f;
+    static_assert(zero_row_floats(W) / 4 <= kWave, "one float4 per lane");
+    if (threadIdx.x < zero_row_floats(W) / 4) reinterpret_cast<float4 *>(zrow)[threadIdx.x] = make_float4(0.f, 0.f, 0.f, 0.f);
 }
 
 template <int N, bool RAG>

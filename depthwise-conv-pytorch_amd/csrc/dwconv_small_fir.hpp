@@ -59,6 +59,8 @@ __global__ __launch_bounds__(kWave) void small_down_kernel(const SmallPlan p)
     float tapv[K * K];
     load_taps<K * K, FLIP>(static_cast<const IO *>(p.taps), static_cast<int>((plane0 + pl) % p.channel), tapv);
     run_to_lds(static_cast<const IO *>(p.in) + (in0 - hin), lds, nplanes * in_plane + hin);
+    const float *zrow = lds + p.zero_off;  // stands in for the rows above and below the plane
+    clear_zero_row<W>(lds + p.zero_off);
     __syncthreads();
 
     float acc[BH][OW];
@@ -70,22 +72,15 @@ __global__ __launch_bounds__(kWave) void small_down_kernel(const SmallPlan p)
     const int oy0 = rb * BH;
     const float *plane = lds + hin + pl * in_plane;
     // rows are read one ahead of their use and the sums pinned after every row (see pin_registers)
+    auto row_at = [&](int iy) { return static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h) ? plane + iy * w_in : zrow; };
     float nxt[W];
-    bool nxt_ok;
-    {
-        const int iy = oy0 * S - p.pad_h;
-        nxt_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
-        lds_load_row_w<W, RAG>(plane + (nxt_ok ? iy : 0) * w_in, nxt);
-    }
+    lds_load_row_w<W, RAG>(row_at(oy0 * S - p.pad_h), nxt, w_in);
 #pragma unroll
     for (int wr = 0; wr < WIN_ROWS; ++wr) {
         float row[W];
-        mask_row<W, RAG>(nxt, row, nxt_ok, w_in);
-        if (wr + 1 < WIN_ROWS) {
-            const int iy = oy0 * S - p.pad_h + wr + 1;
-            nxt_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
-            lds_load_row_w<W, RAG>(plane + (nxt_ok ? iy : 0) * w_in, nxt);
-        }
+#pragma unroll
+        for (int i = 0; i < W; ++i) row[i] = nxt[i];
+        if (wr + 1 < WIN_ROWS) lds_load_row_w<W, RAG>(row_at(oy0 * S - p.pad_h + wr + 1), nxt, w_in);
 #pragma unroll
         for (int b = 0; b < BH; ++b) {
             const int ty = wr - b * S;
@@ -149,6 +144,8 @@ __global__ __launch_bounds__(kWave) void small_up2_kernel(const SmallPlan p)
     float tapv[K * K];
     load_taps<K * K, true>(static_cast<const IO *>(p.taps), static_cast<int>((plane0 + pl) % p.channel), tapv);
     run_to_lds(static_cast<const IO *>(p.in) + (in0 - hin), lds, nplanes * in_plane + hin);
+    const float *zrow = lds + p.zero_off;  // stands in for the rows above and below the plane
+    clear_zero_row<W>(lds + p.zero_off);
     __syncthreads();
 
     float acc[2][OW];
@@ -158,22 +155,15 @@ __global__ __launch_bounds__(kWave) void small_up2_kernel(const SmallPlan p)
         for (int o = 0; o < OW; ++o) acc[r][o] = 0.f;
 
     const float *plane = lds + hin + pl * in_plane;
+    auto row_at = [&](int iy) { return static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h) ? plane + iy * w_in : zrow; };
     float nxt[W];
-    bool nxt_ok;
-    {
-        const int iy = q - p.pad_h;
-        nxt_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
-        lds_load_row_w<W, RAG>(plane + (nxt_ok ? iy : 0) * w_in, nxt);
-    }
+    lds_load_row_w<W, RAG>(row_at(q - p.pad_h), nxt, w_in);
 #pragma unroll
     for (int wr = 0; wr < WIN_ROWS; ++wr) {
         float row[W];
-        mask_row<W, RAG>(nxt, row, nxt_ok, w_in);
-        if (wr + 1 < WIN_ROWS) {
-            const int iy = q - p.pad_h + wr + 1;
-            nxt_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h);
-            lds_load_row_w<W, RAG>(plane + (nxt_ok ? iy : 0) * w_in, nxt);
-        }
+#pragma unroll
+        for (int i = 0; i < W; ++i) row[i] = nxt[i];
+        if (wr + 1 < WIN_ROWS) lds_load_row_w<W, RAG>(row_at(q - p.pad_h + wr + 1), nxt, w_in);
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
             const int a = wr - r;
@@ -214,19 +204,25 @@ size_t small_lds_bytes(int planes, int in_plane, int out_plane, int spare)
     return (static_cast<size_t>(planes) * (in_plane > out_plane ? in_plane : out_plane) + 4 + spare) * 4;
 }
 
+// float offset of the row of zeros: behind the run image and the spare floats
+int small_zero_off(int planes, int in_plane, int out_plane, int spare)
+{
+    return round_up(planes * (in_plane > out_plane ? in_plane : out_plane) + 4 + spare, 4);
+}
+
 // Planes per wavefront: as many as there are lane slots within the LDS budget; when a plane is not a multiple of 4
 // elements a multiple of 4 of them if that costs less than half (every run then starts on a 4-element boundary).
 int planes_per_run(int lanes_per_plane, int in_plane, int out_plane, long planes)
 {
     int P = kWave / lanes_per_plane;
-    while (P > 0 && small_lds_bytes(P, in_plane, out_plane, 0) > 16 * 1024) --P;
+    while (P > 0 && small_lds_bytes(P, in_plane, out_plane, 0) > 16 * 1024 + 16) --P;
     if ((in_plane % 4 != 0 || out_plane % 4 != 0) && P >= 4) P -= P % 4;
     if (static_cast<long>(P) > planes && in_plane % 4 == 0 && out_plane % 4 == 0) P = static_cast<int>(planes);
     return P;
 }
 
 // Fills in the run shape of p (lanes_per_plane set); false when the geometry does not fit a wavefront.
-bool finish_plan(SmallPlan &p, size_t &shmem, long &runs, int spare)
+bool finish_plan(SmallPlan &p, size_t &shmem, long &runs, int spare, int zero_floats)
 {
     if (p.lanes_per_plane < 1 || p.lanes_per_plane > kWave) return false;
     const int in_plane = p.in_h * p.in_w, out_plane = p.out_h * p.out_w;
@@ -235,7 +231,8 @@ bool finish_plan(SmallPlan &p, size_t &shmem, long &runs, int spare)
     p.lpp_magic = magic_u16(p.lanes_per_plane);
     runs = (p.planes + p.planes_per_run - 1) / p.planes_per_run;
     if (runs > 0x7fffffffL) return false;
-    shmem = small_lds_bytes(p.planes_per_run, in_plane, out_plane, spare);
+    p.zero_off = small_zero_off(p.planes_per_run, in_plane, out_plane, spare);
+    shmem = static_cast<size_t>(p.zero_off + zero_floats) * 4;
     return true;
 }
 
@@ -245,7 +242,7 @@ int launch_small_down(SmallPlan &p, hipStream_t stream)
     p.lanes_per_plane = ceil_div(p.out_h, BH);
     size_t shmem;
     long runs;
-    if (!finish_plan(p, shmem, runs, RAG ? W : 0)) return -1;
+    if (!finish_plan(p, shmem, runs, RAG ? W : 0, zero_row_floats(W))) return -1;
     hipLaunchKernelGGL((small_down_kernel<IO, W, RAG, K, S, FLIP, BH>), dim3(static_cast<unsigned>(runs)), dim3(kWave),
                        shmem, stream, p);
     note_variant("small_down%s<%s%d,k%d,s%d,%s,bh%d> P%d", sizeof(IO) == 2 ? "16" : "", RAG ? "r" : "w", W, K, S,
@@ -259,7 +256,7 @@ int launch_small_up2(SmallPlan &p, hipStream_t stream)
     p.lanes_per_plane = ceil_div(p.out_h, 2);
     size_t shmem;
     long runs;
-    if (!finish_plan(p, shmem, runs, RAG ? W : 0)) return -1;
+    if (!finish_plan(p, shmem, runs, RAG ? W : 0, zero_row_floats(W))) return -1;
     hipLaunchKernelGGL((small_up2_kernel<IO, W, RAG, K>), dim3(static_cast<unsigned>(runs)), dim3(kWave), shmem, stream, p);
     note_variant("small_up2%s<%s%d,k%d> P%d", sizeof(IO) == 2 ? "16" : "", RAG ? "r" : "w", W, K, p.planes_per_run);
     return check_launch("small_up2_kernel");
@@ -283,7 +280,9 @@ int launch_small_down_any(SmallPlan &p, int S, bool rot, hipStream_t stream)
     if (S == 1) {
         if constexpr (W <= 8) {
             if constexpr (!RAG) {
-                if (p.planes >= 64l * 2048) { DWCONV_DOWN(W); }
+                const int bh = env_int("DWCONV_SMALL_BH8", p.planes >= 64l * 2048 ? W : 2);
+                if (bh == W) { DWCONV_DOWN(W); }
+                if (bh == 4) { DWCONV_DOWN(4); }
             }
             DWCONV_DOWN(2);
         } else if constexpr (W <= 16) {
