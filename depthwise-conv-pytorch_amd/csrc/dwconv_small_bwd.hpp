@@ -40,6 +40,7 @@ struct SmallBwdPlan {
     int planes_per_run;  // channels per wavefront
     int g_off;           // float offset of the gy run's span in LDS (a multiple of four)
     int zero_off;        // float offset of the row of zeros in LDS (a multiple of four)
+    int lds_x_floats, lds_g_floats;  // LDS images of the two runs (host side only)
     int lanes_per_plane;
     unsigned lpp_magic;
     int chunks, images_per_chunk;
@@ -55,7 +56,7 @@ __device__ __forceinline__ void run_fetch(const IO *__restrict__ g, int n, typen
     for (int u = 0; u < RR; ++u) v[u] = load4_raw<IO>(g + 4 * min(static_cast<int>(threadIdx.x) + u * kWave, n4 - 1));
 }
 
-template <typename IO, int RR>
+template <typename IO, int RR, int GPR = 0>
 __device__ __forceinline__ void run_commit(const IO *__restrict__ g, float *lds, int n,
                                            const typename Raw4<IO>::type (&v)[RR])
 {
@@ -63,18 +64,20 @@ __device__ __forceinline__ void run_commit(const IO *__restrict__ g, float *lds,
 #pragma unroll
     for (int u = 0; u < RR; ++u) {
         // slots past the end of the run hold its last group of four again (run_fetch) and rewrite it in place
-        reinterpret_cast<float4 *>(lds)[min(static_cast<int>(threadIdx.x) + u * kWave, n4 - 1)] = widen4<IO>(v[u]);
+        reinterpret_cast<float4 *>(lds)[lds_group<GPR>(min(static_cast<int>(threadIdx.x) + u * kWave, n4 - 1))] = widen4<IO>(v[u]);
     }
+    // (a run with padded rows is whole groups of four)
     const int tail = n4 * 4 + threadIdx.x;
-    if (tail < n) lds[tail] = Io<IO>::in(g[tail]);
+    if (GPR == 0 && tail < n) lds[tail] = Io<IO>::in(g[tail]);
 }
 
 // PF: the runs of the next image are fetched into registers while the current image is processed
 // (56-64 registers in fp32, half for 16-bit elements; dropped for the fp32 7x7 filter, whose sums and taps already
 // take 98, and for fp32 rows beyond 28 elements, whose row registers do: with it the 32-wide 5x5 instance needs 280
 // registers, one wavefront per SIMD).
-template <typename IO, int W, bool RAG, int K, int S, int BH, bool GX,
-          bool PF = (sizeof(IO) == 2 || (K < 7 && W <= 28))>
+// PAD: LDS rows of 8, 16 or 32 floats get four spare floats (see lds_row_pitch)
+template <typename IO, int W, bool RAG, int K, int S, int BH, bool GX, bool PAD,
+          bool PF = (sizeof(IO) == 2 || (K < 7 && (RAG || W <= 28 || K == 3)))>
 __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -93,7 +96,11 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
     const int nplanes = min(p.planes_per_run, p.channel - c0);
     const int n0 = chunk * p.images_per_chunk;
     const int n1 = min(p.batch, n0 + p.images_per_chunk);
+    // row pitch in LDS (padded for rows of 8, 16 or 32 floats, see lds_row_pitch) and the plane pitch that follows
+    constexpr int GI = PAD ? lds_row_groups(W, RAG) : 0, GO = PAD ? lds_row_groups(OW, RAG) : 0;
+    const int lp_in = GI ? lds_row_pitch(W, RAG) : w_in, lp_out = GO ? lds_row_pitch(OW, RAG) : w_out;
     const int in_plane = p.in_h * w_in, out_plane = p.out_h * w_out;
+    const int lin_plane = p.in_h * lp_in, lout_plane = p.out_h * lp_out;
     const int nx = nplanes * in_plane, ng = nplanes * out_plane;
     float *lds_x = lds;
     float *lds_g = lds + p.g_off;
@@ -133,8 +140,8 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
             run_fetch<IO, RR>(x + (x0 - hx), nx + hx, rx);
             run_fetch<IO, RR>(gy + (g0 - hg), ng + hg, rg);
         }
-        run_commit<IO, RR>(x + (x0 - hx), lds_x, nx + hx, rx);
-        run_commit<IO, RR>(gy + (g0 - hg), lds_g, ng + hg, rg);
+        run_commit<IO, RR, GI>(x + (x0 - hx), lds_x, nx + hx, rx);
+        run_commit<IO, RR, GO>(gy + (g0 - hg), lds_g, ng + hg, rg);
         __syncthreads();
         if (PF && n + 1 < n1) {
             const long x1 = (plane0 + p.channel) * in_plane, g1 = (plane0 + p.channel) * out_plane;
@@ -148,11 +155,11 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
 #pragma unroll
             for (int b = 0; b < BH; ++b) {
                 const bool ok = active && oy0 + b < p.out_h;
-                lds_load_row_w<OW, RAG>(ok ? lds_g + hg + pl * out_plane + (oy0 + b) * w_out : zrow, g[b], w_out);
+                lds_load_row_w<OW, RAG>(ok ? lds_g + hg + pl * lout_plane + (oy0 + b) * lp_out : zrow, g[b], w_out);
             }
-            const float *plane = lds_x + hx + pl * in_plane;
+            const float *plane = lds_x + hx + pl * lin_plane;
             // rows are read one ahead of their use and the sums pinned after every row (see pin_registers)
-            auto row_at = [&](int iy) { return static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h) ? plane + iy * w_in : zrow; };
+            auto row_at = [&](int iy) { return static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h) ? plane + iy * lp_in : zrow; };
             float nxt[W];
             lds_load_row_w<W, RAG>(row_at(oy0 * S - p.pad_h), nxt, w_in);
 #pragma unroll
@@ -186,8 +193,8 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
             for (int b = 0; b < XR; ++b)
 #pragma unroll
                 for (int o = 0; o < W; ++o) xacc[b][o] = 0.f;
-            const float *gplane = lds_g + hg + pl * out_plane;
-            auto grow_at = [&](int gyr) { return static_cast<unsigned>(gyr) < static_cast<unsigned>(p.out_h) ? gplane + gyr * w_out : zrow; };
+            const float *gplane = lds_g + hg + pl * lout_plane;
+            auto grow_at = [&](int gyr) { return static_cast<unsigned>(gyr) < static_cast<unsigned>(p.out_h) ? gplane + gyr * lp_out : zrow; };
             if constexpr (S == 1) {
                 // gx[iy,ix] = sum_{ty,tx} gy[iy - PW + ty, ix - PW + tx] * rot[ty,tx]   (out extent == in extent)
                 float nxt[OW];
@@ -249,14 +256,14 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
             }
             __syncthreads();  // every lane is done with the x run: overwrite it with the gx run
             if (active) {
-                float *dst = lds_x + hx + pl * in_plane;
+                float *dst = lds_x + hx + pl * lin_plane;
                 const int row0 = S == 1 ? oy0 : 2 * rb;
 #pragma unroll
                 for (int b = 0; b < XR; ++b)
-                    if (row0 + b < p.in_h) lds_store_row_w<W, RAG>(dst + (row0 + b) * w_in, xacc[b], w_in);
+                    if (row0 + b < p.in_h) lds_store_row_w<W, RAG>(dst + (row0 + b) * lp_in, xacc[b], w_in);
             }
             __syncthreads();
-            lds_to_run(static_cast<IO *>(p.gx) + (x0 - hx), lds_x, nx + hx, hx);
+            lds_to_run<IO, GI>(static_cast<IO *>(p.gx) + (x0 - hx), lds_x, nx + hx, hx);
         }
     }
 
@@ -273,9 +280,10 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
     }
 }
 
-template <int W, int K, int S, int BH>
+template <int W, bool RAG, int K, int S, int BH, bool PAD>
 bool plan_small_bwd(SmallBwdPlan &p, const WgradGeometry &g)
 {
+    constexpr int OW = (W - 1) / S + 1;
     p.batch = g.batch;
     p.channel = g.channel;
     p.in_h = g.in_h;
@@ -298,7 +306,10 @@ bool plan_small_bwd(SmallBwdPlan &p, const WgradGeometry &g)
     if (P < 1) return false;
     if (in_plane < 4 || out_plane < 4) return false;
     p.planes_per_run = P;
-    p.g_off = round_up(P * in_plane + head, 4);
+    // LDS images: rows at their LDS pitch
+    p.lds_x_floats = P * g.in_h * ((PAD && lds_row_groups(W, RAG)) ? lds_row_pitch(W, RAG) : g.in_w);
+    p.lds_g_floats = P * g.out_h * ((PAD && lds_row_groups(OW, RAG)) ? lds_row_pitch(OW, RAG) : g.out_w);
+    p.g_off = round_up(p.lds_x_floats + head, 4);
     p.lpp_magic = magic_u16(p.lanes_per_plane);
     const int groups = ceil_div(g.channel, P);
     // At these register counts two wavefronts fit a SIMD, 2048 the device: the grid stays within that one resident
@@ -312,11 +323,11 @@ bool plan_small_bwd(SmallBwdPlan &p, const WgradGeometry &g)
     return true;
 }
 
-template <typename IO, int W, bool RAG, int K, int S, int BH>
+template <typename IO, int W, bool RAG, int K, int S, int BH, bool PAD>
 long small_bwd_case(int mode, const SmallBwdArgs &a, const WgradGeometry &g, hipStream_t stream)
 {
     SmallBwdPlan p{};
-    if (!plan_small_bwd<W, K, S, BH>(p, g)) return -1;
+    if (!plan_small_bwd<W, RAG, K, S, BH, PAD>(p, g)) return -1;
     const size_t need = static_cast<size_t>(g.channel) * p.chunks * K * K * sizeof(float);
     if (mode == 0) return static_cast<long>(need);
     if (a.ws == nullptr || a.ws_bytes < need)
@@ -327,19 +338,19 @@ long small_bwd_case(int mode, const SmallBwdArgs &a, const WgradGeometry &g, hip
     p.gx = a.gx;
     p.partial = static_cast<float *>(a.ws);
     // (ragged rows are read up to W - 1 floats past their end: spare floats behind the gy run)
-    p.zero_off = round_up(p.g_off + p.planes_per_run * g.out_h * g.out_w + 4 + (RAG ? W : 0), 4);
+    p.zero_off = round_up(p.g_off + p.lds_g_floats + 4 + (RAG ? W : 0), 4);
     const size_t runs = static_cast<size_t>(p.zero_off + zero_row_floats(W)) * 4;
     const size_t red = static_cast<size_t>(K) * K * kSmallRedPitch * 4;
     const size_t shmem = runs > red ? runs : red;
     const int groups = ceil_div(g.channel, p.planes_per_run);
     if (mode == 2)
-        hipLaunchKernelGGL((small_bwd_kernel<IO, W, RAG, K, S, BH, true>), dim3(groups * p.chunks), dim3(kWave), shmem, stream, p);
+        hipLaunchKernelGGL((small_bwd_kernel<IO, W, RAG, K, S, BH, true, PAD>), dim3(groups * p.chunks), dim3(kWave), shmem, stream, p);
     else
-        hipLaunchKernelGGL((small_bwd_kernel<IO, W, RAG, K, S, BH, false>), dim3(groups * p.chunks), dim3(kWave), shmem, stream, p);
+        hipLaunchKernelGGL((small_bwd_kernel<IO, W, RAG, K, S, BH, false, PAD>), dim3(groups * p.chunks), dim3(kWave), shmem, stream, p);
     const int rc = check_launch("small_bwd_kernel");
     if (rc != DWCONV_OK) return rc;
-    note_variant("%s%s<%s%d,k%d,s%d,bh%d> P%d chunks%d", mode == 2 ? "small_bwd" : "small_wgrad",
-                 sizeof(IO) == 2 ? "16" : "", RAG ? "r" : "w", W, K, S, BH, p.planes_per_run, p.chunks);
+    note_variant("%s%s<%s%d,k%d,s%d,bh%d%s> P%d chunks%d", mode == 2 ? "small_bwd" : "small_wgrad",
+                 sizeof(IO) == 2 ? "16" : "", RAG ? "r" : "w", W, K, S, BH, PAD ? ",pad" : "", p.planes_per_run, p.chunks);
     return launch_wgrad_final(p.partial, static_cast<IO *>(a.gw), g.channel, K * K, p.chunks, stream);
 }
 
@@ -351,8 +362,12 @@ template <typename IO, int W, bool RAG, int K>
 long small_bwd_s(int mode, const SmallBwdArgs &a, const WgradGeometry &g, hipStream_t stream)
 {
     constexpr int BH1 = W <= 8 ? ((sizeof(IO) == 4 && K >= 5) ? 2 : 4) : (W <= 16 ? 2 : 1);
-    if (g.down_h == 1) return small_bwd_case<IO, W, RAG, K, 1, BH1>(mode, a, g, stream);
-    if (g.down_h == 2) return small_bwd_case<IO, W, RAG, K, 2, 1>(mode, a, g, stream);
+    // LDS rows padded where the measurements say so: 32-wide maps (5x5 C=240 115 -> 80 us, 3x3 stride 2 80 -> 54) and
+    // 16-wide ones at stride 2 (one row per lane: 47.5 -> 42.6 us); 16-wide stride 1 (two rows per lane) and 8-wide
+    // maps did not change
+    constexpr bool PAD1 = !RAG && W == 32, PAD2 = !RAG && (W == 32 || W == 16);
+    if (g.down_h == 1) return small_bwd_case<IO, W, RAG, K, 1, BH1, PAD1>(mode, a, g, stream);
+    if (g.down_h == 2) return small_bwd_case<IO, W, RAG, K, 2, 1, PAD2>(mode, a, g, stream);
     return -1;
 }
 

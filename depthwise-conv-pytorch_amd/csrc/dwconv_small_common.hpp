@@ -115,7 +115,25 @@ __device__ __forceinline__ void lds_load_row_w(const float *p, float (&r)[N], in
     }
 }
 
-constexpr int zero_row_floats(int w) { return (w + 3) / 4 * 4 + 4; }
+constexpr int zero_row_floats(int w) { return (w + 3) / 4 * 4 + 8; }
+
+// LDS pitch of a row of n elements.  Lanes sit one or a few rows apart; rows of 8, 16 or 32 floats put them a power
+// of two apart and onto two or four of the 64 banks (row reads of a 32 x 32 plane then take eight times their
+// conflict-free time, and the LDS, not the vector unit, bounds the kernel), so exact instances give such rows four
+// spare floats: lane strides of 12, 20 and 36 floats spread 128-bit reads over all banks.  The flat copies between
+// memory and LDS then skip one group of four after every n / 4 (a shift: lds_group below).  Ragged rows keep the
+// pitch they have in memory.
+constexpr int lds_row_pitch(int n, bool rag) { return (!rag && (n == 8 || n == 16 || n == 32)) ? n + 4 : n; }
+// groups of four per memory row when the LDS rows are padded, else 0
+constexpr int lds_row_groups(int n, bool rag) { return lds_row_pitch(n, rag) != n ? n / 4 : 0; }
+
+// LDS group index of group i of a flat run; GPR = groups of four per row where rows are padded (a power of two), else 0
+template <int GPR>
+__device__ __forceinline__ int lds_group(int i)
+{
+    if constexpr (GPR == 0) return i;
+    else return i + i / GPR;
+}
 
 template <int W>
 __device__ __forceinline__ void clear_zero_row(float *zrow)
@@ -142,7 +160,7 @@ __device__ __forceinline__ void lds_store_row_w(float *p, const float *r, int w)
 // Loads are issued kRunBatch at a time before any of them is consumed, so their latencies overlap.
 constexpr int kRunBatch = 8;
 
-template <typename IO>
+template <typename IO, int GPR = 0>
 __device__ __forceinline__ void run_to_lds(const IO *__restrict__ g, float *lds, int n)
 {
     const int n4 = n >> 2;
@@ -154,10 +172,11 @@ __device__ __forceinline__ void run_to_lds(const IO *__restrict__ g, float *lds,
         for (int u = 0; u < kRunBatch; ++u)
             v[u] = load4<IO>(g + 4 * min(base + u * kWave, n4 - 1));
 #pragma unroll
-        for (int u = 0; u < kRunBatch; ++u) reinterpret_cast<float4 *>(lds)[min(base + u * kWave, n4 - 1)] = v[u];
+        for (int u = 0; u < kRunBatch; ++u) reinterpret_cast<float4 *>(lds)[lds_group<GPR>(min(base + u * kWave, n4 - 1))] = v[u];
     }
+    // (a run with padded rows is whole groups of four)
     const int tail = n4 * 4 + threadIdx.x;
-    if (tail < n) lds[tail] = Io<IO>::in(g[tail]);
+    if (GPR == 0 && tail < n) lds[tail] = Io<IO>::in(g[tail]);
 }
 
 // Two runs at once (grad-weight: x and gy of the same planes): all loads of a batch of both runs fly together.
@@ -190,7 +209,7 @@ __device__ __forceinline__ void runs_to_lds(const IO *__restrict__ ga, float *la
 // `g` points at that boundary, `n` counts the head too, and the run's first element sits at lds[head].  Loading such a
 // span reads up to three elements of the neighbouring run (harmless); storing it must not write them: the first
 // group of four goes out element by element, from `head` on.
-template <typename IO>
+template <typename IO, int GPR = 0>
 __device__ __forceinline__ void lds_to_run(IO *__restrict__ g, const float *lds, int n, int head = 0)
 {
     const int n4 = n >> 2;
@@ -199,7 +218,7 @@ __device__ __forceinline__ void lds_to_run(IO *__restrict__ g, const float *lds,
     for (int base = threadIdx.x; base < n4; base += kWave * U) {
         float4 v[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) v[u] = reinterpret_cast<const float4 *>(lds)[min(base + u * kWave, n4 - 1)];
+        for (int u = 0; u < U; ++u) v[u] = reinterpret_cast<const float4 *>(lds)[lds_group<GPR>(min(base + u * kWave, n4 - 1))];
         // branch-free: groups past the end of the run store out of range of the view and are dropped
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -208,10 +227,12 @@ __device__ __forceinline__ void lds_to_run(IO *__restrict__ g, const float *lds,
             view_store4<IO>(view, whole ? i * 4u * static_cast<unsigned>(sizeof(IO)) : kOob, v[u].x, v[u].y, v[u].z, v[u].w);
         }
     }
-    const int t = threadIdx.x;
-    if (head != 0 && n4 > 0 && t >= head && t < 4) g[t] = Io<IO>::out(lds[t]);
-    const int tail = n4 * 4 + t;
-    if (tail < n && tail >= head) g[tail] = Io<IO>::out(lds[tail]);
+    if constexpr (GPR == 0) {
+        const int t = threadIdx.x;
+        if (head != 0 && n4 > 0 && t >= head && t < 4) g[t] = Io<IO>::out(lds[t]);
+        const int tail = n4 * 4 + t;
+        if (tail < n && tail >= head) g[tail] = Io<IO>::out(lds[tail]);
+    }
 }
 
 // This lane's K*K taps straight from global memory (the lanes of one plane read the same addresses).

@@ -262,9 +262,12 @@ int launch_small_up2(SmallPlan &p, hipStream_t stream)
     return check_launch("small_up2_kernel");
 }
 
-// Rows per lane.  Measured on the 7-, 14- and 28-wide maps and carried over to their neighbours:
-//  * up to 8 wide: a lane takes a whole plane (64 planes per wavefront) when there are enough planes to fill the
-//    device that way, otherwise two rows (four lanes per plane);
+// Rows per lane, measured per width (fp32, batch 128 unless said):
+//  * 7 wide: 3x3 filters a whole plane per lane (64 planes per wavefront) when there are enough planes to fill the
+//    device that way, otherwise two rows; 5x5 and 7x7 filters four rows (C=1152 5x5 17.0 -> 14.8 us; N=256 C=1024
+//    7x7 30.0 -> 27.4; two rows 17.4 / 30.0);
+//  * 8 wide: four rows with 3x3 filters, two with larger ones (C=1152: whole planes 19.0 / 23.2 us, four rows
+//    16.0 / 18.9, two rows 16.4 / 17.4);
 //  * up to 16 wide: one row per lane (twice the lanes per plane, half the planes per wavefront, 80 instead of 140
 //    registers) for fp32 with 3x3 and 5x5 filters (1-2 us per layer), two rows with 7x7 filters or 16-bit
 //    elements (one row loses 1-3 us there);
@@ -279,12 +282,14 @@ int launch_small_down_any(SmallPlan &p, int S, bool rot, hipStream_t stream)
                : launch_small_down<IO, W, RAG, K, 1, false, BHV>(p, stream)
     if (S == 1) {
         if constexpr (W <= 8) {
-            if constexpr (!RAG) {
-                const int bh = env_int("DWCONV_SMALL_BH8", p.planes >= 64l * 2048 ? W : 2);
-                if (bh == W) { DWCONV_DOWN(W); }
-                if (bh == 4) { DWCONV_DOWN(4); }
+            if constexpr (!RAG && W == 7 && K == 3) {
+                if (p.planes >= 64l * 2048) { DWCONV_DOWN(7); }
             }
-            DWCONV_DOWN(2);
+            if constexpr (!RAG && ((W == 7 && K >= 5) || (W == 8 && K == 3))) {
+                DWCONV_DOWN(4);
+            } else {
+                DWCONV_DOWN(2);
+            }
         } else if constexpr (W <= 16) {
             const bool one_row = sizeof(IO) == 4 && K <= 5;
             if (env_int("DWCONV_SMALL_BH", one_row ? 1 : 2) == 1) { DWCONV_DOWN(1); }
