@@ -50,6 +50,7 @@ WORKLOADS = {
     # other input resolutions: 256 -> maps 128, 64, 32, 16, 8; 240 (EfficientNet-B1's) -> 120, 60, 30, 15, 8
     "effnet_b0_256": lambda batch: effnet_at(batch, 256),
     "effnet_b0_240": lambda batch: effnet_at(batch, 240),
+    "effnet_b0_192": lambda batch: effnet_at(batch, 192),   # maps 96, 48, 24, 12, 6
     "cfg1": lambda batch: [(8, 32, 56, 56, 3, 1, 1)],
     "cfg2": lambda batch: [(16, 64, 256, 256, 5, 1, 2)],
     "cfg4": lambda batch: [(256, 1024, 7, 7, 7, 1, 3), (128, 512, 14, 14, 7, 1, 3)],

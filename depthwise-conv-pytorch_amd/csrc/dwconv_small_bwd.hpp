@@ -41,6 +41,9 @@ struct SmallBwdPlan {
     int g_off;           // float offset of the gy run's span in LDS (a multiple of four)
     int zero_off;        // float offset of the row of zeros in LDS (a multiple of four)
     int lds_x_floats, lds_g_floats;  // LDS images of the two runs (host side only)
+    int lds_x_off;       // float offset of the x run's span (0)
+    int lp_in, lp_out;   // ragged instances: LDS row pitch of the x / gy rows (width | 1)
+    unsigned magic_in, magic_out;  // ... and the reciprocals for padded_index (0: pitch == width, flat copies)
     int lanes_per_plane;
     unsigned lpp_magic;
     int chunks, images_per_chunk;
@@ -75,6 +78,25 @@ __device__ __forceinline__ void run_commit(const IO *__restrict__ g, float *lds,
 // (56-64 registers in fp32, half for 16-bit elements; dropped for the fp32 7x7 filter, whose sums and taps already
 // take 98, and for fp32 rows beyond 28 elements, whose row registers do: with it the 32-wide 5x5 instance needs 280
 // registers, one wavefront per SIMD).
+// The same for rows at pitch width + 1 in LDS (ragged even widths; see run_to_lds_rows).
+template <typename IO, int RR>
+__device__ __forceinline__ void run_commit_rows(const IO *__restrict__ g, float *lds, int n, int head, unsigned magic, int dump,
+                                                const typename Raw4<IO>::type (&v)[RR])
+{
+    const int n4 = n >> 2;
+#pragma unroll
+    for (int u = 0; u < RR; ++u) {
+        const float4 w = widen4<IO>(v[u]);
+        const int i = 4 * min(static_cast<int>(threadIdx.x) + u * kWave, n4 - 1) - head;
+        lds[i >= 0 ? padded_index(i, magic) : dump] = w.x;
+        lds[i + 1 >= 0 ? padded_index(i + 1, magic) : dump] = w.y;
+        lds[i + 2 >= 0 ? padded_index(i + 2, magic) : dump] = w.z;
+        lds[padded_index(i + 3, magic)] = w.w;
+    }
+    const int tail = n4 * 4 + threadIdx.x;
+    if (tail < n && tail >= head) lds[padded_index(tail - head, magic)] = Io<IO>::in(g[tail]);
+}
+
 // PAD: LDS rows of 8, 16 or 32 floats get four spare floats (see lds_row_pitch)
 template <typename IO, int W, bool RAG, int K, int S, int BH, bool GX, bool PAD,
           bool PF = (sizeof(IO) == 2 || (K < 7 && (RAG || W <= 28 || K == 3)))>
@@ -98,7 +120,9 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
     const int n1 = min(p.batch, n0 + p.images_per_chunk);
     // row pitch in LDS (padded for rows of 8, 16 or 32 floats, see lds_row_pitch) and the plane pitch that follows
     constexpr int GI = PAD ? lds_row_groups(W, RAG) : 0, GO = PAD ? lds_row_groups(OW, RAG) : 0;
-    const int lp_in = GI ? lds_row_pitch(W, RAG) : w_in, lp_out = GO ? lds_row_pitch(OW, RAG) : w_out;
+    // (ragged even widths: pitch width + 1, element-wise copies)
+    const int lp_in = RAG ? p.lp_in : (GI ? lds_row_pitch(W, RAG) : W), lp_out = RAG ? p.lp_out : (GO ? lds_row_pitch(OW, RAG) : OW);
+    const bool pad_in = RAG && p.magic_in != 0, pad_out = RAG && p.magic_out != 0;
     const int in_plane = p.in_h * w_in, out_plane = p.out_h * w_out;
     const int lin_plane = p.in_h * lp_in, lout_plane = p.out_h * lp_out;
     const int nx = nplanes * in_plane, ng = nplanes * out_plane;
@@ -140,8 +164,10 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
             run_fetch<IO, RR>(x + (x0 - hx), nx + hx, rx);
             run_fetch<IO, RR>(gy + (g0 - hg), ng + hg, rg);
         }
-        run_commit<IO, RR, GI>(x + (x0 - hx), lds_x, nx + hx, rx);
-        run_commit<IO, RR, GO>(gy + (g0 - hg), lds_g, ng + hg, rg);
+        if (pad_in) run_commit_rows<IO, RR>(x + (x0 - hx), lds_x, nx + hx, hx, p.magic_in, p.zero_off - 1 - p.lds_x_off, rx);
+        else run_commit<IO, RR, GI>(x + (x0 - hx), lds_x, nx + hx, rx);
+        if (pad_out) run_commit_rows<IO, RR>(gy + (g0 - hg), lds_g, ng + hg, hg, p.magic_out, p.zero_off - 1 - p.g_off, rg);
+        else run_commit<IO, RR, GO>(gy + (g0 - hg), lds_g, ng + hg, rg);
         __syncthreads();
         if (PF && n + 1 < n1) {
             const long x1 = (plane0 + p.channel) * in_plane, g1 = (plane0 + p.channel) * out_plane;
@@ -155,9 +181,9 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
 #pragma unroll
             for (int b = 0; b < BH; ++b) {
                 const bool ok = active && oy0 + b < p.out_h;
-                lds_load_row_w<OW, RAG>(ok ? lds_g + hg + pl * lout_plane + (oy0 + b) * lp_out : zrow, g[b], w_out);
+                lds_load_row_w<OW, RAG>(ok ? lds_g + (pad_out ? 0 : hg) + pl * lout_plane + (oy0 + b) * lp_out : zrow, g[b], w_out);
             }
-            const float *plane = lds_x + hx + pl * lin_plane;
+            const float *plane = lds_x + (pad_in ? 0 : hx) + pl * lin_plane;
             // rows are read one ahead of their use and the sums pinned after every row (see pin_registers)
             auto row_at = [&](int iy) { return static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h) ? plane + iy * lp_in : zrow; };
             float nxt[W];
@@ -193,7 +219,7 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
             for (int b = 0; b < XR; ++b)
 #pragma unroll
                 for (int o = 0; o < W; ++o) xacc[b][o] = 0.f;
-            const float *gplane = lds_g + hg + pl * lout_plane;
+            const float *gplane = lds_g + (pad_out ? 0 : hg) + pl * lout_plane;
             auto grow_at = [&](int gyr) { return static_cast<unsigned>(gyr) < static_cast<unsigned>(p.out_h) ? gplane + gyr * lp_out : zrow; };
             if constexpr (S == 1) {
                 // gx[iy,ix] = sum_{ty,tx} gy[iy - PW + ty, ix - PW + tx] * rot[ty,tx]   (out extent == in extent)
@@ -256,14 +282,15 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
             }
             __syncthreads();  // every lane is done with the x run: overwrite it with the gx run
             if (active) {
-                float *dst = lds_x + hx + pl * lin_plane;
+                float *dst = lds_x + (pad_in ? 0 : hx) + pl * lin_plane;
                 const int row0 = S == 1 ? oy0 : 2 * rb;
 #pragma unroll
                 for (int b = 0; b < XR; ++b)
                     if (row0 + b < p.in_h) lds_store_row_w<W, RAG>(dst + (row0 + b) * lp_in, xacc[b], w_in);
             }
             __syncthreads();
-            lds_to_run<IO, GI>(static_cast<IO *>(p.gx) + (x0 - hx), lds_x, nx + hx, hx);
+            if (pad_in) lds_to_run_rows(static_cast<IO *>(p.gx) + (x0 - hx), lds_x, nx + hx, hx, p.magic_in);
+            else lds_to_run<IO, GI>(static_cast<IO *>(p.gx) + (x0 - hx), lds_x, nx + hx, hx);
         }
     }
 
@@ -307,8 +334,13 @@ bool plan_small_bwd(SmallBwdPlan &p, const WgradGeometry &g)
     if (in_plane < 4 || out_plane < 4) return false;
     p.planes_per_run = P;
     // LDS images: rows at their LDS pitch
-    p.lds_x_floats = P * g.in_h * ((PAD && lds_row_groups(W, RAG)) ? lds_row_pitch(W, RAG) : g.in_w);
-    p.lds_g_floats = P * g.out_h * ((PAD && lds_row_groups(OW, RAG)) ? lds_row_pitch(OW, RAG) : g.out_w);
+    p.lp_in = RAG ? ragged_pitch(g.in_w) : g.in_w;
+    p.lp_out = RAG ? ragged_pitch(g.out_w) : g.out_w;
+    p.magic_in = RAG ? ragged_magic(g.in_w) : 0;
+    p.magic_out = RAG ? ragged_magic(g.out_w) : 0;
+    p.lds_x_off = 0;
+    p.lds_x_floats = P * g.in_h * ((PAD && lds_row_groups(W, RAG)) ? lds_row_pitch(W, RAG) : p.lp_in);
+    p.lds_g_floats = P * g.out_h * ((PAD && lds_row_groups(OW, RAG)) ? lds_row_pitch(OW, RAG) : p.lp_out);
     p.g_off = round_up(p.lds_x_floats + head, 4);
     p.lpp_magic = magic_u16(p.lanes_per_plane);
     const int groups = ceil_div(g.channel, P);

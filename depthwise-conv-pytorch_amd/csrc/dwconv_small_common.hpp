@@ -32,6 +32,8 @@ struct SmallPlan {
     int lanes_per_plane;   // LPP
     unsigned lpp_magic;
     int zero_off;          // float offset of the row of zeros in LDS (a multiple of four)
+    int lp_in, lp_out;     // ragged instances: LDS row pitch of the input / output rows (width | 1)
+    unsigned magic_in, magic_out;  // ... and the reciprocals for padded_index (0: pitch == width, flat copies)
     Epilogue epi;          // forward kernels: applied to every sum before it is stored
 };
 
@@ -121,8 +123,10 @@ constexpr int zero_row_floats(int w) { return (w + 3) / 4 * 4 + 8; }
 // of two apart and onto two or four of the 64 banks (row reads of a 32 x 32 plane then take eight times their
 // conflict-free time, and the LDS, not the vector unit, bounds the kernel), so exact instances give such rows four
 // spare floats: lane strides of 12, 20 and 36 floats spread 128-bit reads over all banks.  The flat copies between
-// memory and LDS then skip one group of four after every n / 4 (a shift: lds_group below).  Ragged rows keep the
-// pitch they have in memory.
+// memory and LDS then skip one group of four after every n / 4 (a shift: lds_group below).  Ragged rows of an
+// even width (lanes a row apart would meet on 32 / gcd(width, 64) banks with their element reads: a 24-wide map ran
+// at half the speed of a 28-wide one) are laid out at pitch width + 1: the copies between memory and LDS then go
+// element by element (row = index * magic >> 18, see padded_index); odd widths keep the flat copy.
 constexpr int lds_row_pitch(int n, bool rag) { return (!rag && (n == 8 || n == 16 || n == 32)) ? n + 4 : n; }
 // groups of four per memory row when the LDS rows are padded, else 0
 constexpr int lds_row_groups(int n, bool rag) { return lds_row_pitch(n, rag) != n ? n / 4 : 0; }
@@ -134,6 +138,15 @@ __device__ __forceinline__ int lds_group(int i)
     if constexpr (GPR == 0) return i;
     else return i + i / GPR;
 }
+
+// LDS pitch of ragged rows of w elements, and the reciprocal that finds the row of a flat index (0: no padding)
+// (from 10 columns on: on 6-wide maps the element-wise copies cost more than the conflicts, 14.1 -> 16.2 us forward
+// and 25.4 -> 30.3 backward at C=1152; 12-wide maps gain 15-25 %, 24-wide ones 45 %)
+inline bool ragged_padded(int w) { return (w & 1) == 0 && w >= 10; }
+inline int ragged_pitch(int w) { return ragged_padded(w) ? w + 1 : w; }
+inline unsigned ragged_magic(int w) { return ragged_padded(w) ? static_cast<unsigned>(((1u << 18) + w - 1) / w) : 0u; }
+// LDS index of element i (0 <= i < 8192) of a flat run of rows laid out at pitch width + 1
+__device__ __forceinline__ int padded_index(int i, unsigned magic) { return i + static_cast<int>(__umul24(i, magic) >> 18); }
 
 template <int W>
 __device__ __forceinline__ void clear_zero_row(float *zrow)
@@ -177,6 +190,59 @@ __device__ __forceinline__ void run_to_lds(const IO *__restrict__ g, float *lds,
     // (a run with padded rows is whole groups of four)
     const int tail = n4 * 4 + threadIdx.x;
     if (GPR == 0 && tail < n) lds[tail] = Io<IO>::in(g[tail]);
+}
+
+// The same for rows at pitch width + 1 in LDS (ragged even widths): element i of the run proper (the span minus its
+// `head` elements of the neighbouring run, which go to the spare float at `dump`) lands at padded_index(i).
+template <typename IO>
+__device__ __forceinline__ void run_to_lds_rows(const IO *__restrict__ g, float *lds, int n, int head, unsigned magic, int dump)
+{
+    const int n4 = n >> 2;
+    for (int base = threadIdx.x; base < n4; base += kWave * kRunBatch) {
+        float4 v[kRunBatch];
+#pragma unroll
+        for (int u = 0; u < kRunBatch; ++u)
+            v[u] = load4<IO>(g + 4 * min(base + u * kWave, n4 - 1));
+#pragma unroll
+        for (int u = 0; u < kRunBatch; ++u) {
+            const int i = 4 * min(base + u * kWave, n4 - 1) - head;
+            lds[i >= 0 ? padded_index(i, magic) : dump] = v[u].x;
+            lds[i + 1 >= 0 ? padded_index(i + 1, magic) : dump] = v[u].y;
+            lds[i + 2 >= 0 ? padded_index(i + 2, magic) : dump] = v[u].z;
+            lds[padded_index(i + 3, magic)] = v[u].w;
+        }
+    }
+    const int tail = n4 * 4 + threadIdx.x;
+    if (tail < n && tail >= head) lds[padded_index(tail - head, magic)] = Io<IO>::in(g[tail]);
+}
+
+template <typename IO>
+__device__ __forceinline__ void lds_to_run_rows(IO *__restrict__ g, const float *lds, int n, int head, unsigned magic)
+{
+    const int n4 = n >> 2;
+    constexpr int U = 4;
+    const __amdgpu_buffer_rsrc_t view = buffer_view(g, static_cast<long>(n) * sizeof(IO));
+    for (int base = threadIdx.x; base < n4; base += kWave * U) {
+        float4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = 4 * min(base + u * kWave, n4 - 1) - head;
+            v[u].x = lds[padded_index(max(i, 0), magic)];
+            v[u].y = lds[padded_index(max(i + 1, 0), magic)];
+            v[u].z = lds[padded_index(max(i + 2, 0), magic)];
+            v[u].w = lds[padded_index(i + 3, magic)];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = base + u * kWave;
+            const bool whole = i < n4 && (i > 0 || head == 0);
+            view_store4<IO>(view, whole ? i * 4u * static_cast<unsigned>(sizeof(IO)) : kOob, v[u].x, v[u].y, v[u].z, v[u].w);
+        }
+    }
+    const int t = threadIdx.x;
+    if (head != 0 && n4 > 0 && t >= head && t < 4) g[t] = Io<IO>::out(lds[padded_index(t - head, magic)]);
+    const int tail = n4 * 4 + t;
+    if (tail < n && tail >= head) g[tail] = Io<IO>::out(lds[padded_index(tail - head, magic)]);
 }
 
 // Two runs at once (grad-weight: x and gy of the same planes): all loads of a batch of both runs fly together.

@@ -46,6 +46,10 @@ __global__ __launch_bounds__(kWave) void small_down_kernel(const SmallPlan p)
     const long plane0 = static_cast<long>(blockIdx.x) * p.planes_per_run;
     const int nplanes = static_cast<int>(min(static_cast<long>(p.planes_per_run), p.planes - plane0));
     const int in_plane = p.in_h * w_in, out_plane = p.out_h * w_out;
+    // LDS row pitch: the width, or width + 1 for ragged even widths (see ragged_pitch)
+    const int lp_in = RAG ? p.lp_in : W, lp_out = RAG ? p.lp_out : OW;
+    const bool pad_in = RAG && p.magic_in != 0, pad_out = RAG && p.magic_out != 0;
+    const int lin_plane = p.in_h * lp_in, lout_plane = p.out_h * lp_out;
 
     const int pl_raw = fast_div(threadIdx.x, p.lpp_magic);
     const int rb = threadIdx.x - pl_raw * p.lanes_per_plane;
@@ -58,7 +62,10 @@ __global__ __launch_bounds__(kWave) void small_down_kernel(const SmallPlan p)
 
     float tapv[K * K];
     load_taps<K * K, FLIP>(static_cast<const IO *>(p.taps), static_cast<int>((plane0 + pl) % p.channel), tapv);
-    run_to_lds(static_cast<const IO *>(p.in) + (in0 - hin), lds, nplanes * in_plane + hin);
+    if (pad_in)
+        run_to_lds_rows(static_cast<const IO *>(p.in) + (in0 - hin), lds, nplanes * in_plane + hin, hin, p.magic_in, p.zero_off - 1);
+    else
+        run_to_lds(static_cast<const IO *>(p.in) + (in0 - hin), lds, nplanes * in_plane + hin);
     const float *zrow = lds + p.zero_off;  // stands in for the rows above and below the plane
     clear_zero_row<W>(lds + p.zero_off);
     __syncthreads();
@@ -70,9 +77,9 @@ __global__ __launch_bounds__(kWave) void small_down_kernel(const SmallPlan p)
         for (int o = 0; o < OW; ++o) acc[b][o] = 0.f;
 
     const int oy0 = rb * BH;
-    const float *plane = lds + hin + pl * in_plane;
+    const float *plane = lds + (pad_in ? 0 : hin) + pl * lin_plane;
     // rows are read one ahead of their use and the sums pinned after every row (see pin_registers)
-    auto row_at = [&](int iy) { return static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h) ? plane + iy * w_in : zrow; };
+    auto row_at = [&](int iy) { return static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h) ? plane + iy * lp_in : zrow; };
     float nxt[W];
     lds_load_row_w<W, RAG>(row_at(oy0 * S - p.pad_h), nxt, w_in);
 #pragma unroll
@@ -104,13 +111,16 @@ __global__ __launch_bounds__(kWave) void small_down_kernel(const SmallPlan p)
     __syncthreads();  // every lane has read its input rows: the run can be overwritten in place
 
     if (active) {
-        float *dst = lds + hout + pl * out_plane;
+        float *dst = lds + (pad_out ? 0 : hout) + pl * lout_plane;
 #pragma unroll
         for (int b = 0; b < BH; ++b)
-            if (oy0 + b < p.out_h) lds_store_row_w<OW, RAG>(dst + (oy0 + b) * w_out, acc[b], w_out);
+            if (oy0 + b < p.out_h) lds_store_row_w<OW, RAG>(dst + (oy0 + b) * lp_out, acc[b], w_out);
     }
     __syncthreads();
-    lds_to_run(static_cast<IO *>(p.out) + (out0 - hout), lds, nplanes * out_plane + hout, hout);
+    if (pad_out)
+        lds_to_run_rows(static_cast<IO *>(p.out) + (out0 - hout), lds, nplanes * out_plane + hout, hout, p.magic_out);
+    else
+        lds_to_run(static_cast<IO *>(p.out) + (out0 - hout), lds, nplanes * out_plane + hout, hout);
 }
 
 // up = 2, taps rotated, "same" padding of the forward conv (leading pad of the transposed problem = K/2):
@@ -132,6 +142,9 @@ __global__ __launch_bounds__(kWave) void small_up2_kernel(const SmallPlan p)
     const long plane0 = static_cast<long>(blockIdx.x) * p.planes_per_run;
     const int nplanes = static_cast<int>(min(static_cast<long>(p.planes_per_run), p.planes - plane0));
     const int in_plane = p.in_h * w_in, out_plane = p.out_h * w_out;
+    const int lp_in = RAG ? p.lp_in : W, lp_out = RAG ? p.lp_out : OW;
+    const bool pad_in = RAG && p.magic_in != 0, pad_out = RAG && p.magic_out != 0;
+    const int lin_plane = p.in_h * lp_in, lout_plane = p.out_h * lp_out;
 
     const int pl_raw = fast_div(threadIdx.x, p.lpp_magic);
     const int q = threadIdx.x - pl_raw * p.lanes_per_plane;
@@ -143,7 +156,10 @@ __global__ __launch_bounds__(kWave) void small_up2_kernel(const SmallPlan p)
 
     float tapv[K * K];
     load_taps<K * K, true>(static_cast<const IO *>(p.taps), static_cast<int>((plane0 + pl) % p.channel), tapv);
-    run_to_lds(static_cast<const IO *>(p.in) + (in0 - hin), lds, nplanes * in_plane + hin);
+    if (pad_in)
+        run_to_lds_rows(static_cast<const IO *>(p.in) + (in0 - hin), lds, nplanes * in_plane + hin, hin, p.magic_in, p.zero_off - 1);
+    else
+        run_to_lds(static_cast<const IO *>(p.in) + (in0 - hin), lds, nplanes * in_plane + hin);
     const float *zrow = lds + p.zero_off;  // stands in for the rows above and below the plane
     clear_zero_row<W>(lds + p.zero_off);
     __syncthreads();
@@ -154,8 +170,8 @@ __global__ __launch_bounds__(kWave) void small_up2_kernel(const SmallPlan p)
 #pragma unroll
         for (int o = 0; o < OW; ++o) acc[r][o] = 0.f;
 
-    const float *plane = lds + hin + pl * in_plane;
-    auto row_at = [&](int iy) { return static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h) ? plane + iy * w_in : zrow; };
+    const float *plane = lds + (pad_in ? 0 : hin) + pl * lin_plane;
+    auto row_at = [&](int iy) { return static_cast<unsigned>(iy) < static_cast<unsigned>(p.in_h) ? plane + iy * lp_in : zrow; };
     float nxt[W];
     lds_load_row_w<W, RAG>(row_at(q - p.pad_h), nxt, w_in);
 #pragma unroll
@@ -187,13 +203,16 @@ __global__ __launch_bounds__(kWave) void small_up2_kernel(const SmallPlan p)
     __syncthreads();
 
     if (active) {
-        float *dst = lds + hout + pl * out_plane;
+        float *dst = lds + (pad_out ? 0 : hout) + pl * lout_plane;
 #pragma unroll
         for (int r = 0; r < 2; ++r)
-            if (2 * q + r < p.out_h) lds_store_row_w<OW, RAG>(dst + (2 * q + r) * w_out, acc[r], w_out);
+            if (2 * q + r < p.out_h) lds_store_row_w<OW, RAG>(dst + (2 * q + r) * lp_out, acc[r], w_out);
     }
     __syncthreads();
-    lds_to_run(static_cast<IO *>(p.out) + (out0 - hout), lds, nplanes * out_plane + hout, hout);
+    if (pad_out)
+        lds_to_run_rows(static_cast<IO *>(p.out) + (out0 - hout), lds, nplanes * out_plane + hout, hout, p.magic_out);
+    else
+        lds_to_run(static_cast<IO *>(p.out) + (out0 - hout), lds, nplanes * out_plane + hout, hout);
 }
 
 // LDS of a run of `planes` planes (the larger of its input and output image, plus the up to three elements in front
@@ -212,26 +231,31 @@ int small_zero_off(int planes, int in_plane, int out_plane, int spare)
 
 // Planes per wavefront: as many as there are lane slots within the LDS budget; when a plane is not a multiple of 4
 // elements a multiple of 4 of them if that costs less than half (every run then starts on a 4-element boundary).
-int planes_per_run(int lanes_per_plane, int in_plane, int out_plane, long planes)
+int planes_per_run(int lanes_per_plane, int in_plane, int out_plane, int lin_plane, int lout_plane, long planes)
 {
     int P = kWave / lanes_per_plane;
-    while (P > 0 && small_lds_bytes(P, in_plane, out_plane, 0) > 16 * 1024 + 16) --P;
+    while (P > 0 && small_lds_bytes(P, lin_plane, lout_plane, 0) > 16 * 1024 + 16) --P;
     if ((in_plane % 4 != 0 || out_plane % 4 != 0) && P >= 4) P -= P % 4;
     if (static_cast<long>(P) > planes && in_plane % 4 == 0 && out_plane % 4 == 0) P = static_cast<int>(planes);
     return P;
 }
 
 // Fills in the run shape of p (lanes_per_plane set); false when the geometry does not fit a wavefront.
-bool finish_plan(SmallPlan &p, size_t &shmem, long &runs, int spare, int zero_floats)
+bool finish_plan(SmallPlan &p, size_t &shmem, long &runs, int spare, int zero_floats, bool ragged)
 {
     if (p.lanes_per_plane < 1 || p.lanes_per_plane > kWave) return false;
     const int in_plane = p.in_h * p.in_w, out_plane = p.out_h * p.out_w;
-    p.planes_per_run = planes_per_run(p.lanes_per_plane, in_plane, out_plane, p.planes);
+    p.lp_in = ragged ? ragged_pitch(p.in_w) : p.in_w;
+    p.lp_out = ragged ? ragged_pitch(p.out_w) : p.out_w;
+    p.magic_in = ragged ? ragged_magic(p.in_w) : 0;
+    p.magic_out = ragged ? ragged_magic(p.out_w) : 0;
+    const int lin_plane = p.in_h * p.lp_in, lout_plane = p.out_h * p.lp_out;
+    p.planes_per_run = planes_per_run(p.lanes_per_plane, in_plane, out_plane, lin_plane, lout_plane, p.planes);
     if (p.planes_per_run < 1) return false;
     p.lpp_magic = magic_u16(p.lanes_per_plane);
     runs = (p.planes + p.planes_per_run - 1) / p.planes_per_run;
     if (runs > 0x7fffffffL) return false;
-    p.zero_off = small_zero_off(p.planes_per_run, in_plane, out_plane, spare);
+    p.zero_off = small_zero_off(p.planes_per_run, lin_plane, lout_plane, spare);
     shmem = static_cast<size_t>(p.zero_off + zero_floats) * 4;
     return true;
 }
@@ -242,7 +266,7 @@ int launch_small_down(SmallPlan &p, hipStream_t stream)
     p.lanes_per_plane = ceil_div(p.out_h, BH);
     size_t shmem;
     long runs;
-    if (!finish_plan(p, shmem, runs, RAG ? W : 0, zero_row_floats(W))) return -1;
+    if (!finish_plan(p, shmem, runs, RAG ? W : 0, zero_row_floats(W), RAG)) return -1;
     hipLaunchKernelGGL((small_down_kernel<IO, W, RAG, K, S, FLIP, BH>), dim3(static_cast<unsigned>(runs)), dim3(kWave),
                        shmem, stream, p);
     note_variant("small_down%s<%s%d,k%d,s%d,%s,bh%d> P%d", sizeof(IO) == 2 ? "16" : "", RAG ? "r" : "w", W, K, S,
@@ -256,7 +280,7 @@ int launch_small_up2(SmallPlan &p, hipStream_t stream)
     p.lanes_per_plane = ceil_div(p.out_h, 2);
     size_t shmem;
     long runs;
-    if (!finish_plan(p, shmem, runs, RAG ? W : 0, zero_row_floats(W))) return -1;
+    if (!finish_plan(p, shmem, runs, RAG ? W : 0, zero_row_floats(W), RAG)) return -1;
     hipLaunchKernelGGL((small_up2_kernel<IO, W, RAG, K>), dim3(static_cast<unsigned>(runs)), dim3(kWave), shmem, stream, p);
     note_variant("small_up2%s<%s%d,k%d> P%d", sizeof(IO) == 2 ? "16" : "", RAG ? "r" : "w", W, K, p.planes_per_run);
     return check_launch("small_up2_kernel");

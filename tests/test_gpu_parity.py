@@ -119,6 +119,10 @@ SMALL = [
     # runs of planes that start off a 4-element boundary (odd planes, channel groups that are not multiples of four)
     (3, 5, 15, 15, 3, 1, 1), (3, 7, 9, 9, 5, 2, 2), (2, 3, 31, 29, 7, 1, 3), (3, 5, 30, 30, 3, 2, 1), (5, 3, 7, 7, 5, 1, 2),
     (3, 6, 13, 13, 3, 2, 1), (2, 9, 5, 7, 3, 1, 1),
+    # ragged even widths (LDS rows at pitch width + 1, element-wise copies), with and without heads
+    (2, 6, 24, 24, 5, 1, 2), (3, 5, 24, 24, 3, 2, 1), (2, 8, 12, 12, 5, 1, 2), (3, 7, 12, 12, 5, 2, 2), (2, 8, 6, 6, 3, 1, 1),
+    (3, 5, 6, 6, 5, 1, 2), (2, 3, 20, 20, 7, 1, 3), (3, 3, 10, 10, 3, 1, 1), (3, 5, 9, 10, 3, 1, 1), (2, 4, 17, 18, 5, 1, 2),
+    (3, 3, 11, 26, 3, 2, 1), (2, 5, 7, 30, 5, 1, 2), (1, 7, 9, 22, 7, 1, 3),
 ]
 
 
@@ -513,7 +517,7 @@ HALF_SHAPES = [(2, 6, 14, 14, 3, 1, 1), (2, 5, 28, 28, 5, 2, 2), (2, 4, 56, 56, 
                # whole-plane kernels, other widths (exact 8/16/32, ragged classes)
                (2, 8, 8, 8, 5, 1, 2), (2, 6, 16, 16, 3, 1, 1), (2, 4, 32, 32, 5, 2, 2), (2, 8, 15, 15, 5, 1, 2),
                (2, 8, 15, 15, 3, 2, 1), (2, 4, 30, 30, 7, 1, 3), (2, 4, 20, 12, 3, 1, 1), (3, 5, 15, 15, 5, 1, 2),
-               (3, 3, 31, 31, 3, 2, 1),
+               (3, 3, 31, 31, 3, 2, 1), (2, 6, 24, 24, 5, 1, 2), (3, 5, 12, 12, 3, 2, 1), (3, 5, 9, 10, 3, 1, 1),
                # rows of at least 96 elements in whole groups of eight: the kernels with 16-bit LDS images and
                # two-element dot products (7-row and 4-row blocks, several planes per workgroup, odd heights)
                (1, 3, 96, 104, 3, 1, 1), (1, 2, 100, 96, 5, 1, 2), (1, 2, 98, 112, 7, 1, 3), (1, 2, 97, 120, 5, 2, 2),
