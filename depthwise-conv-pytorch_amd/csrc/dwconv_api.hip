@@ -98,6 +98,8 @@ int run_fir(const T *in, const T *taps, T *out, const Geometry &g, hipStream_t s
                 rc = try_launch_fir_tiled16<T>(in, taps, out, g, stream);
                 if (rc >= 0) return rc;
             }
+            rc = try_launch_fir_stack<T>(in, taps, out, g, stream);
+            if (rc >= 0) return rc;
             rc = try_launch_fir_tiled<T>(in, taps, out, g, stream);
             if (rc >= 0) return rc;
         }
@@ -186,6 +188,8 @@ size_t wgrad_workspace(const WgradGeometry &g)
         if (sm > need) need = sm;
         const size_t s2 = bwd_s2_workspace(g);
         if (s2 > need) need = s2;
+        const size_t st = bwd_stack_workspace(g);
+        if (st > need) need = st;
         if constexpr (sizeof(T) == 2) {
             const size_t t16 = bwd_tiled16_workspace(g);
             if (t16 > need) need = t16;
@@ -254,6 +258,8 @@ int backward_any(const T *in, const T *gy, const T *taps, T *gx, T *gw, void *ws
             rc = try_launch_bwd_tiled16<T>(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
             if (rc >= 0) return rc;
         }
+        rc = try_launch_bwd_stack<T>(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+        if (rc >= 0) return rc;
         rc = try_launch_bwd_tiled<T>(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
         if (rc >= 0) return rc;
         rc = try_launch_bwd_s2<T>(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);

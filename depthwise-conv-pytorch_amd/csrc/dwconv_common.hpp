@@ -253,6 +253,15 @@ template <typename IO>
 int try_launch_bwd_tiled16(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
                            const WgradGeometry &g, hipStream_t stream);
 
+// Stride-1 "same" layers with 5x5 / 7x7 filters on maps too wide for several planes per workgroup: one channel per
+// workgroup over a stack of its images, taps in scalar registers (dwconv_stack.hip).  Same return convention.
+size_t bwd_stack_workspace(const WgradGeometry &g);  // 0 when that kernel does not cover g
+template <typename IO>
+int try_launch_bwd_stack(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
+                         const WgradGeometry &g, hipStream_t stream);
+template <typename IO>
+int try_launch_fir_stack(const IO *in, const IO *taps, IO *out, const Geometry &g, hipStream_t stream);
+
 // The same for stride-2 layers: dwconv_bwd_s2.hip.
 size_t bwd_s2_workspace(const WgradGeometry &g);  // 0 when that kernel does not cover g
 template <typename IO>

@@ -1,0 +1,494 @@
+// Stride-1 "same" convolutions with large filters on maps too wide for several planes per workgroup: forward /
+// grad-input, and the fused grad-input + grad-weight sweep (element type fp32, fp16 or bf16; LDS and arithmetic fp32).
+//
+// These shapes (7x7 filters on 56 x 56 maps) are bound by the vector unit, not by HBM, and the general tiled
+// kernels (dwconv_tile.hip, dwconv_wgrad.hip) leave it underused there in two ways, both repaired here:
+//
+//  * Lanes.  A lane owns a 4 x 4 block of outputs and a workgroup a band of one plane: 56 x 56 has 14 x 14 blocks, so
+//    196 of 256 lanes work (112 x 112 and 128 x 96 planes lose the same quarter to bands that do not divide).
+//    Here a workgroup keeps ONE channel and walks that channel's images as one tall stack: image n's rows sit at
+//    stacked rows n * (H + K/2) + K/2 ..., with K/2 rows of zeros between neighbours (the bottom padding of one image
+//    is the top padding of the next).  A tile is U = 256 / (W / 4) consecutive 4-row units of the stack, wherever the
+//    image boundaries fall: 252 of 256 lanes work on a 56-wide map.
+//  * Registers.  All lanes of a workgroup share the channel, so the K*K taps of the grad-input (or forward) pass
+//    are wavefront-uniform: they live in scalar registers and enter the FMAs as scalar operands, not in K*K
+//    vector registers per lane.  The 7x7 fused instance needs about 130 vector registers instead of 188: three
+//    wavefronts per SIMD instead of two.
+//
+//  * Loads.  The vector unit is the bottleneck only if it never waits: a tile image is fetched into registers while
+//    the workgroup computes on the images already in LDS (see stack_kernel), so every load has a whole arithmetic
+//    phase to arrive in.
+//
+// The arithmetic is that of the general kernels: the band (with halo) of x, and of gy in the fused kernel, is
+// staged in LDS with the zero padding materialised; per window row a lane reads aligned float4s once and reuses
+// them for every tap and output row.  Grad-weight sums stay in registers over all tiles of the workgroup's chunk
+// and are reduced in a fixed order (wave64 DPP sum, then the four wavefronts through LDS) into
+// partial[c][chunk][tap]; the second pass is launch_wgrad_final.  Replaces torch_dwconv/dwconv_kernel.cu:69-181
+// (large kernel, both directions at stride 1) and :260-306 (grad-weight) for these shapes.
+#include "dwconv_tile_common.hpp"
+
+namespace dwconv {
+
+namespace {
+
+constexpr int kStackBH = 4;  // rows per unit (the rows of a unit that hangs over the end of an image are masked)
+
+struct StackPlan {
+    const void *x;     // forward: the input; fused backward: x.  Element type IO of the kernel template
+    const void *gy;    // fused backward only
+    const void *taps;
+    void *out;         // forward: the output; fused backward: grad-input
+    float *partial;    // fused backward: partial[c][chunk][tap]
+    int batch, channel;
+    int h, w, plane;
+    int img_stride;        // elements from one image's plane of a channel to the next image's: channel * plane
+    int ru;                // row units per image = ceil(h / 4)
+    int vh;                // rows per image in the stack = h + K/2
+    int ncb;               // 4-wide column blocks per row
+    int units_per_tile;    // U
+    int total_units;       // batch * ru
+    int tiles, chunks;
+    int pitch;             // floats per LDS row
+    int spr;               // float4 slots fetched per row (one of zeros on either side)
+    int img_floats;        // floats of one staged image (x or gy)
+    int rpp;               // rows of an image the workgroup stages per pass: 256 / spr
+    int slots_per_lane;    // loads a lane issues per tile image: ceil(rows / rpp) for the tallest tile
+    int step_n, step_r;    // chunks * units_per_tile units = step_n images + step_r row units
+    unsigned ncb_magic, ru_magic, vh_magic, spr_magic;
+};
+
+// n / d through the reciprocal made by magic_u16(d), for 2 <= d (no test for d == 1: the planner rules it out)
+__device__ __forceinline__ int div_magic(int n, unsigned magic) { return static_cast<int>(__umulhi(static_cast<unsigned>(n), magic)); }
+
+// What a workgroup needs to know about one tile (all uniform).
+struct StackTile {
+    int n0, r0;       // image and row unit of the tile's first unit
+    int units_here;   // units of the tile (the last tile of a channel may be short)
+    int vrel0;        // stacked row, relative to image n0, of LDS row 0
+    int rows;         // stacked rows the tile's windows cover
+    int n_span;       // images from n0 on that the tile may touch
+    long plane0;      // plane index of (image n0, this channel)
+};
+
+// The tile whose first unit is row unit r0 of image n0 (n0 * ru + r0 < total_units).
+__device__ __forceinline__ StackTile stack_tile(const StackPlan &p, int n0, int r0, int c, int K)
+{
+    StackTile t;
+    t.n0 = n0;
+    t.r0 = r0;
+    t.units_here = min(p.units_per_tile, p.total_units - (n0 * p.ru + r0));
+    const int ql = r0 + t.units_here - 1;  // last unit of the tile, counted from image n0's first
+    const int nl = div_magic(ql, p.ru_magic), rl = ql - nl * p.ru;
+    t.vrel0 = r0 * kStackBH;
+    t.rows = nl * p.vh + rl * kStackBH + kStackBH + K - 1 - t.vrel0;
+    t.n_span = min(p.batch - n0, nl + 2);
+    t.plane0 = static_cast<long>(n0) * p.channel + c;
+    return t;
+}
+
+// This lane's part in staging, the same for every tile: one float4 column of the image and every rpp-th row.
+struct StackLane {
+    int jr;        // first LDS row (lanes beyond rpp whole rows stage nothing: jr is then past every image)
+    unsigned coff; // byte offset of the column within a row of the tensor
+    bool col_ok;   // the column lies inside the plane (else it reads as zeros)
+    int dcol;      // float offset of the column within an LDS row
+};
+
+template <typename IO, int K>
+__device__ __forceinline__ StackLane stack_lane(const StackPlan &p)
+{
+    StackLane l;
+    const int jr = div_magic(threadIdx.x, p.spr_magic);
+    const int ix = 4 * (static_cast<int>(threadIdx.x) - jr * p.spr - 1);
+    l.jr = jr < p.rpp ? jr : (1 << 20);
+    l.coff = static_cast<unsigned>(ix) * static_cast<unsigned>(sizeof(IO));
+    l.col_ok = static_cast<unsigned>(ix) < static_cast<unsigned>(p.w);
+    l.dcol = kSlack + ix + K / 2;
+    return l;
+}
+
+// A tile image travels in two steps, so that its loads are in flight while the workgroup computes on the images
+// already in LDS: fetch_stack issues this lane's NS loads into registers (elements as loaded, not yet widened),
+// commit_stack writes them into the LDS image.  LDS row j, column kSlack + ix + K/2 holds column ix of stacked row
+// vrel0 + j of the tensor whose (image n0, channel c) plane starts at `src`; zero rows, columns outside the plane
+// and images past n_span read zeros through the view.
+template <typename IO, int K, int NS>
+__device__ __forceinline__ void fetch_stack(const StackPlan &p, const StackLane &l, const IO *__restrict__ src, const StackTile &t,
+                                            typename Raw4<IO>::type (&v)[NS])
+{
+    constexpr int PW = K / 2;
+    constexpr unsigned ES = sizeof(IO);
+    const long extent = (static_cast<long>(t.n_span - 1) * p.img_stride + p.plane) * ES;
+    const __amdgpu_buffer_rsrc_t view = buffer_view(src, extent);
+#pragma unroll
+    for (int u = 0; u < NS; ++u) {
+        const int j = l.jr + u * p.rpp;
+        const int vr = t.vrel0 + min(j, t.rows);   // (rows past the tile: any row, the load is switched off)
+        const int n = div_magic(vr, p.vh_magic);
+        const int rr = vr - __mul24(n, p.vh) - PW;
+        const bool ok = j < t.rows && l.col_ok && rr >= 0 && n < t.n_span;
+        const unsigned off = (static_cast<unsigned>(n) * static_cast<unsigned>(p.img_stride) + __mul24(rr, p.w)) * ES + l.coff;
+        if constexpr (sizeof(IO) == 4) {
+            const u32x4 q = __builtin_amdgcn_raw_buffer_load_b128(view, ok ? off : kOob, 0, 0);
+            v[u] = make_float4(__uint_as_float(q.x), __uint_as_float(q.y), __uint_as_float(q.z), __uint_as_float(q.w));
+        } else {
+            const u32x2 q = __builtin_amdgcn_raw_buffer_load_b64(view, ok ? off : kOob, 0, 0);
+            v[u] = make_uint2(q.x, q.y);
+        }
+    }
+}
+
+template <typename IO, int K, int NS>
+__device__ __forceinline__ void commit_stack(const StackPlan &p, const StackLane &l, float *lds, const StackTile &t,
+                                             const typename Raw4<IO>::type (&v)[NS])
+{
+    const int dump = p.img_floats - 4;  // right-hand slack of the last row
+#pragma unroll
+    for (int u = 0; u < NS; ++u) {
+        const int j = l.jr + u * p.rpp;
+        float *d = lds + (j < t.rows ? __mul24(j, p.pitch) + l.dcol : dump);
+        const float4 w = widen4<IO>(v[u]);
+        d[0] = w.x;
+        d[1] = w.y;
+        d[2] = w.z;
+        d[3] = w.w;
+    }
+}
+
+// FUSED: grad-input (taps rotated) and grad-weight of one channel's images; otherwise the forward pass (FLIP: taps
+// rotated, the grad-input pass on its own).  NS: loads a lane issues per tile image (the planner's bound).
+//
+// Order of a fused tile, two barriers: [gy of this tile is in registers] commit gy | barrier | issue the loads of x |
+// slide the taps over the gy windows (grad-input out, own gy block kept) | commit x | barrier | issue the loads of the
+// next tile's gy | grad-weight sums over the x windows.  Every image's loads fly during one arithmetic phase.
+template <typename IO, int K, bool FUSED, bool FLIP, int NS>
+__global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
+{
+    extern __shared__ float4 lds_raw[];
+    float *lds = reinterpret_cast<float *>(lds_raw);
+    constexpr int BH = kStackBH;
+    constexpr int PW = K / 2;
+    constexpr int KK = K * K;
+    constexpr int WIN_ROWS = BH - 1 + K;
+    constexpr int NV = (K + 6) / 4;  // float4s that hold a window row: columns 4*cb - K/2 ... 4*cb + 3 + K/2
+    constexpr unsigned ES = sizeof(IO);
+
+    const int c = blockIdx.x / p.chunks;
+    const int chunk = blockIdx.x - c * p.chunks;
+    const IO *const slide_src = static_cast<const IO *>(FUSED ? p.gy : p.x);  // the tensor the taps slide over
+    float *const lds_slide = lds;                   // its image
+    float *const lds_x = lds + p.img_floats;        // fused: the image of x
+
+    typename Raw4<IO>::type staged[NS];
+    const StackLane lane = stack_lane<IO, K>(p);
+    // chunk k takes tiles k, k + chunks, ...: the first unit of the next tile lies step_n images and step_r row
+    // units further on
+    const int u_first = chunk * p.units_per_tile;
+    const int n_first = u_first / p.ru;
+    StackTile cur = stack_tile(p, n_first, u_first - n_first * p.ru, c, K);
+    fetch_stack<IO, K, NS>(p, lane, slide_src + cur.plane0 * p.plane, cur, staged);
+
+    // the taps of the sliding pass, wavefront-uniform: scalar registers
+    float tap[KK];
+#pragma unroll
+    for (int t = 0; t < KK; ++t) {
+        const float v = Io<IO>::in(static_cast<const IO *>(p.taps)[c * KK + ((FUSED || FLIP) ? KK - 1 - t : t)]);
+        tap[t] = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
+    }
+
+    // this lane's place in every tile: unit ul of the tile, column block cb
+    const int ul = div_magic(threadIdx.x, p.ncb_magic);
+    const int cb = threadIdx.x - ul * p.ncb;
+    const int ox = 4 * cb;
+
+    float acc[FUSED ? KK : 1];
+#pragma unroll
+    for (int t = 0; t < (FUSED ? KK : 1); ++t) acc[t] = 0.f;
+
+    // chunk k takes tiles k, k + chunks, ...: at any moment the grid works on a narrow window of images
+    for (int tile = chunk; tile < p.tiles; tile += p.chunks) {
+        const bool more = tile + p.chunks < p.tiles;
+        // (forward: the windows of the previous tile are read until here; fused: the slide image was last read
+        // before the previous tile's second barrier)
+        if (!FUSED && tile != chunk) __syncthreads();
+        commit_stack<IO, K, NS>(p, lane, lds_slide, cur, staged);
+        __syncthreads();
+        StackTile nxt_tile = cur;
+        if (more) {
+            const int r_raw = cur.r0 + p.step_r;
+            const bool carry = r_raw >= p.ru;
+            nxt_tile = stack_tile(p, cur.n0 + p.step_n + (carry ? 1 : 0), carry ? r_raw - p.ru : r_raw, c, K);
+        }
+        if constexpr (FUSED) fetch_stack<IO, K, NS>(p, lane, static_cast<const IO *>(p.x) + cur.plane0 * p.plane, cur, staged);
+        else if (more) fetch_stack<IO, K, NS>(p, lane, slide_src + nxt_tile.plane0 * p.plane, nxt_tile, staged);
+
+        // this lane's unit: image n0 + nrel, row unit r
+        const int q = cur.r0 + ul;
+        const int nrel = div_magic(q, p.ru_magic);
+        const int r = q - __mul24(nrel, p.ru);
+        const bool has_item = ul < cur.units_here;
+        const int base_off = (has_item ? __mul24(nrel, p.vh) + r * BH - cur.vrel0 : 0) * p.pitch + kSlack + ox;
+        const float *sbase = lds_slide + base_off;
+
+        float sums[BH][4];
+        float g[FUSED ? BH : 1][4];
+#pragma unroll
+        for (int b = 0; b < BH; ++b)
+#pragma unroll
+            for (int o = 0; o < 4; ++o) sums[b][o] = 0.f;
+        {
+            float nxt[4 * NV];
+            load_window_row<NV>(sbase, nxt);
+#pragma unroll
+            for (int wr = 0; wr < WIN_ROWS; ++wr) {
+                float win[4 * NV];
+#pragma unroll
+                for (int i = 0; i < 4 * NV; ++i) win[i] = nxt[i];
+                if (wr + 1 < WIN_ROWS) load_window_row<NV>(sbase + (wr + 1) * p.pitch, nxt);
+                if constexpr (FUSED) {
+                    // the lane's own gy block sits K/2 rows and columns into its window
+                    const int gb = wr - PW;
+                    if (gb >= 0 && gb < BH) {
+#pragma unroll
+                        for (int o = 0; o < 4; ++o)
+                            g[gb >= 0 && gb < BH ? gb : 0][o] = (has_item && r * BH + gb < p.h) ? win[o + PW] : 0.f;
+                    }
+                }
+#pragma unroll
+                for (int b = 0; b < BH; ++b) {
+                    const int ty = wr - b;
+                    if (ty < 0 || ty >= K) continue;
+#pragma unroll
+                    for (int tx = 0; tx < K; ++tx)
+#pragma unroll
+                        for (int o = 0; o < 4; ++o) sums[b][o] = fmaf(win[o + tx], tap[ty * K + tx], sums[b][o]);
+                }
+                pin_registers(sums);
+            }
+        }
+        {
+            // branch-free: rows past the end of the image (and lanes without a unit) store out of range
+            const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + cur.plane0 * p.plane,
+                                                            (static_cast<long>(cur.n_span - 1) * p.img_stride + p.plane) * ES);
+            const unsigned o0 = (static_cast<unsigned>(nrel) * static_cast<unsigned>(p.img_stride) + ox) * ES;
+#pragma unroll
+            for (int b = 0; b < BH; ++b) {
+                const int oy = r * BH + b;
+                const bool ok = has_item && oy < p.h;
+                view_store4<IO>(view, ok ? o0 + __mul24(oy, p.w) * ES : kOob, sums[b][0], sums[b][1], sums[b][2], sums[b][3]);
+            }
+        }
+
+        if constexpr (FUSED) {
+            commit_stack<IO, K, NS>(p, lane, lds_x, cur, staged);
+            __syncthreads();
+            if (more) fetch_stack<IO, K, NS>(p, lane, slide_src + nxt_tile.plane0 * p.plane, nxt_tile, staged);
+            const float *base = lds_x + base_off;
+            float nxt[4 * NV];
+            load_window_row<NV>(base, nxt);
+#pragma unroll
+            for (int wr = 0; wr < WIN_ROWS; ++wr) {
+                float win[4 * NV];
+#pragma unroll
+                for (int i = 0; i < 4 * NV; ++i) win[i] = nxt[i];
+                if (wr + 1 < WIN_ROWS) load_window_row<NV>(base + (wr + 1) * p.pitch, nxt);
+#pragma unroll
+                for (int b = 0; b < BH; ++b) {
+                    const int ty = wr - b;
+                    if (ty < 0 || ty >= K) continue;
+#pragma unroll
+                    for (int tx = 0; tx < K; ++tx)
+#pragma unroll
+                        for (int o = 0; o < 4; ++o) acc[ty * K + tx] = fmaf(g[b][o], win[o + tx], acc[ty * K + tx]);
+                }
+                pin_registers(acc);
+            }
+        }
+        cur = nxt_tile;
+    }
+
+    if constexpr (FUSED) {
+        __syncthreads();  // the tile images are dead; their LDS is reused for the reduction
+        // every lane worked on the same channel: wavefront sums, then the four wavefronts in order
+#pragma unroll
+        for (int t = 0; t < KK; ++t) {
+            const float s = wave_sum_to_last_lane(acc[t]);
+            if ((threadIdx.x & 63) == 63) lds[(threadIdx.x >> 6) * KK + t] = s;
+        }
+        __syncthreads();
+        if (threadIdx.x < KK) {
+            float s = lds[threadIdx.x];
+#pragma unroll
+            for (int w = 1; w < kThreads / 64; ++w) s += lds[w * KK + threadIdx.x];
+            p.partial[(static_cast<long>(c) * p.chunks + chunk) * KK + threadIdx.x] = s;
+        }
+    }
+}
+
+// Geometry the stacked kernels take: stride 1, "same" padding, K x K with K in {5, 7}, rows of whole groups of four
+// elements, and a plane too large for two of them to share a workgroup (those shapes keep the several-planes mode of
+// the general kernels).
+bool make_plan(StackPlan &p, int K, int batch, int channel, int h, int w, size_t esize, bool fused, int target_wgs)
+{
+    if (K != 5 && K != 7) return false;
+    if (w % 4 != 0 || w < 16 || h < 8) return false;
+    const int ncb = w / 4;
+    if (ncb > kThreads) return false;
+    const int ru = ceil_div(h, kStackBH);
+    if (2 * ru * ncb <= kThreads) return false;
+    const long plane = static_cast<long>(h) * w;
+    if (plane >= (1l << 23) || static_cast<long>(channel) * plane >= (1l << 28)) return false;
+    p.batch = batch;
+    p.channel = channel;
+    p.h = h;
+    p.w = w;
+    p.plane = static_cast<int>(plane);
+    p.img_stride = static_cast<int>(channel * plane);
+    p.ru = ru;
+    p.vh = h + K / 2;
+    p.ncb = ncb;
+    p.pitch = w + 16;  // kSlack + K/2 columns of zeros + w + zeros up to the last window column + kSlack, rounded up
+    p.spr = ncb + 2;
+    const long total_units = static_cast<long>(batch) * ru;
+    if (total_units >= (1l << 30)) return false;
+    p.total_units = static_cast<int>(total_units);
+    const int budget = env_int("DWCONV_STACK_LDS", 56 * 1024);
+    int units = kThreads / ncb;
+    auto rows_for = [&](int u) { return u * kStackBH + K - 1 + (K / 2) * ((u - 1) / ru + 2); };
+    // (and at most eight loads per lane and image: they wait in registers while the workgroup computes)
+    p.rpp = kThreads / p.spr;
+    while (units > 1 && (static_cast<long>(rows_for(units)) * p.pitch * 4 * (fused ? 2 : 1) > budget ||
+                         rows_for(units) > 8 * p.rpp))
+        --units;
+    if (rows_for(units) > 8 * p.rpp) return false;
+    if (static_cast<long>(rows_for(units)) * p.pitch * 4 * (fused ? 2 : 1) > budget) return false;
+    p.units_per_tile = units;
+    const int rows = rows_for(units);
+    p.img_floats = rows * p.pitch;
+    p.slots_per_lane = ceil_div(rows, p.rpp);
+    // 16-bit reciprocals: slots of an image, stacked rows of a tile, units counted from the tile's first image
+    if (rows + p.vh >= 65536 || ru + units >= 65536) return false;
+    // a tile's images must lie within one buffer view
+    const long span_images = (units - 1) / ru + 3;
+    if ((span_images * p.img_stride + plane) * static_cast<long>(esize) >= static_cast<long>(kOob)) return false;
+    p.tiles = ceil_div(p.total_units, units);
+    int chunks = ceil_div(target_wgs, channel);
+    if (chunks > p.tiles) chunks = p.tiles;
+    if (chunks < 1) chunks = 1;
+    if (static_cast<long>(channel) * chunks > 0x7fffffffL) return false;
+    p.chunks = chunks;
+    const long step = static_cast<long>(chunks) * units;
+    p.step_n = static_cast<int>(step / ru);
+    p.step_r = static_cast<int>(step % ru);
+    p.ncb_magic = magic_u16(ncb);
+    p.ru_magic = magic_u16(ru);
+    p.vh_magic = magic_u16(p.vh);
+    p.spr_magic = magic_u16(p.spr);
+    return true;
+}
+
+size_t lds_bytes(const StackPlan &p, int K, bool fused)
+{
+    const size_t tile = static_cast<size_t>(p.img_floats) * 4 * (fused ? 2 : 1);
+    const size_t red = static_cast<size_t>(kThreads / 64) * K * K * 4;
+    return tile > red ? tile : red;
+}
+
+bool covers_bwd(const WgradGeometry &g)
+{
+    const int K = g.kernel_h;
+    if (!env_int("DWCONV_STACK", 1)) return false;
+    if (g.kernel_w != K || g.down_h != 1 || g.down_w != 1 || g.pad_h != K / 2 || g.pad_w != K / 2) return false;
+    if (g.out_h != g.in_h || g.out_w != g.in_w) return false;
+    return true;
+}
+
+// Workgroups of the fused kernel: one resident round (three per compute unit by its registers and LDS) for 7x7
+// filters (56x56 C=96 at batch 64: 768 workgroups 95 us, 1536 105, 2304 104); 5x5 filters do not care (256x256 C=64:
+// 189-197 us from 768 to 6144).
+int bwd_target_wgs(int K) { return env_int("DWCONV_STACK_WGS", K == 7 ? 768 : 1536); }
+
+}  // namespace
+
+size_t bwd_stack_workspace(const WgradGeometry &g)
+{
+    if (!covers_bwd(g)) return 0;
+    StackPlan p{};
+    // (the plan does not depend on the element size except through the view-extent check: the larger one)
+    if (!make_plan(p, g.kernel_h, g.batch, g.channel, g.in_h, g.in_w, 4, true, bwd_target_wgs(g.kernel_h))) return 0;
+    return static_cast<size_t>(g.channel) * p.chunks * g.kernel_h * g.kernel_w * sizeof(float);
+}
+
+template <typename IO>
+int try_launch_bwd_stack(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
+                         const WgradGeometry &g, hipStream_t stream)
+{
+    if (!covers_bwd(g)) return -1;
+    if (!aligned4(in) || !aligned4(gy) || !aligned4(gx)) return -1;
+    const int K = g.kernel_h;
+    StackPlan p{};
+    if (!make_plan(p, K, g.batch, g.channel, g.in_h, g.in_w, 4, true, bwd_target_wgs(K))) return -1;
+    const size_t need = static_cast<size_t>(g.channel) * p.chunks * K * K * sizeof(float);
+    if (ws == nullptr || ws_bytes < need)
+        return fail(DWCONV_ERR_WORKSPACE, "grad-weight needs a workspace of %zu bytes, got %zu", need, ws_bytes);
+    p.x = in;
+    p.gy = gy;
+    p.taps = taps;
+    p.out = gx;
+    p.partial = static_cast<float *>(ws);
+    const size_t shmem = lds_bytes(p, K, true);
+    const dim3 grid(static_cast<unsigned>(g.channel * p.chunks)), block(kThreads);
+    const bool six = p.slots_per_lane <= 6;
+    if (K == 7 && six) hipLaunchKernelGGL((stack_kernel<IO, 7, true, true, 6>), grid, block, shmem, stream, p);
+    else if (K == 7) hipLaunchKernelGGL((stack_kernel<IO, 7, true, true, 8>), grid, block, shmem, stream, p);
+    else if (six) hipLaunchKernelGGL((stack_kernel<IO, 5, true, true, 6>), grid, block, shmem, stream, p);
+    else hipLaunchKernelGGL((stack_kernel<IO, 5, true, true, 8>), grid, block, shmem, stream, p);
+    const int rc = check_launch("stack_kernel");
+    if (rc != DWCONV_OK) return rc;
+    note_variant("bwd_stack%s<k%d,s1> units%d tiles%d chunks%d", sizeof(IO) == 2 ? "16" : "", K, p.units_per_tile, p.tiles,
+                 p.chunks);
+    return launch_wgrad_final(static_cast<const float *>(ws), gw, g.channel, K * K, p.chunks, stream);
+}
+
+template <typename IO>
+int try_launch_fir_stack(const IO *in, const IO *taps, IO *out, const Geometry &g, hipStream_t stream)
+{
+    if (!env_int("DWCONV_STACK", 1)) return -1;
+    const int K = g.kernel_h;
+    if (g.kernel_w != K || g.up_h != 1 || g.up_w != 1 || g.down_h != 1 || g.down_w != 1) return -1;
+    if (g.pad_h0 != K / 2 || g.pad_w0 != K / 2 || g.out_h != g.in_h || g.out_w != g.in_w) return -1;
+    if (g.epi.enabled()) return -1;  // the fused epilogue stays with the general kernel
+    if (!aligned4(in) || !aligned4(out)) return -1;
+    StackPlan p{};
+    if (!make_plan(p, K, g.batch, g.channel, g.in_h, g.in_w, 4, false, env_int("DWCONV_STACK_FWD_WGS", 8192))) return -1;
+    p.x = in;
+    p.taps = taps;
+    p.out = out;
+    const size_t shmem = lds_bytes(p, K, false);
+    const dim3 grid(static_cast<unsigned>(g.channel * p.chunks)), block(kThreads);
+    const bool rot = !g.forward;
+    const bool six = p.slots_per_lane <= 6;
+#define DWCONV_STACK_FWD(KV, ROT)                                                                            \
+    if (six) hipLaunchKernelGGL((stack_kernel<IO, KV, false, ROT, 6>), grid, block, shmem, stream, p);       \
+    else hipLaunchKernelGGL((stack_kernel<IO, KV, false, ROT, 8>), grid, block, shmem, stream, p)
+    if (K == 7) {
+        if (rot) { DWCONV_STACK_FWD(7, true); } else { DWCONV_STACK_FWD(7, false); }
+    } else {
+        if (rot) { DWCONV_STACK_FWD(5, true); } else { DWCONV_STACK_FWD(5, false); }
+    }
+#undef DWCONV_STACK_FWD
+    note_variant("tile_stack%s<k%d,s1,%s> units%d tiles%d chunks%d", sizeof(IO) == 2 ? "16" : "", K, rot ? "rot" : "fwd",
+                 p.units_per_tile, p.tiles, p.chunks);
+    return check_launch("stack_kernel");
+}
+
+#define DWCONV_INSTANTIATE(IO)                                                                                        \
+    template int try_launch_bwd_stack<IO>(const IO *, const IO *, const IO *, IO *, IO *, void *, size_t,             \
+                                          const WgradGeometry &, hipStream_t);                                        \
+    template int try_launch_fir_stack<IO>(const IO *, const IO *, IO *, const Geometry &, hipStream_t);
+DWCONV_INSTANTIATE(float)
+DWCONV_INSTANTIATE(half_t)
+DWCONV_INSTANTIATE(bf16_t)
+#undef DWCONV_INSTANTIATE
+
+}  // namespace dwconv

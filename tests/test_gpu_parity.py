@@ -123,6 +123,10 @@ SMALL = [
     (2, 6, 24, 24, 5, 1, 2), (3, 5, 24, 24, 3, 2, 1), (2, 8, 12, 12, 5, 1, 2), (3, 7, 12, 12, 5, 2, 2), (2, 8, 6, 6, 3, 1, 1),
     (3, 5, 6, 6, 5, 1, 2), (2, 3, 20, 20, 7, 1, 3), (3, 3, 10, 10, 3, 1, 1), (3, 5, 9, 10, 3, 1, 1), (2, 4, 17, 18, 5, 1, 2),
     (3, 3, 11, 26, 3, 2, 1), (2, 5, 7, 30, 5, 1, 2), (1, 7, 9, 22, 7, 1, 3),
+    # one channel per workgroup over a stack of its images (5x5 / 7x7, stride 1): heights that leave a hanging
+    # 4-row unit (one, two or three rows over), tiles that span two and three images, a last tile that is short
+    (3, 5, 57, 64, 7, 1, 3), (2, 3, 33, 96, 5, 1, 2), (5, 2, 70, 40, 7, 1, 3), (1, 1, 300, 16, 5, 1, 2), (7, 3, 34, 36, 7, 1, 3),
+    (9, 2, 18, 60, 5, 1, 2), (4, 3, 59, 52, 7, 1, 3), (2, 2, 130, 128, 7, 1, 3), (6, 1, 23, 48, 5, 1, 2),
 ]
 
 
@@ -517,6 +521,7 @@ HALF_SHAPES = [(2, 6, 14, 14, 3, 1, 1), (2, 5, 28, 28, 5, 2, 2), (2, 4, 56, 56, 
                # whole-plane kernels, other widths (exact 8/16/32, ragged classes)
                (2, 8, 8, 8, 5, 1, 2), (2, 6, 16, 16, 3, 1, 1), (2, 4, 32, 32, 5, 2, 2), (2, 8, 15, 15, 5, 1, 2),
                (2, 8, 15, 15, 3, 2, 1), (2, 4, 30, 30, 7, 1, 3), (2, 4, 20, 12, 3, 1, 1), (3, 5, 15, 15, 5, 1, 2),
+               (3, 5, 57, 64, 7, 1, 3), (2, 3, 33, 72, 5, 1, 2),
                (3, 3, 31, 31, 3, 2, 1), (2, 6, 24, 24, 5, 1, 2), (3, 5, 12, 12, 3, 2, 1), (3, 5, 9, 10, 3, 1, 1),
                # rows of at least 96 elements in whole groups of eight: the kernels with 16-bit LDS images and
                # two-element dot products (7-row and 4-row blocks, several planes per workgroup, odd heights)
@@ -586,7 +591,8 @@ def test_combined_backward_entry_point(dw, gpu):
     from torch_dwconv import _C
 
     cases = [(2, 6, 14, 14, 3, 1, 1), (2, 6, 30, 33, 5, 2, 2), (2, 3, 40, 44, 3, 1, 0), (1, 4, 64, 64, 5, 1, 2),
-             (2, 4, 64, 48, 3, 2, 1), (1, 2, 20, 20, 4, 2, 1), (2, 3, 31, 29, 7, 2, 3), (2, 3, 48, 52, 5, 2, 0)]
+             (2, 4, 64, 48, 3, 2, 1), (1, 2, 20, 20, 4, 2, 1), (2, 3, 31, 29, 7, 2, 3), (2, 3, 48, 52, 5, 2, 0),
+             (2, 3, 64, 64, 3, 1, 1)]
     seen = set()
     for shape in cases:
         n, c, h, w, k, s, p = shape
@@ -598,7 +604,7 @@ def test_combined_backward_entry_point(dw, gpu):
         gw_ref = oracle.grad_weight(_np(x), _np(gy), wt.shape, s, p)
         np.testing.assert_allclose(_np(gx).astype(np.float64), gx_ref, rtol=1e-5, atol=1e-5)
         np.testing.assert_allclose(_np(gw).astype(np.float64), gw_ref, rtol=1e-4, atol=1e-4 * np.abs(gw_ref).max())
-    assert {"small_bwd", "bwd_tile", "bwd_tile_s2"} <= seen, seen
+    assert {"small_bwd", "bwd_tile", "bwd_stack", "bwd_tile_s2"} <= seen, seen
     # an out_grad whose extent does not belong to the geometry is refused
     x, wt, gy = make_inputs((1, 2, 16, 16, 3, 1, 1), seed=1)
     with pytest.raises(RuntimeError, match="does not match the convolution geometry"):
