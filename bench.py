@@ -51,6 +51,13 @@ WORKLOADS = {
     "effnet_b0_256": lambda batch: effnet_at(batch, 256),
     "effnet_b0_240": lambda batch: effnet_at(batch, 240),
     "effnet_b0_192": lambda batch: effnet_at(batch, 192),   # maps 96, 48, 24, 12, 6
+    # the options the reference's check_options refuses (a shape may carry dilation and depth multiplier as 8th and 9th
+    # entries): the 3x3 stride-1 layers of the stack at dilation 2 (padding 2), a 5x5 one, and the first two layers
+    # with two output channels per input channel
+    "effnet_b0_dil2": lambda batch: [(batch, 32, 112, 112, 3, 1, 2, 2, 1), (batch, 144, 56, 56, 3, 1, 2, 2, 1),
+                                     (batch, 240, 28, 28, 5, 1, 4, 2, 1), (batch, 480, 14, 14, 3, 1, 2, 2, 1),
+                                     (batch, 1152, 7, 7, 3, 1, 2, 2, 1)],
+    "effnet_b0_mult2": lambda batch: [(batch, 32, 112, 112, 3, 1, 1, 1, 2), (batch, 96, 112, 112, 3, 2, 1, 1, 2)],
     "cfg1": lambda batch: [(8, 32, 56, 56, 3, 1, 1)],
     "cfg2": lambda batch: [(16, 64, 256, 256, 5, 1, 2)],
     "cfg4": lambda batch: [(256, 1024, 7, 7, 7, 1, 3), (128, 512, 14, 14, 7, 1, 3)],
@@ -64,7 +71,9 @@ class Layer:
     """Device tensors and the three C-ABI calls of one depthwise layer."""
 
     def __init__(self, shape, lib, torch, dev, gen, dtype="f32", layout="nchw"):
-        n, c, h, w, k, s, p = shape
+        n, c, h, w, k, s, p = shape[:7]
+        dil, mult = (tuple(shape[7:9]) + (1, 1))[:2] if len(shape) > 7 else (1, 1)
+        self.general = (dil, mult) if (dil, mult) != (1, 1) else None
         tdtype = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype]
         es = 4 if dtype == "f32" else 2
         self.fn_fir = getattr(lib, "dwconv2d_" + dtype)
@@ -77,26 +86,34 @@ class Layer:
             self.fn_bwd = getattr(lib, "dwconv2d_backward_nhwc_" + dtype)
         self.shape = shape
         self.lib = lib
-        oh, ow = (h + 2 * p - k) // s + 1, (w + 2 * p - k) // s + 1
+        ke = dil * (k - 1) + 1
+        oh, ow = (h + 2 * p - ke) // s + 1, (w + 2 * p - ke) // s + 1
         self.geom = (n, c, h, w, oh, ow, k, s, p)
         self.x = torch.randn(n, c, h, w, generator=gen).to(dev, tdtype)
-        self.w = (torch.randn(c, 1, k, k, generator=gen) / k).to(dev, tdtype)
-        self.gy = torch.randn(n, c, oh, ow, generator=gen).to(dev, tdtype)
-        self.y = torch.empty(n, c, oh, ow, device=dev, dtype=tdtype)
+        self.w = (torch.randn(c * mult, 1, k, k, generator=gen) / k).to(dev, tdtype)
+        self.gy = torch.randn(n, c * mult, oh, ow, generator=gen).to(dev, tdtype)
+        self.y = torch.empty(n, c * mult, oh, ow, device=dev, dtype=tdtype)
         self.gx = torch.empty_like(self.x)
         self.gw = torch.empty_like(self.w)
         # channels-last: the same element counts, stored (N,H,W,C); values are random either way
-        self.ws_bytes = (lib.dwconv2d_backward_nhwc_workspace_bytes(n, c, h, w, k, k, s, s, p, p, es) if layout == "nhwc"
-                         else lib.dwconv2d_backward_kernel_workspace_bytes(n, c, h, w, oh, ow, k, k, s, s, p, p, es))
+        if self.general:
+            if layout != "nchw":
+                raise SystemExit("dilation / depth multiplier workloads are NCHW")
+            self.fn_gen = getattr(lib, "dwconv2d_general_" + dtype)
+            self.fn_gen_bwd = getattr(lib, "dwconv2d_general_backward_" + dtype)
+            self.ws_bytes = lib.dwconv2d_general_backward_workspace_bytes(n, c, h, w, mult, k, k, s, s, p, p, dil, dil, es)
+        else:
+            self.ws_bytes = (lib.dwconv2d_backward_nhwc_workspace_bytes(n, c, h, w, k, k, s, s, p, p, es) if layout == "nhwc"
+                             else lib.dwconv2d_backward_kernel_workspace_bytes(n, c, h, w, oh, ow, k, k, s, s, p, p, es))
         self.ws = torch.empty(max(self.ws_bytes, 16), dtype=torch.uint8, device=dev)
-        nx, ny, nw = n * c * h * w, n * c * oh * ow, c * k * k
+        nx, ny, nw = n * c * h * w, n * c * mult * oh * ow, c * mult * k * k
         self.bytes = {"fwd": es * (nx + ny + nw), "gx": es * (ny + nx + nw), "gw": es * (nx + ny + nw)}
         # the combined backward call is credited with the bytes of the two passes it replaces
         self.bytes["bwd"] = self.bytes["gx"] + self.bytes["gw"]
         self.flops = 2 * ny * k * k
         # transposed-problem padding, torch_dwconv/dwconv.py:39-44
         self.g_pad = (k - p - 1, h - oh * s + p, k - p - 1, w - ow * s + p)
-        self.name = f"C{c}_{h}x{w}_k{k}s{s}"
+        self.name = f"C{c}_{h}x{w}_k{k}s{s}" + (f"d{dil}" if dil > 1 else "") + (f"m{mult}" if mult > 1 else "")
 
     def _check(self, rc):
         if rc != 0:
@@ -104,6 +121,11 @@ class Layer:
 
     def fwd(self, stream):
         n, c, h, w, oh, ow, k, s, p = self.geom
+        if self.general:
+            dil, mult = self.general
+            self._check(self.fn_gen(self.x.data_ptr(), self.w.data_ptr(), self.y.data_ptr(), n, c, h, w, mult, k, k, s, s,
+                                    p, p, dil, dil, stream))
+            return
         if self.layout == "nhwc":
             self._check(self.fn_fwd_nhwc(self.x.data_ptr(), self.w.data_ptr(), self.y.data_ptr(), n, c, h, w, k, k,
                                          s, s, p, p, stream))
@@ -126,6 +148,12 @@ class Layer:
 
     def bwd(self, stream):
         n, c, h, w, oh, ow, k, s, p = self.geom
+        if self.general:
+            dil, mult = self.general
+            self._check(self.fn_gen_bwd(self.x.data_ptr(), self.gy.data_ptr(), self.w.data_ptr(), self.gx.data_ptr(),
+                                        self.gw.data_ptr(), self.ws.data_ptr(), self.ws_bytes, n, c, h, w, oh, ow, mult,
+                                        k, k, s, s, p, p, dil, dil, stream))
+            return
         self._check(self.fn_bwd(
             self.x.data_ptr(), self.gy.data_ptr(), self.w.data_ptr(), self.gx.data_ptr(), self.gw.data_ptr(),
             self.ws.data_ptr(), self.ws_bytes, n, c, h, w, oh, ow, k, k, s, s, p, p, stream))
@@ -185,7 +213,7 @@ def miopen_native(layers, torch, iters=3):
         for i in range(iters + 2):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            y = F.conv2d(x, wt, stride=s, padding=p, groups=c)
+            y = F.conv2d(x, wt, stride=s, padding=p, dilation=(l.general or (1, 1))[0], groups=c)
             torch.autograd.grad(y, (x, wt), l.gy)
             e1.record()
             torch.cuda.synchronize()
@@ -474,7 +502,7 @@ def main():
                                     "conv_only_ms": round(conv_ms, 4),
                                     "training_fwd_bwd_fused_ms": round(train_fused_ms, 4),
                                     "training_fwd_bwd_conv_then_torch_elementwise_ms": round(train_composed_ms, 4)}
-    if not args.no_cpu_baseline and args.dtype == "f32" and args.layout == "nchw":
+    if not args.no_cpu_baseline and args.dtype == "f32" and args.layout == "nchw" and not any(l.general for l in layers):
         result["cpu_baseline"] = cpu_baseline(layers, torch)
     print(json.dumps(result))
 

@@ -384,6 +384,18 @@ int make_general_geometry(GeneralGeometry &g, int batch, int channel, int in_h, 
 }
 
 inline bool is_plain(const GeneralGeometry &g) { return g.multiplier == 1 && g.dil_h == 1 && g.dil_w == 1; }
+// multiplier 1, stride 1, the same dilation above 1 on both axes: what the whole-plane kernels may take
+inline bool dilated_small(const GeneralGeometry &g)
+{
+    return g.multiplier == 1 && g.dil_h == g.dil_w && g.dil_h > 1 && g.stride_h == 1 && g.stride_w == 1 &&
+           g.kernel_h == g.kernel_w && g.in_w <= 32;
+}
+inline WgradGeometry dilated_wgrad_geometry(const GeneralGeometry &g)
+{
+    WgradGeometry w{g.batch, g.channel, g.in_h, g.in_w, g.out_h, g.out_w, g.kernel_h, g.kernel_w, 1, 1, g.pad_h, g.pad_w};
+    w.dil = g.dil_h;
+    return w;
+}
 
 template <typename T>
 int general_forward_any(const T *in, const T *taps, T *out, int batch, int channel, int in_h, int in_w, int multiplier,
@@ -400,6 +412,18 @@ int general_forward_any(const T *in, const T *taps, T *out, int batch, int chann
     const long long out_elems = 1ll * batch * channel * multiplier * g.out_h * g.out_w;
     if (out_elems > 0 && (in == nullptr || taps == nullptr || out == nullptr))
         return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");
+    if constexpr (!std::is_same<T, double>::value) {
+        if (!force_generic() && out_elems > 0) {
+            int r = try_launch_general_stack_forward<T>(in, taps, out, g, static_cast<hipStream_t>(stream));
+            if (r >= 0) return r;
+            if (dilated_small(g)) {
+                const Geometry gg{batch, channel, in_h, in_w, kernel_h, kernel_w, 1, 1, 1, 1, pad_h, pad_h, pad_w, pad_w,
+                                  g.out_h, g.out_w, 1};
+                r = try_launch_fir_small<T>(in, taps, out, gg, static_cast<hipStream_t>(stream), g.dil_h);
+                if (r >= 0) return r;
+            }
+        }
+    }
     return general_forward<T>(in, taps, out, g, static_cast<hipStream_t>(stream));
 }
 
@@ -411,7 +435,16 @@ size_t general_workspace_any(const GeneralGeometry &g)
                               g.stride_h, g.stride_w, g.pad_h, g.pad_w};
         return wgrad_workspace<T>(w);
     }
-    return general_grad_weight_workspace<T>(g);
+    size_t need = general_grad_weight_workspace<T>(g);
+    if constexpr (!std::is_same<T, double>::value) {
+        const size_t st = general_stack_workspace(g);
+        if (st > need) need = st;
+        if (dilated_small(g)) {
+            const size_t sm = wgrad_small_workspace(dilated_wgrad_geometry(g));
+            if (sm > need) need = sm;
+        }
+    }
+    return need;
 }
 
 template <typename T>
@@ -446,6 +479,16 @@ int general_backward_any(const T *in, const T *gy, const T *taps, T *gx, T *gw, 
     if (has_out && (gy == nullptr || taps == nullptr || (in_h > 0 && in_w > 0 && in == nullptr)))
         return fail(DWCONV_ERR_INVALID_ARGUMENT, "null device pointer");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if constexpr (!std::is_same<T, double>::value) {
+        if (has_out && !force_generic()) {
+            rc = try_launch_general_stack_backward<T>(in, gy, taps, gx, gw, ws, ws_bytes, g, stream);
+            if (rc >= 0) return rc;
+            if (dilated_small(g)) {
+                rc = try_launch_bwd_small<T>(in, gy, taps, gx, gw, ws, ws_bytes, dilated_wgrad_geometry(g), stream);
+                if (rc >= 0) return rc;
+            }
+        }
+    }
     rc = general_grad_input<T>(gy, taps, gx, g, stream);
     if (rc != DWCONV_OK) return rc;
     return general_grad_weight<T>(in, gy, gw, ws, ws_bytes, g, stream);

@@ -159,6 +159,7 @@ struct WgradGeometry {
     int kernel_h, kernel_w;
     int down_h, down_w;
     int pad_h, pad_w;
+    int dil = 1;  // dilation of the taps, both axes (the whole-plane kernels take 2 for 3x3 / 5x5 at stride 1)
 };
 
 // Geometry of a channels-last call: input (N,H,W,C), output (N,OH,OW,C), taps (C,1,KH,KW).
@@ -219,9 +220,10 @@ int try_launch_fir_tiled(const IO *in, const IO *taps, IO *out, const Geometry &
 template <typename IO>
 int try_launch_fir_tiled16(const IO *in, const IO *taps, IO *out, const Geometry &g, hipStream_t stream);
 
-// ---- whole-plane kernels for maps 7, 14 or 28 wide: dwconv_small.hip (same return convention) ----
+// ---- whole-plane kernels for maps up to 32 wide: dwconv_small.hip (same return convention) ----
+// dil: dilation of the taps (1, or 2 for 3x3 / 5x5 forward at stride 1 with padding 2 * (K/2))
 template <typename IO>  // float, half_t or bf16_t
-int try_launch_fir_small(const IO *in, const IO *taps, IO *out, const Geometry &g, hipStream_t stream);
+int try_launch_fir_small(const IO *in, const IO *taps, IO *out, const Geometry &g, hipStream_t stream, int dil = 1);
 
 size_t wgrad_small_workspace(const WgradGeometry &g);  // 0 when the whole-plane kernel does not cover g
 template <typename IO>
@@ -261,6 +263,13 @@ int try_launch_bwd_stack(const IO *in, const IO *gy, const IO *taps, IO *gx, IO 
                          const WgradGeometry &g, hipStream_t stream);
 template <typename IO>
 int try_launch_fir_stack(const IO *in, const IO *taps, IO *out, const Geometry &g, hipStream_t stream);
+// The same kernels at dilation 2 (3x3 and 5x5 taps, multiplier 1, stride 1, padding 2 * (K/2)).
+size_t general_stack_workspace(const GeneralGeometry &g);  // 0 when they do not cover g
+template <typename IO>
+int try_launch_general_stack_forward(const IO *in, const IO *taps, IO *out, const GeneralGeometry &g, hipStream_t stream);
+template <typename IO>
+int try_launch_general_stack_backward(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws,
+                                      size_t ws_bytes, const GeneralGeometry &g, hipStream_t stream);
 
 // The same for stride-2 layers: dwconv_bwd_s2.hip.
 size_t bwd_s2_workspace(const WgradGeometry &g);  // 0 when that kernel does not cover g

@@ -13,12 +13,13 @@ long small_bwd_any(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, 
     if (env_int("DWCONV_NO_SMALL", 0)) return -1;
     const int K = g.kernel_h, S = g.down_h;
     if (g.kernel_w != K || g.down_w != S || (S != 1 && S != 2)) return -1;
-    if (g.pad_w != K / 2 || g.pad_h < 0 || g.pad_h > 7) return -1;
+    if (g.dil != 1 && (g.dil != 2 || S != 1 || K > 5)) return -1;
+    if (g.pad_w != g.dil * (K / 2) || g.pad_h < 0 || g.pad_h > 7) return -1;
     if (g.in_h < 1 || g.in_h > 64 || g.out_h < 1 || g.out_h > 64) return -1;
     if (g.in_w < 1 || g.out_w != (g.in_w - 1) / S + 1) return -1;
     if (mode == 2) {
         // the fused variant writes every gx row from the lane that owns the matching gy rows
-        if (g.pad_h != K / 2) return -1;
+        if (g.pad_h != g.dil * (K / 2)) return -1;
         if (S == 1 && g.out_h != g.in_h) return -1;
         if (S == 2 && g.out_h != (g.in_h - 1) / 2 + 1) return -1;
         if (!aligned4(gx)) return -1;

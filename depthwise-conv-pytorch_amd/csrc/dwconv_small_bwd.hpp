@@ -98,7 +98,8 @@ __device__ __forceinline__ void run_commit_rows(const IO *__restrict__ g, float 
 }
 
 // PAD: LDS rows of 8, 16 or 32 floats get four spare floats (see lds_row_pitch)
-template <typename IO, int W, bool RAG, int K, int S, int BH, bool GX, bool PAD,
+// D: dilation of the taps (stride 1 only; the padding is then D * (K/2)).
+template <typename IO, int W, bool RAG, int K, int S, int BH, bool GX, bool PAD, int D = 1,
           bool PF = (sizeof(IO) == 2 || (K < 7 && (RAG || W <= 28 || K == 3)))>
 __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
 {
@@ -107,9 +108,11 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
     constexpr int OW = (W - 1) / S + 1;  // gy columns a lane handles (the real count when exact)
     constexpr int RR = run_regs(W);
     const int w_in = RAG ? p.in_w : W, w_out = RAG ? p.out_w : OW;
-    constexpr int PW = K / 2;
+    constexpr int KE = (K - 1) * D + 1;  // rows and columns the dilated taps span
+    constexpr int PW = D * (K / 2);
+    static_assert(D == 1 || S == 1, "dilation comes with stride 1");
     constexpr int KK = K * K;
-    constexpr int WIN_ROWS = (BH - 1) * S + K;
+    constexpr int WIN_ROWS = (BH - 1) * S + KE;
     static_assert(S == 1 || BH == 1, "stride-2 lanes own one gy row");
 
     const int group = blockIdx.x / p.chunks;
@@ -196,13 +199,14 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
                 if (wr + 1 < WIN_ROWS) lds_load_row_w<W, RAG>(row_at(oy0 * S - p.pad_h + wr + 1), nxt, w_in);
 #pragma unroll
                 for (int b = 0; b < BH; ++b) {
-                    const int ty = wr - b * S;
-                    if (ty < 0 || ty >= K) continue;
+                    const int dy = wr - b * S;
+                    if (dy < 0 || dy >= KE || dy % D != 0) continue;
+                    const int ty = dy / D;
 #pragma unroll
                     for (int tx = 0; tx < K; ++tx)
 #pragma unroll
                         for (int o = 0; o < OW; ++o) {
-                            const int ix = o * S - PW + tx;
+                            const int ix = o * S - PW + tx * D;
                             if (ix < 0 || ix >= W) continue;
                             wacc[ty * K + tx] = fmaf(g[b][o], row[ix], wacc[ty * K + tx]);
                         }
@@ -226,20 +230,21 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
                 float nxt[OW];
                 lds_load_row_w<OW, RAG>(grow_at(oy0 - PW), nxt, w_out);
 #pragma unroll
-                for (int wr = 0; wr < BH - 1 + K; ++wr) {
+                for (int wr = 0; wr < BH - 1 + KE; ++wr) {
                     float row[OW];
 #pragma unroll
                     for (int i = 0; i < OW; ++i) row[i] = nxt[i];
-                    if (wr + 1 < BH - 1 + K) lds_load_row_w<OW, RAG>(grow_at(oy0 - PW + wr + 1), nxt, w_out);
+                    if (wr + 1 < BH - 1 + KE) lds_load_row_w<OW, RAG>(grow_at(oy0 - PW + wr + 1), nxt, w_out);
 #pragma unroll
                     for (int b = 0; b < BH; ++b) {
-                        const int ty = wr - b;
-                        if (ty < 0 || ty >= K) continue;
+                        const int dy = wr - b;
+                        if (dy < 0 || dy >= KE || dy % D != 0) continue;
+                        const int ty = dy / D;
 #pragma unroll
                         for (int tx = 0; tx < K; ++tx)
 #pragma unroll
                             for (int o = 0; o < W; ++o) {
-                                const int ix = o - PW + tx;
+                                const int ix = o - PW + tx * D;
                                 if (ix < 0 || ix >= OW) continue;
                                 xacc[b][o] = fmaf(row[ix], tapv[ty * K + tx], xacc[b][o]);
                             }
@@ -248,8 +253,8 @@ __global__ __launch_bounds__(kWave) void small_bwd_kernel(const SmallBwdPlan p)
                 }
             } else {
                 // gx[2q + r] = sum_a gy[q - M + r + a] * rot'[r + 2a], rot'[t] = rot[t - E]  (see small_up2_kernel)
-                constexpr int E = PW & 1;
-                constexpr int M = (PW + E) / 2;
+                constexpr int E = (K / 2) & 1;
+                constexpr int M = (K / 2 + E) / 2;
                 constexpr int KA = (K + E + 1) / 2;
                 float nxt[OW];
                 lds_load_row_w<OW, RAG>(grow_at(rb - M), nxt, w_out);
@@ -355,7 +360,7 @@ bool plan_small_bwd(SmallBwdPlan &p, const WgradGeometry &g)
     return true;
 }
 
-template <typename IO, int W, bool RAG, int K, int S, int BH, bool PAD>
+template <typename IO, int W, bool RAG, int K, int S, int BH, bool PAD, int D = 1>
 long small_bwd_case(int mode, const SmallBwdArgs &a, const WgradGeometry &g, hipStream_t stream)
 {
     SmallBwdPlan p{};
@@ -376,13 +381,14 @@ long small_bwd_case(int mode, const SmallBwdArgs &a, const WgradGeometry &g, hip
     const size_t shmem = runs > red ? runs : red;
     const int groups = ceil_div(g.channel, p.planes_per_run);
     if (mode == 2)
-        hipLaunchKernelGGL((small_bwd_kernel<IO, W, RAG, K, S, BH, true, PAD>), dim3(groups * p.chunks), dim3(kWave), shmem, stream, p);
+        hipLaunchKernelGGL((small_bwd_kernel<IO, W, RAG, K, S, BH, true, PAD, D>), dim3(groups * p.chunks), dim3(kWave), shmem, stream, p);
     else
-        hipLaunchKernelGGL((small_bwd_kernel<IO, W, RAG, K, S, BH, false, PAD>), dim3(groups * p.chunks), dim3(kWave), shmem, stream, p);
+        hipLaunchKernelGGL((small_bwd_kernel<IO, W, RAG, K, S, BH, false, PAD, D>), dim3(groups * p.chunks), dim3(kWave), shmem, stream, p);
     const int rc = check_launch("small_bwd_kernel");
     if (rc != DWCONV_OK) return rc;
-    note_variant("%s%s<%s%d,k%d,s%d,bh%d%s> P%d chunks%d", mode == 2 ? "small_bwd" : "small_wgrad",
-                 sizeof(IO) == 2 ? "16" : "", RAG ? "r" : "w", W, K, S, BH, PAD ? ",pad" : "", p.planes_per_run, p.chunks);
+    note_variant("%s%s<%s%d,k%d,s%d,bh%d%s%s> P%d chunks%d", mode == 2 ? "small_bwd" : "small_wgrad",
+                 sizeof(IO) == 2 ? "16" : "", RAG ? "r" : "w", W, K, S, BH, PAD ? ",pad" : "", D == 2 ? ",d2" : "",
+                 p.planes_per_run, p.chunks);
     return launch_wgrad_final(p.partial, static_cast<IO *>(a.gw), g.channel, K * K, p.chunks, stream);
 }
 
@@ -398,6 +404,13 @@ long small_bwd_s(int mode, const SmallBwdArgs &a, const WgradGeometry &g, hipStr
     // 16-wide ones at stride 2 (one row per lane: 47.5 -> 42.6 us); 16-wide stride 1 (two rows per lane) and 8-wide
     // maps did not change
     constexpr bool PAD1 = !RAG && W == 32, PAD2 = !RAG && (W == 32 || W == 16);
+    if (g.dil != 1) {
+        // dilation 2: stride 1, 3x3 and 5x5 taps, both gradients
+        if constexpr (K <= 5) {
+            if (g.dil == 2 && g.down_h == 1) return small_bwd_case<IO, W, RAG, K, 1, BH1, PAD1, 2>(mode, a, g, stream);
+        }
+        return -1;
+    }
     if (g.down_h == 1) return small_bwd_case<IO, W, RAG, K, 1, BH1, PAD1>(mode, a, g, stream);
     if (g.down_h == 2) return small_bwd_case<IO, W, RAG, K, 2, 1, PAD2>(mode, a, g, stream);
     return -1;

@@ -38,10 +38,10 @@ struct SmallPlan {
 };
 
 // Launches the forward / grad-input kernel of width instance (W, RAG) for p: K in {3,5,7}; up2 = false: decimation
-// S in {1,2}, taps rotated if `rot`; up2 = true: the transposed stride-2 problem.  -1 when the instance does not
-// cover the case.
+// S in {1,2}, taps rotated if `rot`, dilation D (2 only for 3x3 / 5x5 forward at stride 1); up2 = true: the
+// transposed stride-2 problem.  -1 when the instance does not cover the case.
 template <int W, bool RAG, typename IO>
-int small_fir_width(SmallPlan &p, int K, int S, bool rot, bool up2, hipStream_t stream);
+int small_fir_width(SmallPlan &p, int K, int S, int D, bool rot, bool up2, hipStream_t stream);
 
 struct SmallBwdArgs {
     const void *x;    // element type IO

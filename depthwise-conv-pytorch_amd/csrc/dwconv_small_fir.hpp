@@ -33,14 +33,16 @@ namespace dwconv {
 namespace {
 
 // out[oy,ox] = sum_{ty,tx} in[oy*S - pad_h + ty, ox*S - K/2 + tx] * f[ty,tx]
-template <typename IO, int W, bool RAG, int K, int S, bool FLIP, int BH>
+// D: dilation of the taps (both axes; the column padding is then D * (K/2)).
+template <typename IO, int W, bool RAG, int K, int S, bool FLIP, int BH, int D = 1>
 __global__ __launch_bounds__(kWave) void small_down_kernel(const SmallPlan p)
 {
     extern __shared__ float4 lds_raw[];
     float *lds = reinterpret_cast<float *>(lds_raw);
     constexpr int OW = (W - 1) / S + 1;  // output columns a lane computes (the real count when exact)
-    constexpr int PW = K / 2;
-    constexpr int WIN_ROWS = (BH - 1) * S + K;
+    constexpr int KE = (K - 1) * D + 1;  // rows and columns the dilated taps span
+    constexpr int PW = D * (K / 2);
+    constexpr int WIN_ROWS = (BH - 1) * S + KE;
     const int w_in = RAG ? p.in_w : W, w_out = RAG ? p.out_w : OW;
 
     const long plane0 = static_cast<long>(blockIdx.x) * p.planes_per_run;
@@ -90,13 +92,14 @@ __global__ __launch_bounds__(kWave) void small_down_kernel(const SmallPlan p)
         if (wr + 1 < WIN_ROWS) lds_load_row_w<W, RAG>(row_at(oy0 * S - p.pad_h + wr + 1), nxt, w_in);
 #pragma unroll
         for (int b = 0; b < BH; ++b) {
-            const int ty = wr - b * S;
-            if (ty < 0 || ty >= K) continue;
+            const int dy = wr - b * S;
+            if (dy < 0 || dy >= KE || dy % D != 0) continue;
+            const int ty = dy / D;
 #pragma unroll
             for (int tx = 0; tx < K; ++tx)
 #pragma unroll
                 for (int o = 0; o < OW; ++o) {
-                    const int ix = o * S - PW + tx;
+                    const int ix = o * S - PW + tx * D;
                     if (ix < 0 || ix >= W) continue;
                     acc[b][o] = fmaf(row[ix], tapv[ty * K + tx], acc[b][o]);
                 }
@@ -260,17 +263,17 @@ bool finish_plan(SmallPlan &p, size_t &shmem, long &runs, int spare, int zero_fl
     return true;
 }
 
-template <typename IO, int W, bool RAG, int K, int S, bool FLIP, int BH>
+template <typename IO, int W, bool RAG, int K, int S, bool FLIP, int BH, int D = 1>
 int launch_small_down(SmallPlan &p, hipStream_t stream)
 {
     p.lanes_per_plane = ceil_div(p.out_h, BH);
     size_t shmem;
     long runs;
     if (!finish_plan(p, shmem, runs, RAG ? W : 0, zero_row_floats(W), RAG)) return -1;
-    hipLaunchKernelGGL((small_down_kernel<IO, W, RAG, K, S, FLIP, BH>), dim3(static_cast<unsigned>(runs)), dim3(kWave),
+    hipLaunchKernelGGL((small_down_kernel<IO, W, RAG, K, S, FLIP, BH, D>), dim3(static_cast<unsigned>(runs)), dim3(kWave),
                        shmem, stream, p);
-    note_variant("small_down%s<%s%d,k%d,s%d,%s,bh%d> P%d", sizeof(IO) == 2 ? "16" : "", RAG ? "r" : "w", W, K, S,
-                 FLIP ? "rot" : "fwd", BH, p.planes_per_run);
+    note_variant("small_down%s<%s%d,k%d,s%d,%s,bh%d%s> P%d", sizeof(IO) == 2 ? "16" : "", RAG ? "r" : "w", W, K, S,
+                 FLIP ? "rot" : "fwd", BH, D == 2 ? ",d2" : "", p.planes_per_run);
     return check_launch("small_down_kernel");
 }
 
@@ -330,8 +333,16 @@ int launch_small_down_any(SmallPlan &p, int S, bool rot, hipStream_t stream)
 }  // namespace
 
 template <int W, bool RAG, typename IO>
-int small_fir_width(SmallPlan &p, int K, int S, bool rot, bool up2, hipStream_t stream)
+int small_fir_width(SmallPlan &p, int K, int S, int D, bool rot, bool up2, hipStream_t stream)
 {
+    if (D != 1) {
+        // dilation 2: forward, stride 1, 3x3 and 5x5 taps; rows per lane as for the undilated filter of the same span
+        if (D != 2 || S != 1 || rot || up2) return -1;
+        constexpr int BHD = W <= 8 ? 2 : (W <= 16 ? 2 : 1);
+        if (K == 3) return launch_small_down<IO, W, RAG, 3, 1, false, BHD, 2>(p, stream);
+        if (K == 5) return launch_small_down<IO, W, RAG, 5, 1, false, BHD, 2>(p, stream);
+        return -1;
+    }
     if (up2) {
         if constexpr (W <= 16) {
             if (K == 3) return launch_small_up2<IO, W, RAG, 3>(p, stream);

@@ -11,7 +11,7 @@
 
 namespace dwconv {
 #define DWCONV_INSTANTIATE(IO) \
-    template int small_fir_width<DWCONV_SMALL_W, DWCONV_SMALL_RAG != 0, IO>(SmallPlan &, int, int, bool, bool, hipStream_t);
+    template int small_fir_width<DWCONV_SMALL_W, DWCONV_SMALL_RAG != 0, IO>(SmallPlan &, int, int, int, bool, bool, hipStream_t);
 DWCONV_INSTANTIATE(float)
 DWCONV_INSTANTIATE(half_t)
 DWCONV_INSTANTIATE(bf16_t)

@@ -71,7 +71,7 @@ struct StackTile {
 };
 
 // The tile whose first unit is row unit r0 of image n0 (n0 * ru + r0 < total_units).
-__device__ __forceinline__ StackTile stack_tile(const StackPlan &p, int n0, int r0, int c, int K)
+__device__ __forceinline__ StackTile stack_tile(const StackPlan &p, int n0, int r0, int c, int KE)
 {
     StackTile t;
     t.n0 = n0;
@@ -80,7 +80,7 @@ __device__ __forceinline__ StackTile stack_tile(const StackPlan &p, int n0, int 
     const int ql = r0 + t.units_here - 1;  // last unit of the tile, counted from image n0's first
     const int nl = div_magic(ql, p.ru_magic), rl = ql - nl * p.ru;
     t.vrel0 = r0 * kStackBH;
-    t.rows = nl * p.vh + rl * kStackBH + kStackBH + K - 1 - t.vrel0;
+    t.rows = nl * p.vh + rl * kStackBH + kStackBH + KE - 1 - t.vrel0;
     t.n_span = min(p.batch - n0, nl + 2);
     t.plane0 = static_cast<long>(n0) * p.channel + c;
     return t;
@@ -94,7 +94,7 @@ struct StackLane {
     int dcol;      // float offset of the column within an LDS row
 };
 
-template <typename IO, int K>
+template <typename IO, int PADW>
 __device__ __forceinline__ StackLane stack_lane(const StackPlan &p)
 {
     StackLane l;
@@ -103,7 +103,7 @@ __device__ __forceinline__ StackLane stack_lane(const StackPlan &p)
     l.jr = jr < p.rpp ? jr : (1 << 20);
     l.coff = static_cast<unsigned>(ix) * static_cast<unsigned>(sizeof(IO));
     l.col_ok = static_cast<unsigned>(ix) < static_cast<unsigned>(p.w);
-    l.dcol = kSlack + ix + K / 2;
+    l.dcol = kSlack + ix + PADW;
     return l;
 }
 
@@ -112,11 +112,10 @@ __device__ __forceinline__ StackLane stack_lane(const StackPlan &p)
 // commit_stack writes them into the LDS image.  LDS row j, column kSlack + ix + K/2 holds column ix of stacked row
 // vrel0 + j of the tensor whose (image n0, channel c) plane starts at `src`; zero rows, columns outside the plane
 // and images past n_span read zeros through the view.
-template <typename IO, int K, int NS>
+template <typename IO, int PADW, int NS>
 __device__ __forceinline__ void fetch_stack(const StackPlan &p, const StackLane &l, const IO *__restrict__ src, const StackTile &t,
                                             typename Raw4<IO>::type (&v)[NS])
 {
-    constexpr int PW = K / 2;
     constexpr unsigned ES = sizeof(IO);
     const long extent = (static_cast<long>(t.n_span - 1) * p.img_stride + p.plane) * ES;
     const __amdgpu_buffer_rsrc_t view = buffer_view(src, extent);
@@ -125,7 +124,7 @@ __device__ __forceinline__ void fetch_stack(const StackPlan &p, const StackLane 
         const int j = l.jr + u * p.rpp;
         const int vr = t.vrel0 + min(j, t.rows);   // (rows past the tile: any row, the load is switched off)
         const int n = div_magic(vr, p.vh_magic);
-        const int rr = vr - __mul24(n, p.vh) - PW;
+        const int rr = vr - __mul24(n, p.vh) - PADW;
         const bool ok = j < t.rows && l.col_ok && rr >= 0 && n < t.n_span;
         const unsigned off = (static_cast<unsigned>(n) * static_cast<unsigned>(p.img_stride) + __mul24(rr, p.w)) * ES + l.coff;
         if constexpr (sizeof(IO) == 4) {
@@ -138,7 +137,7 @@ __device__ __forceinline__ void fetch_stack(const StackPlan &p, const StackLane 
     }
 }
 
-template <typename IO, int K, int NS>
+template <typename IO, int NS>
 __device__ __forceinline__ void commit_stack(const StackPlan &p, const StackLane &l, float *lds, const StackTile &t,
                                              const typename Raw4<IO>::type (&v)[NS])
 {
@@ -161,16 +160,19 @@ __device__ __forceinline__ void commit_stack(const StackPlan &p, const StackLane
 // Order of a fused tile, two barriers: [gy of this tile is in registers] commit gy | barrier | issue the loads of x |
 // slide the taps over the gy windows (grad-input out, own gy block kept) | commit x | barrier | issue the loads of the
 // next tile's gy | grad-weight sums over the x windows.  Every image's loads fly during one arithmetic phase.
-template <typename IO, int K, bool FUSED, bool FLIP, int NS>
+// D: dilation (both axes); the window then spans KE = (K - 1) * D + 1 rows and columns and the "same" padding is
+// D * (K/2).
+template <typename IO, int K, int D, bool FUSED, bool FLIP, int NS>
 __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
 {
     extern __shared__ float4 lds_raw[];
     float *lds = reinterpret_cast<float *>(lds_raw);
     constexpr int BH = kStackBH;
-    constexpr int PW = K / 2;
+    constexpr int KE = (K - 1) * D + 1;
+    constexpr int PW = D * (K / 2);
     constexpr int KK = K * K;
-    constexpr int WIN_ROWS = BH - 1 + K;
-    constexpr int NV = (K + 6) / 4;  // float4s that hold a window row: columns 4*cb - K/2 ... 4*cb + 3 + K/2
+    constexpr int WIN_ROWS = BH - 1 + KE;
+    constexpr int NV = (3 + KE + 3) / 4;  // float4s that hold a window row: columns 4*cb - PW ... 4*cb + 3 + PW
     constexpr unsigned ES = sizeof(IO);
 
     const int c = blockIdx.x / p.chunks;
@@ -180,13 +182,13 @@ __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
     float *const lds_x = lds + p.img_floats;        // fused: the image of x
 
     typename Raw4<IO>::type staged[NS];
-    const StackLane lane = stack_lane<IO, K>(p);
+    const StackLane lane = stack_lane<IO, PW>(p);
     // chunk k takes tiles k, k + chunks, ...: the first unit of the next tile lies step_n images and step_r row
     // units further on
     const int u_first = chunk * p.units_per_tile;
     const int n_first = u_first / p.ru;
-    StackTile cur = stack_tile(p, n_first, u_first - n_first * p.ru, c, K);
-    fetch_stack<IO, K, NS>(p, lane, slide_src + cur.plane0 * p.plane, cur, staged);
+    StackTile cur = stack_tile(p, n_first, u_first - n_first * p.ru, c, KE);
+    fetch_stack<IO, PW, NS>(p, lane, slide_src + cur.plane0 * p.plane, cur, staged);
 
     // the taps of the sliding pass, wavefront-uniform: scalar registers
     float tap[KK];
@@ -211,16 +213,16 @@ __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
         // (forward: the windows of the previous tile are read until here; fused: the slide image was last read
         // before the previous tile's second barrier)
         if (!FUSED && tile != chunk) __syncthreads();
-        commit_stack<IO, K, NS>(p, lane, lds_slide, cur, staged);
+        commit_stack<IO, NS>(p, lane, lds_slide, cur, staged);
         __syncthreads();
         StackTile nxt_tile = cur;
         if (more) {
             const int r_raw = cur.r0 + p.step_r;
             const bool carry = r_raw >= p.ru;
-            nxt_tile = stack_tile(p, cur.n0 + p.step_n + (carry ? 1 : 0), carry ? r_raw - p.ru : r_raw, c, K);
+            nxt_tile = stack_tile(p, cur.n0 + p.step_n + (carry ? 1 : 0), carry ? r_raw - p.ru : r_raw, c, KE);
         }
-        if constexpr (FUSED) fetch_stack<IO, K, NS>(p, lane, static_cast<const IO *>(p.x) + cur.plane0 * p.plane, cur, staged);
-        else if (more) fetch_stack<IO, K, NS>(p, lane, slide_src + nxt_tile.plane0 * p.plane, nxt_tile, staged);
+        if constexpr (FUSED) fetch_stack<IO, PW, NS>(p, lane, static_cast<const IO *>(p.x) + cur.plane0 * p.plane, cur, staged);
+        else if (more) fetch_stack<IO, PW, NS>(p, lane, slide_src + nxt_tile.plane0 * p.plane, nxt_tile, staged);
 
         // this lane's unit: image n0 + nrel, row unit r
         const int q = cur.r0 + ul;
@@ -256,12 +258,13 @@ __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
                 }
 #pragma unroll
                 for (int b = 0; b < BH; ++b) {
-                    const int ty = wr - b;
-                    if (ty < 0 || ty >= K) continue;
+                    const int dy = wr - b;
+                    if (dy < 0 || dy >= KE || dy % D != 0) continue;
+                    const int ty = dy / D;
 #pragma unroll
                     for (int tx = 0; tx < K; ++tx)
 #pragma unroll
-                        for (int o = 0; o < 4; ++o) sums[b][o] = fmaf(win[o + tx], tap[ty * K + tx], sums[b][o]);
+                        for (int o = 0; o < 4; ++o) sums[b][o] = fmaf(win[o + tx * D], tap[ty * K + tx], sums[b][o]);
                 }
                 pin_registers(sums);
             }
@@ -280,9 +283,9 @@ __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
         }
 
         if constexpr (FUSED) {
-            commit_stack<IO, K, NS>(p, lane, lds_x, cur, staged);
+            commit_stack<IO, NS>(p, lane, lds_x, cur, staged);
             __syncthreads();
-            if (more) fetch_stack<IO, K, NS>(p, lane, slide_src + nxt_tile.plane0 * p.plane, nxt_tile, staged);
+            if (more) fetch_stack<IO, PW, NS>(p, lane, slide_src + nxt_tile.plane0 * p.plane, nxt_tile, staged);
             const float *base = lds_x + base_off;
             float nxt[4 * NV];
             load_window_row<NV>(base, nxt);
@@ -294,12 +297,13 @@ __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
                 if (wr + 1 < WIN_ROWS) load_window_row<NV>(base + (wr + 1) * p.pitch, nxt);
 #pragma unroll
                 for (int b = 0; b < BH; ++b) {
-                    const int ty = wr - b;
-                    if (ty < 0 || ty >= K) continue;
+                    const int dy = wr - b;
+                    if (dy < 0 || dy >= KE || dy % D != 0) continue;
+                    const int ty = dy / D;
 #pragma unroll
                     for (int tx = 0; tx < K; ++tx)
 #pragma unroll
-                        for (int o = 0; o < 4; ++o) acc[ty * K + tx] = fmaf(g[b][o], win[o + tx], acc[ty * K + tx]);
+                        for (int o = 0; o < 4; ++o) acc[ty * K + tx] = fmaf(g[b][o], win[o + tx * D], acc[ty * K + tx]);
                 }
                 pin_registers(acc);
             }
@@ -325,12 +329,16 @@ __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
     }
 }
 
-// Geometry the stacked kernels take: stride 1, "same" padding, K x K with K in {5, 7}, rows of whole groups of four
-// elements, and a plane too large for two of them to share a workgroup (those shapes keep the several-planes mode of
-// the general kernels).
-bool make_plan(StackPlan &p, int K, int batch, int channel, int h, int w, size_t esize, bool fused, int target_wgs)
+// Geometry the stacked kernels take: stride 1, "same" padding D * (K/2), K x K taps at dilation D with (K, D) in
+// {(5,1), (7,1), (3,2), (5,2)}, rows of whole groups of four elements, and a plane too large for two of them to share a
+// workgroup (those shapes keep the several-planes mode of the general kernels).
+// (3x3 at dilation 1 stays with the general kernels: they wait for HBM, not for the vector unit, and measured the same
+// or faster: 112x112 C=32 fused backward 124-130 us here against 127, 56x56 C=144 152-158 against 132-144)
+bool stack_shape(int K, int D) { return (D == 1 && (K == 5 || K == 7)) || (D == 2 && (K == 3 || K == 5)); }
+
+bool make_plan(StackPlan &p, int K, int D, int batch, int channel, int h, int w, size_t esize, bool fused, int target_wgs)
 {
-    if (K != 5 && K != 7) return false;
+    if (!stack_shape(K, D)) return false;
     if (w % 4 != 0 || w < 16 || h < 8) return false;
     const int ncb = w / 4;
     if (ncb > kThreads) return false;
@@ -338,6 +346,7 @@ bool make_plan(StackPlan &p, int K, int batch, int channel, int h, int w, size_t
     if (2 * ru * ncb <= kThreads) return false;
     const long plane = static_cast<long>(h) * w;
     if (plane >= (1l << 23) || static_cast<long>(channel) * plane >= (1l << 28)) return false;
+    const int ke = (K - 1) * D + 1, padw = D * (K / 2);
     p.batch = batch;
     p.channel = channel;
     p.h = h;
@@ -345,16 +354,16 @@ bool make_plan(StackPlan &p, int K, int batch, int channel, int h, int w, size_t
     p.plane = static_cast<int>(plane);
     p.img_stride = static_cast<int>(channel * plane);
     p.ru = ru;
-    p.vh = h + K / 2;
+    p.vh = h + padw;
     p.ncb = ncb;
-    p.pitch = w + 16;  // kSlack + K/2 columns of zeros + w + zeros up to the last window column + kSlack, rounded up
+    p.pitch = w + 16;  // kSlack + padw (<= 4) columns of zeros + w + zeros up to the last window column + kSlack, rounded up
     p.spr = ncb + 2;
     const long total_units = static_cast<long>(batch) * ru;
     if (total_units >= (1l << 30)) return false;
     p.total_units = static_cast<int>(total_units);
     const int budget = env_int("DWCONV_STACK_LDS", 56 * 1024);
     int units = kThreads / ncb;
-    auto rows_for = [&](int u) { return u * kStackBH + K - 1 + (K / 2) * ((u - 1) / ru + 2); };
+    auto rows_for = [&](int u) { return u * kStackBH + ke - 1 + padw * ((u - 1) / ru + 2); };
     // (and at most eight loads per lane and image: they wait in registers while the workgroup computes)
     p.rpp = kThreads / p.spr;
     while (units > 1 && (static_cast<long>(rows_for(units)) * p.pitch * 4 * (fused ? 2 : 1) > budget ||
@@ -366,7 +375,7 @@ bool make_plan(StackPlan &p, int K, int batch, int channel, int h, int w, size_t
     const int rows = rows_for(units);
     p.img_floats = rows * p.pitch;
     p.slots_per_lane = ceil_div(rows, p.rpp);
-    // 16-bit reciprocals: slots of an image, stacked rows of a tile, units counted from the tile's first image
+    // 16-bit reciprocals: stacked rows of a tile, units counted from the tile's first image
     if (rows + p.vh >= 65536 || ru + units >= 65536) return false;
     // a tile's images must lie within one buffer view
     const long span_images = (units - 1) / ru + 3;
@@ -394,41 +403,63 @@ size_t lds_bytes(const StackPlan &p, int K, bool fused)
     return tile > red ? tile : red;
 }
 
-bool covers_bwd(const WgradGeometry &g)
-{
-    const int K = g.kernel_h;
-    if (!env_int("DWCONV_STACK", 1)) return false;
-    if (g.kernel_w != K || g.down_h != 1 || g.down_w != 1 || g.pad_h != K / 2 || g.pad_w != K / 2) return false;
-    if (g.out_h != g.in_h || g.out_w != g.in_w) return false;
-    return true;
-}
-
 // Workgroups of the fused kernel: one resident round (three per compute unit by its registers and LDS) for 7x7
 // filters (56x56 C=96 at batch 64: 768 workgroups 95 us, 1536 105, 2304 104); 5x5 filters do not care (256x256 C=64:
 // 189-197 us from 768 to 6144).
 int bwd_target_wgs(int K) { return env_int("DWCONV_STACK_WGS", K == 7 ? 768 : 1536); }
 
-}  // namespace
-
-size_t bwd_stack_workspace(const WgradGeometry &g)
+// fn.template operator()<K, D>() for the supported (K, D)
+template <typename Fn>
+void for_shape(int K, int D, Fn &&fn)
 {
-    if (!covers_bwd(g)) return 0;
+    if (K == 5 && D == 1) fn.template operator()<5, 1>();
+    if (K == 7 && D == 1) fn.template operator()<7, 1>();
+    if (K == 3 && D == 2) fn.template operator()<3, 2>();
+    if (K == 5 && D == 2) fn.template operator()<5, 2>();
+}
+
+template <typename IO, bool FUSED>
+struct StackLaunch {
+    const StackPlan &p;
+    bool rot;
+    size_t shmem;
+    hipStream_t stream;
+    template <int K, int D>
+    void operator()()
+    {
+        const dim3 grid(static_cast<unsigned>(p.channel * p.chunks)), block(kThreads);
+        const bool six = p.slots_per_lane <= 6;
+        if constexpr (FUSED) {
+            if (six) hipLaunchKernelGGL((stack_kernel<IO, K, D, true, true, 6>), grid, block, shmem, stream, p);
+            else hipLaunchKernelGGL((stack_kernel<IO, K, D, true, true, 8>), grid, block, shmem, stream, p);
+        } else if (rot) {
+            if (six) hipLaunchKernelGGL((stack_kernel<IO, K, D, false, true, 6>), grid, block, shmem, stream, p);
+            else hipLaunchKernelGGL((stack_kernel<IO, K, D, false, true, 8>), grid, block, shmem, stream, p);
+        } else {
+            if (six) hipLaunchKernelGGL((stack_kernel<IO, K, D, false, false, 6>), grid, block, shmem, stream, p);
+            else hipLaunchKernelGGL((stack_kernel<IO, K, D, false, false, 8>), grid, block, shmem, stream, p);
+        }
+    }
+};
+
+size_t stack_backward_workspace(int K, int D, int batch, int channel, int h, int w)
+{
+    if (!env_int("DWCONV_STACK", 1)) return 0;
     StackPlan p{};
     // (the plan does not depend on the element size except through the view-extent check: the larger one)
-    if (!make_plan(p, g.kernel_h, g.batch, g.channel, g.in_h, g.in_w, 4, true, bwd_target_wgs(g.kernel_h))) return 0;
-    return static_cast<size_t>(g.channel) * p.chunks * g.kernel_h * g.kernel_w * sizeof(float);
+    if (!make_plan(p, K, D, batch, channel, h, w, 4, true, bwd_target_wgs(K))) return 0;
+    return static_cast<size_t>(channel) * p.chunks * K * K * sizeof(float);
 }
 
 template <typename IO>
-int try_launch_bwd_stack(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
-                         const WgradGeometry &g, hipStream_t stream)
+int launch_stack_backward(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes, int K, int D,
+                          int batch, int channel, int h, int w, hipStream_t stream)
 {
-    if (!covers_bwd(g)) return -1;
+    if (!env_int("DWCONV_STACK", 1)) return -1;
     if (!aligned4(in) || !aligned4(gy) || !aligned4(gx)) return -1;
-    const int K = g.kernel_h;
     StackPlan p{};
-    if (!make_plan(p, K, g.batch, g.channel, g.in_h, g.in_w, 4, true, bwd_target_wgs(K))) return -1;
-    const size_t need = static_cast<size_t>(g.channel) * p.chunks * K * K * sizeof(float);
+    if (!make_plan(p, K, D, batch, channel, h, w, 4, true, bwd_target_wgs(K))) return -1;
+    const size_t need = static_cast<size_t>(channel) * p.chunks * K * K * sizeof(float);
     if (ws == nullptr || ws_bytes < need)
         return fail(DWCONV_ERR_WORKSPACE, "grad-weight needs a workspace of %zu bytes, got %zu", need, ws_bytes);
     p.x = in;
@@ -436,56 +467,106 @@ int try_launch_bwd_stack(const IO *in, const IO *gy, const IO *taps, IO *gx, IO 
     p.taps = taps;
     p.out = gx;
     p.partial = static_cast<float *>(ws);
-    const size_t shmem = lds_bytes(p, K, true);
-    const dim3 grid(static_cast<unsigned>(g.channel * p.chunks)), block(kThreads);
-    const bool six = p.slots_per_lane <= 6;
-    if (K == 7 && six) hipLaunchKernelGGL((stack_kernel<IO, 7, true, true, 6>), grid, block, shmem, stream, p);
-    else if (K == 7) hipLaunchKernelGGL((stack_kernel<IO, 7, true, true, 8>), grid, block, shmem, stream, p);
-    else if (six) hipLaunchKernelGGL((stack_kernel<IO, 5, true, true, 6>), grid, block, shmem, stream, p);
-    else hipLaunchKernelGGL((stack_kernel<IO, 5, true, true, 8>), grid, block, shmem, stream, p);
+    for_shape(K, D, StackLaunch<IO, true>{p, true, lds_bytes(p, K, true), stream});
     const int rc = check_launch("stack_kernel");
     if (rc != DWCONV_OK) return rc;
-    note_variant("bwd_stack%s<k%d,s1> units%d tiles%d chunks%d", sizeof(IO) == 2 ? "16" : "", K, p.units_per_tile, p.tiles,
-                 p.chunks);
-    return launch_wgrad_final(static_cast<const float *>(ws), gw, g.channel, K * K, p.chunks, stream);
+    note_variant("bwd_stack%s<k%d,d%d,s1> units%d tiles%d chunks%d", sizeof(IO) == 2 ? "16" : "", K, D, p.units_per_tile,
+                 p.tiles, p.chunks);
+    return launch_wgrad_final(static_cast<const float *>(ws), gw, channel, K * K, p.chunks, stream);
+}
+
+template <typename IO>
+int launch_stack_forward(const IO *in, const IO *taps, IO *out, int K, int D, int batch, int channel, int h, int w, bool rot,
+                         hipStream_t stream)
+{
+    if (!env_int("DWCONV_STACK", 1)) return -1;
+    if (!aligned4(in) || !aligned4(out)) return -1;
+    StackPlan p{};
+    // (short-lived workgroups of one tile each measured best: 56x56 C=96 7x7 43 us with 4800, 46-50 with 1280-4096)
+    if (!make_plan(p, K, D, batch, channel, h, w, 4, false, env_int("DWCONV_STACK_FWD_WGS", 8192))) return -1;
+    p.x = in;
+    p.taps = taps;
+    p.out = out;
+    for_shape(K, D, StackLaunch<IO, false>{p, rot, lds_bytes(p, K, false), stream});
+    note_variant("tile_stack%s<k%d,d%d,s1,%s> units%d tiles%d chunks%d", sizeof(IO) == 2 ? "16" : "", K, D, rot ? "rot" : "fwd",
+                 p.units_per_tile, p.tiles, p.chunks);
+    return check_launch("stack_kernel");
+}
+
+bool covers_bwd(const WgradGeometry &g)
+{
+    const int K = g.kernel_h;
+    if (g.kernel_w != K || g.down_h != 1 || g.down_w != 1 || g.pad_h != K / 2 || g.pad_w != K / 2) return false;
+    if (g.out_h != g.in_h || g.out_w != g.in_w) return false;
+    return true;
+}
+
+// dilated, multiplier 1, stride 1, "same" padding: the geometry the dilated instances take
+bool covers_general(const GeneralGeometry &g)
+{
+    const int K = g.kernel_h, D = g.dil_h;
+    if (g.multiplier != 1 || g.kernel_w != K || g.dil_w != D || D < 2) return false;
+    if (g.stride_h != 1 || g.stride_w != 1 || g.pad_h != D * (K / 2) || g.pad_w != D * (K / 2)) return false;
+    if (g.out_h != g.in_h || g.out_w != g.in_w) return false;
+    return stack_shape(K, D);
+}
+
+}  // namespace
+
+size_t bwd_stack_workspace(const WgradGeometry &g)
+{
+    if (!covers_bwd(g)) return 0;
+    return stack_backward_workspace(g.kernel_h, 1, g.batch, g.channel, g.in_h, g.in_w);
+}
+
+template <typename IO>
+int try_launch_bwd_stack(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
+                         const WgradGeometry &g, hipStream_t stream)
+{
+    if (!covers_bwd(g)) return -1;
+    return launch_stack_backward<IO>(in, gy, taps, gx, gw, ws, ws_bytes, g.kernel_h, 1, g.batch, g.channel, g.in_h, g.in_w, stream);
 }
 
 template <typename IO>
 int try_launch_fir_stack(const IO *in, const IO *taps, IO *out, const Geometry &g, hipStream_t stream)
 {
-    if (!env_int("DWCONV_STACK", 1)) return -1;
     const int K = g.kernel_h;
     if (g.kernel_w != K || g.up_h != 1 || g.up_w != 1 || g.down_h != 1 || g.down_w != 1) return -1;
     if (g.pad_h0 != K / 2 || g.pad_w0 != K / 2 || g.out_h != g.in_h || g.out_w != g.in_w) return -1;
     if (g.epi.enabled()) return -1;  // the fused epilogue stays with the general kernel
-    if (!aligned4(in) || !aligned4(out)) return -1;
-    StackPlan p{};
-    if (!make_plan(p, K, g.batch, g.channel, g.in_h, g.in_w, 4, false, env_int("DWCONV_STACK_FWD_WGS", 8192))) return -1;
-    p.x = in;
-    p.taps = taps;
-    p.out = out;
-    const size_t shmem = lds_bytes(p, K, false);
-    const dim3 grid(static_cast<unsigned>(g.channel * p.chunks)), block(kThreads);
-    const bool rot = !g.forward;
-    const bool six = p.slots_per_lane <= 6;
-#define DWCONV_STACK_FWD(KV, ROT)                                                                            \
-    if (six) hipLaunchKernelGGL((stack_kernel<IO, KV, false, ROT, 6>), grid, block, shmem, stream, p);       \
-    else hipLaunchKernelGGL((stack_kernel<IO, KV, false, ROT, 8>), grid, block, shmem, stream, p)
-    if (K == 7) {
-        if (rot) { DWCONV_STACK_FWD(7, true); } else { DWCONV_STACK_FWD(7, false); }
-    } else {
-        if (rot) { DWCONV_STACK_FWD(5, true); } else { DWCONV_STACK_FWD(5, false); }
-    }
-#undef DWCONV_STACK_FWD
-    note_variant("tile_stack%s<k%d,s1,%s> units%d tiles%d chunks%d", sizeof(IO) == 2 ? "16" : "", K, rot ? "rot" : "fwd",
-                 p.units_per_tile, p.tiles, p.chunks);
-    return check_launch("stack_kernel");
+    return launch_stack_forward<IO>(in, taps, out, K, 1, g.batch, g.channel, g.in_h, g.in_w, !g.forward, stream);
+}
+
+size_t general_stack_workspace(const GeneralGeometry &g)
+{
+    if (!covers_general(g)) return 0;
+    return stack_backward_workspace(g.kernel_h, g.dil_h, g.batch, g.channel, g.in_h, g.in_w);
+}
+
+template <typename IO>
+int try_launch_general_stack_forward(const IO *in, const IO *taps, IO *out, const GeneralGeometry &g, hipStream_t stream)
+{
+    if (!covers_general(g)) return -1;
+    return launch_stack_forward<IO>(in, taps, out, g.kernel_h, g.dil_h, g.batch, g.channel, g.in_h, g.in_w, false, stream);
+}
+
+template <typename IO>
+int try_launch_general_stack_backward(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
+                                      const GeneralGeometry &g, hipStream_t stream)
+{
+    if (!covers_general(g)) return -1;
+    return launch_stack_backward<IO>(in, gy, taps, gx, gw, ws, ws_bytes, g.kernel_h, g.dil_h, g.batch, g.channel, g.in_h,
+                                     g.in_w, stream);
 }
 
 #define DWCONV_INSTANTIATE(IO)                                                                                        \
     template int try_launch_bwd_stack<IO>(const IO *, const IO *, const IO *, IO *, IO *, void *, size_t,             \
                                           const WgradGeometry &, hipStream_t);                                        \
-    template int try_launch_fir_stack<IO>(const IO *, const IO *, IO *, const Geometry &, hipStream_t);
+    template int try_launch_fir_stack<IO>(const IO *, const IO *, IO *, const Geometry &, hipStream_t);               \
+    template int try_launch_general_stack_forward<IO>(const IO *, const IO *, IO *, const GeneralGeometry &,          \
+                                                      hipStream_t);                                                   \
+    template int try_launch_general_stack_backward<IO>(const IO *, const IO *, const IO *, IO *, IO *, void *,        \
+                                                       size_t, const GeneralGeometry &, hipStream_t);
 DWCONV_INSTANTIATE(float)
 DWCONV_INSTANTIATE(half_t)
 DWCONV_INSTANTIATE(bf16_t)

@@ -1282,6 +1282,13 @@ GENERAL_CASES = [
     (2, 4, 1, 14, 14, 3, 3, 1, 2, 2), (2, 3, 2, 9, 11, 3, 3, 1, 1, 1), (1, 5, 3, 13, 12, 5, 3, 2, 2, 2),
     (2, 8, 1, 16, 16, 3, 3, 2, 3, 3), (2, 2, 4, 7, 7, 3, 3, 1, 0, 1), (1, 3, 2, 6, 6, 3, 3, 1, 1, 3),
     (2, 6, 1, 20, 24, 3, 3, 1, 1, 1),
+    # dilation 2, stride 1, "same" padding on maps wide enough for the stacked-image kernels (3x3 and 5x5 taps): heights
+    # that leave a hanging unit, tiles across two and three images
+    (2, 3, 1, 40, 48, 3, 3, 1, 2, 2), (3, 2, 1, 33, 64, 5, 5, 1, 4, 2), (5, 2, 1, 57, 52, 3, 3, 1, 2, 2),
+    (7, 1, 1, 18, 96, 5, 5, 1, 4, 2), (2, 2, 1, 130, 128, 3, 3, 1, 2, 2),
+    # dilation 2 on maps up to 32 wide: the whole-plane kernels (exact and ragged widths, odd planes)
+    (3, 8, 1, 14, 14, 3, 3, 1, 2, 2), (2, 6, 1, 28, 28, 5, 5, 1, 4, 2), (3, 8, 1, 7, 7, 3, 3, 1, 2, 2), (2, 4, 1, 16, 16, 5, 5, 1, 4, 2),
+    (2, 8, 1, 15, 15, 3, 3, 1, 2, 2), (3, 5, 1, 9, 30, 5, 5, 1, 4, 2), (2, 3, 1, 32, 32, 3, 3, 1, 2, 2), (2, 4, 1, 20, 24, 3, 3, 1, 2, 2),
 ]
 
 
@@ -1303,7 +1310,16 @@ def test_dilation_and_depth_multiplier(dw, gpu, case, dtype):
     gx, gw = torch.autograd.grad(y, (xg, wg), gy.to(gpu))
     _announce(case, str(dtype), v_fwd, "|", _C.last_variant())
     plain = m == 1 and d == 1
-    assert v_fwd.startswith("general_fwd") != plain, v_fwd  # the plain case runs the tuned kernels
+    stacked = (m == 1 and d == 2 and s == 1 and kh == kw and kh in (3, 5) and p == d * (kh // 2) and w % 4 == 0 and w >= 16
+               and h >= 8 and 2 * ((h + 3) // 4) * (w // 4) > 256 and dtype != torch.float64)
+    small = (m == 1 and d == 2 and s == 1 and kh == kw and kh in (3, 5) and p == d * (kh // 2) and w <= 32 and h <= 64
+             and dtype != torch.float64)
+    if stacked:
+        assert v_fwd.startswith("tile_stack") and _C.last_variant() is not None, v_fwd
+    elif small:
+        assert v_fwd.startswith("small_down") and ",d2" in v_fwd, v_fwd
+    else:
+        assert v_fwd.startswith("general_fwd") != plain, v_fwd  # the plain case runs the tuned kernels
     y_ref, gx_ref, gw_ref = oracle.torch_reference_general(x, wt, gy, s, p, d)
     tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-12, atol=1e-12)
     np.testing.assert_allclose(_np(y.detach()).astype(np.float64), y_ref.numpy(), **tol)
