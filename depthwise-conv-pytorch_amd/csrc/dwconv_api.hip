@@ -511,8 +511,9 @@ constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 void *g_scratch_ptr[kMaxDevices] = {};
 
-// Address of `scratch` on the current device (looked up once per device).
-int scratch_of_current_device(void **ptr)
+// Address of `scratch` on the current device (looked up once per device).  The lookup is not a call to make
+// while `stream` records a graph: a first call that arrives under capture is refused instead.
+int scratch_of_current_device(void **ptr, hipStream_t stream)
 {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
@@ -520,6 +521,14 @@ int scratch_of_current_device(void **ptr)
     if (dev < 0 || dev >= kMaxDevices) return fail(DWCONV_ERR_UNSUPPORTED, "device ordinal %d out of range", dev);
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
     if (g_scratch_ptr[dev] == nullptr) {
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        e = hipStreamIsCapturing(stream, &capture);
+        if (e != hipSuccess) return fail(DWCONV_ERR_LAUNCH, "hipStreamIsCapturing: %s", hipGetErrorString(e));
+        if (capture != hipStreamCaptureStatusNone)
+            return fail(DWCONV_ERR_UNSUPPORTED,
+                        "dwconv2d_backward_noalloc_f32: the first call on device %d looks up the scratch buffer's "
+                        "address and must be made outside stream capture",
+                        dev);
         void *p = nullptr;
         e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
         if (e != hipSuccess || p == nullptr)
@@ -697,7 +706,7 @@ int dwconv2d_backward_noalloc_f32(const float *input, const float *out_grad, con
                     "buffer holds %zu; call dwconv2d_backward_f32 with a workspace of your own",
                     need, sizeof(scratch));
     void *ws = nullptr;
-    const int rs = scratch_of_current_device(&ws);
+    const int rs = scratch_of_current_device(&ws, static_cast<hipStream_t>(stream));
     if (rs != DWCONV_OK) return rs;
     return backward_any<float>(input, out_grad, kernel, in_grad, kernel_grad, ws, sizeof(scratch), batch, channel, in_h,
                                in_w, out_h, out_w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w, stream);

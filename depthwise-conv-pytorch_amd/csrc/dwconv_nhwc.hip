@@ -902,7 +902,7 @@ bool plan_nhwc(NhwcPlan &p, const NhwcGeometry &g, int bh, int tw, int blocks_h,
     cap = std::max(1, std::min(cap, 128));
     while (cap > 1 && static_cast<size_t>(cap) * CV * K * K * 4 > static_cast<size_t>(kNhwcTapLds)) --cap;
     p.lanes_c = pick_lanes_c(g.channel / CV, cap, env_int("DWCONV_NHWC_ALIGN", 1) ? 32 / CV : 1);
-    if (exact_lanes > 0 && getenv(lanes_env) == nullptr && (g.channel / CV) % exact_lanes == 0) p.lanes_c = exact_lanes;
+    if (exact_lanes > 0 && !env_set(lanes_env) && (g.channel / CV) % exact_lanes == 0) p.lanes_c = exact_lanes;
     p.lanes_c_magic = magic_u16(p.lanes_c);
     p.blocks_per_wg = kNhwcThreads / p.lanes_c;
     p.blocks_y = ceil_div(blocks_h, bh);

@@ -10,7 +10,7 @@ namespace {
 template <typename IO>
 int small_fir_any_width(SmallPlan &p, int width, bool exact_ok, int K, int S, int D, bool rot, bool up2, hipStream_t stream)
 {
-    if (exact_ok && small_width_is_exact(width) && !env_int("DWCONV_SMALL_FORCE_RAGGED", 0)) {
+    if (exact_ok && small_width_is_exact(width)) {
 #define DWCONV_CASE(WV) \
         if (width == WV) return small_fir_width<WV, false, IO>(p, K, S, D, rot, up2, stream);
         DWCONV_SMALL_EXACT_WIDTHS(DWCONV_CASE)

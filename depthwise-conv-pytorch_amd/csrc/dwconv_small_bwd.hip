@@ -27,7 +27,7 @@ long small_bwd_any(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, 
     if (mode != 0 && (!aligned4(x) || !aligned4(gy))) return -1;
     const SmallBwdArgs a{x, gy, taps, gx, gw, ws, ws_bytes};
     const int width = g.in_w;
-    if (small_width_is_exact(width) && !env_int("DWCONV_SMALL_FORCE_RAGGED", 0)) {
+    if (small_width_is_exact(width)) {
 #define DWCONV_CASE(WV) \
         if (width == WV) return small_bwd_width<WV, false, IO>(mode, a, g, stream);
         DWCONV_SMALL_EXACT_WIDTHS(DWCONV_CASE)

@@ -310,7 +310,7 @@ template <typename RowsFor>
 bool plan_tiles(TilePlan &p, int row_units, int unit_rows, int used_cols, int taps_per_plane, RowsFor rows_for,
                 int lds_budget = dwconv::kLdsBudget)
 {
-    const int threads = env_int("DWCONV_TILE_THREADS", kThreads);
+    const int threads = kThreads;
     const int target_items = env_int("DWCONV_TILE_ITEMS", threads);
     const int kLdsBudget = env_int("DWCONV_TILE_LDS", lds_budget);
     layout_columns(p.st, used_cols);
@@ -384,8 +384,8 @@ int launch_down(TilePlan &p, hipStream_t stream)
     // on a 5x5 stride-2 layer).
     const bool lds_out_pays = sizeof(IO) == 4 && K == 3 && S == 1 && p.row_tiles == 1 && (p.out_w * sizeof(IO)) % 128 != 0;
     p.lds_out = env_int("DWCONV_TILE_LDS_OUT", lds_out_pays) && p.vec_out == 2 &&
-                p.planes_per_tile * p.items_per_plane <= env_int("DWCONV_TILE_THREADS", kThreads);
-    hipLaunchKernelGGL((fir_down_kernel<IO, K, S, FLIP, BH>), dim3(p.n_tiles), dim3(env_int("DWCONV_TILE_THREADS", kThreads)), lds_bytes(p, K * K),
+                p.planes_per_tile * p.items_per_plane <= kThreads;
+    hipLaunchKernelGGL((fir_down_kernel<IO, K, S, FLIP, BH>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K),
                        stream, p);
     note_variant("tile_down%s<k%d,s%d,%s,bh%d> P%d rows%d vin%d vout%d%s", sizeof(IO) == 2 ? "16" : "", K, S, FLIP ? "rot" : "fwd", BH,
                  p.planes_per_tile, p.rows_per_tile, p.st.vec_in, p.vec_out, p.lds_out ? " ldsout" : "");
@@ -412,7 +412,7 @@ int launch_up2(TilePlan &p, hipStream_t stream)
     if (!plan_tiles(p, ceil_div(ceil_div(p.out_h, 2), BQ), BQ, used_cols, K * K, rows_for)) return -1;
     if (p.st.vec_in) p.st.vec_in = stage_vector_mode(p.st, p.planes_per_tile, sizeof(IO));
     if (p.vec_out) p.vec_out = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
-    hipLaunchKernelGGL((fir_up2_kernel<IO, K, EY, EX, BQ>), dim3(p.n_tiles), dim3(env_int("DWCONV_TILE_THREADS", kThreads)), lds_bytes(p, K * K), stream,
+    hipLaunchKernelGGL((fir_up2_kernel<IO, K, EY, EX, BQ>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K), stream,
                        p);
     note_variant("tile_up2%s<k%d,e%d%d,bq%d> P%d rows%d vin%d vout%d", sizeof(IO) == 2 ? "16" : "", K, EY, EX, BQ, p.planes_per_tile,
                  p.rows_per_tile, p.st.vec_in, p.vec_out);

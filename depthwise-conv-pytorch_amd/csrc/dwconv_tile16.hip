@@ -174,34 +174,37 @@ __global__ __launch_bounds__(kThreads) void fir_down16_kernel(const Tile16Plan p
         const int rows_here = min(p.rows_per_tile, p.out_h - oy0);
         const int run = rows_here * p.out_w;  // elements per plane, a multiple of eight
         // Wavefronts with no item at all skip the arithmetic; lanes without one in the others compute item 0 again.
-        // Both arms meet the same barriers, and the sums never leave their arm (merging them with the arm that has
-        // none would have every sum zeroed first).
+        // The sums never leave the arm that makes them (merged with the arm that has none, every sum would be zeroed
+        // first); what leaves it are the packed rows, and every wavefront meets the one barrier after the branch.
+        uint32_t packed[BH][OWI / 2];
+#pragma unroll
+        for (int b = 0; b < BH; ++b)
+#pragma unroll
+            for (int i = 0; i < OWI / 2; ++i) packed[b][i] = 0u;
         if (__builtin_amdgcn_readfirstlane(threadIdx.x) < n_items) {
             float acc[BH][OWI];
             convolve(pl, rb, cb, acc);
-            __syncthreads();  // every window has been read: the image can be overwritten
-            if (has_item) {
 #pragma unroll
-                for (int b = 0; b < BH; ++b) {
-                    if (rb * BH + b < rows_here) {
-                        uint32_t t[OWI / 2];
-                        pack_row(acc[b], t);
-                        // (one 128- or 64-bit write per lane at a multiple of its size: conflict-free)
-                        uint32_t *d = lds32 + ((__mul24(pl, run) + __mul24(rb * BH + b, p.out_w) + cb * OWI) >> 1);
-                        if constexpr (OWI == 8) {
-                            u32x4 v;
-                            v.x = t[0]; v.y = t[1]; v.z = t[2]; v.w = t[3];
-                            *reinterpret_cast<u32x4 *>(d) = v;
-                        } else {
-                            u32x2 v;
-                            v.x = t[0]; v.y = t[1];
-                            *reinterpret_cast<u32x2 *>(d) = v;
-                        }
+            for (int b = 0; b < BH; ++b) pack_row(acc[b], packed[b]);
+        }
+        __syncthreads();  // every window has been read: the image can be overwritten
+        if (has_item) {
+#pragma unroll
+            for (int b = 0; b < BH; ++b) {
+                if (rb * BH + b < rows_here) {
+                    // (one 128- or 64-bit write per lane at a multiple of its size: conflict-free)
+                    uint32_t *d = lds32 + ((__mul24(pl, run) + __mul24(rb * BH + b, p.out_w) + cb * OWI) >> 1);
+                    if constexpr (OWI == 8) {
+                        u32x4 v;
+                        v.x = packed[b][0]; v.y = packed[b][1]; v.z = packed[b][2]; v.w = packed[b][3];
+                        *reinterpret_cast<u32x4 *>(d) = v;
+                    } else {
+                        u32x2 v;
+                        v.x = packed[b][0]; v.y = packed[b][1];
+                        *reinterpret_cast<u32x2 *>(d) = v;
                     }
                 }
             }
-        } else {
-            __syncthreads();
         }
         __syncthreads();
         const u32x4 *image = reinterpret_cast<const u32x4 *>(lds_raw);

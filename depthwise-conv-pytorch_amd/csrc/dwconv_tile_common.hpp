@@ -508,11 +508,33 @@ inline int floor_div(int a, int b)
     return q;
 }
 
+// Tuning overrides.  The planners' choices (rows per lane, workgroups, LDS budgets, which kernel family) can be
+// overridden through DWCONV_* environment variables for measurements.  They are honoured only while DWCONV_TUNING=1 is
+// set as well, so that a stray variable in a user's environment changes nothing; values that are not plain
+// non-negative numbers up to 2^24 are ignored.
+inline bool tuning_enabled()
+{
+    const char *t = std::getenv("DWCONV_TUNING");
+    return t != nullptr && t[0] == '1' && t[1] == '\0';
+}
+
 inline int env_int(const char *name, int dflt)
 {
+    if (!tuning_enabled()) return dflt;
     const char *e = std::getenv(name);
     if (e == nullptr || e[0] == '\0') return dflt;
-    return std::atoi(e);
+    char *end = nullptr;
+    const long v = std::strtol(e, &end, 10);
+    if (end == e || *end != '\0' || v < 0 || v > (1l << 24)) return dflt;
+    return static_cast<int>(v);
+}
+
+// True when the override `name` is set (and overrides are enabled at all).
+inline bool env_set(const char *name)
+{
+    if (!tuning_enabled()) return false;
+    const char *e = std::getenv(name);
+    return e != nullptr && e[0] != '\0';
 }
 
 // vec_in for a tile of `planes` planes of `in_plane` elements of `esize` bytes whose rows allow vector loads.

@@ -209,7 +209,8 @@ int dwconv2d_backward_bf16(const unsigned short *input, const unsigned short *ou
  * device holds one such buffer, shared by all calls on it: the kernels overwrite what they read from it,
  * so nothing needs clearing between calls, but two calls that overlap in time on one device (different
  * streams or threads) race on it -- run them on one stream or order them yourself.  The buffer's address
- * is looked up on the first call on each device; make that call outside stream capture. */
+ * is looked up on the first call on each device; make that call outside stream capture (a first call on
+ * a capturing stream returns DWCONV_ERR_UNSUPPORTED and launches nothing). */
 #define DWCONV_NOALLOC_SCRATCH_BYTES (32u << 20)
 int dwconv2d_backward_noalloc_f32(const float *input, const float *out_grad, const float *kernel,
                                   float *in_grad, float *kernel_grad, int batch, int channel,

@@ -428,6 +428,7 @@ def test_half_precision_several_tiles_per_workgroup(dw, gpu, dtype, monkeypatch)
     """A workgroup of the fused 16-bit backward that walks three or more tiles (sums carried over tiles, strided
     chunk walk, grad-input streamed out of LDS between tiles), forced on a small tensor by capping the grid."""
     monkeypatch.setenv("DWCONV_WGRAD_WGS", "8")
+    monkeypatch.setenv("DWCONV_TUNING", "1")
     shape = (9, 4, 40, 104, 3, 1, 1)
     check_full_size(dw, gpu, shape, seed=45, dtype=dtype, expect=("tile_down16_dot2", "bwd_tile16_dot2"))
     check_full_size(dw, gpu, (13, 3, 37, 96, 5, 1, 2), seed=46, dtype=dtype, expect=("tile_down16_dot2", "bwd_tile16_dot2"))
@@ -584,6 +585,26 @@ def test_half_precision_uses_the_fast_kernels(dw, gpu):
         assert _C.last_variant().startswith(fwd), _C.last_variant()
         _C.dwconv2d_backward(x, gy, wt, s, s, p, p)
         assert _C.last_variant().startswith(bwd), _C.last_variant()
+
+
+def test_tuning_overrides_need_the_master_switch(dw, gpu, monkeypatch):
+    """DWCONV_* overrides of the planners are ignored unless DWCONV_TUNING=1 is set too, and ill-formed values always."""
+    from torch_dwconv import _C
+
+    x, wt, _ = make_inputs((2, 8, 14, 14, 3, 1, 1), seed=2)
+    xg, wg = x.to(gpu), wt.to(gpu)
+    monkeypatch.setenv("DWCONV_NO_SMALL", "1")
+    dw.depthwise_conv2d(xg, wg, padding=1)
+    assert _C.last_variant().startswith("small_down"), _C.last_variant()
+    monkeypatch.setenv("DWCONV_TUNING", "1")
+    dw.depthwise_conv2d(xg, wg, padding=1)
+    assert _C.last_variant().startswith("tile_down"), _C.last_variant()
+    monkeypatch.setenv("DWCONV_NO_SMALL", "yes")   # not a number: ignored
+    dw.depthwise_conv2d(xg, wg, padding=1)
+    assert _C.last_variant().startswith("small_down"), _C.last_variant()
+    monkeypatch.setenv("DWCONV_NO_SMALL", "-1")    # out of range: ignored
+    dw.depthwise_conv2d(xg, wg, padding=1)
+    assert _C.last_variant().startswith("small_down"), _C.last_variant()
 
 
 def test_combined_backward_entry_point(dw, gpu):
@@ -813,6 +834,7 @@ def test_channels_last_fused_backward(dw, gpu, shape, monkeypatch):
     assert none is None and not _C.last_variant().startswith("nhwc_bwd"), _C.last_variant()
     np.testing.assert_allclose(_np(gx_only), _np(gx), rtol=1e-6, atol=1e-6)
     monkeypatch.setenv("DWCONV_NHWC_FUSED_BWD", "0")
+    monkeypatch.setenv("DWCONV_TUNING", "1")
     gx3, gw3 = _C.dwconv2d_backward_nhwc(xg, gyg, wg, s, s, p, p)
     assert "nhwc_wgrad" in _C.last_variant(), _C.last_variant()
     np.testing.assert_allclose(_np(gx3), _np(gx), rtol=1e-6, atol=1e-6)
@@ -861,6 +883,7 @@ def test_channels_last_fused_backward_other_layers(dw, gpu, case, monkeypatch):
     gx2, gw2 = _C.dwconv2d_backward_nhwc(xg, gyg, wg, s, s, p, p)
     assert torch.equal(gw, gw2) and torch.equal(gx, gx2)
     monkeypatch.setenv("DWCONV_NHWC_FUSED_BWD", "0")
+    monkeypatch.setenv("DWCONV_TUNING", "1")
     gx3, gw3 = _C.dwconv2d_backward_nhwc(xg, gyg, wg, s, s, p, p)
     assert "nhwc_wgrad" in _C.last_variant() and not _C.last_variant().startswith("nhwc_bwd"), _C.last_variant()
     np.testing.assert_allclose(_np(gx3), _np(gx), rtol=1e-6, atol=1e-6)

@@ -134,3 +134,49 @@ def test_noalloc_inside_a_hip_graph():
         gx_ref, gw_ref, _, _ = _reference(x, gy, w, s, p)
         torch.cuda.synchronize()
         assert torch.equal(gx, gx_ref) and torch.equal(gw, gw_ref), replay
+
+
+_FIRST_CALL_UNDER_CAPTURE = r"""
+import ctypes, sys
+import torch
+sys.path[:0] = {paths!r}
+from torch_dwconv import _C
+
+hip = ctypes.CDLL("libamdhip64.so")
+x = torch.zeros(2, 4, 8, 8, device="cuda:0"); w = torch.zeros(4, 1, 3, 3, device="cuda:0")
+gx = torch.empty_like(x); gw = torch.empty_like(w)
+side = torch.cuda.Stream()
+torch.cuda.synchronize()
+stream = ctypes.c_void_p(side.cuda_stream)
+assert hip.hipStreamBeginCapture(stream, 2) == 0  # relaxed mode
+rc = _C._lib.dwconv2d_backward_noalloc_f32(x.data_ptr(), x.data_ptr(), w.data_ptr(), gx.data_ptr(), gw.data_ptr(),
+                                           2, 4, 8, 8, 8, 8, 3, 3, 1, 1, 1, 1, stream)
+message = _C._lib.dwconv_last_error().decode()
+graph = ctypes.c_void_p()
+assert hip.hipStreamEndCapture(stream, ctypes.byref(graph)) == 0
+if graph.value:
+    hip.hipGraphDestroy(graph)
+assert rc == 2, (rc, message)  # DWCONV_ERR_UNSUPPORTED, nothing recorded
+assert "outside stream capture" in message, message
+# the same call outside capture then works
+rc = _C._lib.dwconv2d_backward_noalloc_f32(x.data_ptr(), x.data_ptr(), w.data_ptr(), gx.data_ptr(), gw.data_ptr(),
+                                           2, 4, 8, 8, 8, 8, 3, 3, 1, 1, 1, 1, stream)
+assert rc == 0, _C._lib.dwconv_last_error().decode()
+torch.cuda.synchronize()
+assert float(gx.abs().sum()) == 0.0
+print("ok")
+"""
+
+
+def test_noalloc_first_call_under_capture_is_refused():
+    """The scratch buffer's address is looked up on the first call on a device; a first call on a capturing stream
+    is refused with a clear error instead of recording the lookup.  Needs a process of its own (first call)."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    paths = [root, os.path.join(root, "depthwise-conv-pytorch_amd")]
+    out = subprocess.run([sys.executable, "-c", _FIRST_CALL_UNDER_CAPTURE.format(paths=paths)], capture_output=True,
+                         text=True, timeout=170)
+    assert out.returncode == 0 and "ok" in out.stdout, out.stdout + out.stderr
