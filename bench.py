@@ -321,6 +321,9 @@ def main():
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB first (a kernel of known traffic, "
                          "to scale rocprofv3 FETCH_SIZE/WRITE_SIZE readings)")
+    ap.add_argument("--call-markers", action="store_true",
+                    help="launch a one-element fill kernel after every C-ABI call, so that a profile's list of "
+                         "dispatches can be split into calls (profiling aid; adds launches to the timed region)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: depthwise conv2d is a single-GPU kernel path; run with --gpus 1")
@@ -355,9 +358,13 @@ def main():
     step_bytes = sum(l.bytes["fwd"] + l.bytes["gx"] + l.bytes["gw"] for l in layers)
     turn = [0]
 
+    marker = torch.zeros(1, device=dev) if args.call_markers else None
+
     def step():
         for _, _, fn in call_sets[turn[0] % ring]:
             fn(stream)
+            if marker is not None:
+                marker.zero_()
         turn[0] += 1
 
     def timed(n_steps):
@@ -424,15 +431,18 @@ def main():
     dom_name, dom = max(((k, v) for k, v in by_kernel.items() if v["ms"] >= 0.95 * top_ms),
                         key=lambda kv: kv[1]["bytes"] / kv[1]["launches"])
     achieved = dom["bytes"] / dom["ms"] / 1e6
-    # measured HBM bytes per launch of that kernel, from the committed rocprofv3 --pmc summary (null if the
-    # summary does not cover this variant)
-    traffic = None
-    profiled = args.workload == "effnet_b0" and args.dtype == "f32" and args.batch == 128 and not args.only
-    try:
-        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json" if args.layout == "nchw" else "hbm_traffic_nhwc.json")) as f:
-            traffic = json.load(f)["bytes_per_launch"].get(dom_name) if profiled else None
-    except (OSError, ValueError, KeyError):
-        traffic = None
+    # measured HBM bytes (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE, scaled by a plain copy's readings) from the
+    # committed summary of this very configuration: per launch of the dominant kernel, and per step (null where the
+    # summary does not cover the configuration)
+    traffic = measured_step = None
+    if not args.only and not args.separate_backward:
+        try:
+            with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+                entry = json.load(f)["workloads"][f"{args.workload}/{args.dtype}/{args.layout}/b{shapes[0][0]}"]
+            traffic = entry["bytes_per_launch"].get(dom_name)
+            measured_step = entry["measured_bytes_per_step"]
+        except (OSError, ValueError, KeyError):
+            pass
     # the device function behind the variant name, as rocprofv3 lists it (backward calls end with a ~4.5 us
     # *_final_kernel that the per-call timing includes)
     family = dom_name.split("<")[0].rstrip("16")
@@ -442,6 +452,7 @@ def main():
                 "bwd_tile": "wgrad_tile_kernel + wgrad_tile_final_kernel",
                 "wgrad_tile": "wgrad_tile_kernel + wgrad_tile_final_kernel",
                 "bwd_tile_s2": "bwd_s2_kernel + wgrad_tile_final_kernel",
+                "tile_stack": "stack_kernel", "bwd_stack": "stack_kernel + wgrad_tile_final_kernel",
                 "nhwc_bwd": "nhwc_bwd_fused_kernel + nhwc_wgrad_final_kernel"}.get(family, family)
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": dom_name, "kernel_function": function,
@@ -468,6 +479,10 @@ def main():
                                f"{len(calls)} C-ABI calls per step",
                    "layers": [l.name for l in layers], "algorithmic_bytes_per_step": step_bytes},
         "frac_of_hbm_roofline": round(step_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, 4),
+        # the same with the HBM bytes the counters saw in one step instead of the algorithmic ones: how busy the
+        # memory system was, re-reads and write-backs included
+        "measured_traffic_frac": round(measured_step / ms_per_step / 1e6 / HBM_PEAK_GBS, 4) if measured_step else None,
+        "measured_over_algorithmic_bytes": round(measured_step / step_bytes, 3) if measured_step else None,
         # arithmetic side (matters for the 7x7-filter shapes): nominal FLOPs 2*|y|*k^2 per pass, three passes
         "tflops": round(3 * sum(l.flops for l in layers) / ms_per_step / 1e9, 2),
         "frac_of_fp32_vector_peak": round(3 * sum(l.flops for l in layers) / ms_per_step / 1e9 / FP32_VECTOR_PEAK_TFLOPS, 4),

@@ -191,7 +191,13 @@ class DepthwiseConv2dFusedFunction(Function):
     Forward: one kernel; only the inputs are kept for the backward pass (no pre-activation tensor).  Backward:
     the convolution result is recomputed with the plain forward kernel, one sweep turns it and ``grad_output``
     into the gradient of the convolution result plus the gradients of ``scale`` and ``shift``
-    (``_C.dwconv2d_epilogue_backward``), and that goes through the ordinary backward kernels."""
+    (``_C.dwconv2d_epilogue_backward``), and that goes through the ordinary backward kernels.
+
+    Corner behaviour with float16 / bfloat16 tensors and ReLU / ReLU6: the forward kernel applies the activation to
+    its fp32 sum, the backward pass takes the mask from the recomputed result after that was rounded to 16 bits.
+    An output whose pre-activation lies within one 16-bit rounding step of 0 (or of 6) can therefore get the slope
+    of the other side of the corner; no other output is affected (with fp32 tensors the window shrinks to the last
+    bit of the fp32 sum)."""
 
     @staticmethod
     def forward(ctx, input, kernel, scale, shift, activation, stride, pad):

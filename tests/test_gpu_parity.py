@@ -1210,6 +1210,52 @@ def test_fused_epilogue_training_partial_gradients_and_dtypes(dw, gpu):
             np.testing.assert_allclose(_np(a.double()), b.numpy(), rtol=4 * step + 1e-3, atol=(4 * step + 1e-3) * float(b.abs().max()))
 
 
+@pytest.mark.parametrize("activation", ["relu", "relu6"])
+@pytest.mark.parametrize("dtype,step", [(torch.float16, 2.0 ** -11), (torch.bfloat16, 2.0 ** -8)], ids=["f16", "bf16"])
+def test_fused_epilogue_training_16bit_piecewise_activations(dw, gpu, dtype, step, activation):
+    """ReLU / ReLU6 training on 16-bit tensors.  The backward pass takes the activation's mask from the recomputed
+    convolution result, which is rounded to 16 bits, whereas the fused forward applied the activation to the fp32 sum:
+    an output whose pre-activation lies within one rounding step of a corner (0, or 6 for ReLU6) may get the slope of
+    the other side.  Those outputs, and only those, are given the full size of their contribution as extra tolerance;
+    everywhere else the gradients meet the bounds of the smooth-activation test."""
+    import torch.nn.functional as F
+    from torch_dwconv.dwconv import depthwise_conv2d_fused
+
+    shape = (3, 8, 28, 28, 5, 1, 2)
+    n, c, h, w, k, s, p = shape
+    x, wt, gy = make_inputs(shape, seed=53)
+    scale, shift = torch.linspace(0.5, 2.0, c), torch.linspace(-1.0, 3.0, c)
+    xs, ws, gs = x.to(dtype), wt.to(dtype), gy.to(dtype)
+    _, ref = _fused_reference_grads(xs, ws, scale, shift, gs, activation, s, p)
+    xd, wd, gd, sd = xs.double(), ws.double(), gs.double(), scale.double().view(1, -1, 1, 1)
+    conv = F.conv2d(xd, wd, stride=s, padding=p, groups=c)
+    z = conv * sd + shift.double().view(1, -1, 1, 1)
+    reach = conv.abs() * sd * step * 1.01  # how far rounding the convolution result can move z
+    near = z.abs() <= reach
+    if activation == "relu6":
+        near |= (z - 6).abs() <= reach
+    frac = float(near.double().mean())
+    assert 0 < frac < 0.02, frac  # some such outputs exist, and they are few
+    flipped = near.double() * gd.abs()  # the most a flipped slope changes the gradient of the activation's input
+    extra = [F.conv_transpose2d(flipped * sd, wd.abs(), stride=s, padding=p, groups=c),
+             (flipped * sd).sum((0, 2, 3)).view(c, 1, 1, 1) * float(xd.abs().max()),
+             (flipped * conv.abs()).sum((0, 2, 3)), flipped.sum((0, 2, 3))]
+    leaves = [xs.to(gpu).requires_grad_(True), ws.to(gpu).requires_grad_(True), scale.to(gpu).requires_grad_(True),
+              shift.to(gpu).requires_grad_(True)]
+    y = depthwise_conv2d_fused(leaves[0], leaves[1], leaves[3], leaves[2], activation, s, p)
+    got = torch.autograd.grad(y, leaves, gs.to(gpu))
+    for i, (a, b, e) in enumerate(zip(got, ref, extra)):
+        rel = 4 * step + (1e-3 if i else 0.0)
+        bound = rel * b.abs() + rel * float(b.abs().max()) + e.view_as(b)
+        worst = ((a.double().cpu() - b).abs() - bound).max()
+        assert float(worst) <= 0.0, (i, float(worst))
+    # where no such output is in reach the input gradient is as exact as under a smooth activation
+    clean = extra[0] == 0
+    assert float(clean.double().mean()) > 0.3
+    err = (got[0].double().cpu() - ref[0]).abs()[clean]
+    assert float(err.max()) <= 4 * step * float(ref[0].abs().max()) * 2
+
+
 def test_plane_beyond_two_gib(dw, gpu):
     """One fp32 plane of more than 2 GiB: byte offsets inside it pass 2^31, where the kernels' 32-bit buffer-view
     offsets end, so the library must take its 64-bit addressing path.  Corners (with their zero padding) and an
