@@ -1246,7 +1246,7 @@ def test_fused_epilogue_training_16bit_piecewise_activations(dw, gpu, dtype, ste
     got = torch.autograd.grad(y, leaves, gs.to(gpu))
     for i, (a, b, e) in enumerate(zip(got, ref, extra)):
         rel = 4 * step + (1e-3 if i else 0.0)
-        bound = rel * b.abs() + rel * float(b.abs().max()) + e.view_as(b)
+        bound = rel * b.abs() + rel * float(b.abs().max()) + e.expand_as(b)
         worst = ((a.double().cpu() - b).abs() - bound).max()
         assert float(worst) <= 0.0, (i, float(worst))
     # where no such output is in reach the input gradient is as exact as under a smooth activation
