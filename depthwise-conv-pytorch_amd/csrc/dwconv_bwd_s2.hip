@@ -42,13 +42,20 @@ struct BwdS2Plan {
     int n_items;
     int bq;
     int vec_gx;
+    bool prefetch;    // two-step staging, if the tensors turn out to be reachable through buffer views
 };
 
 
 // E = parity of the transposed problem's leading pad K - 1 - pad (the same on both axes).
 // BQ: half-resolution rows per lane (4; 2 for planes too low to give every lane a block of 4).
 // VIEWS: x, gy and gx all go through buffer views (sx.vec_in == sg.vec_in == vec_gx == 2), nothing else compiled in.
-template <typename IO, int K, int E, int BQ, bool VIEWS>
+// PF (with VIEWS): the images travel in two steps (fetch_rows / commit_rows), each one's loads in flight during an
+// arithmetic phase.  Order of a tile, two barriers as without PF: [gy of this tile is in registers] commit gy |
+// barrier | issue the loads of x | grad-input from the gy windows | commit x | barrier | issue the loads of the next
+// tile's gy | grad-weight sums over the x windows.
+constexpr int kPrefetchSlots = 8;  // loads per lane and image at most (the planner checks rows_fit)
+
+template <typename IO, int K, int E, int BQ, bool VIEWS, bool PF = false>
 __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -82,18 +89,39 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
 #pragma unroll
     for (int t = 0; t < KK; ++t) wacc[t] = 0.f;
 
+    static_assert(!PF || VIEWS, "the two-step staging goes through buffer views");
+    RowLane lane_x{}, lane_g{};
+    typename Raw4<IO>::type staged[PF ? kPrefetchSlots : 1];
+    if constexpr (PF) {
+        lane_x = row_lane<IO>(p.sx);
+        lane_g = row_lane<IO>(p.sg);
+        if (chunk < p.tiles_per_group) {
+            const int n = chunk / p.row_tiles, rt = chunk - n * p.row_tiles;
+            fetch_rows<IO, kPrefetchSlots>(p.sg, lane_g, gy + (static_cast<long>(n) * p.channel + c) * p.sg.in_plane,
+                                           rt * p.rows_per_tile - p.m, staged);
+        }
+    }
+
     for (int tile = chunk; tile < p.tiles_per_group; tile += p.chunks) {
         const int n = tile / p.row_tiles, rt = tile - n * p.row_tiles;
         const long plane0 = static_cast<long>(n) * p.channel + c;
         const int q0 = rt * p.rows_per_tile;
 
-        if (tile != chunk) __syncthreads();  // the previous tile's window reads are done
-        // fp32: two 16-byte loads in flight per lane and image (not four): -3 % on the 112x112 layer, the two images'
-        // loads overlap.  16-bit elements: four 8-byte loads, the same bytes in flight (112x112 C=96 176 -> 166 us).
-        constexpr int kInFlight = sizeof(IO) == 2 ? 4 : 2;
-        stage_tile<IO, VIEWS, kInFlight>(p.sx, x, lds, plane0, 1, 2 * q0 - p.pad);
-        stage_tile<IO, VIEWS, kInFlight>(p.sg, gy, lds + p.g_base, plane0, 1, q0 - p.m);
-        __syncthreads();
+        if constexpr (PF) {
+            // (every lane read its gy windows of the previous tile before that tile's second barrier)
+            commit_rows<IO, kPrefetchSlots>(p.sg, lane_g, lds + p.g_base, staged);
+            __syncthreads();
+            fetch_rows<IO, kPrefetchSlots>(p.sx, lane_x, x + plane0 * p.sx.in_plane, 2 * q0 - p.pad, staged);
+        } else {
+            if (tile != chunk) __syncthreads();  // the previous tile's window reads are done
+            // fp32: two 16-byte loads in flight per lane and image (not four): -3 % on the 112x112 layer, the two
+            // images' loads overlap.  16-bit elements: four 8-byte loads, the same bytes in flight (112x112 C=96
+            // 176 -> 166 us).
+            constexpr int kInFlight = sizeof(IO) == 2 ? 4 : 2;
+            stage_tile<IO, VIEWS, kInFlight>(p.sx, x, lds, plane0, 1, 2 * q0 - p.pad);
+            stage_tile<IO, VIEWS, kInFlight>(p.sg, gy, lds + p.g_base, plane0, 1, q0 - p.m);
+            __syncthreads();
+        }
 
         // ---- gy window: grad-input block, and this lane's gy elements from the window's centre
         float g[BQ][2];
@@ -168,6 +196,18 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
                     for (int o = 0; o < 4; ++o)
                         if (ox + o < p.sx.in_w) row[o] = Io<IO>::out(xacc[b][o]);
                 }
+            }
+        }
+
+        if constexpr (PF) {
+            // (every lane read its x windows of the previous tile before this tile's first barrier)
+            commit_rows<IO, kPrefetchSlots>(p.sx, lane_x, lds, staged);
+            __syncthreads();
+            const int next = tile + p.chunks;
+            if (next < p.tiles_per_group) {
+                const int nn = next / p.row_tiles, nrt = next - nn * p.row_tiles;
+                fetch_rows<IO, kPrefetchSlots>(p.sg, lane_g, gy + (static_cast<long>(nn) * p.channel + c) * p.sg.in_plane,
+                                               nrt * p.rows_per_tile - p.m, staged);
             }
         }
 
@@ -261,8 +301,26 @@ bool plan_bwd_s2(BwdS2Plan &p, const WgradGeometry &g, int kBq, size_t esize)
     // Workgroups in all.  The fp32 5x5 / 7x7 kernels gain from four times as many, shorter chunks (-7 % on a
     // 56x56 layer, -4 % at 128x96); the 3x3 one does not, and with 16-bit elements, where the kernel is bound by
     // instruction issue, the per-workgroup prologue and reduction make more chunks 8-15 % slower.
-    const int wgs = K >= 5 && esize == 4 ? 12288 : 3072;
-    int chunks = ceil_div(env_int("DWCONV_WGRAD_WGS", wgs), g.channel);
+    // Two-step staging (see the kernel) is for 16-bit elements, where the arithmetic is long against the bytes: 56x56
+    // 5x5 bf16 88 -> 81 us, 112x112 3x3 bf16 162 -> 156.  It needs several tiles per workgroup, and its registers
+    // leave room for four workgroups per CU (three with 7x7 filters), so the workgroups are counted to fill the chip
+    // three times over, rounded down (with one chunk more per channel, a fourth, nearly empty round: +5 %).  With fp32
+    // elements it gains on some layers and loses on others inside a training step (48x48 5x5 92 -> 85 us, 56x56 117 ->
+    // 124, 64x64 137 -> 142; 3x3 112x112 274 -> 287): those kernels wait for memory with all their loads in flight
+    // as they are, and stay as they were.  The choice is made from the geometry alone, so that the workspace query
+    // and the launch agree; tensors that then turn out to be misaligned run the one-step kernel on the same chunks.
+    const int pf_mode = env_int("DWCONV_S2_PREFETCH", 1);  // 0: never, 1: 16-bit elements, 2: wherever it fits
+    p.prefetch = (pf_mode == 2 || (pf_mode == 1 && esize == 2)) && rows_fit(p.sx, kPrefetchSlots) &&
+                 rows_fit(p.sg, kPrefetchSlots) && g.in_w % 4 == 0 && g.out_w % 4 == 0 &&
+                 stage_vector_mode(p.sx, 1, esize) == 2 && stage_vector_mode(p.sg, 1, esize) == 2 &&
+                 vector_mode(1, p.sx.in_plane, esize) == 2;
+    int chunks;
+    if (p.prefetch) {
+        chunks = env_int("DWCONV_WGRAD_WGS", kCus * (K == 7 ? 3 : 4) * 3) / g.channel;
+    } else {
+        const int wgs = K >= 5 && esize == 4 ? 12288 : 3072;
+        chunks = ceil_div(env_int("DWCONV_WGRAD_WGS", wgs), g.channel);
+    }
     if (chunks > p.tiles_per_group) chunks = p.tiles_per_group;
     if (chunks < 1) chunks = 1;
     p.chunks = chunks;
@@ -300,10 +358,12 @@ long bwd_s2_case(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO
     const int E = (K - 1 - g.pad_h) & 1;
     const dim3 grid(g.channel * p.chunks), block(kThreads)  /* all 256 lanes stage the images even when the tile has fewer items */;
     const bool views = p.sx.vec_in == 2 && p.sg.vec_in == 2 && p.vec_gx == 2 && !env_int("DWCONV_NO_VIEW_ONLY", 0);
+    const bool prefetch = views && p.prefetch;
     auto launch = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, block, shmem, stream, p); };
     auto pick = [&](auto e, auto b) {
         constexpr int kE = decltype(e)::value, kB = decltype(b)::value;
-        if (views) launch(bwd_s2_kernel<IO, K, kE, kB, true>);
+        if (prefetch) launch(bwd_s2_kernel<IO, K, kE, kB, true, true>);
+        else if (views) launch(bwd_s2_kernel<IO, K, kE, kB, true>);
         else launch(bwd_s2_kernel<IO, K, kE, kB, false>);
     };
     using std::integral_constant;
@@ -314,8 +374,8 @@ long bwd_s2_case(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO
     else pick(integral_constant<int, 0>{}, integral_constant<int, 4>{});
     const int rc = check_launch("bwd_s2_kernel");
     if (rc != DWCONV_OK) return rc;
-    note_variant("bwd_tile_s2%s<k%d,e%d,bq%d> rows%d chunks%d vin%d vgy%d vgx%d", sizeof(IO) == 2 ? "16" : "", K, E, bq,
-                 p.rows_per_tile, p.chunks, p.sx.vec_in, p.sg.vec_in, p.vec_gx);
+    note_variant("bwd_tile_s2%s<k%d,e%d,bq%d> rows%d chunks%d vin%d vgy%d vgx%d%s", sizeof(IO) == 2 ? "16" : "", K, E, bq,
+                 p.rows_per_tile, p.chunks, p.sx.vec_in, p.sg.vec_in, p.vec_gx, prefetch ? " pf" : "");
     return launch_wgrad_final(p.partial, gw, g.channel, K * K, p.chunks, stream);
 }
 

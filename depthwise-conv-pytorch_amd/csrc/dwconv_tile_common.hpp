@@ -13,6 +13,7 @@ constexpr int kThreads = 256;           // lanes per workgroup (4 wavefronts)
 constexpr int kSlack = 4;               // spare floats on both sides of every LDS row
 constexpr int kLdsBudget = 48 * 1024;   // bytes of LDS one tile may take
 constexpr int kXcds = 8;
+constexpr int kCus = 256;                 // compute units of an MI355X
 
 // The LDS image of a tile: `planes` images of `lds_rows` rows of `pitch` floats.
 // Row r, column c (after the slack) of an image holds input row iy0 + r, column c - col_shift,
@@ -542,6 +543,88 @@ inline int vector_mode(long planes, long in_plane, size_t esize)
 {
     const bool fits = planes * in_plane * static_cast<long>(esize) < static_cast<long>(kOob);
     return fits && env_int("DWCONV_STAGE_VIEW", 1) ? 2 : 1;
+}
+
+// ---- a one-plane image staged in two steps --------------------------------------------------------------
+// fetch_rows issues a lane's loads into registers (elements as loaded), commit_rows writes them into the LDS image
+// later: between the two the workgroup computes on the images already in LDS, with the next image's loads in
+// flight.  A lane owns one float4 column and every rpp-th row (rpp = whole rows per sweep of the workgroup); trips
+// that lie past the image for every lane are skipped under a uniform bound.  The planner checks rows_fit().
+struct RowLane {
+    int rl;         // first row (lanes beyond rpp whole rows stage nothing: rl is then past every image)
+    int rpp;        // rows per sweep
+    unsigned coff;  // byte offset of the column within a row of the tensor
+    bool col_ok;    // the column lies inside the plane (else it reads as zeros)
+    int dcol;       // float offset of the column within an LDS row
+};
+
+template <typename IO>
+__device__ __forceinline__ RowLane row_lane(const StageLayout &s)
+{
+    RowLane l;
+    l.rpp = fast_div(kThreads, s.spr_magic);
+    const int rl = fast_div(threadIdx.x, s.spr_magic);
+    const int ix = 4 * (s.g_lo + static_cast<int>(threadIdx.x) - __mul24(rl, s.spr));
+    l.rl = rl < l.rpp ? rl : (1 << 20);
+    l.coff = static_cast<unsigned>(ix) * static_cast<unsigned>(sizeof(IO));
+    l.col_ok = static_cast<unsigned>(ix) < static_cast<unsigned>(s.in_w);
+    l.dcol = kSlack + ix + s.col_shift;
+    return l;
+}
+
+// `plane`: the tensor plane the image is cut from; LDS row r holds its row iy0 + r (zeros outside the plane).
+template <typename IO, int NS>
+__device__ __forceinline__ void fetch_rows(const StageLayout &s, const RowLane &l, const IO *__restrict__ plane, int iy0,
+                                           typename Raw4<IO>::type (&v)[NS])
+{
+    constexpr unsigned ES = sizeof(IO);
+    const __amdgpu_buffer_rsrc_t view = buffer_view(plane, static_cast<long>(s.in_plane) * ES);
+    // (the lane's row is made opaque here and in commit_rows: what derives from it is then worked out where it is
+    // used, an add and a select per slot, instead of being kept in registers from one tile to the next)
+    int rl = l.rl;
+    asm volatile("" : "+v"(rl));
+#pragma unroll
+    for (int u = 0; u < NS; ++u) {
+        if (u * l.rpp >= s.lds_rows) break;  // uniform
+        const int r = rl + u * l.rpp;
+        const int iy = iy0 + r;
+        const bool ok = r < s.lds_rows && l.col_ok && static_cast<unsigned>(iy) < static_cast<unsigned>(s.in_h);
+        const unsigned off = __mul24(iy, s.in_w) * ES + l.coff;
+        if constexpr (sizeof(IO) == 4) {
+            const u32x4 q = __builtin_amdgcn_raw_buffer_load_b128(view, ok ? off : kOob, 0, 0);
+            v[u] = make_float4(__uint_as_float(q.x), __uint_as_float(q.y), __uint_as_float(q.z), __uint_as_float(q.w));
+        } else {
+            const u32x2 q = __builtin_amdgcn_raw_buffer_load_b64(view, ok ? off : kOob, 0, 0);
+            v[u] = make_uint2(q.x, q.y);
+        }
+    }
+}
+
+template <typename IO, int NS>
+__device__ __forceinline__ void commit_rows(const StageLayout &s, const RowLane &l, float *lds,
+                                            const typename Raw4<IO>::type (&v)[NS])
+{
+    const int dump = s.plane_pitch - 4;  // right-hand slack of the last row
+    int rl = l.rl;
+    asm volatile("" : "+v"(rl));
+#pragma unroll
+    for (int u = 0; u < NS; ++u) {
+        if (u * l.rpp >= s.lds_rows) break;  // uniform
+        const int r = rl + u * l.rpp;
+        float *d = lds + (r < s.lds_rows ? __mul24(r, s.pitch) + l.dcol : dump);
+        const float4 w = widen4<IO>(v[u]);
+        d[0] = w.x;
+        d[1] = w.y;
+        d[2] = w.z;
+        d[3] = w.w;
+    }
+}
+
+// Whether an image can be staged that way with at most `ns` loads per lane.
+inline bool rows_fit(const StageLayout &s, int ns)
+{
+    if (s.spr < 1 || s.spr > kThreads) return false;
+    return s.lds_rows <= ns * (kThreads / s.spr);
 }
 
 // vec_in of a staged image: the view path also needs operands that fit its 24-bit multiplies.
