@@ -190,12 +190,23 @@ __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
     StackTile cur = stack_tile(p, n_first, u_first - n_first * p.ru, c, KE);
     fetch_stack<IO, PW, NS>(p, lane, slide_src + cur.plane0 * p.plane, cur, staged);
 
-    // the taps of the sliding pass, wavefront-uniform: scalar registers
-    float tap[KK];
+    // The taps of the sliding pass, wavefront-uniform: scalar registers.  The fused 7x7 kernel has no room for 49 of
+    // them beside its other scalars (the compiler then parks those in vector lanes and fetches them back around every
+    // staging step, some 230 lane reads per tile): it keeps the taps in the lanes of one vector register and brings
+    // each filter row into scalar registers when the window walk reaches it, 49 lane reads per tile and four rows
+    // live at a time.
+    constexpr bool kRollTaps = FUSED && K == 7;
+    float tap[kRollTaps ? 1 : KK];
+    float tap_lanes = 0.f;
+    if constexpr (kRollTaps) {
+        const int t = min(static_cast<int>(threadIdx.x) & 63, KK - 1);
+        tap_lanes = Io<IO>::in(static_cast<const IO *>(p.taps)[c * KK + KK - 1 - t]);
+    } else {
 #pragma unroll
-    for (int t = 0; t < KK; ++t) {
-        const float v = Io<IO>::in(static_cast<const IO *>(p.taps)[c * KK + ((FUSED || FLIP) ? KK - 1 - t : t)]);
-        tap[t] = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
+        for (int t = 0; t < KK; ++t) {
+            const float v = Io<IO>::in(static_cast<const IO *>(p.taps)[c * KK + ((FUSED || FLIP) ? KK - 1 - t : t)]);
+            tap[t] = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
+        }
     }
 
     // this lane's place in every tile: unit ul of the tile, column block cb
@@ -241,12 +252,22 @@ __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
         {
             float nxt[4 * NV];
             load_window_row<NV>(sbase, nxt);
+            float trow[kRollTaps ? K : 1][K];
+            if constexpr (kRollTaps) asm volatile("" : "+v"(tap_lanes));  // (keeps the lane reads inside the tile loop)
 #pragma unroll
             for (int wr = 0; wr < WIN_ROWS; ++wr) {
                 float win[4 * NV];
 #pragma unroll
                 for (int i = 0; i < 4 * NV; ++i) win[i] = nxt[i];
                 if (wr + 1 < WIN_ROWS) load_window_row<NV>(sbase + (wr + 1) * p.pitch, nxt);
+                if constexpr (kRollTaps) {
+                    if (wr % D == 0 && wr / D < K) {
+#pragma unroll
+                        for (int tx = 0; tx < K; ++tx)
+                            trow[wr / D < K ? wr / D : 0][tx] =
+                                __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tap_lanes), (wr / D) * K + tx));
+                    }
+                }
                 if constexpr (FUSED) {
                     // the lane's own gy block sits K/2 rows and columns into its window
                     const int gb = wr - PW;
@@ -264,7 +285,8 @@ __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
 #pragma unroll
                     for (int tx = 0; tx < K; ++tx)
 #pragma unroll
-                        for (int o = 0; o < 4; ++o) sums[b][o] = fmaf(win[o + tx * D], tap[ty * K + tx], sums[b][o]);
+                        for (int o = 0; o < 4; ++o)
+                            sums[b][o] = fmaf(win[o + tx * D], kRollTaps ? trow[kRollTaps ? ty : 0][tx] : tap[kRollTaps ? 0 : ty * K + tx], sums[b][o]);
                 }
                 pin_registers(sums);
             }
