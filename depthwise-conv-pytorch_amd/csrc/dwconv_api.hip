@@ -397,6 +397,21 @@ inline WgradGeometry dilated_wgrad_geometry(const GeneralGeometry &g)
     return w;
 }
 
+// Depth multiplier above 1 with the taps at dilation 1, square filters and one stride of 1 or 2: what the tiled
+// kernels may take on maps large enough for one plane per tile (Geometry::mult, WgradGeometry::mult).
+inline bool multiplied_tiled(const GeneralGeometry &g)
+{
+    return g.multiplier > 1 && g.dil_h == 1 && g.dil_w == 1 && g.kernel_h == g.kernel_w && g.stride_h == g.stride_w &&
+           (g.stride_h == 1 || g.stride_h == 2);
+}
+inline WgradGeometry multiplied_wgrad_geometry(const GeneralGeometry &g)
+{
+    WgradGeometry w{g.batch, g.channel * g.multiplier, g.in_h, g.in_w, g.out_h, g.out_w, g.kernel_h, g.kernel_w,
+                    g.stride_h, g.stride_w, g.pad_h, g.pad_w};
+    w.mult = g.multiplier;
+    return w;
+}
+
 template <typename T>
 int general_forward_any(const T *in, const T *taps, T *out, int batch, int channel, int in_h, int in_w, int multiplier,
                         int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w, int dil_h,
@@ -422,6 +437,13 @@ int general_forward_any(const T *in, const T *taps, T *out, int batch, int chann
                 r = try_launch_fir_small<T>(in, taps, out, gg, static_cast<hipStream_t>(stream), g.dil_h);
                 if (r >= 0) return r;
             }
+            if (multiplied_tiled(g)) {
+                Geometry gg{batch, channel * multiplier, in_h, in_w, kernel_h, kernel_w, 1, 1, stride_h, stride_w,
+                            pad_h, pad_h, pad_w, pad_w, g.out_h, g.out_w, 1};
+                gg.mult = multiplier;
+                r = try_launch_fir_tiled<T>(in, taps, out, gg, static_cast<hipStream_t>(stream));
+                if (r >= 0) return r;
+            }
         }
     }
     return general_forward<T>(in, taps, out, g, static_cast<hipStream_t>(stream));
@@ -442,6 +464,10 @@ size_t general_workspace_any(const GeneralGeometry &g)
         if (dilated_small(g)) {
             const size_t sm = wgrad_small_workspace(dilated_wgrad_geometry(g));
             if (sm > need) need = sm;
+        }
+        if (multiplied_tiled(g)) {
+            const size_t mt = wgrad_tiled_workspace(multiplied_wgrad_geometry(g));
+            if (mt > need) need = mt;
         }
     }
     return need;
@@ -486,6 +512,26 @@ int general_backward_any(const T *in, const T *gy, const T *taps, T *gx, T *gw, 
             if (dilated_small(g)) {
                 rc = try_launch_bwd_small<T>(in, gy, taps, gx, gw, ws, ws_bytes, dilated_wgrad_geometry(g), stream);
                 if (rc >= 0) return rc;
+            }
+            if (multiplied_tiled(g)) {
+                // the two passes on their own; either falls back to the per-element kernels where the tiled one
+                // does not take the shape
+                const int s = g.stride_h;
+                Geometry gi{batch, channel, g.out_h, g.out_w, kernel_h, kernel_w, s, s, 1, 1, kernel_h - pad_h - 1,
+                            in_h - g.out_h * s + pad_h, kernel_w - pad_w - 1, in_w - g.out_w * s + pad_w, in_h, in_w, 0};
+                gi.mult = multiplier;
+                rc = gi.pad_h1 >= 0 && gi.pad_w1 >= 0 ? try_launch_fir_tiled<T>(gy, taps, gx, gi, stream) : -1;
+                if (rc < 0) rc = general_grad_input<T>(gy, taps, gx, g, stream);
+                if (rc != DWCONV_OK) return rc;
+                char first[sizeof(g_variant)];
+                std::snprintf(first, sizeof(first), "%s", g_variant);
+                rc = try_launch_wgrad_tiled<T>(in, gy, gw, ws, ws_bytes, multiplied_wgrad_geometry(g), stream);
+                if (rc < 0) rc = general_grad_weight<T>(in, gy, gw, ws, ws_bytes, g, stream);
+                if (rc != DWCONV_OK) return rc;
+                char second[sizeof(g_variant)];
+                std::snprintf(second, sizeof(second), "%s", g_variant);
+                note_variant("%.60s + %.60s", first, second);
+                return DWCONV_OK;
             }
         }
     }

@@ -148,6 +148,11 @@ struct Geometry {
     int out_h, out_w;
     int forward;
     Epilogue epi;  // forward convolutions only
+    // Depth multiplier M (tiled kernels on larger maps only).  `channel` and planes() count the result's channels.
+    // Forward: result plane (n, c) reads input plane (n, c / M) of an input with channel / M channels.  Backward:
+    // result plane (n, c) adds up the planes (n, c * M + m) of an operand with channel * M channels, each with the
+    // taps of its own channel.
+    int mult = 1;
     long planes() const { return static_cast<long>(batch) * channel; }
 };
 
@@ -160,6 +165,8 @@ struct WgradGeometry {
     int down_h, down_w;
     int pad_h, pad_w;
     int dil = 1;  // dilation of the taps, both axes (the whole-plane kernels take 2 for 3x3 / 5x5 at stride 1)
+    int mult = 1; // depth multiplier M (tiled grad-weight kernel only): `channel` counts the channels of out_grad and of
+                  // the taps, the input has channel / M of them and plane (n, c) of out_grad meets input plane (n, c / M)
 };
 
 // Geometry of a channels-last call: input (N,H,W,C), output (N,OH,OW,C), taps (C,1,KH,KW).

@@ -48,16 +48,20 @@ struct TilePlan {
     int tap_base;              // float offset of the tap table in LDS
     int vec_out;               // 128-bit global stores are legal
     int lds_out;               // fir_down: results go back through LDS and out as one linear stream per plane
+    int mult;                  // depth multiplier M (one plane per tile when > 1).  Forward: `channel` counts the output's
+                               // channels and output plane (n, c) reads input plane (n, c / M); backward (taps rotated):
+                               // `channel` counts the result's channels and plane (n, c) adds up the M planes
+                               // (n, c * M + m) of the operand, each with the taps of its own channel
     Epilogue epi;              // forward kernels: applied to every sum before it is stored
 };
 
 // Copies the tap tables of the tile's planes into LDS, rotated by 180 degrees if FLIP.
 template <typename IO, int KK, bool FLIP>
-__device__ __forceinline__ void stage_taps(const TilePlan &p, float *lds, long plane0, int nplanes)
+__device__ __forceinline__ void stage_taps(const TilePlan &p, float *lds, long plane0, int nplanes, int channels)
 {
     for (int i = threadIdx.x; i < nplanes * KK; i += blockDim.x) {
         const int pl = i / KK, t = i - pl * KK;
-        const int c = static_cast<int>((plane0 + pl) % p.channel);
+        const int c = static_cast<int>((plane0 + pl) % channels);
         lds[p.tap_base + i] = Io<IO>::in(static_cast<const IO *>(p.taps)[c * KK + (FLIP ? KK - 1 - t : t)]);
     }
 }
@@ -78,7 +82,7 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
     const int nplanes = static_cast<int>(min(static_cast<long>(p.planes_per_tile), p.planes - plane0));
     const int oy0 = rt * p.rows_per_tile;
 
-    stage_taps<IO, KK, FLIP>(p, lds, plane0, nplanes);
+    stage_taps<IO, KK, FLIP>(p, lds, plane0, nplanes, p.channel);
     stage_tile<IO, false, kStageBatch, true>(p.st, static_cast<const IO *>(p.in), lds, plane0, nplanes, oy0 * S - p.row_shift);
     __syncthreads();
 
@@ -197,6 +201,186 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
     }
 }
 
+// fir_down_kernel for a depth multiplier above 1 (TilePlan::mult), one plane per tile: a kernel of its own, so that the
+// plain one carries none of this.
+template <typename IO, int K, int S, bool FLIP, int BH>
+__global__ __launch_bounds__(kThreads) void fir_down_mult_kernel(const TilePlan p)
+{
+    extern __shared__ float4 lds_raw[];
+    float *lds = reinterpret_cast<float *>(lds_raw);
+    constexpr int KK = K * K;
+    constexpr int WIN_ROWS = (BH - 1) * S + K;
+    constexpr int NV = (3 * S + K + 3) / 4;  // float4s covering the columns 4 outputs touch
+
+    const int tile = xcd_contiguous_tile(blockIdx.x, p.n_tiles);
+    const int pg = tile / p.row_tiles, rt = tile - pg * p.row_tiles;
+    const long plane0 = static_cast<long>(pg) * p.planes_per_tile;
+    const int nplanes = static_cast<int>(min(static_cast<long>(p.planes_per_tile), p.planes - plane0));
+    const int oy0 = rt * p.rows_per_tile;
+
+    // the operand's first plane and the channel count its taps are indexed by (depth multiplier: see TilePlan::mult)
+    long src0 = plane0;
+    int tap_channels = p.channel;
+    {
+        if constexpr (FLIP) {
+            src0 = plane0 * p.mult;
+            tap_channels = p.channel * p.mult;
+        } else {
+            const int n = pg / p.channel;
+            src0 = static_cast<long>(n) * (p.channel / p.mult) + (pg - n * p.channel) / p.mult;
+        }
+    }
+    stage_taps<IO, KK, FLIP>(p, lds, FLIP ? src0 : plane0, nplanes, tap_channels);
+    stage_tile<IO, false, kStageBatch, true>(p.st, static_cast<const IO *>(p.in), lds, src0, nplanes, oy0 * S - p.row_shift);
+    __syncthreads();
+
+    const int n_items = nplanes * p.items_per_plane;
+    // adds the windows of one item to its block of BH x 4 sums
+    auto accumulate = [&](int pl, int rb, int cb, float(&acc)[BH][4]) {
+        float tapv[KK];
+#pragma unroll
+        for (int t = 0; t < KK; ++t) tapv[t] = lds[p.tap_base + pl * KK + t];
+
+        const float *base = lds + __mul24(pl, p.st.plane_pitch) + __mul24(rb * BH * S, p.st.pitch) + kSlack + 4 * cb * S;
+        // window rows are read one ahead of their use and the sums pinned after every row (see pin_registers)
+        float nxt[4 * NV];
+        load_window_row<NV>(base, nxt);
+#pragma unroll
+        for (int wr = 0; wr < WIN_ROWS; ++wr) {
+            float win[4 * NV];
+#pragma unroll
+            for (int i = 0; i < 4 * NV; ++i) win[i] = nxt[i];
+            if (wr + 1 < WIN_ROWS) load_window_row<NV>(base + (wr + 1) * p.st.pitch, nxt);
+#pragma unroll
+            for (int b = 0; b < BH; ++b) {
+                const int ty = wr - b * S;
+                if (ty < 0 || ty >= K) continue;
+#pragma unroll
+                for (int tx = 0; tx < K; ++tx)
+#pragma unroll
+                    for (int o = 0; o < 4; ++o)
+                        acc[b][o] = fmaf(win[o * S + tx], tapv[ty * K + tx], acc[b][o]);
+            }
+            pin_registers(acc);
+        }
+    };
+    // the block of BH x 4 sums of one item
+    auto convolve = [&](int pl, int rb, int cb, float(&acc)[BH][4]) {
+#pragma unroll
+        for (int b = 0; b < BH; ++b)
+#pragma unroll
+            for (int o = 0; o < 4; ++o) acc[b][o] = 0.f;
+        accumulate(pl, rb, cb, acc);
+        if constexpr (!FLIP) {
+            if (p.epi.enabled()) {
+                epilogue_apply_block<1>(acc, p.epi, static_cast<int>((plane0 + pl) % p.channel));
+            }
+        }
+    };
+    // a finished block to memory
+    auto store_block = [&](int pl, int rb, int cb, const float(&acc)[BH][4]) {
+        const int ox = 4 * cb;
+        if (p.vec_out == 2) {
+            // branch-free: rows past the end of the plane store out of range
+            const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO));
+            const unsigned o0 = (pl * p.out_plane + ox) * static_cast<unsigned>(sizeof(IO));
+#pragma unroll
+            for (int b = 0; b < BH; ++b) {
+                const int oy = oy0 + rb * BH + b;
+                view_store4<IO>(view, oy < p.out_h ? o0 + oy * p.out_w * static_cast<unsigned>(sizeof(IO)) : kOob, acc[b][0],
+                                acc[b][1], acc[b][2], acc[b][3]);
+            }
+            return;
+        }
+        IO *dst = static_cast<IO *>(p.out) + (plane0 + pl) * p.out_plane + ox;
+#pragma unroll
+        for (int b = 0; b < BH; ++b) {
+            const int oy = oy0 + rb * BH + b;
+            if (oy >= p.out_h) continue;
+            IO *row = dst + static_cast<long>(oy) * p.out_w;
+            if (p.vec_out) {
+                store4<IO>(row, acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+            } else {
+#pragma unroll
+                for (int o = 0; o < 4; ++o)
+                    if (ox + o < p.out_w) row[o] = Io<IO>::out(acc[b][o]);
+            }
+        }
+    };
+
+    if constexpr (FLIP) {
+        {
+            // One plane per tile and one item per lane (the launcher's rule): the lane keeps its sums while the M
+            // operand planes of its result plane pass through LDS one after the other.
+            const bool has_item = static_cast<int>(threadIdx.x) < n_items;
+            const int item = has_item ? threadIdx.x : 0;
+            const int rb = fast_div(item, p.ncb_magic);
+            const int cb = item - __mul24(rb, p.ncb);
+            float acc[BH][4];
+#pragma unroll
+            for (int b = 0; b < BH; ++b)
+#pragma unroll
+                for (int o = 0; o < 4; ++o) acc[b][o] = 0.f;
+            for (int m = 0;;) {
+                accumulate(0, rb, cb, acc);
+                if (++m == p.mult) break;
+                __syncthreads();
+                stage_taps<IO, KK, FLIP>(p, lds, src0 + m, 1, tap_channels);
+                stage_tile<IO, false, kStageBatch, true>(p.st, static_cast<const IO *>(p.in), lds, src0 + m, 1, oy0 * S - p.row_shift);
+                __syncthreads();
+            }
+            if (has_item) store_block(0, rb, cb, acc);
+            return;
+        }
+    }
+
+    if (p.lds_out) {
+        // One item per lane (the planner guarantees it).  The sums go back into LDS in the layout the band has in
+        // memory, over the input image, and leave as one linear stream per plane: every store instruction of a
+        // wavefront then covers 1 KiB of consecutive bytes, where lane-owned blocks write a row segment at a time
+        // and leave the 128-byte lines that straddle two rows to two partial writes.
+        const bool has_item = static_cast<int>(threadIdx.x) < n_items;
+        const int item = has_item ? threadIdx.x : 0;
+        const int pl = fast_div(item, p.ipp_magic);
+        const int rem = item - __mul24(pl, p.items_per_plane);
+        const int rb = fast_div(rem, p.ncb_magic);
+        const int cb = rem - __mul24(rb, p.ncb);
+        float acc[BH][4];
+        convolve(pl, rb, cb, acc);
+        const int rows_here = min(p.rows_per_tile, p.out_h - oy0);
+        const int run = rows_here * p.out_w;  // elements per plane, a multiple of four
+        __syncthreads();  // every window has been read: the image can be overwritten
+        if (has_item) {
+#pragma unroll
+            for (int b = 0; b < BH; ++b)
+                if (rb * BH + b < rows_here)
+                    *reinterpret_cast<float4 *>(lds + pl * run + (rb * BH + b) * p.out_w + 4 * cb) =
+                        make_float4(acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+        }
+        __syncthreads();
+        const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO));
+        const int run4 = run >> 2, total4 = nplanes * run4;
+        for (int i = threadIdx.x; i < total4; i += blockDim.x) {
+            const int q = nplanes == 1 ? 0 : i / run4;
+            const float4 v = reinterpret_cast<const float4 *>(lds)[i];
+            const unsigned off = (q * p.out_plane + oy0 * p.out_w + (i - q * run4) * 4) * static_cast<unsigned>(sizeof(IO));
+            view_store4<IO>(view, off, v.x, v.y, v.z, v.w);
+        }
+        return;
+    }
+
+    for (int item = threadIdx.x; item < n_items; item += blockDim.x) {
+        // (24-bit multiplies: full rate, and every operand here is an LDS-sized quantity)
+        const int pl = fast_div(item, p.ipp_magic);
+        const int rem = item - __mul24(pl, p.items_per_plane);
+        const int rb = fast_div(rem, p.ncb_magic);
+        const int cb = rem - __mul24(rb, p.ncb);
+        float acc[BH][4];
+        convolve(pl, rb, cb, acc);
+        store_block(pl, rb, cb, acc);
+    }
+}
+
 // up = 2, no decimation, taps rotated.  With pad0 = 2m - E (E = pad0 & 1, m = (pad0+E)/2) and the
 // rotated filter g shifted by E (g'[t] = g[t-E]):
 //   out[2q + r] = sum_a in[q - m + r + a] * g'[r + 2a]      along each axis,
@@ -219,28 +403,21 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
     const int nplanes = static_cast<int>(min(static_cast<long>(p.planes_per_tile), p.planes - plane0));
     const int qy0 = rt * p.rows_per_tile;
 
-    stage_taps<IO, KK, true>(p, lds, plane0, nplanes);
-    stage_tile<IO, false, kStageBatch, true>(p.st, static_cast<const IO *>(p.in), lds, plane0, nplanes, qy0 - p.row_shift);
+    // depth multiplier (see TilePlan::mult): result plane (n, c) adds up the operand's planes (n, c * M + m)
+    const long src0 = p.mult > 1 ? plane0 * p.mult : plane0;
+    const int tap_channels = p.mult > 1 ? p.channel * p.mult : p.channel;
+    stage_taps<IO, KK, true>(p, lds, src0, nplanes, tap_channels);
+    stage_tile<IO, false, kStageBatch, true>(p.st, static_cast<const IO *>(p.in), lds, src0, nplanes, qy0 - p.row_shift);
     __syncthreads();
 
     const int n_items = nplanes * p.items_per_plane;
-    for (int item = threadIdx.x; item < n_items; item += blockDim.x) {
-        const int pl = fast_div(item, p.ipp_magic);
-        const int rem = item - pl * p.items_per_plane;
-        const int rb = fast_div(rem, p.ncb_magic);
-        const int cb = rem - rb * p.ncb;
-
+    // adds the windows of one item to its block of 2*BQ x 4 sums
+    auto accumulate = [&](int pl, int rb, int cb, float(&acc)[2 * BQ][4]) {
         float tapv[KK];
 #pragma unroll
         for (int t = 0; t < KK; ++t) tapv[t] = lds[p.tap_base + pl * KK + t];
 
         const float *base = lds + pl * p.st.plane_pitch + (rb * BQ) * p.st.pitch + kSlack + 2 * cb;
-        float acc[2 * BQ][4];
-#pragma unroll
-        for (int b = 0; b < 2 * BQ; ++b)
-#pragma unroll
-            for (int o = 0; o < 4; ++o) acc[b][o] = 0.f;
-
         float nxt[NW];
         load_window_row2<NW / 2>(base, nxt);
 #pragma unroll
@@ -271,7 +448,9 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
                 }
             pin_registers(acc);
         }
-
+    };
+    // a finished block to memory
+    auto store_block = [&](int pl, int rb, int cb, const float(&acc)[2 * BQ][4]) {
         const int ox = 4 * cb;
         if (p.vec_out == 2) {
             // branch-free: rows past the end of the plane store out of range
@@ -283,7 +462,7 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
                 view_store4<IO>(view, oy < p.out_h ? o0 + oy * p.out_w * static_cast<unsigned>(sizeof(IO)) : kOob, acc[b][0],
                                 acc[b][1], acc[b][2], acc[b][3]);
             }
-            continue;
+            return;
         }
         IO *dst = static_cast<IO *>(p.out) + (plane0 + pl) * p.out_plane + ox;
 #pragma unroll
@@ -299,6 +478,43 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
                     if (ox + o < p.out_w) row[o] = Io<IO>::out(acc[b][o]);
             }
         }
+    };
+
+    if (p.mult > 1) {
+        // one plane per tile and one item per lane (the launcher's rule), as in fir_down_kernel
+        const bool has_item = static_cast<int>(threadIdx.x) < n_items;
+        const int item = has_item ? threadIdx.x : 0;
+        const int rb = fast_div(item, p.ncb_magic);
+        const int cb = item - rb * p.ncb;
+        float acc[2 * BQ][4];
+#pragma unroll
+        for (int b = 0; b < 2 * BQ; ++b)
+#pragma unroll
+            for (int o = 0; o < 4; ++o) acc[b][o] = 0.f;
+        for (int m = 0;;) {
+            accumulate(0, rb, cb, acc);
+            if (++m == p.mult) break;
+            __syncthreads();
+            stage_taps<IO, KK, true>(p, lds, src0 + m, 1, tap_channels);
+            stage_tile<IO, false, kStageBatch, true>(p.st, static_cast<const IO *>(p.in), lds, src0 + m, 1, qy0 - p.row_shift);
+            __syncthreads();
+        }
+        if (has_item) store_block(0, rb, cb, acc);
+        return;
+    }
+
+    for (int item = threadIdx.x; item < n_items; item += blockDim.x) {
+        const int pl = fast_div(item, p.ipp_magic);
+        const int rem = item - pl * p.items_per_plane;
+        const int rb = fast_div(rem, p.ncb_magic);
+        const int cb = rem - rb * p.ncb;
+        float acc[2 * BQ][4];
+#pragma unroll
+        for (int b = 0; b < 2 * BQ; ++b)
+#pragma unroll
+            for (int o = 0; o < 4; ++o) acc[b][o] = 0.f;
+        accumulate(pl, rb, cb, acc);
+        store_block(pl, rb, cb, acc);
     }
 }
 
@@ -377,18 +593,26 @@ int launch_down(TilePlan &p, hipStream_t stream)
     // on the 112x112 3x3 layer, -12 %.)
     constexpr int kBudget = S == 2 ? (sizeof(IO) == 2 ? 28 : 20) * 1024 : dwconv::kLdsBudget;
     if (!plan_tiles(p, ceil_div(p.out_h, BH), BH, used_cols, K * K, rows_for, kBudget)) return -1;
+    // a depth multiplier is served where a tile is one plane (and, backward, a lane has one item): larger maps
+    if (p.mult > 1 && (p.planes_per_tile != 1 || p.items_per_plane > kThreads)) return -1;
     if (p.st.vec_in) p.st.vec_in = stage_vector_mode(p.st, p.planes_per_tile, sizeof(IO));
     if (p.vec_out) p.vec_out = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
     // Results through LDS: measured to pay where a workgroup owns a whole fp32 plane of a 3x3 stride-1 layer whose
     // rows are not whole 128-byte lines (56x56: -10 %); neutral or worse elsewhere (+2 % with 16-bit elements, +9 %
     // on a 5x5 stride-2 layer).
     const bool lds_out_pays = sizeof(IO) == 4 && K == 3 && S == 1 && p.row_tiles == 1 && (p.out_w * sizeof(IO)) % 128 != 0;
-    p.lds_out = env_int("DWCONV_TILE_LDS_OUT", lds_out_pays) && p.vec_out == 2 &&
+    p.lds_out = env_int("DWCONV_TILE_LDS_OUT", lds_out_pays) && p.vec_out == 2 && p.mult == 1 &&
                 p.planes_per_tile * p.items_per_plane <= kThreads;
-    hipLaunchKernelGGL((fir_down_kernel<IO, K, S, FLIP, BH>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K),
-                       stream, p);
-    note_variant("tile_down%s<k%d,s%d,%s,bh%d> P%d rows%d vin%d vout%d%s", sizeof(IO) == 2 ? "16" : "", K, S, FLIP ? "rot" : "fwd", BH,
-                 p.planes_per_tile, p.rows_per_tile, p.st.vec_in, p.vec_out, p.lds_out ? " ldsout" : "");
+    if (p.mult > 1)
+        hipLaunchKernelGGL((fir_down_mult_kernel<IO, K, S, FLIP, BH>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K),
+                           stream, p);
+    else
+        hipLaunchKernelGGL((fir_down_kernel<IO, K, S, FLIP, BH>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K),
+                           stream, p);
+    char mult[16] = "";
+    if (p.mult > 1) std::snprintf(mult, sizeof(mult), " m%d", p.mult);
+    note_variant("tile_down%s<k%d,s%d,%s,bh%d> P%d rows%d vin%d vout%d%s%s", sizeof(IO) == 2 ? "16" : "", K, S, FLIP ? "rot" : "fwd", BH,
+                 p.planes_per_tile, p.rows_per_tile, p.st.vec_in, p.vec_out, p.lds_out ? " ldsout" : "", mult);
     return check_launch("fir_down_kernel");
 }
 
@@ -410,12 +634,15 @@ int launch_up2(TilePlan &p, hipStream_t stream)
     const int used_cols = 2 * (p.ncb - 1) + NW;
     auto rows_for = [](int units) { return units * BQ + KAY; };
     if (!plan_tiles(p, ceil_div(ceil_div(p.out_h, 2), BQ), BQ, used_cols, K * K, rows_for)) return -1;
+    if (p.mult > 1 && (p.planes_per_tile != 1 || p.items_per_plane > kThreads)) return -1;
     if (p.st.vec_in) p.st.vec_in = stage_vector_mode(p.st, p.planes_per_tile, sizeof(IO));
     if (p.vec_out) p.vec_out = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
     hipLaunchKernelGGL((fir_up2_kernel<IO, K, EY, EX, BQ>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K), stream,
                        p);
-    note_variant("tile_up2%s<k%d,e%d%d,bq%d> P%d rows%d vin%d vout%d", sizeof(IO) == 2 ? "16" : "", K, EY, EX, BQ, p.planes_per_tile,
-                 p.rows_per_tile, p.st.vec_in, p.vec_out);
+    char mult[16] = "";
+    if (p.mult > 1) std::snprintf(mult, sizeof(mult), " m%d", p.mult);
+    note_variant("tile_up2%s<k%d,e%d%d,bq%d> P%d rows%d vin%d vout%d%s", sizeof(IO) == 2 ? "16" : "", K, EY, EX, BQ, p.planes_per_tile,
+                 p.rows_per_tile, p.st.vec_in, p.vec_out, mult);
     return check_launch("fir_up2_kernel");
 }
 
@@ -447,6 +674,8 @@ int try_launch_fir_tiled(const IO *in, const IO *taps, IO *out, const Geometry &
     p.out = out;
     p.planes = g.planes();
     p.channel = g.channel;
+    p.mult = g.mult;
+    if (g.mult > 1 && g.forward && g.channel % g.mult != 0) return -1;
     p.epi = g.epi;
     p.st.in_h = g.in_h;
     p.st.in_w = g.in_w;

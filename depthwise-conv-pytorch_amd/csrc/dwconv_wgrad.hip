@@ -48,6 +48,8 @@ struct WgradPlan {
     int vec_gx;
     int strided;           // chunk k takes tiles k, k+chunks, ... instead of a contiguous range
     int lds_gx;            // fused: grad-input goes back through LDS and leaves as one linear stream (one plane per tile)
+    int mult;              // depth multiplier M (grad-weight alone, one plane per tile): `channel` counts the channels of
+                           // gy and of the taps; plane (n, c) of gy meets plane (n, c / M) of an x with channel / M channels
 };
 
 // GX (stride 1, pad = K/2 only): the band of gy is staged in LDS next to the band of x, with the same
@@ -134,7 +136,8 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
         }
 
         if (tile != t_begin) __syncthreads();  // the previous tile's window reads are done
-        stage_tile(p.st, x, lds, plane0, nplanes, oy0 * S - p.pad_h);
+        stage_tile(p.st, x, lds, p.mult > 1 ? static_cast<long>(n) * (p.channel / p.mult) + c0 / p.mult : plane0, nplanes,
+                   oy0 * S - p.pad_h);
         if constexpr (GX) stage_tile(p.st, gy, lds + p.g_base, plane0, nplanes, oy0 - p.pad_h);
         __syncthreads();
 
@@ -454,8 +457,11 @@ struct Launcher {
     {
         const bool fused = gx != nullptr;
         if (fused && S != 1) return;
+        if (g.mult > 1 && (fused || g.channel % g.mult != 0)) return;
         WgradPlan p{};
         if (!make_plan<K, S, BH>(p, g, fused)) return;
+        if (g.mult > 1 && p.planes_per_tile != 1) return;  // (larger maps only)
+        p.mult = g.mult;
         const size_t need = static_cast<size_t>(p.groups) * p.planes_per_tile * p.chunks * K * K * sizeof(float);
         if (ws == nullptr || ws_bytes < need) {
             rc = fail(DWCONV_ERR_WORKSPACE, "grad-weight needs a workspace of %zu bytes, got %zu", need, ws_bytes);
@@ -487,9 +493,11 @@ struct Launcher {
         if (!fused) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, false>), grid, block, shmem, stream, p);
         rc = check_launch("wgrad_tile_kernel");
         if (rc != DWCONV_OK) return;
-        note_variant("%s%s<k%d,s%d,bh%d> P%d rows%d chunks%d vin%d vgy%d%s", fused ? "bwd_tile" : "wgrad_tile",
+        char mult[16] = "";
+        if (p.mult > 1) std::snprintf(mult, sizeof(mult), " m%d", p.mult);
+        note_variant("%s%s<k%d,s%d,bh%d> P%d rows%d chunks%d vin%d vgy%d%s%s", fused ? "bwd_tile" : "wgrad_tile",
                      sizeof(IO) == 2 ? "16" : "", K, S, BH, p.planes_per_tile, p.rows_per_tile, p.chunks, p.st.vec_in, p.vec_gy,
-                     p.lds_gx ? " ldsgx" : "");
+                     p.lds_gx ? " ldsgx" : "", mult);
         rc = launch_wgrad_final(static_cast<const float *>(ws), gw, g.channel, K * K, p.chunks, stream);
     }
 };

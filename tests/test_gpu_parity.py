@@ -1368,6 +1368,14 @@ def test_tensor_beyond_two_gib(dw, gpu, layout):
 
 
 # ---- dilation and depth multiplier ---------------------------------------------------------------------------
+# depth multiplier on maps large enough for one plane per tile: the tiled kernels (forward with the input plane c / M,
+# grad-input summed over the M planes of out_grad, grad-weight against the shared input plane); both strides, 3x3 / 5x5 /
+# 7x7, odd extents and widths that are not whole groups of four (scalar loads and stores), no padding
+MULTIPLIED_TILED = [
+    (2, 3, 2, 56, 56, 3, 3, 1, 1, 1), (2, 2, 3, 113, 120, 3, 3, 2, 1, 1), (3, 2, 2, 64, 48, 5, 5, 1, 2, 1),
+    (2, 2, 4, 140, 144, 5, 5, 2, 2, 1), (1, 3, 2, 130, 128, 3, 3, 2, 1, 1), (2, 2, 2, 50, 49, 3, 3, 1, 1, 1),
+    (2, 2, 2, 60, 64, 3, 3, 1, 0, 1), (2, 2, 2, 56, 56, 7, 7, 1, 3, 1), (2, 1, 5, 127, 130, 3, 3, 2, 1, 1),
+]
 GENERAL_CASES = [
     # (N, C, M, H, W, KH, KW, stride, pad, dilation)
     (2, 4, 1, 14, 14, 3, 3, 1, 2, 2), (2, 3, 2, 9, 11, 3, 3, 1, 1, 1), (1, 5, 3, 13, 12, 5, 3, 2, 2, 2),
@@ -1380,7 +1388,7 @@ GENERAL_CASES = [
     # dilation 2 on maps up to 32 wide: the whole-plane kernels (exact and ragged widths, odd planes)
     (3, 8, 1, 14, 14, 3, 3, 1, 2, 2), (2, 6, 1, 28, 28, 5, 5, 1, 4, 2), (3, 8, 1, 7, 7, 3, 3, 1, 2, 2), (2, 4, 1, 16, 16, 5, 5, 1, 4, 2),
     (2, 8, 1, 15, 15, 3, 3, 1, 2, 2), (3, 5, 1, 9, 30, 5, 5, 1, 4, 2), (2, 3, 1, 32, 32, 3, 3, 1, 2, 2), (2, 4, 1, 20, 24, 3, 3, 1, 2, 2),
-]
+] + MULTIPLIED_TILED
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
@@ -1405,7 +1413,13 @@ def test_dilation_and_depth_multiplier(dw, gpu, case, dtype):
                and h >= 8 and 2 * ((h + 3) // 4) * (w // 4) > 256 and dtype != torch.float64)
     small = (m == 1 and d == 2 and s == 1 and kh == kw and kh in (3, 5) and p == d * (kh // 2) and w <= 32 and h <= 64
              and dtype != torch.float64)
-    if stacked:
+    if case in MULTIPLIED_TILED and dtype != torch.float64:
+        # (autograd runs the backward on its own thread; the variant note is per thread)
+        _C.dwconv2d_general_backward(xg.detach(), gy.to(gpu), wg.detach(), s, s, p, p, d, d)
+        v_bwd = _C.last_variant()
+        assert v_fwd.startswith("tile_down") and v_fwd.endswith(" m%d" % m), v_fwd
+        assert v_bwd.startswith("tile_down" if s == 1 else "tile_up2") and "wgrad_tile" in v_bwd and v_bwd.count(" m%d" % m) == 2, v_bwd
+    elif stacked:
         assert v_fwd.startswith("tile_stack") and _C.last_variant() is not None, v_fwd
     elif small:
         assert v_fwd.startswith("small_down") and ",d2" in v_fwd, v_fwd
