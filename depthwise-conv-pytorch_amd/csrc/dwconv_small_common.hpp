@@ -12,10 +12,20 @@ constexpr int kWave = 64;
 // Width instances of the whole-plane kernels: exact widths, and ragged capacity classes for every other width.
 // Each instance is its own translation unit (dwconv_small_width.hip); the dispatchers call them through the
 // function templates declared below.
-#define DWCONV_SMALL_EXACT_WIDTHS(X) X(7) X(8) X(14) X(16) X(28) X(32)
+#define DWCONV_SMALL_EXACT_WIDTHS(X) X(6) X(7) X(8) X(9) X(10) X(12) X(14) X(15) X(16) X(18) X(20) X(24) X(28) X(30) X(32)
 #define DWCONV_SMALL_RAGGED_WIDTHS(X) X(8) X(16) X(24) X(32)
 
-inline bool small_width_is_exact(int w) { return w == 7 || w == 8 || w == 14 || w == 16 || w == 28 || w == 32; }
+inline bool small_width_is_exact(int w)
+{
+    switch (w) {
+#define DWCONV_CASE(WV) case WV:
+        DWCONV_SMALL_EXACT_WIDTHS(DWCONV_CASE)
+#undef DWCONV_CASE
+        return true;
+    default:
+        return false;
+    }
+}
 // capacity class of a width that has no exact instance; 0 when it is too wide for this family
 inline int small_ragged_class(int w) { return w < 1 || w > 32 ? 0 : (w + 7) / 8 * 8; }
 

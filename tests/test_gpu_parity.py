@@ -105,8 +105,7 @@ SMALL = [
     (3, 12, 7, 7, 5, 1, 2), (5, 20, 7, 7, 3, 1, 1), (3, 8, 7, 7, 7, 1, 3), (2, 13, 14, 14, 3, 1, 1),
     (3, 10, 14, 14, 5, 2, 2), (5, 11, 28, 28, 3, 2, 1), (3, 6, 28, 28, 5, 1, 2), (2, 4, 28, 28, 7, 2, 3),
     (2, 70, 14, 14, 7, 1, 3), (2, 68, 7, 7, 5, 1, 2), (2, 3, 20, 14, 3, 1, 1), (2, 4, 10, 7, 5, 1, 2),
-    # whole-plane kernels at the other widths up to 32: exact instances (8, 16, 32) and ragged classes (any other
-    # width), both strides, odd extents (stride 2 of an odd plane: gx is 2*gy - 1 wide), planes that are not a
+    # whole-plane kernels at the other widths up to 32: exact instances and ragged classes (any width without one), both strides, odd extents (stride 2 of an odd plane: gx is 2*gy - 1 wide), planes that are not a
     # multiple of four elements
     (3, 8, 8, 8, 3, 1, 1), (2, 12, 8, 8, 5, 1, 2), (2, 8, 8, 8, 7, 1, 3), (3, 8, 8, 8, 5, 2, 2),
     (2, 6, 16, 16, 3, 1, 1), (2, 5, 16, 16, 5, 1, 2), (2, 4, 16, 16, 7, 1, 3), (3, 6, 16, 16, 5, 2, 2), (2, 4, 16, 16, 3, 2, 1),
@@ -123,6 +122,9 @@ SMALL = [
     (2, 6, 24, 24, 5, 1, 2), (3, 5, 24, 24, 3, 2, 1), (2, 8, 12, 12, 5, 1, 2), (3, 7, 12, 12, 5, 2, 2), (2, 8, 6, 6, 3, 1, 1),
     (3, 5, 6, 6, 5, 1, 2), (2, 3, 20, 20, 7, 1, 3), (3, 3, 10, 10, 3, 1, 1), (3, 5, 9, 10, 3, 1, 1), (2, 4, 17, 18, 5, 1, 2),
     (3, 3, 11, 26, 3, 2, 1), (2, 5, 7, 30, 5, 1, 2), (1, 7, 9, 22, 7, 1, 3),
+    # widths that keep a ragged class now that 6, 9, 10, 12, 15, 18, 20, 24 and 30 have exact instances
+    (3, 5, 11, 22, 3, 1, 1), (2, 3, 27, 26, 5, 2, 2), (3, 4, 19, 21, 5, 1, 2), (2, 6, 13, 11, 3, 1, 1), (3, 3, 23, 27, 7, 1, 3),
+    (2, 5, 18, 18, 5, 1, 2), (3, 4, 10, 10, 5, 2, 2), (2, 3, 20, 20, 3, 1, 1), (3, 7, 9, 9, 7, 1, 3),
     # one channel per workgroup over a stack of its images (5x5 / 7x7, stride 1): heights that leave a hanging
     # 4-row unit (one, two or three rows over), tiles that span two and three images, a last tile that is short
     (3, 5, 57, 64, 7, 1, 3), (2, 3, 33, 96, 5, 1, 2), (5, 2, 70, 40, 7, 1, 3), (1, 1, 300, 16, 5, 1, 2), (7, 3, 34, 36, 7, 1, 3),
