@@ -363,7 +363,7 @@ def test_large_kernel_small_map_layers(dw, gpu, shape):
 
 
 def effnet_layers_at(res, batch=128):
-    """The 12 layers for a res x res network input (224: the BASELINE maps; 256: 128/64/32/16/8; 240: 120/60/30/15/8)."""
+    """The 12 layers for a res x res network input (224: 112/56/28/14/7; 256: 128/64/32/16/8; 240: 120/60/30/15/8)."""
     from shapes import EFFNET_B0
 
     shapes, h = [], res // 2
