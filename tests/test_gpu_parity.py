@@ -1437,6 +1437,33 @@ def test_dilation_and_depth_multiplier(dw, gpu, case, dtype):
     assert torch.equal(gw, gw2)
 
 
+@pytest.mark.parametrize("dtype,step", [(torch.float16, 2.0 ** -11), (torch.bfloat16, 2.0 ** -8)], ids=["f16", "bf16"])
+def test_depth_multiplier_tiled_half_precision(dw, gpu, dtype, step):
+    """The tiled kernels' depth-multiplier route with 16-bit tensors (fp32 sums, one rounding per result): forward,
+    grad-input summed over the M planes of out_grad, grad-weight, against fp64 on the rounded inputs."""
+    from torch_dwconv import _C
+    from torch_dwconv.dwconv import depthwise_conv2d_general
+
+    for case in [(2, 3, 2, 56, 56, 3, 3, 1, 1, 1), (2, 2, 3, 113, 120, 3, 3, 2, 1, 1), (2, 2, 4, 140, 144, 5, 5, 2, 2, 1),
+                 (2, 2, 2, 50, 49, 3, 3, 1, 1, 1), (2, 2, 2, 56, 56, 7, 7, 1, 3, 1)]:
+        n, c, m, h, w, kh, kw, s, p, d = case
+        g = torch.Generator("cpu").manual_seed(59)
+        x = torch.randn(n, c, h, w, generator=g).to(dtype)
+        wt = (torch.randn(c * m, 1, kh, kw, generator=g) / kh).to(dtype)
+        xg = x.to(gpu).requires_grad_(True)
+        wg = wt.to(gpu).requires_grad_(True)
+        y = depthwise_conv2d_general(xg, wg, stride=s, padding=p, dilation=d)
+        v_fwd = _C.last_variant()
+        assert v_fwd.startswith("tile_down16") and v_fwd.endswith(" m%d" % m), v_fwd
+        gy = torch.randn(y.shape, generator=g).to(dtype)
+        gx, gw = torch.autograd.grad(y, (xg, wg), gy.to(gpu))
+        assert y.dtype == dtype and gx.dtype == dtype and gw.dtype == dtype
+        y_ref, gx_ref, gw_ref = oracle.torch_reference_general(x.double(), wt.double(), gy.double(), s, p, d)
+        for got, ref in ((y.detach(), y_ref), (gx, gx_ref)):
+            np.testing.assert_allclose(_np(got.double()), ref.numpy(), rtol=1e-5 + step, atol=1e-5 + step * float(ref.abs().max()))
+        np.testing.assert_allclose(_np(gw.double()), gw_ref.numpy(), rtol=1e-4 + step, atol=(1e-4 + step) * float(gw_ref.abs().max()))
+
+
 def test_general_entry_point_errors(dw, gpu):
     from torch_dwconv import _C
     from torch_dwconv.dwconv import depthwise_conv2d_general
