@@ -175,7 +175,9 @@ def depthwise_conv2d_general(input, weight, stride=1, padding=0, dilation=1):
     """``F.conv2d(input, weight, stride=stride, padding=padding, dilation=dilation, groups=C)`` for a ``weight`` of
     shape ``(C*M, 1, KH, KW)``: the dilation and the depth multiplier ``M`` that ``depthwise_conv2d`` refuses, as the
     reference does (torch_dwconv/dwconv.py:99-106).  With ``M == 1`` and no dilation it runs the same kernels as
-    ``depthwise_conv2d``; otherwise per-element kernels (correct for every geometry, not tuned)."""
+    ``depthwise_conv2d``.  Tuned as well: dilation 2 with 3x3 / 5x5 filters at stride 1 and "same" padding, and a depth
+    multiplier with square 3x3 / 5x5 / 7x7 filters at stride 1 or 2 on maps from about 46x46 up.  Everything else runs
+    per-element kernels (correct for every geometry, not tuned)."""
     stride = make_tuple(stride, 2)
     padding = make_tuple(padding, 2)
     dilation = make_tuple(dilation, 2)
