@@ -357,10 +357,15 @@ __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
 // (3x3 at dilation 1 stays with the general kernels: they wait for HBM, not for the vector unit, and measured the same
 // or faster: 112x112 C=32 fused backward 124-130 us here against 127, 56x56 C=144 152-158 against 132-144)
 bool stack_shape(int K, int D) { return (D == 1 && (K == 5 || K == 7)) || (D == 2 && (K == 3 || K == 5)); }
+// 16-bit elements, 3x3 at dilation 1, rows under 96 elements (from there on the kernels with 16-bit LDS images serve):
+// the general kernels are bound by their vector instructions with such tensors (the fused 56x56 backward keeps the
+// vector units 91 % busy with 196 of 256 lanes at work, 144 on a 48x48 map), and full lanes pay.
+bool stack_shape_half(int K, int D, int w) { return K == 3 && D == 1 && w < 96 && env_int("DWCONV_STACK_K3_16", 1); }
 
-bool make_plan(StackPlan &p, int K, int D, int batch, int channel, int h, int w, size_t esize, bool fused, int target_wgs)
+bool make_plan(StackPlan &p, int K, int D, int batch, int channel, int h, int w, size_t esize, bool fused, int target_wgs,
+               bool half_io = false)
 {
-    if (!stack_shape(K, D)) return false;
+    if (!stack_shape(K, D) && !(half_io && stack_shape_half(K, D, w))) return false;
     if (w % 4 != 0 || w < 16 || h < 8) return false;
     const int ncb = w / 4;
     if (ncb > kThreads) return false;
@@ -434,6 +439,7 @@ int bwd_target_wgs(int K) { return env_int("DWCONV_STACK_WGS", K == 7 ? 768 : 15
 template <typename Fn>
 void for_shape(int K, int D, Fn &&fn)
 {
+    if (K == 3 && D == 1) fn.template operator()<3, 1>();
     if (K == 5 && D == 1) fn.template operator()<5, 1>();
     if (K == 7 && D == 1) fn.template operator()<7, 1>();
     if (K == 3 && D == 2) fn.template operator()<3, 2>();
@@ -449,6 +455,7 @@ struct StackLaunch {
     template <int K, int D>
     void operator()()
     {
+        if constexpr (K == 3 && D == 1 && sizeof(IO) == 4) return;  // (16-bit elements only: stack_shape_half)
         const dim3 grid(static_cast<unsigned>(p.channel * p.chunks)), block(kThreads);
         const bool six = p.slots_per_lane <= 6;
         if constexpr (FUSED) {
@@ -469,7 +476,8 @@ size_t stack_backward_workspace(int K, int D, int batch, int channel, int h, int
     if (!env_int("DWCONV_STACK", 1)) return 0;
     StackPlan p{};
     // (the plan does not depend on the element size except through the view-extent check: the larger one)
-    if (!make_plan(p, K, D, batch, channel, h, w, 4, true, bwd_target_wgs(K))) return 0;
+    // (and a 16-bit caller may take the 3x3 instance)
+    if (!make_plan(p, K, D, batch, channel, h, w, 4, true, bwd_target_wgs(K), true)) return 0;
     return static_cast<size_t>(channel) * p.chunks * K * K * sizeof(float);
 }
 
@@ -480,7 +488,7 @@ int launch_stack_backward(const IO *in, const IO *gy, const IO *taps, IO *gx, IO
     if (!env_int("DWCONV_STACK", 1)) return -1;
     if (!aligned4(in) || !aligned4(gy) || !aligned4(gx)) return -1;
     StackPlan p{};
-    if (!make_plan(p, K, D, batch, channel, h, w, 4, true, bwd_target_wgs(K))) return -1;
+    if (!make_plan(p, K, D, batch, channel, h, w, 4, true, bwd_target_wgs(K), sizeof(IO) == 2)) return -1;
     const size_t need = static_cast<size_t>(channel) * p.chunks * K * K * sizeof(float);
     if (ws == nullptr || ws_bytes < need)
         return fail(DWCONV_ERR_WORKSPACE, "grad-weight needs a workspace of %zu bytes, got %zu", need, ws_bytes);
@@ -505,7 +513,7 @@ int launch_stack_forward(const IO *in, const IO *taps, IO *out, int K, int D, in
     if (!aligned4(in) || !aligned4(out)) return -1;
     StackPlan p{};
     // (short-lived workgroups of one tile each measured best: 56x56 C=96 7x7 43 us with 4800, 46-50 with 1280-4096)
-    if (!make_plan(p, K, D, batch, channel, h, w, 4, false, env_int("DWCONV_STACK_FWD_WGS", 8192))) return -1;
+    if (!make_plan(p, K, D, batch, channel, h, w, 4, false, env_int("DWCONV_STACK_FWD_WGS", 8192), sizeof(IO) == 2)) return -1;
     p.x = in;
     p.taps = taps;
     p.out = out;
