@@ -359,13 +359,24 @@ __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
 bool stack_shape(int K, int D) { return (D == 1 && (K == 5 || K == 7)) || (D == 2 && (K == 3 || K == 5)); }
 // 16-bit elements, 3x3 at dilation 1, rows under 96 elements (from there on the kernels with 16-bit LDS images serve):
 // the general kernels are bound by their vector instructions with such tensors (the fused 56x56 backward keeps the
-// vector units 91 % busy with 196 of 256 lanes at work, 144 on a 48x48 map), and full lanes pay.
-bool stack_shape_half(int K, int D, int w) { return K == 3 && D == 1 && w < 96 && env_int("DWCONV_STACK_K3_16", 1); }
+// vector units 91 % busy with 196 of 256 lanes at work, 144 on a 48x48 map), and full lanes pay.  Measured by width
+// with square bf16 maps, C = 144, batch 128, us stacked / general: fused backward 48: 78 / 95, 52: 90 / 97, 56: 97 / 98,
+// 60: 114 / 139, 64: 120 / 142, 72: 155 / 174, 80: 187 / 191, 88: 209 / 260, 92: 285 / 269; forward 48: 48 / 50,
+// 52: 60 / 52, 56: 64 / 56, 60: 70 / 76, 64: 62 / 69, 68: 103 / 97, 72: 94 / 100, 76: 117 / 104, 80: 129 / 107,
+// 84: 143 / 130, 88: 138 / 140, 92: 173 / 152.  The forward pass takes the stacked kernel only at the widths where it
+// won by more than the noise.
+bool stack_shape_half(int K, int D, int w, bool fused)
+{
+    if (K != 3 || D != 1 || !env_int("DWCONV_STACK_K3_16", 1)) return false;
+    if (fused) return w <= 88;
+    if (env_set("DWCONV_STACK_K3_16_FWD_W")) return w <= env_int("DWCONV_STACK_K3_16_FWD_W", 0);
+    return w == 48 || w == 60 || w == 64 || w == 72;
+}
 
 bool make_plan(StackPlan &p, int K, int D, int batch, int channel, int h, int w, size_t esize, bool fused, int target_wgs,
                bool half_io = false)
 {
-    if (!stack_shape(K, D) && !(half_io && stack_shape_half(K, D, w))) return false;
+    if (!stack_shape(K, D) && !(half_io && stack_shape_half(K, D, w, fused))) return false;
     if (w % 4 != 0 || w < 16 || h < 8) return false;
     const int ncb = w / 4;
     if (ncb > kThreads) return false;

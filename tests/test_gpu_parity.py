@@ -404,7 +404,7 @@ def test_stress_grad_weight_determinism(dw, gpu):
 HALF_FULL_SIZE = {
     0: ("tile_down16_dot2", "bwd_tile16_dot2"),    # 112x112 C32 3x3: 16-bit LDS images, fused backward
     1: ("tile_down16_dot2", "bwd_tile_s216"),      # 112x112 C96 3x3 stride 2
-    2: ("tile_stack16<k3", "bwd_stack16<k3"),      # 56x56 C144 3x3: one channel per workgroup over its stacked images
+    2: ("tile_down16<", "bwd_stack16<k3"),         # 56x56 C144 3x3: backward one channel per workgroup over its stacked images
     3: ("tile_down16<", "bwd_tile_s216"),          # 56x56 C144 5x5 stride 2
     4: ("small_down16", "small_bwd16"),            # 28x28 C240 5x5
     5: ("small_down16", "small_bwd16"),            # 28x28 C240 3x3 stride 2
@@ -420,6 +420,13 @@ def test_half_precision_full_batch(dw, gpu, layer, dtype):
     """EfficientNet-B0 layers at batch 128 with 16-bit tensors: whole tensors against the fp64 reference on the
     rounded inputs (outputs start as NaN), one rounding step of tolerance, bit-identical grad-weight."""
     check_full_size(dw, gpu, effnet_layers()[layer], seed=41, dtype=dtype, expect=HALF_FULL_SIZE[layer])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+def test_half_precision_full_batch_stacked_forward(dw, gpu, dtype):
+    """The 3x3 instance of the stacked-image kernel in the forward pass (taken at the widths where it measured faster
+    than the general tiled kernel: 48, 60, 64, 72), at the batch of the benchmark."""
+    check_full_size(dw, gpu, (128, 144, 48, 48, 3, 1, 1), seed=45, dtype=dtype, expect=("tile_stack16<k3", "bwd_stack16<k3"))
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
@@ -609,7 +616,8 @@ def test_half_precision_uses_the_fast_kernels(dw, gpu):
 
     for shape, fwd, bwd in [((2, 8, 112, 112, 3, 1, 1), "tile_down16_dot2", "bwd_tile16_dot2"),
                             ((2, 8, 112, 112, 3, 2, 1), "tile_down16_dot2", "bwd_tile_s216"),
-                            ((2, 8, 56, 56, 3, 1, 1), "tile_stack16<k3", "bwd_stack16<k3"),
+                            ((2, 8, 56, 56, 3, 1, 1), "tile_down16<", "bwd_stack16<k3"),
+                            ((2, 8, 48, 48, 3, 1, 1), "tile_stack16<k3", "bwd_stack16<k3"),
                             ((2, 8, 56, 54, 3, 1, 1), "tile_down16<", "bwd_tile16<"),
                             ((2, 8, 14, 14, 5, 1, 2), "small_down16", "small_bwd16"),
                             ((2, 8, 28, 28, 3, 1, 1), "small_down16", "small_bwd16")]:
