@@ -51,6 +51,8 @@ WORKLOADS = {
     "effnet_b0_256": lambda batch: effnet_at(batch, 256),
     "effnet_b0_240": lambda batch: effnet_at(batch, 240),
     "effnet_b0_192": lambda batch: effnet_at(batch, 192),   # maps 96, 48, 24, 12, 6
+    # EfficientNet-B3's resolution: maps 150, 75, 38, 19, 10, none of them whole groups of four elements wide
+    "effnet_b0_300": lambda batch: effnet_at(batch, 300),
     # the options the reference's check_options refuses (a shape may carry dilation and depth multiplier as 8th and 9th
     # entries): the 3x3 stride-1 layers of the stack at dilation 2 (padding 2), a 5x5 one, and the first two layers
     # with two output channels per input channel

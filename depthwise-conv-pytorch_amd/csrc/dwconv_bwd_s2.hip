@@ -169,17 +169,32 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
                 }
             pin_registers(xacc);
         }
-        if (VIEWS || p.vec_gx == 2) {
+        if (VIEWS || p.vec_gx >= 2) {
             // branch-free: rows and column blocks past the end of the plane store out of range
             const int ox = 4 * cb;
             const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.gx) + plane0 * p.sx.in_plane, static_cast<long>(p.sx.in_plane) * sizeof(IO));  // this plane only
             const bool col_ok = has_item && ox < p.sx.in_w;
+            bool done = false;
+            if constexpr (!VIEWS && sizeof(IO) == 4) {
+                if (p.vec_gx == 3) {  // rows of any width: the block that ends a row may be short
 #pragma unroll
-            for (int b = 0; b < 2 * BQ; ++b) {
-                const int oy = 2 * (q0 + rb * BQ) + b;
-                const bool ok = col_ok && oy < p.sx.in_h;
-                view_store4<IO>(view, ok ? (oy * p.sx.in_w + ox) * static_cast<unsigned>(sizeof(IO)) : kOob, xacc[b][0],
-                                xacc[b][1], xacc[b][2], xacc[b][3]);
+                    for (int b = 0; b < 2 * BQ; ++b) {
+                        const int oy = 2 * (q0 + rb * BQ) + b;
+                        const bool ok = col_ok && oy < p.sx.in_h;
+                        view_store_first<IO>(view, ok ? (oy * p.sx.in_w + ox) * static_cast<unsigned>(sizeof(IO)) : kOob,
+                                             p.sx.in_w - ox, xacc[b][0], xacc[b][1], xacc[b][2], xacc[b][3]);
+                    }
+                    done = true;
+                }
+            }
+            if (!done) {
+#pragma unroll
+                for (int b = 0; b < 2 * BQ; ++b) {
+                    const int oy = 2 * (q0 + rb * BQ) + b;
+                    const bool ok = col_ok && oy < p.sx.in_h;
+                    view_store4<IO>(view, ok ? (oy * p.sx.in_w + ox) * static_cast<unsigned>(sizeof(IO)) : kOob, xacc[b][0],
+                                    xacc[b][1], xacc[b][2], xacc[b][3]);
+                }
             }
         } else if (!VIEWS && has_item) {
             const int ox = 4 * cb;
@@ -346,12 +361,15 @@ long bwd_s2_case(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO
     p.taps = taps;
     p.gx = gx;
     p.partial = static_cast<float *>(ws);
-    p.sx.vec_in = (g.in_w % 4 == 0) && aligned4(x);
-    p.sg.vec_in = (g.out_w % 4 == 0) && aligned4(gy);
-    p.vec_gx = (g.in_w % 4 == 0) && aligned4(gx);
-    if (p.sx.vec_in) p.sx.vec_in = stage_vector_mode(p.sx, 1, sizeof(IO));
-    if (p.sg.vec_in) p.sg.vec_in = stage_vector_mode(p.sg, 1, sizeof(IO));
-    if (p.vec_gx) p.vec_gx = vector_mode(1, p.sx.in_plane, sizeof(IO));
+    p.sx.vec_in = row_vector_mode(g.in_w, x);
+    p.sg.vec_in = row_vector_mode(g.out_w, gy);
+    p.vec_gx = row_vector_mode(g.in_w, gx);
+    // (rows of any width, mode 3, need the view; the aligned modes choose between pointer and view)
+    const int x_view = stage_vector_mode(p.sx, 1, sizeof(IO)), g_view = stage_vector_mode(p.sg, 1, sizeof(IO));
+    const int gx_view = vector_mode(1, p.sx.in_plane, sizeof(IO));
+    p.sx.vec_in = p.sx.vec_in == 1 ? x_view : (p.sx.vec_in == 3 && x_view == 2 ? 3 : 0);
+    p.sg.vec_in = p.sg.vec_in == 1 ? g_view : (p.sg.vec_in == 3 && g_view == 2 ? 3 : 0);
+    p.vec_gx = p.vec_gx == 1 ? gx_view : (p.vec_gx == 3 && gx_view == 2 ? 3 : 0);
     const size_t images = static_cast<size_t>(p.sx.plane_pitch + p.sg.plane_pitch) * 4;
     const size_t red = static_cast<size_t>(kThreads / 64) * K * K * 4;
     const size_t shmem = images > red ? images : red;

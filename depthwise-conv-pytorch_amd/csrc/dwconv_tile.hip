@@ -67,7 +67,8 @@ __device__ __forceinline__ void stage_taps(const TilePlan &p, float *lds, long p
 }
 
 // up = 1, decimation S.  out[oy,ox] = sum_{ty,tx} in[oy*S - pad_h0 + ty, ox*S - pad_w0 + tx] * f[ty,tx].
-template <typename IO, int K, int S, bool FLIP, int BH>
+// ANY_WIDTH: the instance for rows that are not whole, aligned groups of four elements (vec_in or vec_out == 3; fp32).
+template <typename IO, int K, int S, bool FLIP, int BH, bool ANY_WIDTH = false>
 __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -83,7 +84,7 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
     const int oy0 = rt * p.rows_per_tile;
 
     stage_taps<IO, KK, FLIP>(p, lds, plane0, nplanes, p.channel);
-    stage_tile<IO, false, kStageBatch, true>(p.st, static_cast<const IO *>(p.in), lds, plane0, nplanes, oy0 * S - p.row_shift);
+    stage_tile<IO, false, kStageBatch, true, ANY_WIDTH>(p.st, static_cast<const IO *>(p.in), lds, plane0, nplanes, oy0 * S - p.row_shift);
     __syncthreads();
 
     const int n_items = nplanes * p.items_per_plane;
@@ -172,10 +173,21 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
         float acc[BH][4];
         convolve(pl, rb, cb, acc);
         const int ox = 4 * cb;
-        if (p.vec_out == 2) {
+        if (p.vec_out == 2 || (ANY_WIDTH && p.vec_out == 3)) {
             // branch-free: rows past the end of the plane store out of range
             const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO));
             const unsigned o0 = (pl * p.out_plane + ox) * static_cast<unsigned>(sizeof(IO));
+            if constexpr (ANY_WIDTH && sizeof(IO) == 4) {
+                if (p.vec_out == 3) {  // the block that ends a row may be short
+#pragma unroll
+                    for (int b = 0; b < BH; ++b) {
+                        const int oy = oy0 + rb * BH + b;
+                        view_store_first<IO>(view, oy < p.out_h ? o0 + oy * p.out_w * static_cast<unsigned>(sizeof(IO)) : kOob,
+                                             p.out_w - ox, acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+                    }
+                    continue;
+                }
+            }
 #pragma unroll
             for (int b = 0; b < BH; ++b) {
                 const int oy = oy0 + rb * BH + b;
@@ -280,10 +292,21 @@ __global__ __launch_bounds__(kThreads) void fir_down_mult_kernel(const TilePlan 
     // a finished block to memory
     auto store_block = [&](int pl, int rb, int cb, const float(&acc)[BH][4]) {
         const int ox = 4 * cb;
-        if (p.vec_out == 2) {
+        if (p.vec_out >= 2) {
             // branch-free: rows past the end of the plane store out of range
             const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO));
             const unsigned o0 = (pl * p.out_plane + ox) * static_cast<unsigned>(sizeof(IO));
+            if constexpr (sizeof(IO) == 4) {
+                if (p.vec_out == 3) {  // rows of any width: the block that ends a row may be short
+#pragma unroll
+                    for (int b = 0; b < BH; ++b) {
+                        const int oy = oy0 + rb * BH + b;
+                        view_store_first<IO>(view, oy < p.out_h ? o0 + oy * p.out_w * static_cast<unsigned>(sizeof(IO)) : kOob,
+                                             p.out_w - ox, acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+                    }
+                    return;
+                }
+            }
 #pragma unroll
             for (int b = 0; b < BH; ++b) {
                 const int oy = oy0 + rb * BH + b;
@@ -452,10 +475,21 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
     // a finished block to memory
     auto store_block = [&](int pl, int rb, int cb, const float(&acc)[2 * BQ][4]) {
         const int ox = 4 * cb;
-        if (p.vec_out == 2) {
+        if (p.vec_out >= 2) {
             // branch-free: rows past the end of the plane store out of range
             const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO));
             const unsigned o0 = (pl * p.out_plane + ox) * static_cast<unsigned>(sizeof(IO));
+            if constexpr (sizeof(IO) == 4) {
+                if (p.vec_out == 3) {  // rows of any width: the block that ends a row may be short
+#pragma unroll
+                    for (int b = 0; b < 2 * BQ; ++b) {
+                        const int oy = 2 * (qy0 + rb * BQ) + b;
+                        view_store_first<IO>(view, oy < p.out_h ? o0 + oy * p.out_w * static_cast<unsigned>(sizeof(IO)) : kOob,
+                                             p.out_w - ox, acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+                    }
+                    return;
+                }
+            }
 #pragma unroll
             for (int b = 0; b < 2 * BQ; ++b) {
                 const int oy = 2 * (qy0 + rb * BQ) + b;
@@ -575,6 +609,19 @@ bool plan_tiles(TilePlan &p, int row_units, int unit_rows, int used_cols, int ta
     return true;
 }
 
+// The tile is known: whether its planes fit a buffer view decides between modes 1 and 2, and whether rows of any
+// width (mode 3) can be served at all.
+template <typename IO>
+void settle_vector_modes(TilePlan &p)
+{
+    const int in_view = stage_vector_mode(p.st, p.planes_per_tile, sizeof(IO));
+    const int out_view = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
+    if (p.st.vec_in == 1) p.st.vec_in = in_view;
+    else if (p.st.vec_in == 3 && in_view != 2) p.st.vec_in = 0;
+    if (p.vec_out == 1) p.vec_out = out_view;
+    else if (p.vec_out == 3 && out_view != 2) p.vec_out = 0;
+}
+
 size_t lds_bytes(const TilePlan &p, int taps_per_plane)
 {
     return static_cast<size_t>(p.planes_per_tile) * (p.st.plane_pitch + taps_per_plane) * 4;
@@ -595,8 +642,7 @@ int launch_down(TilePlan &p, hipStream_t stream)
     if (!plan_tiles(p, ceil_div(p.out_h, BH), BH, used_cols, K * K, rows_for, kBudget)) return -1;
     // a depth multiplier is served where a tile is one plane (and, backward, a lane has one item): larger maps
     if (p.mult > 1 && (p.planes_per_tile != 1 || p.items_per_plane > kThreads)) return -1;
-    if (p.st.vec_in) p.st.vec_in = stage_vector_mode(p.st, p.planes_per_tile, sizeof(IO));
-    if (p.vec_out) p.vec_out = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
+    settle_vector_modes<IO>(p);
     // Results through LDS: measured to pay where a workgroup owns a whole fp32 plane of a 3x3 stride-1 layer whose
     // rows are not whole 128-byte lines (56x56: -10 %); neutral or worse elsewhere (+2 % with 16-bit elements, +9 %
     // on a 5x5 stride-2 layer).
@@ -606,7 +652,11 @@ int launch_down(TilePlan &p, hipStream_t stream)
     if (p.mult > 1)
         hipLaunchKernelGGL((fir_down_mult_kernel<IO, K, S, FLIP, BH>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K),
                            stream, p);
-    else
+    else if (p.st.vec_in == 3 || p.vec_out == 3) {
+        if constexpr (sizeof(IO) == 4)
+            hipLaunchKernelGGL((fir_down_kernel<IO, K, S, FLIP, BH, true>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K),
+                               stream, p);
+    } else
         hipLaunchKernelGGL((fir_down_kernel<IO, K, S, FLIP, BH>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K),
                            stream, p);
     char mult[16] = "";
@@ -635,8 +685,7 @@ int launch_up2(TilePlan &p, hipStream_t stream)
     auto rows_for = [](int units) { return units * BQ + KAY; };
     if (!plan_tiles(p, ceil_div(ceil_div(p.out_h, 2), BQ), BQ, used_cols, K * K, rows_for)) return -1;
     if (p.mult > 1 && (p.planes_per_tile != 1 || p.items_per_plane > kThreads)) return -1;
-    if (p.st.vec_in) p.st.vec_in = stage_vector_mode(p.st, p.planes_per_tile, sizeof(IO));
-    if (p.vec_out) p.vec_out = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
+    settle_vector_modes<IO>(p);
     hipLaunchKernelGGL((fir_up2_kernel<IO, K, EY, EX, BQ>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K), stream,
                        p);
     char mult[16] = "";
@@ -683,8 +732,8 @@ int try_launch_fir_tiled(const IO *in, const IO *taps, IO *out, const Geometry &
     p.out_w = g.out_w;
     p.st.in_plane = g.in_h * g.in_w;
     p.out_plane = g.out_h * g.out_w;
-    p.st.vec_in = (g.in_w % 4 == 0) && aligned4(in);
-    p.vec_out = (g.out_w % 4 == 0) && aligned4(out);
+    p.st.vec_in = row_vector_mode(g.in_w, in);
+    p.vec_out = row_vector_mode(g.out_w, out);
 
     if (g.up_h == 1 && g.up_w == 1 && g.down_h == g.down_w && (g.down_h == 1 || g.down_h == 2)) {
         p.row_shift = g.pad_h0;

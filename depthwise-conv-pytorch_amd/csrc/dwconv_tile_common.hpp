@@ -29,7 +29,9 @@ struct StageLayout {
     int pitch;        // floats per LDS row, slack included
     int plane_pitch;  // floats per plane image
     int vec_in;       // 0: element loads; 1: four elements per load (in_w % 4 == 0, base aligned to four elements);
-                      // 2: the same through a buffer view (the tile's planes span less than kOob bytes)
+                      // 2: the same through a buffer view (the tile's planes span less than kOob bytes);
+                      // 3: through a view with rows of any width at any element alignment (fp32): a slot's load starts
+                      //    on an element boundary only, and what it reads past the end of its row is zeroed
 };
 
 // Four consecutive elements (aligned to four elements) as fp32, and back.
@@ -215,6 +217,28 @@ __device__ __forceinline__ void view_store1(__amdgpu_buffer_rsrc_t view, unsigne
     __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(a), view, off, 0, POLICY);
 }
 
+// The first `n` of four results (n >= 4: all four) at byte offset `off`, which need only be a multiple of the element
+// size: one 128-bit store for a whole block, a 64-bit and / or a 32-bit one for the block that ends a row whose width
+// is not a multiple of four.  Branch-free: the stores that do not apply go out of range.  Dropped when `off` is at or
+// beyond kOob.
+template <typename IO, int POLICY = kStoreStreaming>
+__device__ __forceinline__ void view_store_first(__amdgpu_buffer_rsrc_t view, unsigned off, int n, float a, float b, float c, float d)
+{
+    static_assert(sizeof(IO) == 4, "rows of any width are served for fp32 elements");
+    const bool row = off < kOob;
+    view_store4<IO, POLICY>(view, n >= 4 ? off : kOob, a, b, c, d);
+    view_store2<IO, POLICY>(view, row && (n == 2 || n == 3) ? off : kOob, a, b);
+    view_store1<IO, POLICY>(view, row && (n == 1 || n == 3) ? off + (n == 3 ? 8u : 0u) : kOob, n == 3 ? c : a);
+}
+
+// Zeroes what a four-element load read past the `n` elements that were left of its row.
+__device__ __forceinline__ void keep_first(float4 &v, int n)
+{
+    v.y = n > 1 ? v.y : 0.f;
+    v.z = n > 2 ? v.z : 0.f;
+    v.w = n > 3 ? v.w : 0.f;
+}
+
 // True when groups of four elements starting at `p` may be moved with one vector access.
 template <typename IO>
 inline bool aligned4(const IO *p)
@@ -251,13 +275,17 @@ constexpr int kStageBatch = 4;
 // BY_ROWS: the view path walks rows per lane instead of linear slots (see there).  It needs fewer vector instructions
 // and more registers: the forward kernels, which stage once, gain a few per cent from it (up to 10 % with 7x7
 // filters); the backward kernels, which stage two images per chunk, lose a wavefront of occupancy and 2-8 %.
-template <typename IO, bool VIEW_ONLY = false, int BATCH = kStageBatch, bool BY_ROWS = false>
+// ANY_WIDTH: vec_in == 3 (rows of any width) is looked for at run time; kernels that keep an instance of their own for
+// such rows switch it off in the other one, which then carries none of it.
+template <typename IO, bool VIEW_ONLY = false, int BATCH = kStageBatch, bool BY_ROWS = false, bool ANY_WIDTH = true>
 __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__restrict__ in, float *lds,
                                            long plane0, int nplanes, int iy0)
 {
     constexpr int kStageBatch = BATCH;  // shadows the default within this function
     const int total = nplanes * s.lds_rows * s.spr;
-    if (VIEW_ONLY || s.vec_in == 2) {
+    if (VIEW_ONLY || s.vec_in == 2 || (ANY_WIDTH && s.vec_in == 3)) {
+        // (rows of any width, vec_in == 3: see StageLayout)
+        const bool ragged = ANY_WIDTH && !VIEW_ONLY && s.vec_in == 3;
         // groups of four elements through a view of the tile's planes: slots outside the image read zeros
         const __amdgpu_buffer_rsrc_t view = buffer_view(in + plane0 * s.in_plane, static_cast<long>(nplanes) * s.in_plane * sizeof(IO));
         if constexpr (BY_ROWS) {
@@ -277,6 +305,7 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__res
                 const int ix = 4 * (s.g_lo + sc);
                 const bool col_ok = static_cast<unsigned>(ix) < static_cast<unsigned>(s.in_w);
                 const int dcol = kSlack + ix + s.col_shift;
+                const int left = s.in_w - ix;  // elements of the row from this column on
                 if (nplanes == 1) {
                     // rows of the image that exist in the plane: [lo, lo + span)
                     const int lo = max(iy0, 0);
@@ -298,6 +327,10 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__res
                             const bool ok = col_ok && static_cast<unsigned>(iy + u * rpp - lo) < span;
                             v[u] = view_load4<IO>(view, ok ? off + u * off_step : kOob);
                         }
+                        if (ragged) {
+#pragma unroll
+                            for (int u = 0; u < kStageBatch; ++u) keep_first(v[u], left);
+                        }
 #pragma unroll
                         for (int u = 0; u < kStageBatch; ++u) {
                             float *d = lds + dst + u * dst_step;  // (col_shift need not be a multiple of four)
@@ -316,6 +349,10 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__res
                         for (int u = 0; u < kStageBatch; ++u) {
                             const bool ok = col_ok && static_cast<unsigned>(iy + u * rpp - lo) < span;
                             v[u] = view_load4<IO>(view, ok ? off + u * off_step : kOob);
+                        }
+                        if (ragged) {
+#pragma unroll
+                            for (int u = 0; u < kStageBatch; ++u) keep_first(v[u], left);
                         }
 #pragma unroll
                         for (int u = 0; u < kStageBatch; ++u) {
@@ -342,6 +379,10 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__res
                             const unsigned off = (__mul24(pl, s.in_plane) + __mul24(iy, s.in_w) + ix) * ES;
                             v[u] = view_load4<IO>(view, ok ? off : kOob);
                             dst[u] = live ? __mul24(pl, s.plane_pitch) + __mul24(r, s.pitch) + dcol : dump;
+                        }
+                        if (ragged) {
+#pragma unroll
+                            for (int u = 0; u < kStageBatch; ++u) keep_first(v[u], left);
                         }
 #pragma unroll
                         for (int u = 0; u < kStageBatch; ++u) {
@@ -375,6 +416,7 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__res
                                 static_cast<unsigned>(ix) < static_cast<unsigned>(s.in_w);
                 const unsigned off = (__mul24(pl, s.in_plane) + __mul24(iy, s.in_w) + ix) * static_cast<unsigned>(sizeof(IO));
                 v[u] = view_load4<IO>(view, ok ? off : kOob);
+                if (ragged) keep_first(v[u], s.in_w - ix);
                 // slots past the end of the image (they hold zeros) go to the spare floats that end the image:
                 // the right-hand slack of its last row, which no stored output depends on
                 dst[u] = live ? __mul24(pl, s.plane_pitch) + __mul24(r, s.pitch) + kSlack + ix + s.col_shift
@@ -543,6 +585,21 @@ inline int vector_mode(long planes, long in_plane, size_t esize)
 {
     const bool fits = planes * in_plane * static_cast<long>(esize) < static_cast<long>(kOob);
     return fits && env_int("DWCONV_STAGE_VIEW", 1) ? 2 : 1;
+}
+
+// How a tensor whose rows are `width` elements wide and which starts at `base` is moved, before the view conditions are
+// known: 1 = groups of four aligned elements (stage_vector_mode / vector_mode then decide between 1 and 2), 3 = groups
+// of four at any element alignment through a view (fp32 only; the caller drops to 0 where the view does not fit), 0 =
+// element by element.
+template <typename IO>
+inline int unaligned_vector_mode()
+{
+    return sizeof(IO) == 4 && env_int("DWCONV_RAGGED_VIEWS", 1) ? 3 : 0;
+}
+template <typename IO>
+inline int row_vector_mode(int width, const IO *base)
+{
+    return width % 4 == 0 && aligned4(base) ? 1 : unaligned_vector_mode<IO>();
 }
 
 // ---- a one-plane image staged in two steps --------------------------------------------------------------

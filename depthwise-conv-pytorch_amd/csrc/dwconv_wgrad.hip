@@ -57,7 +57,9 @@ struct WgradPlan {
 // rotated taps, stored straight to memory) and, from the window's centre, its block of gy for the
 // grad-weight sums.  gy is read from HBM once for both gradients.
 
-template <typename IO, int K, int S, int BH, bool GX>
+// ANY_WIDTH: the instance for rows that are not whole, aligned groups of four elements (a mode 3 among st.vec_in,
+// vec_gy, vec_gx; fp32); the other instance carries none of it.
+template <typename IO, int K, int S, int BH, bool GX, bool ANY_WIDTH = false>
 __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -115,10 +117,11 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
             const int oy = oy0 + rb * BH + b;
             const IO *row = gsrc + static_cast<long>(oy) * p.out_w;
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (p.vec_gy == 2) {
+            if (p.vec_gy == 2 || (ANY_WIDTH && p.vec_gy == 3)) {
                 // branch-free: rows past the plane (and lanes without an item) read zeros through the view
                 const unsigned off = ((pl * p.out_plane + ox) + oy * p.out_w) * static_cast<unsigned>(sizeof(IO));
                 v = view_load4<IO>(buffer_view(gy + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO)), has_item && oy < p.out_h ? off : kOob);
+                if (ANY_WIDTH && p.vec_gy == 3) keep_first(v, p.out_w - ox);  // the block that ends a row
             } else if (has_item && oy < p.out_h) {
                 if (p.vec_gy) {
                     v = load4<IO>(row);
@@ -136,9 +139,9 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
         }
 
         if (tile != t_begin) __syncthreads();  // the previous tile's window reads are done
-        stage_tile(p.st, x, lds, p.mult > 1 ? static_cast<long>(n) * (p.channel / p.mult) + c0 / p.mult : plane0, nplanes,
-                   oy0 * S - p.pad_h);
-        if constexpr (GX) stage_tile(p.st, gy, lds + p.g_base, plane0, nplanes, oy0 - p.pad_h);
+        stage_tile<IO, false, kStageBatch, false, ANY_WIDTH>(p.st, x, lds, p.mult > 1 ? static_cast<long>(n) * (p.channel / p.mult) + c0 / p.mult : plane0,
+                                                             nplanes, oy0 * S - p.pad_h);
+        if constexpr (GX) stage_tile<IO, false, kStageBatch, false, ANY_WIDTH>(p.st, gy, lds + p.g_base, plane0, nplanes, oy0 - p.pad_h);
         __syncthreads();
 
         float xacc[GX ? BH : 1][4];  // grad-input block (kept until the tile's window reads are over when it leaves through LDS)
@@ -174,16 +177,31 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
             }
             if (p.lds_gx) {
                 // stored after the grad-weight sums, below
-            } else if (p.vec_gx == 2) {
+            } else if (p.vec_gx == 2 || (ANY_WIDTH && p.vec_gx == 3)) {
                 // branch-free: rows past the end of the plane (and lanes without an item) store out of range
                 const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.gx) + plane0 * p.st.in_plane, static_cast<long>(nplanes) * p.st.in_plane * sizeof(IO));
                 const unsigned o0 = (pl * p.st.in_plane + ox) * static_cast<unsigned>(sizeof(IO));
+                bool done = false;
+                if constexpr (ANY_WIDTH && sizeof(IO) == 4) {
+                    if (p.vec_gx == 3) {  // the block that ends a row may be short
 #pragma unroll
-                for (int b = 0; b < BH; ++b) {
-                    const int oy = oy0 + rb * BH + b;
-                    const bool ok = has_item && oy < p.st.in_h;
-                    view_store4<IO>(view, ok ? o0 + oy * p.st.in_w * static_cast<unsigned>(sizeof(IO)) : kOob, xacc[b][0],
-                                    xacc[b][1], xacc[b][2], xacc[b][3]);
+                        for (int b = 0; b < BH; ++b) {
+                            const int oy = oy0 + rb * BH + b;
+                            const bool ok = has_item && oy < p.st.in_h;
+                            view_store_first<IO>(view, ok ? o0 + oy * p.st.in_w * static_cast<unsigned>(sizeof(IO)) : kOob,
+                                                 p.st.in_w - ox, xacc[b][0], xacc[b][1], xacc[b][2], xacc[b][3]);
+                        }
+                        done = true;
+                    }
+                }
+                if (!done) {
+#pragma unroll
+                    for (int b = 0; b < BH; ++b) {
+                        const int oy = oy0 + rb * BH + b;
+                        const bool ok = has_item && oy < p.st.in_h;
+                        view_store4<IO>(view, ok ? o0 + oy * p.st.in_w * static_cast<unsigned>(sizeof(IO)) : kOob, xacc[b][0],
+                                        xacc[b][1], xacc[b][2], xacc[b][3]);
+                    }
                 }
             } else if (has_item) {
                 IO *dst = static_cast<IO *>(p.gx) + (plane0 + pl) * p.st.in_plane + ox;
@@ -470,27 +488,39 @@ struct Launcher {
         p.x = x;
         p.gy = gy;
         p.partial = static_cast<float *>(ws);
-        p.st.vec_in = (g.in_w % 4 == 0) && aligned4(x);
-        p.vec_gy = (g.out_w % 4 == 0) && aligned4(gy);
+        p.st.vec_in = row_vector_mode(g.in_w, x);
+        p.vec_gy = row_vector_mode(g.out_w, gy);
         p.strided = env_int("DWCONV_WGRAD_STRIDED", 1);
         p.taps = taps;
         p.gx = gx;
-        p.vec_gx = (g.in_w % 4 == 0) && aligned4(gx);
+        p.vec_gx = row_vector_mode(g.in_w, gx);
         const size_t shmem = lds_bytes<K, S, BH>(p, fused);
         const dim3 grid(p.groups * p.chunks), block(kThreads);
-        if (fused) p.st.vec_in = p.st.vec_in && aligned4(gy);  // gy is staged with the x image's layout
-        if (p.st.vec_in) p.st.vec_in = stage_vector_mode(p.st, p.planes_per_tile, sizeof(IO));
-        if (p.vec_gx) p.vec_gx = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
-        if (p.vec_gy) p.vec_gy = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
+        // gy is staged with the x image's layout and mode
+        if (fused && p.st.vec_in == 1 && !aligned4(gy)) p.st.vec_in = unaligned_vector_mode<IO>();
+        const int in_view = stage_vector_mode(p.st, p.planes_per_tile, sizeof(IO));
+        const int gx_view = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
+        const int gy_view = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
+        // (rows of any width, mode 3, need the view; the aligned modes choose between pointer and view)
+        p.st.vec_in = p.st.vec_in == 1 ? in_view : (p.st.vec_in == 3 && in_view == 2 ? 3 : 0);
+        p.vec_gx = p.vec_gx == 1 ? gx_view : (p.vec_gx == 3 && gx_view == 2 ? 3 : 0);
+        p.vec_gy = p.vec_gy == 1 ? gy_view : (p.vec_gy == 3 && gy_view == 2 ? 3 : 0);
         // grad-input through LDS: 3x3 filters on fp32 rows that are not whole 64-byte bursts, one plane per tile
         // (56x56: 148 -> 143 us; rows of 112 or 256 floats: unchanged or 1.5 % slower; 7x7 filters, which are bound
         // by arithmetic, 3 % slower; 16-bit elements 2 % slower)
         const bool lds_gx_pays = sizeof(IO) == 4 && K == 3 && (g.in_w * sizeof(IO)) % 64 != 0;
         p.lds_gx = fused && p.planes_per_tile == 1 && p.vec_gx == 2 && env_int("DWCONV_WGRAD_LDS_GX", lds_gx_pays);
-        if constexpr (S == 1) {
-            if (fused) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, true>), grid, block, shmem, stream, p);
+        const bool any_width = p.st.vec_in == 3 || p.vec_gy == 3 || (fused && p.vec_gx == 3);
+        if constexpr (sizeof(IO) == 4) {
+            if constexpr (S == 1) {
+                if (fused && any_width) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, true, true>), grid, block, shmem, stream, p);
+            }
+            if (!fused && any_width) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, false, true>), grid, block, shmem, stream, p);
         }
-        if (!fused) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, false>), grid, block, shmem, stream, p);
+        if constexpr (S == 1) {
+            if (fused && !any_width) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, true>), grid, block, shmem, stream, p);
+        }
+        if (!fused && !any_width) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, false>), grid, block, shmem, stream, p);
         rc = check_launch("wgrad_tile_kernel");
         if (rc != DWCONV_OK) return;
         char mult[16] = "";
