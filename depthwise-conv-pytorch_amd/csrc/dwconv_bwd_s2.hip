@@ -175,14 +175,14 @@ __global__ __launch_bounds__(kThreads) void bwd_s2_kernel(const BwdS2Plan p)
             const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.gx) + plane0 * p.sx.in_plane, static_cast<long>(p.sx.in_plane) * sizeof(IO));  // this plane only
             const bool col_ok = has_item && ox < p.sx.in_w;
             bool done = false;
-            if constexpr (!VIEWS && sizeof(IO) == 4) {
+            if constexpr (!VIEWS) {
                 if (p.vec_gx == 3) {  // rows of any width: the block that ends a row may be short
 #pragma unroll
                     for (int b = 0; b < 2 * BQ; ++b) {
                         const int oy = 2 * (q0 + rb * BQ) + b;
                         const bool ok = col_ok && oy < p.sx.in_h;
                         view_store_first<IO>(view, ok ? (oy * p.sx.in_w + ox) * static_cast<unsigned>(sizeof(IO)) : kOob,
-                                             p.sx.in_w - ox, xacc[b][0], xacc[b][1], xacc[b][2], xacc[b][3]);
+                                             p.sx.in_w - ox, p.sx.in_w & 3, xacc[b][0], xacc[b][1], xacc[b][2], xacc[b][3]);
                     }
                     done = true;
                 }

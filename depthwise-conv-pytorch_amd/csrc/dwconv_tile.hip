@@ -67,7 +67,7 @@ __device__ __forceinline__ void stage_taps(const TilePlan &p, float *lds, long p
 }
 
 // up = 1, decimation S.  out[oy,ox] = sum_{ty,tx} in[oy*S - pad_h0 + ty, ox*S - pad_w0 + tx] * f[ty,tx].
-// ANY_WIDTH: the instance for rows that are not whole, aligned groups of four elements (vec_in or vec_out == 3; fp32).
+// ANY_WIDTH: the instance for rows that are not whole, aligned groups of four elements (vec_in or vec_out == 3).
 template <typename IO, int K, int S, bool FLIP, int BH, bool ANY_WIDTH = false>
 __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
 {
@@ -177,13 +177,13 @@ __global__ __launch_bounds__(kThreads) void fir_down_kernel(const TilePlan p)
             // branch-free: rows past the end of the plane store out of range
             const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO));
             const unsigned o0 = (pl * p.out_plane + ox) * static_cast<unsigned>(sizeof(IO));
-            if constexpr (ANY_WIDTH && sizeof(IO) == 4) {
+            if constexpr (ANY_WIDTH) {
                 if (p.vec_out == 3) {  // the block that ends a row may be short
 #pragma unroll
                     for (int b = 0; b < BH; ++b) {
                         const int oy = oy0 + rb * BH + b;
                         view_store_first<IO>(view, oy < p.out_h ? o0 + oy * p.out_w * static_cast<unsigned>(sizeof(IO)) : kOob,
-                                             p.out_w - ox, acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+                                             p.out_w - ox, p.out_w & 3, acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
                     }
                     continue;
                 }
@@ -296,13 +296,13 @@ __global__ __launch_bounds__(kThreads) void fir_down_mult_kernel(const TilePlan 
             // branch-free: rows past the end of the plane store out of range
             const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO));
             const unsigned o0 = (pl * p.out_plane + ox) * static_cast<unsigned>(sizeof(IO));
-            if constexpr (sizeof(IO) == 4) {
+            {
                 if (p.vec_out == 3) {  // rows of any width: the block that ends a row may be short
 #pragma unroll
                     for (int b = 0; b < BH; ++b) {
                         const int oy = oy0 + rb * BH + b;
                         view_store_first<IO>(view, oy < p.out_h ? o0 + oy * p.out_w * static_cast<unsigned>(sizeof(IO)) : kOob,
-                                             p.out_w - ox, acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+                                             p.out_w - ox, p.out_w & 3, acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
                     }
                     return;
                 }
@@ -479,13 +479,13 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
             // branch-free: rows past the end of the plane store out of range
             const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO));
             const unsigned o0 = (pl * p.out_plane + ox) * static_cast<unsigned>(sizeof(IO));
-            if constexpr (sizeof(IO) == 4) {
+            {
                 if (p.vec_out == 3) {  // rows of any width: the block that ends a row may be short
 #pragma unroll
                     for (int b = 0; b < 2 * BQ; ++b) {
                         const int oy = 2 * (qy0 + rb * BQ) + b;
                         view_store_first<IO>(view, oy < p.out_h ? o0 + oy * p.out_w * static_cast<unsigned>(sizeof(IO)) : kOob,
-                                             p.out_w - ox, acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+                                             p.out_w - ox, p.out_w & 3, acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
                     }
                     return;
                 }
@@ -652,11 +652,10 @@ int launch_down(TilePlan &p, hipStream_t stream)
     if (p.mult > 1)
         hipLaunchKernelGGL((fir_down_mult_kernel<IO, K, S, FLIP, BH>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K),
                            stream, p);
-    else if (p.st.vec_in == 3 || p.vec_out == 3) {
-        if constexpr (sizeof(IO) == 4)
-            hipLaunchKernelGGL((fir_down_kernel<IO, K, S, FLIP, BH, true>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K),
-                               stream, p);
-    } else
+    else if (p.st.vec_in == 3 || p.vec_out == 3)
+        hipLaunchKernelGGL((fir_down_kernel<IO, K, S, FLIP, BH, true>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K),
+                           stream, p);
+    else
         hipLaunchKernelGGL((fir_down_kernel<IO, K, S, FLIP, BH>), dim3(p.n_tiles), dim3(kThreads), lds_bytes(p, K * K),
                            stream, p);
     char mult[16] = "";
@@ -670,7 +669,10 @@ template <typename IO, int K, int S, bool FLIP>
 int launch_down_bh(TilePlan &p, hipStream_t stream)
 {
     const int forced = env_int("DWCONV_TILE_BH", 0);
-    const bool seven = forced ? forced == 7 : (p.out_h % 7 == 0 || p.out_h > 64) && p.out_h % 4 != 0;
+    // Seven rows per lane where four would leave rows over and seven would not, and (stride 2) on tall planes that
+    // four does not divide; stride-1 layers measured better with four there (150x150 3x3: 159 -> 152 us, 75x75: 221
+    // -> 206; stride 2, 150 -> 75: 254 against 259 with four).
+    const bool seven = forced ? forced == 7 : (p.out_h % 7 == 0 || (S == 2 && p.out_h > 64)) && p.out_h % 4 != 0;
     return seven ? launch_down<IO, K, S, FLIP, 7>(p, stream) : launch_down<IO, K, S, FLIP, 4>(p, stream);
 }
 

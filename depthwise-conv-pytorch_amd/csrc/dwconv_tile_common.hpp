@@ -30,7 +30,7 @@ struct StageLayout {
     int plane_pitch;  // floats per plane image
     int vec_in;       // 0: element loads; 1: four elements per load (in_w % 4 == 0, base aligned to four elements);
                       // 2: the same through a buffer view (the tile's planes span less than kOob bytes);
-                      // 3: through a view with rows of any width at any element alignment (fp32): a slot's load starts
+                      // 3: through a view with rows of any width at any element alignment: a slot's load starts
                       //    on an element boundary only, and what it reads past the end of its row is zeroed
 };
 
@@ -217,18 +217,30 @@ __device__ __forceinline__ void view_store1(__amdgpu_buffer_rsrc_t view, unsigne
     __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(a), view, off, 0, POLICY);
 }
 
-// The first `n` of four results (n >= 4: all four) at byte offset `off`, which need only be a multiple of the element
-// size: one 128-bit store for a whole block, a 64-bit and / or a 32-bit one for the block that ends a row whose width
-// is not a multiple of four.  Branch-free: the stores that do not apply go out of range.  Dropped when `off` is at or
-// beyond kOob.
+// A block of four results at byte offset `off`, which need only be a multiple of the element size, of a row whose width
+// leaves `rem` = width % 4 elements (uniform) to its last block: `n` is what is left of the row from the block's first
+// column on, so n >= 4 for a whole block (one 128-bit store) and n == rem for the last one (a 64-bit and / or a 32-bit
+// store; with 16-bit elements a 64-bit store, then a 32-bit and / or a 16-bit one).  Branch-free per lane: the stores that do not apply to a lane go out of range; the ones no lane needs are
+// skipped under the uniform `rem`.  Dropped when `off` is at or beyond kOob.
 template <typename IO, int POLICY = kStoreStreaming>
-__device__ __forceinline__ void view_store_first(__amdgpu_buffer_rsrc_t view, unsigned off, int n, float a, float b, float c, float d)
+__device__ __forceinline__ void view_store_first(__amdgpu_buffer_rsrc_t view, unsigned off, int n, int rem, float a, float b, float c,
+                                                 float d)
 {
-    static_assert(sizeof(IO) == 4, "rows of any width are served for fp32 elements");
-    const bool row = off < kOob;
+    const bool tail = off < kOob && n < 4;
     view_store4<IO, POLICY>(view, n >= 4 ? off : kOob, a, b, c, d);
-    view_store2<IO, POLICY>(view, row && (n == 2 || n == 3) ? off : kOob, a, b);
-    view_store1<IO, POLICY>(view, row && (n == 1 || n == 3) ? off + (n == 3 ? 8u : 0u) : kOob, n == 3 ? c : a);
+    if (rem & 2) view_store2<IO, POLICY>(view, tail ? off : kOob, a, b);
+    if (rem & 1) {
+        const unsigned at = tail ? off + (rem == 3 ? 2u * static_cast<unsigned>(sizeof(IO)) : 0u) : kOob;
+        const float last = rem == 3 ? c : a;
+        if constexpr (sizeof(IO) == 4) {
+            view_store1<IO, POLICY>(view, at, last);
+        } else {
+            unsigned t;
+            if constexpr (std::is_same<IO, bf16_t>::value) t = bf16_pack2(last, 0.f);
+            else t = f16_pack2(last, 0.f);
+            __builtin_amdgcn_raw_buffer_store_b16(static_cast<unsigned short>(t & 0xffffu), view, at, 0, POLICY);
+        }
+    }
 }
 
 // Zeroes what a four-element load read past the `n` elements that were left of its row.
@@ -589,17 +601,20 @@ inline int vector_mode(long planes, long in_plane, size_t esize)
 
 // How a tensor whose rows are `width` elements wide and which starts at `base` is moved, before the view conditions are
 // known: 1 = groups of four aligned elements (stage_vector_mode / vector_mode then decide between 1 and 2), 3 = groups
-// of four at any element alignment through a view (fp32 only; the caller drops to 0 where the view does not fit), 0 =
+// of four at any element alignment through a view (the caller drops to 0 where the view does not fit), 0 =
 // element by element.
+// (Mode 3 needs every row to start on a 32-bit boundary: the 64-bit loads of four 16-bit elements returned wrong
+// data from 2-byte-aligned addresses, so odd widths of 16-bit tensors stay with mode 0.)
 template <typename IO>
-inline int unaligned_vector_mode()
+inline int unaligned_vector_mode(int width, const IO *base)
 {
-    return sizeof(IO) == 4 && env_int("DWCONV_RAGGED_VIEWS", 1) ? 3 : 0;
+    const bool dword_rows = sizeof(IO) == 4 || (width % 2 == 0 && (reinterpret_cast<uintptr_t>(base) & 3) == 0);
+    return dword_rows && env_int("DWCONV_RAGGED_VIEWS", 1) ? 3 : 0;
 }
 template <typename IO>
 inline int row_vector_mode(int width, const IO *base)
 {
-    return width % 4 == 0 && aligned4(base) ? 1 : unaligned_vector_mode<IO>();
+    return width % 4 == 0 && aligned4(base) ? 1 : unaligned_vector_mode<IO>(width, base);
 }
 
 // ---- a one-plane image staged in two steps --------------------------------------------------------------

@@ -58,7 +58,7 @@ struct WgradPlan {
 // grad-weight sums.  gy is read from HBM once for both gradients.
 
 // ANY_WIDTH: the instance for rows that are not whole, aligned groups of four elements (a mode 3 among st.vec_in,
-// vec_gy, vec_gx; fp32); the other instance carries none of it.
+// vec_gy, vec_gx); the other instance carries none of it.
 template <typename IO, int K, int S, int BH, bool GX, bool ANY_WIDTH = false>
 __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
 {
@@ -182,14 +182,14 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
                 const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.gx) + plane0 * p.st.in_plane, static_cast<long>(nplanes) * p.st.in_plane * sizeof(IO));
                 const unsigned o0 = (pl * p.st.in_plane + ox) * static_cast<unsigned>(sizeof(IO));
                 bool done = false;
-                if constexpr (ANY_WIDTH && sizeof(IO) == 4) {
+                if constexpr (ANY_WIDTH) {
                     if (p.vec_gx == 3) {  // the block that ends a row may be short
 #pragma unroll
                         for (int b = 0; b < BH; ++b) {
                             const int oy = oy0 + rb * BH + b;
                             const bool ok = has_item && oy < p.st.in_h;
                             view_store_first<IO>(view, ok ? o0 + oy * p.st.in_w * static_cast<unsigned>(sizeof(IO)) : kOob,
-                                                 p.st.in_w - ox, xacc[b][0], xacc[b][1], xacc[b][2], xacc[b][3]);
+                                                 p.st.in_w - ox, p.st.in_w & 3, xacc[b][0], xacc[b][1], xacc[b][2], xacc[b][3]);
                         }
                         done = true;
                     }
@@ -426,7 +426,9 @@ bool dispatch(const WgradGeometry &g, Fn &&fn)
     if ((g.out_h - 1) * S - g.pad_h + K - 1 > g.in_h - 1 + 7 || (g.out_w - 1) * S - g.pad_w + K - 1 > g.in_w - 1 + 7)
         return false;
     const int forced = env_int("DWCONV_TILE_BH", 0);
-    const bool seven = forced ? forced == 7 : (g.out_h % 7 == 0 || g.out_h > 64) && g.out_h % 4 != 0;
+    // (as in the forward launcher; the fused stride-1 backward of a 150x150 3x3 layer: 289 -> 270 us with four rows per
+    // lane, of a 74x74 5x5 one 289 -> 220)
+    const bool seven = forced ? forced == 7 : (g.out_h % 7 == 0 || (S == 2 && g.out_h > 64)) && g.out_h % 4 != 0;
 #define DWCONV_WGRAD_CASE(KV, SV)                                                   \
     if (K == KV && S == SV) {                                                       \
         if (seven) fn.template operator()<KV, SV, 7>();                            \
@@ -497,7 +499,11 @@ struct Launcher {
         const size_t shmem = lds_bytes<K, S, BH>(p, fused);
         const dim3 grid(p.groups * p.chunks), block(kThreads);
         // gy is staged with the x image's layout and mode
-        if (fused && p.st.vec_in == 1 && !aligned4(gy)) p.st.vec_in = unaligned_vector_mode<IO>();
+        if (fused && p.st.vec_in != 0) {
+            const int gy_mode = row_vector_mode(g.in_w, gy);
+            if (gy_mode == 0) p.st.vec_in = 0;
+            else if (gy_mode == 3) p.st.vec_in = 3;
+        }
         const int in_view = stage_vector_mode(p.st, p.planes_per_tile, sizeof(IO));
         const int gx_view = vector_mode(p.planes_per_tile, p.st.in_plane, sizeof(IO));
         const int gy_view = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
@@ -511,12 +517,10 @@ struct Launcher {
         const bool lds_gx_pays = sizeof(IO) == 4 && K == 3 && (g.in_w * sizeof(IO)) % 64 != 0;
         p.lds_gx = fused && p.planes_per_tile == 1 && p.vec_gx == 2 && env_int("DWCONV_WGRAD_LDS_GX", lds_gx_pays);
         const bool any_width = p.st.vec_in == 3 || p.vec_gy == 3 || (fused && p.vec_gx == 3);
-        if constexpr (sizeof(IO) == 4) {
-            if constexpr (S == 1) {
-                if (fused && any_width) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, true, true>), grid, block, shmem, stream, p);
-            }
-            if (!fused && any_width) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, false, true>), grid, block, shmem, stream, p);
+        if constexpr (S == 1) {
+            if (fused && any_width) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, true, true>), grid, block, shmem, stream, p);
         }
+        if (!fused && any_width) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, false, true>), grid, block, shmem, stream, p);
         if constexpr (S == 1) {
             if (fused && !any_width) hipLaunchKernelGGL((wgrad_tile_kernel<IO, K, S, BH, true>), grid, block, shmem, stream, p);
         }
