@@ -363,7 +363,7 @@ long bwd_s2_case(int mode, const IO *x, const IO *gy, const IO *taps, IO *gx, IO
     p.partial = static_cast<float *>(ws);
     p.sx.vec_in = row_vector_mode(g.in_w, x);
     p.sg.vec_in = row_vector_mode(g.out_w, gy);
-    p.vec_gx = row_vector_mode(g.in_w, gx);
+    p.vec_gx = row_vector_mode(g.in_w, gx, false);
     // (rows of any width, mode 3, need the view; the aligned modes choose between pointer and view)
     const int x_view = stage_vector_mode(p.sx, 1, sizeof(IO)), g_view = stage_vector_mode(p.sg, 1, sizeof(IO));
     const int gx_view = vector_mode(1, p.sx.in_plane, sizeof(IO));

@@ -735,7 +735,7 @@ int try_launch_fir_tiled(const IO *in, const IO *taps, IO *out, const Geometry &
     p.st.in_plane = g.in_h * g.in_w;
     p.out_plane = g.out_h * g.out_w;
     p.st.vec_in = row_vector_mode(g.in_w, in);
-    p.vec_out = row_vector_mode(g.out_w, out);
+    p.vec_out = row_vector_mode(g.out_w, out, false);
 
     if (g.up_h == 1 && g.up_w == 1 && g.down_h == g.down_w && (g.down_h == 1 || g.down_h == 2)) {
         p.row_shift = g.pad_h0;

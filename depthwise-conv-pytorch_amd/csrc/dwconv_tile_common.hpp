@@ -217,11 +217,13 @@ __device__ __forceinline__ void view_store1(__amdgpu_buffer_rsrc_t view, unsigne
     __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(a), view, off, 0, POLICY);
 }
 
-// A block of four results at byte offset `off`, which need only be a multiple of the element size, of a row whose width
-// leaves `rem` = width % 4 elements (uniform) to its last block: `n` is what is left of the row from the block's first
-// column on, so n >= 4 for a whole block (one 128-bit store) and n == rem for the last one (a 64-bit and / or a 32-bit
-// store; with 16-bit elements a 64-bit store, then a 32-bit and / or a 16-bit one).  Branch-free per lane: the stores that do not apply to a lane go out of range; the ones no lane needs are
-// skipped under the uniform `rem`.  Dropped when `off` is at or beyond kOob.
+// A block of four results at byte offset `off`, which need only be a multiple of 4 bytes, of a row whose width leaves
+// `rem` = width % 4 elements (uniform) to its last block: `n` is what is left of the row from the block's first column
+// on, so n >= 4 for a whole block (one 128-bit store; 64 bits for 16-bit elements) and n == rem for the last one (a
+// 64-bit and / or a 32-bit store; 16-bit elements, whose rows are even here: a 32-bit store).  Branch-free per lane: the
+// stores that do not apply to a lane go out of range; the ones no lane needs are skipped under the uniform `rem`.
+// Dropped when `off` is at or beyond kOob.  (16-bit tensors with rows that start 2 bytes past a 32-bit boundary do not
+// come here: stored as 16 + 32 + 16 bits they measured slower than element by element.)
 template <typename IO, int POLICY = kStoreStreaming>
 __device__ __forceinline__ void view_store_first(__amdgpu_buffer_rsrc_t view, unsigned off, int n, int rem, float a, float b, float c,
                                                  float d)
@@ -229,18 +231,16 @@ __device__ __forceinline__ void view_store_first(__amdgpu_buffer_rsrc_t view, un
     const bool tail = off < kOob && n < 4;
     view_store4<IO, POLICY>(view, n >= 4 ? off : kOob, a, b, c, d);
     if (rem & 2) view_store2<IO, POLICY>(view, tail ? off : kOob, a, b);
-    if (rem & 1) {
-        const unsigned at = tail ? off + (rem == 3 ? 2u * static_cast<unsigned>(sizeof(IO)) : 0u) : kOob;
-        const float last = rem == 3 ? c : a;
-        if constexpr (sizeof(IO) == 4) {
-            view_store1<IO, POLICY>(view, at, last);
-        } else {
-            unsigned t;
-            if constexpr (std::is_same<IO, bf16_t>::value) t = bf16_pack2(last, 0.f);
-            else t = f16_pack2(last, 0.f);
-            __builtin_amdgcn_raw_buffer_store_b16(static_cast<unsigned short>(t & 0xffffu), view, at, 0, POLICY);
-        }
+    if constexpr (sizeof(IO) == 4) {
+        if (rem & 1) view_store1<IO, POLICY>(view, tail ? off + (rem == 3 ? 8u : 0u) : kOob, rem == 3 ? c : a);
     }
+}
+
+// Whether some row of a 16-bit tensor `width` elements wide that starts at `base` begins 2 bytes past a 32-bit boundary.
+template <typename IO>
+__device__ __forceinline__ bool mixed_row_starts(const IO *base, int width)
+{
+    return sizeof(IO) == 2 && ((width & 1) != 0 || (reinterpret_cast<uintptr_t>(base) & 2) != 0);
 }
 
 // Zeroes what a four-element load read past the `n` elements that were left of its row.
@@ -249,6 +249,43 @@ __device__ __forceinline__ void keep_first(float4 &v, int n)
     v.y = n > 1 ? v.y : 0.f;
     v.z = n > 2 ? v.z : 0.f;
     v.w = n > 3 ? v.w : 0.f;
+}
+
+// Views for rows of any width (vec_in == 3).  fp32: the plain view.  16 bits: every load must start on a 32-bit boundary,
+// so the view starts at the boundary at or before `base` and ends at the one at or after the last byte (at most two
+// bytes of the neighbouring planes, or of the allocation's own padding, on either side); `bias` is what a byte offset
+// relative to `base` is increased by.
+struct AnyWidthView {
+    __amdgpu_buffer_rsrc_t view;
+    unsigned bias;
+};
+template <typename IO>
+__device__ __forceinline__ AnyWidthView any_width_view(const IO *base, long bytes)
+{
+    AnyWidthView v;
+    if constexpr (sizeof(IO) == 4) {
+        v.bias = 0;
+        v.view = buffer_view(base, bytes);
+    } else {
+        v.bias = static_cast<unsigned>(reinterpret_cast<uintptr_t>(base) & 2);
+        v.view = buffer_view(reinterpret_cast<const char *>(base) - v.bias, (bytes + v.bias + 3) & ~3l);
+    }
+    return v;
+}
+// Four consecutive elements at byte offset `off` (relative to the view's tensor; kOob: zeros) as fp32.  16 bits: three
+// aligned dwords and two funnel shifts when the elements start in the middle of a dword.
+template <typename IO>
+__device__ __forceinline__ float4 any_width_load4(const AnyWidthView &v, unsigned off)
+{
+    if constexpr (sizeof(IO) == 4) {
+        return view_load4<IO>(v.view, off);
+    } else {
+        typedef unsigned int u32x3 __attribute__((ext_vector_type(3)));
+        const unsigned at = off < kOob ? off + v.bias : kOob;
+        const u32x3 d = __builtin_amdgcn_raw_buffer_load_b96(v.view, at & ~3u, 0, 0);
+        const unsigned sh = (at & 2u) << 3;
+        return widen4<IO>(make_uint2(__builtin_amdgcn_alignbit(d.y, d.x, sh), __builtin_amdgcn_alignbit(d.z, d.y, sh)));
+    }
 }
 
 // True when groups of four elements starting at `p` may be moved with one vector access.
@@ -300,6 +337,19 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__res
         const bool ragged = ANY_WIDTH && !VIEW_ONLY && s.vec_in == 3;
         // groups of four elements through a view of the tile's planes: slots outside the image read zeros
         const __amdgpu_buffer_rsrc_t view = buffer_view(in + plane0 * s.in_plane, static_cast<long>(nplanes) * s.in_plane * sizeof(IO));
+        // (16-bit rows that do not all start on 32-bit boundaries are loaded from such boundaries: see any_width_view)
+        AnyWidthView wide{view, 0};
+        bool split = false;
+        if constexpr (sizeof(IO) == 2 && ANY_WIDTH && !VIEW_ONLY) {
+            split = ragged && mixed_row_starts(in + plane0 * s.in_plane, s.in_w);
+            if (split) wide = any_width_view(in + plane0 * s.in_plane, static_cast<long>(nplanes) * s.in_plane * sizeof(IO));
+        }
+        auto load_slot = [&](unsigned off) -> float4 {
+            if constexpr (sizeof(IO) == 2 && ANY_WIDTH && !VIEW_ONLY) {
+                if (split) return any_width_load4<IO>(wide, off);
+            }
+            return view_load4<IO>(view, off);
+        };
         if constexpr (BY_ROWS) {
             // A lane owns one float4 column and every rpp-th row: column, column check and the LDS column are
             // computed once, and per slot only the row moves (two additions, a range check, a select), where the
@@ -337,7 +387,7 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__res
 #pragma unroll
                         for (int u = 0; u < kStageBatch; ++u) {
                             const bool ok = col_ok && static_cast<unsigned>(iy + u * rpp - lo) < span;
-                            v[u] = view_load4<IO>(view, ok ? off + u * off_step : kOob);
+                            v[u] = load_slot(ok ? off + u * off_step : kOob);
                         }
                         if (ragged) {
 #pragma unroll
@@ -360,7 +410,7 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__res
 #pragma unroll
                         for (int u = 0; u < kStageBatch; ++u) {
                             const bool ok = col_ok && static_cast<unsigned>(iy + u * rpp - lo) < span;
-                            v[u] = view_load4<IO>(view, ok ? off + u * off_step : kOob);
+                            v[u] = load_slot(ok ? off + u * off_step : kOob);
                         }
                         if (ragged) {
 #pragma unroll
@@ -389,7 +439,7 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__res
                             const int iy = iy0 + r;
                             const bool ok = live && col_ok && static_cast<unsigned>(iy) < static_cast<unsigned>(s.in_h);
                             const unsigned off = (__mul24(pl, s.in_plane) + __mul24(iy, s.in_w) + ix) * ES;
-                            v[u] = view_load4<IO>(view, ok ? off : kOob);
+                            v[u] = load_slot(ok ? off : kOob);
                             dst[u] = live ? __mul24(pl, s.plane_pitch) + __mul24(r, s.pitch) + dcol : dump;
                         }
                         if (ragged) {
@@ -427,7 +477,7 @@ __device__ __forceinline__ void stage_tile(const StageLayout &s, const IO *__res
                 const bool ok = live && static_cast<unsigned>(iy) < static_cast<unsigned>(s.in_h) &&
                                 static_cast<unsigned>(ix) < static_cast<unsigned>(s.in_w);
                 const unsigned off = (__mul24(pl, s.in_plane) + __mul24(iy, s.in_w) + ix) * static_cast<unsigned>(sizeof(IO));
-                v[u] = view_load4<IO>(view, ok ? off : kOob);
+                v[u] = load_slot(ok ? off : kOob);
                 if (ragged) keep_first(v[u], s.in_w - ix);
                 // slots past the end of the image (they hold zeros) go to the spare floats that end the image:
                 // the right-hand slack of its last row, which no stored output depends on
@@ -603,18 +653,21 @@ inline int vector_mode(long planes, long in_plane, size_t esize)
 // known: 1 = groups of four aligned elements (stage_vector_mode / vector_mode then decide between 1 and 2), 3 = groups
 // of four at any element alignment through a view (the caller drops to 0 where the view does not fit), 0 =
 // element by element.
-// (Mode 3 needs every row to start on a 32-bit boundary: the 64-bit loads of four 16-bit elements returned wrong
-// data from 2-byte-aligned addresses, so odd widths of 16-bit tensors stay with mode 0.)
+// `mixed_ok`: whether mode 3 is wanted also where rows of a 16-bit tensor start 2 bytes past a 32-bit boundary (odd
+// widths, or a base there).  64- and 32-bit accesses from such addresses returned wrong data; loads are then made from
+// the boundary before (any_width_load4: 150x150 -> 75x75 5x5 stride-2 forward in bf16 209 -> 130 us), stores stay
+// element by element (`mixed_ok` false for results: in aligned pieces of 16 + 32 + 16 bits they were 3-10 % slower).
 template <typename IO>
-inline int unaligned_vector_mode(int width, const IO *base)
+inline int unaligned_vector_mode(int width, const IO *base, bool mixed_ok)
 {
-    const bool dword_rows = sizeof(IO) == 4 || (width % 2 == 0 && (reinterpret_cast<uintptr_t>(base) & 3) == 0);
-    return dword_rows && env_int("DWCONV_RAGGED_VIEWS", 1) ? 3 : 0;
+    const bool mixed = sizeof(IO) == 2 && ((width & 1) != 0 || (reinterpret_cast<uintptr_t>(base) & 2) != 0);
+    if (mixed && !mixed_ok) return 0;
+    return env_int("DWCONV_RAGGED_VIEWS", 1) ? 3 : 0;
 }
 template <typename IO>
-inline int row_vector_mode(int width, const IO *base)
+inline int row_vector_mode(int width, const IO *base, bool mixed_ok = true)
 {
-    return width % 4 == 0 && aligned4(base) ? 1 : unaligned_vector_mode<IO>(width, base);
+    return width % 4 == 0 && aligned4(base) ? 1 : unaligned_vector_mode<IO>(width, base, mixed_ok);
 }
 
 // ---- a one-plane image staged in two steps --------------------------------------------------------------

@@ -120,8 +120,17 @@ __global__ __launch_bounds__(kThreads) void wgrad_tile_kernel(const WgradPlan p)
             if (p.vec_gy == 2 || (ANY_WIDTH && p.vec_gy == 3)) {
                 // branch-free: rows past the plane (and lanes without an item) read zeros through the view
                 const unsigned off = ((pl * p.out_plane + ox) + oy * p.out_w) * static_cast<unsigned>(sizeof(IO));
-                v = view_load4<IO>(buffer_view(gy + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO)), has_item && oy < p.out_h ? off : kOob);
-                if (ANY_WIDTH && p.vec_gy == 3) keep_first(v, p.out_w - ox);  // the block that ends a row
+                if (ANY_WIDTH && p.vec_gy == 3 && mixed_row_starts(gy + plane0 * p.out_plane, p.out_w)) {
+                    // (16-bit rows that do not all start on 32-bit boundaries)
+                    v = any_width_load4<IO>(any_width_view(gy + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO)),
+                                            has_item && oy < p.out_h ? off : kOob);
+                    keep_first(v, p.out_w - ox);
+                } else if (ANY_WIDTH && p.vec_gy == 3) {  // rows of any width: the block that ends a row is cut short
+                    v = view_load4<IO>(buffer_view(gy + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO)), has_item && oy < p.out_h ? off : kOob);
+                    keep_first(v, p.out_w - ox);
+                } else {
+                    v = view_load4<IO>(buffer_view(gy + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO)), has_item && oy < p.out_h ? off : kOob);
+                }
             } else if (has_item && oy < p.out_h) {
                 if (p.vec_gy) {
                     v = load4<IO>(row);
@@ -495,7 +504,7 @@ struct Launcher {
         p.strided = env_int("DWCONV_WGRAD_STRIDED", 1);
         p.taps = taps;
         p.gx = gx;
-        p.vec_gx = row_vector_mode(g.in_w, gx);
+        p.vec_gx = row_vector_mode(g.in_w, gx, false);
         const size_t shmem = lds_bytes<K, S, BH>(p, fused);
         const dim3 grid(p.groups * p.chunks), block(kThreads);
         // gy is staged with the x image's layout and mode

@@ -380,6 +380,88 @@ def test_small_maps_of_other_resolutions_full_batch(dw, gpu, shape):
     check_full_size(dw, gpu, shape, seed=51, expect=("small_down", "small_bwd"))
 
 
+# Rows that are not whole groups of four elements (EfficientNet at a 300-pixel input: maps 150, 75, 38 wide): the tiled
+# kernels move them with four-element accesses at element alignment through buffer views (modes "vin3", "vout3", "vgy3",
+# "vgx3" of the variant strings).
+ANY_WIDTH = [(2, 3, 40, 150, 3, 1, 1), (2, 3, 41, 75, 3, 1, 1), (2, 3, 38, 38, 5, 1, 2), (2, 3, 75, 75, 5, 2, 2),
+             (2, 2, 44, 150, 3, 2, 1), (3, 2, 38, 38, 3, 2, 1), (1, 3, 47, 57, 7, 1, 3), (2, 2, 66, 61, 7, 2, 3),
+             (2, 3, 35, 33, 3, 1, 0), (1, 2, 90, 201, 5, 1, 2), (2, 5, 34, 37, 5, 2, 1), (1, 2, 130, 65, 3, 1, 1)]
+
+
+@pytest.mark.parametrize("shape", ANY_WIDTH, ids=shape_id)
+def test_rows_of_any_width_fp32(dw, gpu, shape):
+    """Forward, both separate backward passes and the fused backward on rows of 33 ... 201 elements, against the C
+    oracle; every pass must have taken the view path, not the element-by-element one."""
+    from torch_dwconv import _C
+
+    n, c, h, w, k, s, p = shape
+    variant = check_against_c_oracle(dw, gpu, shape, seed=61)
+    assert " vin3 " in variant and variant.endswith("vout3"), variant
+    x, wt, gy = make_inputs(shape, seed=61)
+    xg, wg, gg = x.to(gpu), wt.to(gpu), gy.to(gpu)
+    ow = gy.shape[3]
+    _C.dwconv2d_backward(xg, gg, wg, s, s, p, p)
+    fused = _C.last_variant()
+    assert "vin3" in fused and ("vgy3" in fused or ow % 4 == 0), fused
+    if s == 2:
+        assert "vgx3" in fused, fused
+    _C.dwconv2d_backward_kernel(xg, gg, wg, 1, 1, s, s, p, p)
+    sep = _C.last_variant()
+    assert sep.startswith("wgrad_tile") and "vin3" in sep, sep
+
+
+def test_rows_of_any_width_unaligned_base(dw, gpu):
+    """Rows of whole groups of four whose tensor starts one element past a 16-byte boundary: the same view path."""
+    from torch_dwconv import _C
+
+    shape = (2, 3, 40, 48, 3, 1, 1)
+    x, wt, gy = make_inputs(shape, seed=62)
+    y_ref = oracle.forward(_np(x), _np(wt), 1, 1)
+    flat = torch.empty(x.numel() + 1, device=gpu)
+    flat[1:] = x.to(gpu).flatten()
+    xv = flat[1:].view_as(x)
+    y = dw.depthwise_conv2d(xv, wt.to(gpu), padding=1)
+    assert " vin3 " in _C.last_variant(), _C.last_variant()
+    np.testing.assert_allclose(_np(y), y_ref, rtol=1e-5, atol=1e-5)
+    gflat = torch.empty(gy.numel() + 1, device=gpu)
+    gflat[1:] = gy.to(gpu).flatten()
+    gx, gw = _C.dwconv2d_backward(xv, gflat[1:].view_as(gy), wt.to(gpu), 1, 1, 1, 1)
+    assert "vin3" in _C.last_variant() and "vgy3" in _C.last_variant(), _C.last_variant()
+    np.testing.assert_allclose(_np(gx), oracle.grad_input(_np(gy), _np(wt), (40, 48), 1, 1), rtol=1e-5, atol=1e-5)
+    gw_ref = oracle.grad_weight(_np(x), _np(gy), wt.shape, 1, 1)
+    np.testing.assert_allclose(_np(gw), gw_ref, rtol=1e-4, atol=1e-4 * float(np.abs(gw_ref).max()))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+def test_rows_of_any_width_half_precision(dw, gpu, dtype):
+    """16-bit tensors, even and odd widths (odd: every other row starts 2 bytes past a 32-bit boundary; such rows are
+    loaded from the boundary before and stored element by element), against the fp64 reference on the rounded inputs."""
+    from torch_dwconv import _C
+
+    step = 2.0 ** -11 if dtype == torch.float16 else 2.0 ** -8
+    for shape, mode in (((2, 3, 40, 150, 3, 1, 1), "vin3"), ((2, 3, 38, 38, 5, 2, 2), "vin3"), ((2, 2, 41, 75, 3, 1, 1), "vin3 vout0"),
+                        ((3, 3, 37, 39, 5, 2, 2), "vin3"), ((2, 3, 45, 67, 7, 1, 3), "vin3 vout0"), ((1, 5, 33, 35, 3, 2, 0), "vin3"),
+                        ((2, 2, 44, 54, 5, 1, 2), "vin3"), ((1, 3, 50, 70, 7, 2, 3), "vin3")):
+        n, c, h, w, k, s, p = shape
+        x, wt, gy = (t.to(dtype) for t in make_inputs(shape, seed=63))
+        y, gx, gw, variant = run_three_passes(dw, x.to(gpu), wt.to(gpu), gy.to(gpu), s, p)
+        _announce(shape_id(shape), str(dtype), variant)
+        assert mode in variant, variant
+        y_ref = oracle.forward(_np(x.double()), _np(wt.double()), s, p)
+        gx_ref = oracle.grad_input(_np(gy.double()), _np(wt.double()), (h, w), s, p)
+        gw_ref = oracle.grad_weight(_np(x.double()), _np(gy.double()), wt.shape, s, p)
+        np.testing.assert_allclose(_np(y.double()), y_ref, rtol=step, atol=1e-5 + step * 1e-2)
+        np.testing.assert_allclose(_np(gx.double()), gx_ref, rtol=step, atol=1e-5 + step * 1e-2)
+        np.testing.assert_allclose(_np(gw.double()), gw_ref, rtol=step + 1e-4, atol=(step + 1e-4) * float(np.abs(gw_ref).max()))
+
+
+@pytest.mark.parametrize("shape", [effnet_layers_at(300)[i] for i in (0, 1, 3, 4)], ids=shape_id)
+def test_rows_of_any_width_full_batch(dw, gpu, shape):
+    """Layers of the 300-pixel stack (150x150 3x3 stride 1 and 2, 75x75 5x5 stride 2, 38x38 5x5) at batch 128: whole
+    tensors against the fp64 reference, outputs start as NaN."""
+    check_full_size(dw, gpu, shape, seed=64, expect=("tile_down<", "bwd_tile"))
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
 @pytest.mark.parametrize("shape", [effnet_layers_at(256)[i] for i in (4, 5, 7, 10)] + [effnet_layers_at(240)[i] for i in (4, 5, 8, 9)], ids=shape_id)
 def test_small_maps_of_other_resolutions_half_precision(dw, gpu, shape, dtype):
