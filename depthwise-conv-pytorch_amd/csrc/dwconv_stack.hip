@@ -27,6 +27,8 @@
 // (large kernel, both directions at stride 1) and :260-306 (grad-weight) for these shapes.
 #include "dwconv_tile_common.hpp"
 
+#include <initializer_list>
+
 namespace dwconv {
 
 namespace {
@@ -92,6 +94,7 @@ struct StackLane {
     unsigned coff; // byte offset of the column within a row of the tensor
     bool col_ok;   // the column lies inside the plane (else it reads as zeros)
     int dcol;      // float offset of the column within an LDS row
+    int left;      // elements of the row from this column on (rows of any width: what a load reads past them is zeroed)
 };
 
 template <typename IO, int PADW>
@@ -104,6 +107,7 @@ __device__ __forceinline__ StackLane stack_lane(const StackPlan &p)
     l.coff = static_cast<unsigned>(ix) * static_cast<unsigned>(sizeof(IO));
     l.col_ok = static_cast<unsigned>(ix) < static_cast<unsigned>(p.w);
     l.dcol = kSlack + ix + PADW;
+    l.left = p.w - ix;
     return l;
 }
 
@@ -137,7 +141,8 @@ __device__ __forceinline__ void fetch_stack(const StackPlan &p, const StackLane 
     }
 }
 
-template <typename IO, int NS>
+// ANY_WIDTH: rows that are not whole groups of four elements (the last slot of a row has read into the next row).
+template <typename IO, int NS, bool ANY_WIDTH>
 __device__ __forceinline__ void commit_stack(const StackPlan &p, const StackLane &l, float *lds, const StackTile &t,
                                              const typename Raw4<IO>::type (&v)[NS])
 {
@@ -146,7 +151,8 @@ __device__ __forceinline__ void commit_stack(const StackPlan &p, const StackLane
     for (int u = 0; u < NS; ++u) {
         const int j = l.jr + u * p.rpp;
         float *d = lds + (j < t.rows ? __mul24(j, p.pitch) + l.dcol : dump);
-        const float4 w = widen4<IO>(v[u]);
+        float4 w = widen4<IO>(v[u]);
+        if constexpr (ANY_WIDTH) keep_first(w, l.left);
         d[0] = w.x;
         d[1] = w.y;
         d[2] = w.z;
@@ -162,7 +168,9 @@ __device__ __forceinline__ void commit_stack(const StackPlan &p, const StackLane
 // next tile's gy | grad-weight sums over the x windows.  Every image's loads fly during one arithmetic phase.
 // D: dilation (both axes); the window then spans KE = (K - 1) * D + 1 rows and columns and the "same" padding is
 // D * (K/2).
-template <typename IO, int K, int D, bool FUSED, bool FLIP, int NS>
+// ANY_WIDTH: the instance for rows that are not whole, 16-byte-aligned groups of four elements (loads and stores at
+// element alignment through the same views, the block that ends a row cut short); the other instance carries none of it.
+template <typename IO, int K, int D, bool FUSED, bool FLIP, int NS, bool ANY_WIDTH = false>
 __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -224,7 +232,7 @@ __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
         // (forward: the windows of the previous tile are read until here; fused: the slide image was last read
         // before the previous tile's second barrier)
         if (!FUSED && tile != chunk) __syncthreads();
-        commit_stack<IO, NS>(p, lane, lds_slide, cur, staged);
+        commit_stack<IO, NS, ANY_WIDTH>(p, lane, lds_slide, cur, staged);
         __syncthreads();
         StackTile nxt_tile = cur;
         if (more) {
@@ -300,12 +308,16 @@ __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
             for (int b = 0; b < BH; ++b) {
                 const int oy = r * BH + b;
                 const bool ok = has_item && oy < p.h;
-                view_store4<IO>(view, ok ? o0 + __mul24(oy, p.w) * ES : kOob, sums[b][0], sums[b][1], sums[b][2], sums[b][3]);
+                if constexpr (ANY_WIDTH)
+                    view_store_first<IO>(view, ok ? o0 + __mul24(oy, p.w) * ES : kOob, p.w - ox, p.w & 3, sums[b][0], sums[b][1],
+                                         sums[b][2], sums[b][3]);
+                else
+                    view_store4<IO>(view, ok ? o0 + __mul24(oy, p.w) * ES : kOob, sums[b][0], sums[b][1], sums[b][2], sums[b][3]);
             }
         }
 
         if constexpr (FUSED) {
-            commit_stack<IO, NS>(p, lane, lds_x, cur, staged);
+            commit_stack<IO, NS, ANY_WIDTH>(p, lane, lds_x, cur, staged);
             __syncthreads();
             if (more) fetch_stack<IO, PW, NS>(p, lane, slide_src + nxt_tile.plane0 * p.plane, nxt_tile, staged);
             const float *base = lds_x + base_off;
@@ -377,8 +389,8 @@ bool make_plan(StackPlan &p, int K, int D, int batch, int channel, int h, int w,
                bool half_io = false)
 {
     if (!stack_shape(K, D) && !(half_io && stack_shape_half(K, D, w, fused))) return false;
-    if (w % 4 != 0 || w < 16 || h < 8) return false;
-    const int ncb = w / 4;
+    if (w < 16 || h < 8) return false;
+    const int ncb = ceil_div(w, 4);
     if (ncb > kThreads) return false;
     const int ru = ceil_div(h, kStackBH);
     if (2 * ru * ncb <= kThreads) return false;
@@ -394,7 +406,7 @@ bool make_plan(StackPlan &p, int K, int D, int batch, int channel, int h, int w,
     p.ru = ru;
     p.vh = h + padw;
     p.ncb = ncb;
-    p.pitch = w + 16;  // kSlack + padw (<= 4) columns of zeros + w + zeros up to the last window column + kSlack, rounded up
+    p.pitch = round_up(w, 4) + 16;  // kSlack + padw (<= 4) columns of zeros + w + zeros up to the last window column + kSlack, rounded up
     p.spr = ncb + 2;
     const long total_units = static_cast<long>(batch) * ru;
     if (total_units >= (1l << 30)) return false;
@@ -463,24 +475,45 @@ struct StackLaunch {
     bool rot;
     size_t shmem;
     hipStream_t stream;
+    bool any_width = false;
     template <int K, int D>
     void operator()()
     {
         if constexpr (K == 3 && D == 1 && sizeof(IO) == 4) return;  // (16-bit elements only: stack_shape_half)
         const dim3 grid(static_cast<unsigned>(p.channel * p.chunks)), block(kThreads);
         const bool six = p.slots_per_lane <= 6;
+        if (any_width) launch<K, D, true>(grid, block, six);
+        else launch<K, D, false>(grid, block, six);
+    }
+    template <int K, int D, bool AW>
+    void launch(dim3 grid, dim3 block, bool six)
+    {
         if constexpr (FUSED) {
-            if (six) hipLaunchKernelGGL((stack_kernel<IO, K, D, true, true, 6>), grid, block, shmem, stream, p);
-            else hipLaunchKernelGGL((stack_kernel<IO, K, D, true, true, 8>), grid, block, shmem, stream, p);
+            if (six) hipLaunchKernelGGL((stack_kernel<IO, K, D, true, true, 6, AW>), grid, block, shmem, stream, p);
+            else hipLaunchKernelGGL((stack_kernel<IO, K, D, true, true, 8, AW>), grid, block, shmem, stream, p);
         } else if (rot) {
-            if (six) hipLaunchKernelGGL((stack_kernel<IO, K, D, false, true, 6>), grid, block, shmem, stream, p);
-            else hipLaunchKernelGGL((stack_kernel<IO, K, D, false, true, 8>), grid, block, shmem, stream, p);
+            if (six) hipLaunchKernelGGL((stack_kernel<IO, K, D, false, true, 6, AW>), grid, block, shmem, stream, p);
+            else hipLaunchKernelGGL((stack_kernel<IO, K, D, false, true, 8, AW>), grid, block, shmem, stream, p);
         } else {
-            if (six) hipLaunchKernelGGL((stack_kernel<IO, K, D, false, false, 6>), grid, block, shmem, stream, p);
-            else hipLaunchKernelGGL((stack_kernel<IO, K, D, false, false, 8>), grid, block, shmem, stream, p);
+            if (six) hipLaunchKernelGGL((stack_kernel<IO, K, D, false, false, 6, AW>), grid, block, shmem, stream, p);
+            else hipLaunchKernelGGL((stack_kernel<IO, K, D, false, false, 8, AW>), grid, block, shmem, stream, p);
         }
     }
 };
+
+// Which instance serves tensors of rows `w` wide at these bases: 0 = the aligned one, 1 = ANY_WIDTH, -1 = neither
+// (16-bit rows that do not all start on 32-bit boundaries: the general kernels take those).
+template <typename IO>
+int stack_width_mode(int w, std::initializer_list<const IO *> bases)
+{
+    bool aligned = w % 4 == 0, dword = sizeof(IO) == 4 || w % 2 == 0;
+    for (const IO *b : bases) {
+        aligned = aligned && aligned4(b);
+        dword = dword && (reinterpret_cast<uintptr_t>(b) & 3) == 0;
+    }
+    if (aligned) return 0;
+    return dword && env_int("DWCONV_RAGGED_VIEWS", 1) ? 1 : -1;
+}
 
 size_t stack_backward_workspace(int K, int D, int batch, int channel, int h, int w)
 {
@@ -497,7 +530,8 @@ int launch_stack_backward(const IO *in, const IO *gy, const IO *taps, IO *gx, IO
                           int batch, int channel, int h, int w, hipStream_t stream)
 {
     if (!env_int("DWCONV_STACK", 1)) return -1;
-    if (!aligned4(in) || !aligned4(gy) || !aligned4(gx)) return -1;
+    const int width_mode = stack_width_mode<IO>(w, {in, gy, gx});
+    if (width_mode < 0) return -1;
     StackPlan p{};
     if (!make_plan(p, K, D, batch, channel, h, w, 4, true, bwd_target_wgs(K), sizeof(IO) == 2)) return -1;
     const size_t need = static_cast<size_t>(channel) * p.chunks * K * K * sizeof(float);
@@ -508,11 +542,11 @@ int launch_stack_backward(const IO *in, const IO *gy, const IO *taps, IO *gx, IO
     p.taps = taps;
     p.out = gx;
     p.partial = static_cast<float *>(ws);
-    for_shape(K, D, StackLaunch<IO, true>{p, true, lds_bytes(p, K, true), stream});
+    for_shape(K, D, StackLaunch<IO, true>{p, true, lds_bytes(p, K, true), stream, width_mode == 1});
     const int rc = check_launch("stack_kernel");
     if (rc != DWCONV_OK) return rc;
-    note_variant("bwd_stack%s<k%d,d%d,s1> units%d tiles%d chunks%d", sizeof(IO) == 2 ? "16" : "", K, D, p.units_per_tile,
-                 p.tiles, p.chunks);
+    note_variant("bwd_stack%s<k%d,d%d,s1> units%d tiles%d chunks%d%s", sizeof(IO) == 2 ? "16" : "", K, D, p.units_per_tile,
+                 p.tiles, p.chunks, width_mode == 1 ? " anywidth" : "");
     return launch_wgrad_final(static_cast<const float *>(ws), gw, channel, K * K, p.chunks, stream);
 }
 
@@ -520,17 +554,22 @@ template <typename IO>
 int launch_stack_forward(const IO *in, const IO *taps, IO *out, int K, int D, int batch, int channel, int h, int w, bool rot,
                          hipStream_t stream)
 {
-    if (!env_int("DWCONV_STACK", 1)) return -1;
-    if (!aligned4(in) || !aligned4(out)) return -1;
+    if (!env_int("DWCONV_STACK", 1) || !env_int("DWCONV_STACK_FWD", 1)) return -1;
+    const int width_mode = stack_width_mode<IO>(w, {in, static_cast<const IO *>(out)});
+    if (width_mode < 0) return -1;
+    // fp32 at dilation 1: the general tiled kernel has overtaken this one on 5x5 filters (square maps 48-256 wide: 2-29 %
+    // faster; the 256x256 C=64 layer 104 against 114 us) and on 7x7 filters on wide rows (128: 9 %, 256: 38 %); 7x7 on
+    // rows up to 116 stays here (56x56 C=96: 43 against 48 us), whole groups of four only (57-75 wide: even or slower).
+    if (D == 1 && sizeof(IO) == 4 && !env_set("DWCONV_STACK_FWD") && (K == 5 || w > 116 || width_mode == 1)) return -1;
     StackPlan p{};
     // (short-lived workgroups of one tile each measured best: 56x56 C=96 7x7 43 us with 4800, 46-50 with 1280-4096)
     if (!make_plan(p, K, D, batch, channel, h, w, 4, false, env_int("DWCONV_STACK_FWD_WGS", 8192), sizeof(IO) == 2)) return -1;
     p.x = in;
     p.taps = taps;
     p.out = out;
-    for_shape(K, D, StackLaunch<IO, false>{p, rot, lds_bytes(p, K, false), stream});
-    note_variant("tile_stack%s<k%d,d%d,s1,%s> units%d tiles%d chunks%d", sizeof(IO) == 2 ? "16" : "", K, D, rot ? "rot" : "fwd",
-                 p.units_per_tile, p.tiles, p.chunks);
+    for_shape(K, D, StackLaunch<IO, false>{p, rot, lds_bytes(p, K, false), stream, width_mode == 1});
+    note_variant("tile_stack%s<k%d,d%d,s1,%s> units%d tiles%d chunks%d%s", sizeof(IO) == 2 ? "16" : "", K, D, rot ? "rot" : "fwd",
+                 p.units_per_tile, p.tiles, p.chunks, width_mode == 1 ? " anywidth" : "");
     return check_launch("stack_kernel");
 }
 

@@ -402,7 +402,10 @@ def test_rows_of_any_width_fp32(dw, gpu, shape):
     ow = gy.shape[3]
     _C.dwconv2d_backward(xg, gg, wg, s, s, p, p)
     fused = _C.last_variant()
-    assert "vin3" in fused and ("vgy3" in fused or ow % 4 == 0), fused
+    if fused.startswith("bwd_stack"):  # (5x5 / 7x7 stride-1 "same" layers: the stacked kernel's own any-width instance)
+        assert fused.endswith(" anywidth"), fused
+    else:
+        assert "vin3" in fused and ("vgy3" in fused or ow % 4 == 0), fused
     if s == 2:
         assert "vgx3" in fused, fused
     _C.dwconv2d_backward_kernel(xg, gg, wg, 1, 1, s, s, p, p)
@@ -446,7 +449,7 @@ def test_rows_of_any_width_half_precision(dw, gpu, dtype):
         x, wt, gy = (t.to(dtype) for t in make_inputs(shape, seed=63))
         y, gx, gw, variant = run_three_passes(dw, x.to(gpu), wt.to(gpu), gy.to(gpu), s, p)
         _announce(shape_id(shape), str(dtype), variant)
-        assert mode in variant, variant
+        assert mode in variant or variant.endswith(" anywidth"), variant  # (5x5 / 7x7 "same" layers: the stacked kernel)
         y_ref = oracle.forward(_np(x.double()), _np(wt.double()), s, p)
         gx_ref = oracle.grad_input(_np(gy.double()), _np(wt.double()), (h, w), s, p)
         gw_ref = oracle.grad_weight(_np(x.double()), _np(gy.double()), wt.shape, s, p)
@@ -514,7 +517,7 @@ def test_half_precision_full_batch_stacked_forward(dw, gpu, dtype):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
 def test_half_precision_full_batch_general_tiled_kernels(dw, gpu, dtype, monkeypatch):
     """The 16-bit instances of the general tiled kernels on the 56x56 3x3 layer (they serve what the stacked-image
-    kernel does not take: rows that are not whole groups of four, unaligned tensors, small planes)."""
+    kernel does not take: rows of odd width, tensors off a 32-bit boundary, small planes)."""
     monkeypatch.setenv("DWCONV_TUNING", "1")
     monkeypatch.setenv("DWCONV_STACK_K3_16", "0")
     check_full_size(dw, gpu, effnet_layers()[2], seed=41, dtype=dtype, expect=("tile_down16<", "bwd_tile16<"))
@@ -700,7 +703,8 @@ def test_half_precision_uses_the_fast_kernels(dw, gpu):
                             ((2, 8, 112, 112, 3, 2, 1), "tile_down16_dot2", "bwd_tile_s216"),
                             ((2, 8, 56, 56, 3, 1, 1), "tile_down16<", "bwd_stack16<k3"),
                             ((2, 8, 48, 48, 3, 1, 1), "tile_stack16<k3", "bwd_stack16<k3"),
-                            ((2, 8, 56, 54, 3, 1, 1), "tile_down16<", "bwd_tile16<"),
+                            ((2, 8, 56, 54, 3, 1, 1), "tile_down16<", "bwd_stack16<k3"),
+                            ((2, 8, 56, 55, 3, 1, 1), "tile_down16<", "bwd_tile16<"),
                             ((2, 8, 14, 14, 5, 1, 2), "small_down16", "small_bwd16"),
                             ((2, 8, 28, 28, 3, 1, 1), "small_down16", "small_bwd16")]:
         n, c, h, w, k, s, p = shape
@@ -709,6 +713,26 @@ def test_half_precision_uses_the_fast_kernels(dw, gpu):
         assert _C.last_variant().startswith(fwd), _C.last_variant()
         _C.dwconv2d_backward(x, gy, wt, s, s, p, p)
         assert _C.last_variant().startswith(bwd), _C.last_variant()
+
+
+def test_stacked_kernel_routes(dw, gpu):
+    """Which stride-1 "same" layers the stacked-image kernel takes: fp32 forward only 7x7 filters on aligned rows up to
+    116 elements (the general tiled kernel measured faster elsewhere); the fused backward 5x5 and 7x7 at any width,
+    with its own instance for rows that are not whole groups of four."""
+    from torch_dwconv import _C
+
+    for shape, fwd, bwd in [((2, 4, 64, 64, 5, 1, 2), "tile_down<k5", "bwd_stack<k5"),
+                            ((2, 4, 56, 56, 7, 1, 3), "tile_stack<k7", "bwd_stack<k7"),
+                            ((1, 3, 40, 128, 7, 1, 3), "tile_down<k7", "bwd_stack<k7"),
+                            ((2, 3, 57, 57, 5, 1, 2), "tile_down<k5", "bwd_stack<k5"),
+                            ((2, 3, 46, 66, 7, 1, 3), "tile_down<k7", "bwd_stack<k7")]:
+        n, c, h, w, k, s, p = shape
+        variant = check_against_c_oracle(dw, gpu, shape, seed=71)
+        assert variant.startswith(fwd), variant
+        x, wt, gy = (t.to(gpu) for t in make_inputs(shape, seed=71))
+        _C.dwconv2d_backward(x, gy, wt, s, s, p, p)
+        assert _C.last_variant().startswith(bwd), _C.last_variant()
+        assert _C.last_variant().endswith(" anywidth") == (w % 4 != 0), _C.last_variant()
 
 
 def test_tuning_overrides_need_the_master_switch(dw, gpu, monkeypatch):
@@ -1487,6 +1511,8 @@ GENERAL_CASES = [
     # that leave a hanging unit, tiles across two and three images
     (2, 3, 1, 40, 48, 3, 3, 1, 2, 2), (3, 2, 1, 33, 64, 5, 5, 1, 4, 2), (5, 2, 1, 57, 52, 3, 3, 1, 2, 2),
     (7, 1, 1, 18, 96, 5, 5, 1, 4, 2), (2, 2, 1, 130, 128, 3, 3, 1, 2, 2),
+    # the same on rows that are not whole groups of four elements
+    (2, 3, 1, 40, 50, 3, 3, 1, 2, 2), (2, 2, 1, 45, 75, 5, 5, 1, 4, 2), (3, 2, 1, 37, 33, 3, 3, 1, 2, 2),
     # dilation 2 on maps up to 32 wide: the whole-plane kernels (exact and ragged widths, odd planes)
     (3, 8, 1, 14, 14, 3, 3, 1, 2, 2), (2, 6, 1, 28, 28, 5, 5, 1, 4, 2), (3, 8, 1, 7, 7, 3, 3, 1, 2, 2), (2, 4, 1, 16, 16, 5, 5, 1, 4, 2),
     (2, 8, 1, 15, 15, 3, 3, 1, 2, 2), (3, 5, 1, 9, 30, 5, 5, 1, 4, 2), (2, 3, 1, 32, 32, 3, 3, 1, 2, 2), (2, 4, 1, 20, 24, 3, 3, 1, 2, 2),
@@ -1511,8 +1537,8 @@ def test_dilation_and_depth_multiplier(dw, gpu, case, dtype):
     gx, gw = torch.autograd.grad(y, (xg, wg), gy.to(gpu))
     _announce(case, str(dtype), v_fwd, "|", _C.last_variant())
     plain = m == 1 and d == 1
-    stacked = (m == 1 and d == 2 and s == 1 and kh == kw and kh in (3, 5) and p == d * (kh // 2) and w % 4 == 0 and w >= 16
-               and h >= 8 and 2 * ((h + 3) // 4) * (w // 4) > 256 and dtype != torch.float64)
+    stacked = (m == 1 and d == 2 and s == 1 and kh == kw and kh in (3, 5) and p == d * (kh // 2) and w >= 16
+               and h >= 8 and 2 * ((h + 3) // 4) * ((w + 3) // 4) > 256 and dtype != torch.float64)
     small = (m == 1 and d == 2 and s == 1 and kh == kw and kh in (3, 5) and p == d * (kh // 2) and w <= 32 and h <= 64
              and dtype != torch.float64)
     if case in MULTIPLIED_TILED and dtype != torch.float64:
@@ -1523,6 +1549,7 @@ def test_dilation_and_depth_multiplier(dw, gpu, case, dtype):
         assert v_bwd.startswith("tile_down" if s == 1 else "tile_up2") and "wgrad_tile" in v_bwd and v_bwd.count(" m%d" % m) == 2, v_bwd
     elif stacked:
         assert v_fwd.startswith("tile_stack") and _C.last_variant() is not None, v_fwd
+        assert v_fwd.endswith(" anywidth") == (w % 4 != 0), v_fwd
     elif small:
         assert v_fwd.startswith("small_down") and ",d2" in v_fwd, v_fwd
     else:
