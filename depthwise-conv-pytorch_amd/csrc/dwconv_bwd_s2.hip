@@ -313,8 +313,7 @@ bool plan_bwd_s2(BwdS2Plan &p, const WgradGeometry &g, int kBq, size_t esize)
     const long tiles = static_cast<long>(g.batch) * bands;
     if (tiles > 0x7fffffffL) return false;
     p.tiles_per_group = static_cast<int>(tiles);
-    // Workgroups in all.  The fp32 5x5 / 7x7 kernels gain from four times as many, shorter chunks (-7 % on a
-    // 56x56 layer, -4 % at 128x96); the 3x3 one does not, and with 16-bit elements, where the kernel is bound by
+    // Workgroups in all.  The fp32 5x5 / 7x7 kernels gain from twice as many, shorter chunks; the 3x3 one does not, and with 16-bit elements, where the kernel is bound by
     // instruction issue, the per-workgroup prologue and reduction make more chunks 8-15 % slower.
     // Two-step staging (see the kernel) is for 16-bit elements, where the arithmetic is long against the bytes: 56x56
     // 5x5 bf16 88 -> 81 us, 112x112 3x3 bf16 162 -> 156.  It needs several tiles per workgroup, and its registers
@@ -333,7 +332,8 @@ bool plan_bwd_s2(BwdS2Plan &p, const WgradGeometry &g, int kBq, size_t esize)
     if (p.prefetch) {
         chunks = env_int("DWCONV_WGRAD_WGS", kCus * (K == 7 ? 3 : 4) * 3) / g.channel;
     } else {
-        const int wgs = K >= 5 && esize == 4 ? 12288 : 3072;
+        // (5x5 fp32: 6144 against 12288 measured 3-8 % faster on 48- to 64-wide maps, the same at 75 and 128 x 96)
+        const int wgs = K >= 5 && esize == 4 ? 6144 : 3072;
         chunks = ceil_div(env_int("DWCONV_WGRAD_WGS", wgs), g.channel);
     }
     if (chunks > p.tiles_per_group) chunks = p.tiles_per_group;

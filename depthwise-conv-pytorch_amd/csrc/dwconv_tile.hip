@@ -637,8 +637,10 @@ int launch_down(TilePlan &p, hipStream_t stream)
     // A stride-2 layer reads four times what it writes: smaller tiles (more workgroups per CU, more loads in flight)
     // beat the halo rows they add: -17 % on a 56x56 5x5 layer, -3 % on a 112x112 3x3 one, -6 % on 128x96 5x5.
     // (16-bit elements land in an fp32 image, so the same bytes in flight need twice the LDS: 28 KiB measured best
-    // on the 112x112 3x3 layer, -12 %.)
-    constexpr int kBudget = S == 2 ? (sizeof(IO) == 2 ? 28 : 20) * 1024 : dwconv::kLdsBudget;
+    // on the 112x112 3x3 layer, -12 %.)  With four rows per lane 16 KiB is another 1-3 % better on 3x3 layers 112-128
+    // wide (bands of 12 rows instead of 16-20) and changes nothing for 5x5 ones; with seven rows per lane it would halve
+    // the band (150 -> 75: 248 -> 305 us) and 20 KiB stays.
+    constexpr int kBudget = S == 2 ? (sizeof(IO) == 2 ? 28 : (BH == 7 ? 20 : 16)) * 1024 : dwconv::kLdsBudget;
     if (!plan_tiles(p, ceil_div(p.out_h, BH), BH, used_cols, K * K, rows_for, kBudget)) return -1;
     // a depth multiplier is served where a tile is one plane (and, backward, a lane has one item): larger maps
     if (p.mult > 1 && (p.planes_per_tile != 1 || p.items_per_plane > kThreads)) return -1;
