@@ -66,6 +66,8 @@ WORKLOADS = {
     "convnext_t": lambda batch: [(64, 96, 56, 56, 7, 1, 3), (64, 192, 28, 28, 7, 1, 3),
                                  (64, 384, 14, 14, 7, 1, 3), (64, 768, 7, 7, 7, 1, 3)],
     "stress": lambda batch: [(64, 256, 128, 96, 5, 2, 2)],
+    # ConvNeXt-T's first three stages with the larger filters of its successors (9x9, 11x11, 13x13)
+    "large_filters": lambda batch: [(64, 96, 56, 56, 9, 1, 4), (64, 192, 28, 28, 11, 1, 5), (64, 384, 14, 14, 13, 1, 6)],
 }
 
 

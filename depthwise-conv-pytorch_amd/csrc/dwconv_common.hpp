@@ -242,6 +242,16 @@ int try_launch_bwd_small(const IO *in, const IO *gy, const IO *taps, IO *gx, IO 
                          const WgradGeometry &g, hipStream_t stream);
 // Pass 2 shared by the tiled and whole-plane grad-weight kernels:
 // gw[c][tap] = sum over chunks of partial[c][chunk][tap] (fp32 partial sums, added in fp64 in a fixed order).
+// The stacked-image kernels (dwconv_stack.hip) of one large filter size each, K = 9, 11, 13: translation units of their
+// own.  -1 when the geometry is not covered.
+template <int K>
+size_t stack_bigk_workspace(int batch, int channel, int h, int w);
+template <int K, typename IO>
+int stack_bigk_forward(const IO *in, const IO *taps, IO *out, int batch, int channel, int h, int w, bool rot, hipStream_t stream);
+template <int K, typename IO>
+int stack_bigk_backward(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes, int batch,
+                        int channel, int h, int w, hipStream_t stream);
+
 template <typename IO>
 int launch_wgrad_final(const float *partial, IO *gw, int channel, int taps, int chunks, hipStream_t stream);
 

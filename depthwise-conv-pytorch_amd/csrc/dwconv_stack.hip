@@ -25,9 +25,17 @@
 // and are reduced in a fixed order (wave64 DPP sum, then the four wavefronts through LDS) into
 // partial[c][chunk][tap]; the second pass is launch_wgrad_final.  Replaces torch_dwconv/dwconv_kernel.cu:69-181
 // (large kernel, both directions at stride 1) and :260-306 (grad-weight) for these shapes.
+//
+// One source, several translation units: built as it is, it holds the instances for 5x5 / 7x7 filters and the dilated
+// 3x3 / 5x5 ones (and 3x3 for 16-bit tensors); built with DWCONV_STACK_BIGK = 9, 11 or 13 it holds the instances of
+// that one filter size and exports them as stack_bigk_* (dwconv_common.hpp), which the first unit calls.
 #include "dwconv_tile_common.hpp"
 
 #include <initializer_list>
+
+#ifndef DWCONV_STACK_BIGK
+#define DWCONV_STACK_BIGK 0
+#endif
 
 namespace dwconv {
 
@@ -51,7 +59,7 @@ struct StackPlan {
     int total_units;       // batch * ru
     int tiles, chunks;
     int pitch;             // floats per LDS row
-    int spr;               // float4 slots fetched per row (one of zeros on either side)
+    int spr;               // float4 slots fetched per row (ceil(padding / 4) of zeros on either side)
     int img_floats;        // floats of one staged image (x or gy)
     int rpp;               // rows of an image the workgroup stages per pass: 256 / spr
     int slots_per_lane;    // loads a lane issues per tile image: ceil(rows / rpp) for the tallest tile
@@ -102,7 +110,7 @@ __device__ __forceinline__ StackLane stack_lane(const StackPlan &p)
 {
     StackLane l;
     const int jr = div_magic(threadIdx.x, p.spr_magic);
-    const int ix = 4 * (static_cast<int>(threadIdx.x) - jr * p.spr - 1);
+    const int ix = 4 * (static_cast<int>(threadIdx.x) - jr * p.spr - (PADW + 3) / 4);
     l.jr = jr < p.rpp ? jr : (1 << 20);
     l.coff = static_cast<unsigned>(ix) * static_cast<unsigned>(sizeof(IO));
     l.col_ok = static_cast<unsigned>(ix) < static_cast<unsigned>(p.w);
@@ -200,15 +208,19 @@ __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
 
     // The taps of the sliding pass, wavefront-uniform: scalar registers.  The fused 7x7 kernel has no room for 49 of
     // them beside its other scalars (the compiler then parks those in vector lanes and fetches them back around every
-    // staging step, some 230 lane reads per tile): it keeps the taps in the lanes of one vector register and brings
-    // each filter row into scalar registers when the window walk reaches it, 49 lane reads per tile and four rows
-    // live at a time.
-    constexpr bool kRollTaps = FUSED && K == 7;
+    // staging step, some 230 lane reads per tile), and filters from 9x9 up have more taps than there are scalar
+    // registers: those keep the taps in the lanes of one to three vector registers and bring each filter row into
+    // scalar registers when the window walk reaches it, K*K lane reads per tile and four rows live at a time.
+    constexpr bool kRollTaps = (FUSED && K == 7) || K > 7;
+    constexpr int kTapRegs = (KK + 63) / 64;
     float tap[kRollTaps ? 1 : KK];
-    float tap_lanes = 0.f;
+    float tap_lanes[kRollTaps ? kTapRegs : 1];
     if constexpr (kRollTaps) {
-        const int t = min(static_cast<int>(threadIdx.x) & 63, KK - 1);
-        tap_lanes = Io<IO>::in(static_cast<const IO *>(p.taps)[c * KK + KK - 1 - t]);
+#pragma unroll
+        for (int i = 0; i < kTapRegs; ++i) {
+            const int t = min(64 * i + (static_cast<int>(threadIdx.x) & 63), KK - 1);
+            tap_lanes[i] = Io<IO>::in(static_cast<const IO *>(p.taps)[c * KK + ((FUSED || FLIP) ? KK - 1 - t : t)]);
+        }
     } else {
 #pragma unroll
         for (int t = 0; t < KK; ++t) {
@@ -261,7 +273,10 @@ __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
             float nxt[4 * NV];
             load_window_row<NV>(sbase, nxt);
             float trow[kRollTaps ? K : 1][K];
-            if constexpr (kRollTaps) asm volatile("" : "+v"(tap_lanes));  // (keeps the lane reads inside the tile loop)
+            if constexpr (kRollTaps) {  // (keeps the lane reads inside the tile loop)
+#pragma unroll
+                for (int i = 0; i < kTapRegs; ++i) asm volatile("" : "+v"(tap_lanes[i]));
+            }
 #pragma unroll
             for (int wr = 0; wr < WIN_ROWS; ++wr) {
                 float win[4 * NV];
@@ -272,8 +287,8 @@ __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
                     if (wr % D == 0 && wr / D < K) {
 #pragma unroll
                         for (int tx = 0; tx < K; ++tx)
-                            trow[wr / D < K ? wr / D : 0][tx] =
-                                __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tap_lanes), (wr / D) * K + tx));
+                            trow[wr / D < K ? wr / D : 0][tx] = __int_as_float(__builtin_amdgcn_readlane(
+                                __float_as_int(tap_lanes[((wr / D) * K + tx) / 64]), ((wr / D) * K + tx) % 64));
                     }
                 }
                 if constexpr (FUSED) {
@@ -368,7 +383,11 @@ __global__ __launch_bounds__(kThreads) void stack_kernel(const StackPlan p)
 // workgroup (those shapes keep the several-planes mode of the general kernels).
 // (3x3 at dilation 1 stays with the general kernels: they wait for HBM, not for the vector unit, and measured the same
 // or faster: 112x112 C=32 fused backward 124-130 us here against 127, 56x56 C=144 152-158 against 132-144)
-bool stack_shape(int K, int D) { return (D == 1 && (K == 5 || K == 7)) || (D == 2 && (K == 3 || K == 5)); }
+bool stack_shape(int K, int D)
+{
+    if (DWCONV_STACK_BIGK) return D == 1 && K == DWCONV_STACK_BIGK;
+    return (D == 1 && (K == 5 || K == 7)) || (D == 2 && (K == 3 || K == 5));
+}
 // 16-bit elements, 3x3 at dilation 1, rows under 96 elements (from there on the kernels with 16-bit LDS images serve):
 // the general kernels are bound by their vector instructions with such tensors (the fused 56x56 backward keeps the
 // vector units 91 % busy with 196 of 256 lanes at work, 144 on a 48x48 map), and full lanes pay.  Measured by width
@@ -379,7 +398,7 @@ bool stack_shape(int K, int D) { return (D == 1 && (K == 5 || K == 7)) || (D == 
 // won by more than the noise.
 bool stack_shape_half(int K, int D, int w, bool fused)
 {
-    if (K != 3 || D != 1 || !env_int("DWCONV_STACK_K3_16", 1)) return false;
+    if (DWCONV_STACK_BIGK || K != 3 || D != 1 || !env_int("DWCONV_STACK_K3_16", 1)) return false;
     if (fused) return w <= 88;
     if (env_set("DWCONV_STACK_K3_16_FWD_W")) return w <= env_int("DWCONV_STACK_K3_16_FWD_W", 0);
     return w == 48 || w == 60 || w == 64 || w == 72;
@@ -389,11 +408,13 @@ bool make_plan(StackPlan &p, int K, int D, int batch, int channel, int h, int w,
                bool half_io = false)
 {
     if (!stack_shape(K, D) && !(half_io && stack_shape_half(K, D, w, fused))) return false;
-    if (w < 16 || h < 8) return false;
+    // (filters from 9x9 up have no other tuned kernel: their small planes come here too, from two row units and two
+    // column blocks on: the in-kernel divisions need divisors of at least 2)
+    if (w < (K > 7 ? 8 : 16) || h < (K > 7 ? 5 : 8)) return false;
     const int ncb = ceil_div(w, 4);
     if (ncb > kThreads) return false;
     const int ru = ceil_div(h, kStackBH);
-    if (2 * ru * ncb <= kThreads) return false;
+    if (K <= 7 && 2 * ru * ncb <= kThreads) return false;
     const long plane = static_cast<long>(h) * w;
     if (plane >= (1l << 23) || static_cast<long>(channel) * plane >= (1l << 28)) return false;
     const int ke = (K - 1) * D + 1, padw = D * (K / 2);
@@ -406,8 +427,9 @@ bool make_plan(StackPlan &p, int K, int D, int batch, int channel, int h, int w,
     p.ru = ru;
     p.vh = h + padw;
     p.ncb = ncb;
-    p.pitch = round_up(w, 4) + 16;  // kSlack + padw (<= 4) columns of zeros + w + zeros up to the last window column + kSlack, rounded up
-    p.spr = ncb + 2;
+    const int side = ceil_div(padw, 4);  // float4 slots of zeros on either side of a row
+    p.pitch = round_up(w, 4) + 8 * side + 8;  // kSlack + 4 * side columns of zeros + w + as many zeros + kSlack
+    p.spr = ncb + 2 * side;
     const long total_units = static_cast<long>(batch) * ru;
     if (total_units >= (1l << 30)) return false;
     p.total_units = static_cast<int>(total_units);
@@ -456,17 +478,23 @@ size_t lds_bytes(const StackPlan &p, int K, bool fused)
 // Workgroups of the fused kernel: one resident round (three per compute unit by its registers and LDS) for 7x7
 // filters (56x56 C=96 at batch 64: 768 workgroups 95 us, 1536 105, 2304 104); 5x5 filters do not care (256x256 C=64:
 // 189-197 us from 768 to 6144).
-int bwd_target_wgs(int K) { return env_int("DWCONV_STACK_WGS", K == 7 ? 768 : 1536); }
+// Larger filters like 7x7: 768 against 1536 on 56x56 9x9 126 against 136 us, 28x28 11x11 131 against 150, 14x14 13x13
+// 220 against 277 (the K*K sums of a workgroup are reduced once per workgroup).
+int bwd_target_wgs(int K) { return env_int("DWCONV_STACK_WGS", K >= 7 ? 768 : 1536); }
 
 // fn.template operator()<K, D>() for the supported (K, D)
 template <typename Fn>
 void for_shape(int K, int D, Fn &&fn)
 {
+#if DWCONV_STACK_BIGK
+    if (K == DWCONV_STACK_BIGK && D == 1) fn.template operator()<DWCONV_STACK_BIGK, 1>();
+#else
     if (K == 3 && D == 1) fn.template operator()<3, 1>();
     if (K == 5 && D == 1) fn.template operator()<5, 1>();
     if (K == 7 && D == 1) fn.template operator()<7, 1>();
     if (K == 3 && D == 2) fn.template operator()<3, 2>();
     if (K == 5 && D == 2) fn.template operator()<5, 2>();
+#endif
 }
 
 template <typename IO, bool FUSED>
@@ -518,6 +546,11 @@ int stack_width_mode(int w, std::initializer_list<const IO *> bases)
 size_t stack_backward_workspace(int K, int D, int batch, int channel, int h, int w)
 {
     if (!env_int("DWCONV_STACK", 1)) return 0;
+#if !DWCONV_STACK_BIGK
+    if (D == 1 && K == 9) return stack_bigk_workspace<9>(batch, channel, h, w);
+    if (D == 1 && K == 11) return stack_bigk_workspace<11>(batch, channel, h, w);
+    if (D == 1 && K == 13) return stack_bigk_workspace<13>(batch, channel, h, w);
+#endif
     StackPlan p{};
     // (the plan does not depend on the element size except through the view-extent check: the larger one)
     // (and a 16-bit caller may take the 3x3 instance)
@@ -530,6 +563,11 @@ int launch_stack_backward(const IO *in, const IO *gy, const IO *taps, IO *gx, IO
                           int batch, int channel, int h, int w, hipStream_t stream)
 {
     if (!env_int("DWCONV_STACK", 1)) return -1;
+#if !DWCONV_STACK_BIGK
+    if (D == 1 && K == 9) return stack_bigk_backward<9, IO>(in, gy, taps, gx, gw, ws, ws_bytes, batch, channel, h, w, stream);
+    if (D == 1 && K == 11) return stack_bigk_backward<11, IO>(in, gy, taps, gx, gw, ws, ws_bytes, batch, channel, h, w, stream);
+    if (D == 1 && K == 13) return stack_bigk_backward<13, IO>(in, gy, taps, gx, gw, ws, ws_bytes, batch, channel, h, w, stream);
+#endif
     const int width_mode = stack_width_mode<IO>(w, {in, gy, gx});
     if (width_mode < 0) return -1;
     StackPlan p{};
@@ -555,12 +593,17 @@ int launch_stack_forward(const IO *in, const IO *taps, IO *out, int K, int D, in
                          hipStream_t stream)
 {
     if (!env_int("DWCONV_STACK", 1) || !env_int("DWCONV_STACK_FWD", 1)) return -1;
+#if !DWCONV_STACK_BIGK
+    if (D == 1 && K == 9) return stack_bigk_forward<9, IO>(in, taps, out, batch, channel, h, w, rot, stream);
+    if (D == 1 && K == 11) return stack_bigk_forward<11, IO>(in, taps, out, batch, channel, h, w, rot, stream);
+    if (D == 1 && K == 13) return stack_bigk_forward<13, IO>(in, taps, out, batch, channel, h, w, rot, stream);
+#endif
     const int width_mode = stack_width_mode<IO>(w, {in, static_cast<const IO *>(out)});
     if (width_mode < 0) return -1;
     // fp32 at dilation 1: the general tiled kernel has overtaken this one on 5x5 filters (square maps 48-256 wide: 2-29 %
     // faster; the 256x256 C=64 layer 104 against 114 us) and on 7x7 filters on wide rows (128: 9 %, 256: 38 %); 7x7 on
     // rows up to 116 stays here (56x56 C=96: 43 against 48 us), whole groups of four only (57-75 wide: even or slower).
-    if (D == 1 && sizeof(IO) == 4 && !env_set("DWCONV_STACK_FWD") && (K == 5 || w > 116 || width_mode == 1)) return -1;
+    if (D == 1 && K <= 7 && sizeof(IO) == 4 && !env_set("DWCONV_STACK_FWD") && (K == 5 || w > 116 || width_mode == 1)) return -1;
     StackPlan p{};
     // (short-lived workgroups of one tile each measured best: 56x56 C=96 7x7 43 us with 4800, 46-50 with 1280-4096)
     if (!make_plan(p, K, D, batch, channel, h, w, 4, false, env_int("DWCONV_STACK_FWD_WGS", 8192), sizeof(IO) == 2)) return -1;
@@ -592,6 +635,35 @@ bool covers_general(const GeneralGeometry &g)
 }
 
 }  // namespace
+
+#if DWCONV_STACK_BIGK
+
+template <>
+size_t stack_bigk_workspace<DWCONV_STACK_BIGK>(int batch, int channel, int h, int w)
+{
+    return stack_backward_workspace(DWCONV_STACK_BIGK, 1, batch, channel, h, w);
+}
+template <int K, typename IO>
+int stack_bigk_forward(const IO *in, const IO *taps, IO *out, int batch, int channel, int h, int w, bool rot, hipStream_t stream)
+{
+    return launch_stack_forward<IO>(in, taps, out, K, 1, batch, channel, h, w, rot, stream);
+}
+template <int K, typename IO>
+int stack_bigk_backward(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes, int batch,
+                        int channel, int h, int w, hipStream_t stream)
+{
+    return launch_stack_backward<IO>(in, gy, taps, gx, gw, ws, ws_bytes, K, 1, batch, channel, h, w, stream);
+}
+#define DWCONV_INSTANTIATE(IO)                                                                                                \
+    template int stack_bigk_forward<DWCONV_STACK_BIGK, IO>(const IO *, const IO *, IO *, int, int, int, int, bool, hipStream_t); \
+    template int stack_bigk_backward<DWCONV_STACK_BIGK, IO>(const IO *, const IO *, const IO *, IO *, IO *, void *, size_t, int,  \
+                                                            int, int, int, hipStream_t);
+DWCONV_INSTANTIATE(float)
+DWCONV_INSTANTIATE(half_t)
+DWCONV_INSTANTIATE(bf16_t)
+#undef DWCONV_INSTANTIATE
+
+#else
 
 size_t bwd_stack_workspace(const WgradGeometry &g)
 {
@@ -651,5 +723,7 @@ DWCONV_INSTANTIATE(float)
 DWCONV_INSTANTIATE(half_t)
 DWCONV_INSTANTIATE(bf16_t)
 #undef DWCONV_INSTANTIATE
+
+#endif  // DWCONV_STACK_BIGK
 
 }  // namespace dwconv

@@ -735,6 +735,54 @@ def test_stacked_kernel_routes(dw, gpu):
         assert _C.last_variant().endswith(" anywidth") == (w % 4 != 0), _C.last_variant()
 
 
+LARGE_FILTERS = [(2, 3, 20, 24, 9, 1, 4), (3, 2, 33, 57, 9, 1, 4), (1, 4, 9, 12, 9, 1, 4), (2, 2, 41, 40, 11, 1, 5),
+                 (2, 3, 14, 14, 11, 1, 5), (1, 2, 70, 31, 11, 1, 5), (2, 2, 28, 28, 13, 1, 6), (3, 1, 37, 66, 13, 1, 6),
+                 (1, 3, 5, 8, 13, 1, 6), (5, 2, 6, 97, 13, 1, 6)]
+
+
+@pytest.mark.parametrize("shape", LARGE_FILTERS, ids=shape_id)
+def test_large_filters_take_the_stacked_kernels(dw, gpu, shape):
+    """9x9, 11x11 and 13x13 stride-1 "same" layers (planes from 5 rows and 8 columns on, any width): forward, both
+    separate passes and the fused backward through the stacked-image kernels, against the C oracle."""
+    from torch_dwconv import _C
+
+    n, c, h, w, k, s, p = shape
+    variant = check_against_c_oracle(dw, gpu, shape, seed=81)
+    assert variant.startswith("tile_stack<k%d,d1,s1,fwd>" % k), variant
+    x, wt, gy = (t.to(gpu) for t in make_inputs(shape, seed=81))
+    gx, gw = _C.dwconv2d_backward(x, gy, wt, s, s, p, p)
+    assert _C.last_variant().startswith("bwd_stack<k%d,d1,s1>" % k), _C.last_variant()
+    gx2, gw2 = _C.dwconv2d_backward(x, gy, wt, s, s, p, p)
+    assert torch.equal(gw, gw2) and torch.equal(gx, gx2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+def test_large_filters_half_precision(dw, gpu, dtype):
+    from torch_dwconv import _C
+
+    step = 2.0 ** -11 if dtype == torch.float16 else 2.0 ** -8
+    for shape in [(2, 3, 20, 24, 9, 1, 4), (2, 2, 33, 58, 11, 1, 5), (2, 2, 28, 28, 13, 1, 6)]:
+        n, c, h, w, k, s, p = shape
+        x, wt, gy = (t.to(dtype) for t in make_inputs(shape, seed=82))
+        y, gx, gw, variant = run_three_passes(dw, x.to(gpu), wt.to(gpu), gy.to(gpu), s, p)
+        _announce(shape_id(shape), str(dtype), variant)
+        assert variant.startswith("tile_stack16<k%d" % k), variant
+        y_ref = oracle.forward(_np(x.double()), _np(wt.double()), s, p)
+        gx_ref = oracle.grad_input(_np(gy.double()), _np(wt.double()), (h, w), s, p)
+        gw_ref = oracle.grad_weight(_np(x.double()), _np(gy.double()), wt.shape, s, p)
+        np.testing.assert_allclose(_np(y.double()), y_ref, rtol=step, atol=1e-5 + step * 2e-2)
+        np.testing.assert_allclose(_np(gx.double()), gx_ref, rtol=step, atol=1e-5 + step * 2e-2)
+        np.testing.assert_allclose(_np(gw.double()), gw_ref, rtol=step + 1e-4, atol=(step + 1e-4) * float(np.abs(gw_ref).max()))
+
+
+@pytest.mark.parametrize("shape", [(64, 96, 56, 56, 9, 1, 4), (64, 192, 28, 28, 11, 1, 5), (64, 384, 14, 14, 13, 1, 6)], ids=shape_id)
+def test_large_filters_full_size(dw, gpu, shape):
+    """ConvNeXt-T's first three stages with 9x9, 11x11 and 13x13 filters at batch 64: whole tensors against the fp64
+    reference, outputs start as NaN."""
+    k = shape[4]
+    check_full_size(dw, gpu, shape, seed=83, expect=("tile_stack<k%d" % k, "bwd_stack<k%d" % k))
+
+
 def test_tuning_overrides_need_the_master_switch(dw, gpu, monkeypatch):
     """DWCONV_* overrides of the planners are ignored unless DWCONV_TUNING=1 is set too, and ill-formed values always."""
     from torch_dwconv import _C
