@@ -102,6 +102,8 @@ int run_fir(const T *in, const T *taps, T *out, const Geometry &g, hipStream_t s
             if (rc >= 0) return rc;
             rc = try_launch_fir_tiled<T>(in, taps, out, g, stream);
             if (rc >= 0) return rc;
+            rc = try_launch_fir_any<T>(in, taps, out, g, stream);
+            if (rc >= 0) return rc;
         }
     }
     return launch_fir_direct<T>(in, taps, out, g, stream);
@@ -442,6 +444,14 @@ int general_forward_any(const T *in, const T *taps, T *out, int batch, int chann
                             pad_h, pad_h, pad_w, pad_w, g.out_h, g.out_w, 1};
                 gg.mult = multiplier;
                 r = try_launch_fir_tiled<T>(in, taps, out, gg, static_cast<hipStream_t>(stream));
+                if (r >= 0) return r;
+            }
+            if (multiplier == 1) {  // any other dilation, stride or filter extent: the any-geometry tiled kernel
+                Geometry gg{batch, channel, in_h, in_w, kernel_h, kernel_w, 1, 1, stride_h, stride_w,
+                            pad_h, pad_h, pad_w, pad_w, g.out_h, g.out_w, 1};
+                gg.dil_h = dil_h;
+                gg.dil_w = dil_w;
+                r = try_launch_fir_any<T>(in, taps, out, gg, static_cast<hipStream_t>(stream));
                 if (r >= 0) return r;
             }
         }

@@ -153,6 +153,8 @@ struct Geometry {
     // result plane (n, c) adds up the planes (n, c * M + m) of an operand with channel * M channels, each with the
     // taps of its own channel.
     int mult = 1;
+    // Dilation of the taps (the any-geometry tiled kernel only; every other kernel is handed 1).
+    int dil_h = 1, dil_w = 1;
     long planes() const { return static_cast<long>(batch) * channel; }
 };
 
@@ -222,6 +224,9 @@ int launch_wgrad_direct(const T *in, const T *gy, T *gw, void *ws, size_t ws_byt
 // or a positive dwconv_status on a launch error.
 template <typename IO>  // float, half_t or bf16_t
 int try_launch_fir_tiled(const IO *in, const IO *taps, IO *out, const Geometry &g, hipStream_t stream);
+// The same for any filter extent, stride and dilation (up = 1): taps looped over at run time (dwconv_tile.hip).
+template <typename IO>
+int try_launch_fir_any(const IO *in, const IO *taps, IO *out, const Geometry &g, hipStream_t stream);
 // The same for 16-bit tensors whose rows are whole groups of eight elements: raw 16-bit LDS image and two-element
 // dot products (dwconv_tile16.hip).  -1 when it does not cover g.
 template <typename IO>

@@ -53,6 +53,8 @@ struct TilePlan {
                                // `channel` counts the result's channels and plane (n, c) adds up the M planes
                                // (n, c * M + m) of the operand, each with the taps of its own channel
     Epilogue epi;              // forward kernels: applied to every sum before it is stored
+    // fir_any_kernel: filter extent, decimation and dilation per axis, and whether the taps are rotated
+    int kh, kw, sh, sw, dh, dw, flip;
 };
 
 // Copies the tap tables of the tile's planes into LDS, rotated by 180 degrees if FLIP.
@@ -552,6 +554,93 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
     }
 }
 
+// Any filter extent, stride and dilation (up = 1): what has no kernel of its own above (rectangular and even-sized
+// filters, strip filters such as 1 x 7 or 21 x 1, 15 x 15 and larger, strides above 2, dilations above 2).  The same
+// tiles and the same LDS image; the taps are looped over at run time, so a lane reads its BH x 4 inputs from LDS for
+// every tap instead of keeping window rows in registers: one LDS read per multiply-add, which still leaves filters of
+// few taps bound by HBM.  Replaces the generic instantiation of torch_dwconv/dwconv_kernel.cu:69-181 (kernel sizes of
+// -1) for these shapes.
+// SW: the column stride when it is 1 or 2 (the four inputs of a row then sit at immediate offsets), 0 = any.
+template <typename IO, int BH, int SW>
+__global__ __launch_bounds__(kThreads) void fir_any_kernel(const TilePlan p)
+{
+    extern __shared__ float4 lds_raw[];
+    float *lds = reinterpret_cast<float *>(lds_raw);
+    const int KK = p.kh * p.kw;
+    const int sw = SW ? SW : p.sw;
+
+    const int tile = xcd_contiguous_tile(blockIdx.x, p.n_tiles);
+    const int pg = tile / p.row_tiles, rt = tile - pg * p.row_tiles;
+    const long plane0 = static_cast<long>(pg) * p.planes_per_tile;
+    const int nplanes = static_cast<int>(min(static_cast<long>(p.planes_per_tile), p.planes - plane0));
+    const int oy0 = rt * p.rows_per_tile;
+
+    for (int i = threadIdx.x; i < nplanes * KK; i += blockDim.x) {
+        const int pl = i / KK, t = i - pl * KK;
+        const int c = static_cast<int>((plane0 + pl) % p.channel);
+        lds[p.tap_base + i] = Io<IO>::in(static_cast<const IO *>(p.taps)[c * KK + (p.flip ? KK - 1 - t : t)]);
+    }
+    stage_tile<IO, false, kStageBatch, true>(p.st, static_cast<const IO *>(p.in), lds, plane0, nplanes, oy0 * p.sh - p.row_shift);
+    __syncthreads();
+
+    const int n_items = nplanes * p.items_per_plane;
+    const int row_step = p.sh * p.st.pitch;
+    for (int item = threadIdx.x; item < n_items; item += blockDim.x) {
+        const int pl = fast_div(item, p.ipp_magic);
+        const int rem = item - __mul24(pl, p.items_per_plane);
+        const int rb = fast_div(rem, p.ncb_magic);
+        const int cb = rem - __mul24(rb, p.ncb);
+        float acc[BH][4];
+#pragma unroll
+        for (int b = 0; b < BH; ++b)
+#pragma unroll
+            for (int o = 0; o < 4; ++o) acc[b][o] = 0.f;
+        const float *base = lds + __mul24(pl, p.st.plane_pitch) + __mul24(rb * BH, row_step) + kSlack + 4 * cb * sw;
+        const float *tp = lds + p.tap_base + pl * KK;
+        for (int ty = 0; ty < p.kh; ++ty) {
+            const float *trow = base + __mul24(ty * p.dh, p.st.pitch);
+            for (int tx = 0; tx < p.kw; ++tx) {
+                const float t = tp[ty * p.kw + tx];
+                const float *r = trow + tx * p.dw;
+#pragma unroll
+                for (int b = 0; b < BH; ++b)
+#pragma unroll
+                    for (int o = 0; o < 4; ++o) acc[b][o] = fmaf(r[b * row_step + o * sw], t, acc[b][o]);
+            }
+        }
+        if (!p.flip && p.epi.enabled()) epilogue_apply_block<1>(acc, p.epi, static_cast<int>((plane0 + pl) % p.channel));
+
+        const int ox = 4 * cb;
+        if (p.vec_out >= 2) {
+            // branch-free: rows past the end of the plane store out of range
+            const __amdgpu_buffer_rsrc_t view = buffer_view(static_cast<IO *>(p.out) + plane0 * p.out_plane, static_cast<long>(nplanes) * p.out_plane * sizeof(IO));
+            const unsigned o0 = (pl * p.out_plane + ox) * static_cast<unsigned>(sizeof(IO));
+#pragma unroll
+            for (int b = 0; b < BH; ++b) {
+                const int oy = oy0 + rb * BH + b;
+                const unsigned off = oy < p.out_h ? o0 + oy * p.out_w * static_cast<unsigned>(sizeof(IO)) : kOob;
+                if (p.vec_out == 3) view_store_first<IO>(view, off, p.out_w - ox, p.out_w & 3, acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+                else view_store4<IO>(view, off, acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+            }
+            continue;
+        }
+        IO *dst = static_cast<IO *>(p.out) + (plane0 + pl) * p.out_plane + ox;
+#pragma unroll
+        for (int b = 0; b < BH; ++b) {
+            const int oy = oy0 + rb * BH + b;
+            if (oy >= p.out_h) continue;
+            IO *row = dst + static_cast<long>(oy) * p.out_w;
+            if (p.vec_out) {
+                store4<IO>(row, acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+            } else {
+#pragma unroll
+                for (int o = 0; o < 4; ++o)
+                    if (ox + o < p.out_w) row[o] = Io<IO>::out(acc[b][o]);
+            }
+        }
+    }
+}
+
 // Fills in the tiling of `p` for a plane whose output is split into `row_units`
 // units of rows (BH output rows or BQ half-resolution rows each) and `ncb` column
 // blocks.  `rows_for(units)` gives the LDS rows a band of that many units needs.
@@ -709,6 +798,66 @@ int launch_up2_parity(TilePlan &p, int ey, int ex, hipStream_t stream)
 }
 
 }  // namespace
+
+template <typename IO>
+int try_launch_fir_any(const IO *in, const IO *taps, IO *out, const Geometry &g, hipStream_t stream)
+{
+    if (!env_int("DWCONV_FIR_ANY", 1)) return -1;
+    if (g.up_h != 1 || g.up_w != 1 || g.mult != 1) return -1;
+    if (g.kernel_h < 1 || g.kernel_w < 1 || g.down_h < 1 || g.down_w < 1 || g.dil_h < 1 || g.dil_w < 1) return -1;
+    if (g.pad_h0 < 0 || g.pad_w0 < 0 || g.in_h < 1 || g.in_w < 1) return -1;
+    if (static_cast<long>(g.kernel_h) * g.kernel_w > 4096) return -1;
+    if (static_cast<long>(g.in_h) * g.in_w >= (1l << 30) || static_cast<long>(g.out_h) * g.out_w >= (1l << 30)) return -1;
+    // (everything the staging multiplies must stay far below 2^23)
+    const long span_h = static_cast<long>(g.kernel_h - 1) * g.dil_h, span_w = static_cast<long>(g.kernel_w - 1) * g.dil_w;
+    if (span_h > 4096 || span_w > 4096 || g.down_h > 64 || g.down_w > 64 || g.pad_h0 > 4096 || g.pad_w0 > 4096) return -1;
+
+    constexpr int BH = 4;
+    TilePlan p{};
+    p.in = in;
+    p.taps = taps;
+    p.out = out;
+    p.planes = g.planes();
+    p.channel = g.channel;
+    p.mult = 1;
+    p.epi = g.epi;
+    p.st.in_h = g.in_h;
+    p.st.in_w = g.in_w;
+    p.out_h = g.out_h;
+    p.out_w = g.out_w;
+    p.st.in_plane = g.in_h * g.in_w;
+    p.out_plane = g.out_h * g.out_w;
+    p.st.vec_in = row_vector_mode(g.in_w, in);
+    p.vec_out = row_vector_mode(g.out_w, out, false);
+    p.row_shift = g.pad_h0;
+    p.st.col_shift = g.pad_w0;
+    p.kh = g.kernel_h;
+    p.kw = g.kernel_w;
+    p.sh = g.down_h;
+    p.sw = g.down_w;
+    p.dh = g.dil_h;
+    p.dw = g.dil_w;
+    p.flip = !g.forward;
+    p.ncb = ceil_div(p.out_w, 4);
+    const long used_cols = static_cast<long>(4 * p.ncb - 1) * p.sw + span_w + 1;
+    if (used_cols > (1 << 16)) return -1;
+    const int sh = p.sh, span = static_cast<int>(span_h);
+    auto rows_for = [sh, span](int units) { return (units * BH - 1) * sh + span + 1; };
+    if (!plan_tiles(p, ceil_div(p.out_h, BH), BH, static_cast<int>(used_cols), p.kh * p.kw, rows_for)) return -1;
+    settle_vector_modes<IO>(p);
+    const dim3 grid(p.n_tiles), block(kThreads);
+    const size_t shmem = lds_bytes(p, p.kh * p.kw);
+    if (p.sw == 1) hipLaunchKernelGGL((fir_any_kernel<IO, BH, 1>), grid, block, shmem, stream, p);
+    else if (p.sw == 2) hipLaunchKernelGGL((fir_any_kernel<IO, BH, 2>), grid, block, shmem, stream, p);
+    else hipLaunchKernelGGL((fir_any_kernel<IO, BH, 0>), grid, block, shmem, stream, p);
+    note_variant("tile_any%s<k%dx%d,s%dx%d,d%dx%d,%s> P%d rows%d vin%d vout%d", sizeof(IO) == 2 ? "16" : "", p.kh, p.kw, p.sh, p.sw,
+                 p.dh, p.dw, p.flip ? "rot" : "fwd", p.planes_per_tile, p.rows_per_tile, p.st.vec_in, p.vec_out);
+    return check_launch("fir_any_kernel");
+}
+
+template int try_launch_fir_any<float>(const float *, const float *, float *, const Geometry &, hipStream_t);
+template int try_launch_fir_any<half_t>(const half_t *, const half_t *, half_t *, const Geometry &, hipStream_t);
+template int try_launch_fir_any<bf16_t>(const bf16_t *, const bf16_t *, bf16_t *, const Geometry &, hipStream_t);
 
 template <typename IO>
 int try_launch_fir_tiled(const IO *in, const IO *taps, IO *out, const Geometry &g, hipStream_t stream)

@@ -1200,7 +1200,7 @@ FUSED_CASES = [
     # (shape, channels_last, expected kernel family)
     ((2, 8, 56, 56, 3, 1, 1), False, "tile_down"), ((2, 6, 57, 44, 5, 2, 2), False, "tile_down"),
     ((3, 8, 14, 14, 5, 1, 2), False, "small_down"), ((2, 12, 28, 28, 3, 2, 1), False, "small_down"),
-    ((2, 3, 9, 11, 4, 1, 1), False, "direct"), ((2, 16, 20, 24, 3, 1, 1), True, "nhwc_down"),
+    ((2, 3, 9, 11, 4, 1, 1), False, "tile_any"), ((2, 16, 20, 24, 3, 1, 1), True, "nhwc_down"),
     ((2, 8, 15, 13, 5, 2, 2), True, "nhwc_down"), ((2, 5, 9, 9, 3, 1, 1), True, "nhwc_fwd_direct"),
 ]
 
@@ -1226,6 +1226,27 @@ def test_fused_epilogue(dw, gpu, case, activation):
         assert y.is_contiguous(memory_format=torch.channels_last) == nhwc or y.is_contiguous()
         ref = oracle.torch_reference_fused(x, wt, sc, sh, activation, s, p)
         np.testing.assert_allclose(_np(y).astype(np.float64), ref.numpy(), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("activation", [None, "relu6", "silu"])
+def test_fused_epilogue_per_element_kernel(dw, gpu, activation, monkeypatch):
+    """The epilogue inside the per-element kernel, which serves what no tiled kernel takes (here: with the any-geometry
+    tiled kernel switched off)."""
+    from torch_dwconv import _C
+    from torch_dwconv.dwconv import depthwise_conv2d_fused
+
+    monkeypatch.setenv("DWCONV_TUNING", "1")
+    monkeypatch.setenv("DWCONV_FIR_ANY", "0")
+    shape = (2, 3, 9, 11, 4, 1, 1)
+    n, c, h, w, k, s, p = shape
+    x, wt, _ = make_inputs(shape, seed=43)
+    x = x * 2
+    g = torch.Generator("cpu").manual_seed(44)
+    scale, shift = torch.randn(c, generator=g) + 1.5, torch.randn(c, generator=g)
+    y = depthwise_conv2d_fused(x.to(gpu), wt.to(gpu), bias=shift.to(gpu), scale=scale.to(gpu), activation=activation, stride=s, padding=p)
+    assert _C.last_variant().startswith("direct"), _C.last_variant()
+    ref = oracle.torch_reference_fused(x, wt, scale, shift, activation, s, p)
+    np.testing.assert_allclose(_np(y).astype(np.float64), ref.numpy(), rtol=1e-5, atol=1e-5)
 
 
 def test_fused_epilogue_other_dtypes_and_autograd(dw, gpu):
@@ -1600,8 +1621,12 @@ def test_dilation_and_depth_multiplier(dw, gpu, case, dtype):
         assert v_fwd.endswith(" anywidth") == (w % 4 != 0), v_fwd
     elif small:
         assert v_fwd.startswith("small_down") and ",d2" in v_fwd, v_fwd
+    elif plain:
+        assert not v_fwd.startswith("general_fwd"), v_fwd  # the plain case runs the tuned kernels
+    elif m == 1 and dtype != torch.float64:
+        assert v_fwd.startswith("tile_any<k%dx%d,s%dx%d,d%dx%d" % (kh, kw, s, s, d, d)), v_fwd  # any other dilation / stride
     else:
-        assert v_fwd.startswith("general_fwd") != plain, v_fwd  # the plain case runs the tuned kernels
+        assert v_fwd.startswith("general_fwd"), v_fwd
     y_ref, gx_ref, gw_ref = oracle.torch_reference_general(x, wt, gy, s, p, d)
     tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-12, atol=1e-12)
     np.testing.assert_allclose(_np(y.detach()).astype(np.float64), y_ref.numpy(), **tol)
