@@ -53,8 +53,6 @@ int check_launch(const char *what)
 
 namespace {
 
-constexpr int kMaxSmallKernel = 15;
-
 int make_geometry(Geometry &g, const void *in, const void *taps, const void *out, int batch,
                   int channel, int in_h, int in_w, int kernel_h, int kernel_w, int up_h, int up_w,
                   int down_h, int down_w, int pad_h0, int pad_h1, int pad_w0, int pad_w1, int forward)
@@ -141,9 +139,8 @@ int dwconv2d_small_any(const T *in, const T *taps, T *out, int batch, int channe
     if (in_h > 32 || in_w > 32)
         return fail(DWCONV_ERR_UNSUPPORTED, "dwconv2d_small handles planes up to 32x32, got %dx%d",
                     in_h, in_w);
-    if (kernel_h < 1 || kernel_w < 1 || kernel_h > kMaxSmallKernel || kernel_w > kMaxSmallKernel)
-        return fail(DWCONV_ERR_UNSUPPORTED, "dwconv2d_small handles kernels from 1x1 to %dx%d, got %dx%d",
-                    kMaxSmallKernel, kMaxSmallKernel, kernel_h, kernel_w);
+    if (kernel_h < 1 || kernel_w < 1)
+        return fail(DWCONV_ERR_UNSUPPORTED, "dwconv2d_small needs a kernel of at least 1x1, got %dx%d", kernel_h, kernel_w);
     if (pad_h < 0 || pad_h >= kernel_h || pad_w < 0 || pad_w >= kernel_w)
         return fail(DWCONV_ERR_UNSUPPORTED, "dwconv2d_small needs 0 <= pad < kernel, got pad %dx%d kernel %dx%d",
                     pad_h, pad_w, kernel_h, kernel_w);
@@ -192,6 +189,8 @@ size_t wgrad_workspace(const WgradGeometry &g)
         if (s2 > need) need = s2;
         const size_t st = bwd_stack_workspace(g);
         if (st > need) need = st;
+        const size_t any = wgrad_any_workspace(g, 1, 1);
+        if (any > need) need = any;
         if constexpr (sizeof(T) == 2) {
             const size_t t16 = bwd_tiled16_workspace(g);
             if (t16 > need) need = t16;
@@ -231,6 +230,8 @@ int wgrad_any(const T *in, const T *gy, T *gw, void *ws, size_t ws_bytes, int ba
                 const int r = try_launch_wgrad_tiled<T>(in, gy, gw, ws, ws_bytes, g, stream);
                 if (r >= 0) return r;
             }
+            const int r = try_launch_wgrad_any<T>(in, gy, gw, ws, ws_bytes, g, 1, 1, stream);
+            if (r >= 0) return r;
         }
     }
     return launch_wgrad_direct<T>(in, gy, gw, ws, ws_bytes, g, stream);
@@ -475,6 +476,12 @@ size_t general_workspace_any(const GeneralGeometry &g)
             const size_t sm = wgrad_small_workspace(dilated_wgrad_geometry(g));
             if (sm > need) need = sm;
         }
+        if (g.multiplier == 1) {
+            const WgradGeometry wg{g.batch, g.channel, g.in_h, g.in_w, g.out_h, g.out_w, g.kernel_h, g.kernel_w,
+                                   g.stride_h, g.stride_w, g.pad_h, g.pad_w};
+            const size_t any = wgrad_any_workspace(wg, g.dil_h, g.dil_w);
+            if (any > need) need = any;
+        }
         if (multiplied_tiled(g)) {
             const size_t mt = wgrad_tiled_workspace(multiplied_wgrad_geometry(g));
             if (mt > need) need = mt;
@@ -536,6 +543,32 @@ int general_backward_any(const T *in, const T *gy, const T *taps, T *gx, T *gw, 
                 char first[sizeof(g_variant)];
                 std::snprintf(first, sizeof(first), "%s", g_variant);
                 rc = try_launch_wgrad_tiled<T>(in, gy, gw, ws, ws_bytes, multiplied_wgrad_geometry(g), stream);
+                if (rc < 0) rc = general_grad_weight<T>(in, gy, gw, ws, ws_bytes, g, stream);
+                if (rc != DWCONV_OK) return rc;
+                char second[sizeof(g_variant)];
+                std::snprintf(second, sizeof(second), "%s", g_variant);
+                note_variant("%.60s + %.60s", first, second);
+                return DWCONV_OK;
+            }
+            if (multiplier == 1 && in_h > 0 && in_w > 0) {
+                // any other dilation, stride or filter extent: the two passes through the any-geometry tiled kernels
+                // (grad-input of a stride-1 layer is the correlation with the rotated taps; above stride 1 it stays
+                // with the gather kernel); either falls back to the per-element kernels
+                rc = -1;
+                if (stride_h == 1 && stride_w == 1) {
+                    Geometry gi{batch, channel, g.out_h, g.out_w, kernel_h, kernel_w, 1, 1, 1, 1,
+                                dil_h * (kernel_h - 1) - pad_h, in_h - g.out_h + pad_h, dil_w * (kernel_w - 1) - pad_w,
+                                in_w - g.out_w + pad_w, in_h, in_w, 0};
+                    gi.dil_h = dil_h;
+                    gi.dil_w = dil_w;
+                    if (gi.pad_h0 >= 0 && gi.pad_w0 >= 0) rc = try_launch_fir_any<T>(gy, taps, gx, gi, stream);
+                }
+                if (rc < 0) rc = general_grad_input<T>(gy, taps, gx, g, stream);
+                if (rc != DWCONV_OK) return rc;
+                char first[sizeof(g_variant)];
+                std::snprintf(first, sizeof(first), "%s", g_variant);
+                const WgradGeometry wg{batch, channel, in_h, in_w, g.out_h, g.out_w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w};
+                rc = try_launch_wgrad_any<T>(in, gy, gw, ws, ws_bytes, wg, dil_h, dil_w, stream);
                 if (rc < 0) rc = general_grad_weight<T>(in, gy, gw, ws, ws_bytes, g, stream);
                 if (rc != DWCONV_OK) return rc;
                 char second[sizeof(g_variant)];

@@ -257,6 +257,12 @@ template <int K, typename IO>
 int stack_bigk_backward(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes, int batch,
                         int channel, int h, int w, hipStream_t stream);
 
+// Grad-weight for any filter extent, stride and dilation (dwconv_wgrad.hip); workspace bytes (0: not covered) and launch.
+size_t wgrad_any_workspace(const WgradGeometry &g, int dil_h, int dil_w);
+template <typename IO>
+int try_launch_wgrad_any(const IO *in, const IO *gy, IO *gw, void *ws, size_t ws_bytes, const WgradGeometry &g, int dil_h,
+                         int dil_w, hipStream_t stream);
+
 template <typename IO>
 int launch_wgrad_final(const float *partial, IO *gw, int channel, int taps, int chunks, hipStream_t stream);
 

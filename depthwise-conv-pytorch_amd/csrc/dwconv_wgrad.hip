@@ -342,6 +342,178 @@ __global__ __launch_bounds__(256) void wgrad_tile_final_kernel(const float *__re
     if (live && part == 0) gw[e] = Io<IO>::out(static_cast<float>(s));
 }
 
+// Grad-weight for any filter extent, stride and dilation (what make_plan's filter sizes do not cover: rectangular,
+// even-sized and strip filters, strides above 2, dilated taps): one channel per workgroup, the same chunks and
+// partial sums, the taps looped over at run time.  A workgroup keeps up to kAnyTaps sums per lane (the loop over
+// them is unrolled under a uniform bound, so the sums stay in registers); larger filters are cut into passes of
+// kAnyTaps taps (blockIdx.y), each of which stages the x bands again.  One LDS read per multiply-add.
+constexpr int kAnyTaps = 64;
+
+struct AnyTaps {
+    int kh, kw, sh, sw, dh, dw;
+};
+
+template <typename IO, int BH, int SW>
+__global__ __launch_bounds__(kThreads) void wgrad_any_kernel(const WgradPlan p, const AnyTaps a)
+{
+    extern __shared__ float4 lds_raw[];
+    float *lds = reinterpret_cast<float *>(lds_raw);
+    const IO *const x = static_cast<const IO *>(p.x);
+    const IO *const gy = static_cast<const IO *>(p.gy);
+    const int KK = a.kh * a.kw;
+    const int sw = SW ? SW : a.sw;
+    const int t_first = blockIdx.y * kAnyTaps;
+    const int nt = min(kAnyTaps, KK - t_first);
+
+    const int c = blockIdx.x / p.chunks;
+    const int chunk = blockIdx.x - c * p.chunks;
+
+    float acc[kAnyTaps];
+#pragma unroll
+    for (int t = 0; t < kAnyTaps; ++t) acc[t] = 0.f;
+
+    const bool has_item = static_cast<int>(threadIdx.x) < p.items_per_plane;
+    const int item = has_item ? threadIdx.x : 0;
+    const int rb = fast_div(item, p.ncb_magic);
+    const int cb = item - rb * p.ncb;
+    const int ox = 4 * cb;
+    const int row_step = a.sh * p.st.pitch;
+    const float *base = lds + __mul24(rb * BH, row_step) + kSlack + 4 * cb * sw;
+    const int ty_first = t_first / a.kw, tx_first = t_first - ty_first * a.kw;
+
+    for (int tile = chunk; tile < p.tiles_per_group; tile += p.chunks) {
+        const int n = tile / p.row_tiles, rt = tile - n * p.row_tiles;
+        const long plane0 = static_cast<long>(n) * p.channel + c;
+        const int oy0 = rt * p.rows_per_tile;
+
+        // this lane's block of gy (zero where it hangs over the edge of the plane, and for lanes without an item)
+        float g[BH][4];
+        const IO *gsrc = gy + plane0 * p.out_plane + ox;
+#pragma unroll
+        for (int b = 0; b < BH; ++b) {
+            const int oy = oy0 + rb * BH + b;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (p.vec_gy >= 2) {
+                const unsigned off = (ox + oy * p.out_w) * static_cast<unsigned>(sizeof(IO));
+                const bool ok = has_item && oy < p.out_h;
+                if (p.vec_gy == 3 && mixed_row_starts(gy + plane0 * p.out_plane, p.out_w))
+                    v = any_width_load4<IO>(any_width_view(gy + plane0 * p.out_plane, static_cast<long>(p.out_plane) * sizeof(IO)), ok ? off : kOob);
+                else
+                    v = view_load4<IO>(buffer_view(gy + plane0 * p.out_plane, static_cast<long>(p.out_plane) * sizeof(IO)), ok ? off : kOob);
+                if (p.vec_gy == 3) keep_first(v, p.out_w - ox);
+            } else if (has_item && oy < p.out_h) {
+                const IO *row = gsrc + static_cast<long>(oy) * p.out_w;
+                if (p.vec_gy) {
+                    v = load4<IO>(row);
+                } else {
+                    if (ox + 0 < p.out_w) v.x = Io<IO>::in(row[0]);
+                    if (ox + 1 < p.out_w) v.y = Io<IO>::in(row[1]);
+                    if (ox + 2 < p.out_w) v.z = Io<IO>::in(row[2]);
+                    if (ox + 3 < p.out_w) v.w = Io<IO>::in(row[3]);
+                }
+            }
+            g[b][0] = v.x;
+            g[b][1] = v.y;
+            g[b][2] = v.z;
+            g[b][3] = v.w;
+        }
+
+        if (tile != chunk) __syncthreads();  // the previous tile's window reads are done
+        stage_tile(p.st, x, lds, plane0, 1, oy0 * a.sh - p.pad_h);
+        __syncthreads();
+
+        int ty = ty_first, tx = tx_first;
+#pragma unroll
+        for (int t = 0; t < kAnyTaps; ++t) {
+            if (t < nt) {  // (uniform)
+                const float *r = base + __mul24(ty * a.dh, p.st.pitch) + tx * a.dw;
+                float sum = acc[t];
+#pragma unroll
+                for (int b = 0; b < BH; ++b)
+#pragma unroll
+                    for (int o = 0; o < 4; ++o) sum = fmaf(g[b][o], r[b * row_step + o * sw], sum);
+                acc[t] = sum;
+                if (++tx == a.kw) {
+                    tx = 0;
+                    ++ty;
+                }
+            }
+        }
+    }
+
+    __syncthreads();  // the tile image is dead; its LDS is reused for the reduction
+    // every lane worked on the same channel: wavefront sums, then the four wavefronts in order
+#pragma unroll
+    for (int t = 0; t < kAnyTaps; ++t) {
+        if (t < nt) {
+            const float sum = wave_sum_to_last_lane(acc[t]);
+            if ((threadIdx.x & 63) == 63) lds[(threadIdx.x >> 6) * kAnyTaps + t] = sum;
+        }
+    }
+    __syncthreads();
+    if (static_cast<int>(threadIdx.x) < nt) {
+        float sum = lds[threadIdx.x];
+#pragma unroll
+        for (int w = 1; w < kThreads / 64; ++w) sum += lds[w * kAnyTaps + threadIdx.x];
+        p.partial[(static_cast<long>(c) * p.chunks + chunk) * KK + t_first + threadIdx.x] = sum;
+    }
+}
+
+// The plan of wgrad_any_kernel for g (dilation dil_h x dil_w), or false.
+bool make_any_plan(WgradPlan &p, AnyTaps &a, const WgradGeometry &g, int dil_h, int dil_w)
+{
+    constexpr int BH = 4;
+    if (g.mult != 1 || g.kernel_h < 1 || g.kernel_w < 1 || g.down_h < 1 || g.down_w < 1 || dil_h < 1 || dil_w < 1) return false;
+    if (g.pad_h < 0 || g.pad_w < 0 || g.in_h < 1 || g.in_w < 1 || g.out_h < 1 || g.out_w < 1) return false;
+    const long KK = static_cast<long>(g.kernel_h) * g.kernel_w;
+    if (KK > 4096) return false;
+    if (static_cast<long>(g.in_h) * g.in_w >= (1l << 30) || static_cast<long>(g.out_h) * g.out_w >= (1l << 30)) return false;
+    const long span_h = static_cast<long>(g.kernel_h - 1) * dil_h, span_w = static_cast<long>(g.kernel_w - 1) * dil_w;
+    if (span_h > 4096 || span_w > 4096 || g.down_h > 64 || g.down_w > 64 || g.pad_h > 4096 || g.pad_w > 4096) return false;
+    a = AnyTaps{g.kernel_h, g.kernel_w, g.down_h, g.down_w, dil_h, dil_w};
+    p.batch = g.batch;
+    p.channel = g.channel;
+    p.out_h = g.out_h;
+    p.out_w = g.out_w;
+    p.out_plane = g.out_h * g.out_w;
+    p.pad_h = g.pad_h;
+    p.st.in_h = g.in_h;
+    p.st.in_w = g.in_w;
+    p.st.in_plane = g.in_h * g.in_w;
+    p.st.col_shift = g.pad_w;
+    p.ncb = ceil_div(g.out_w, 4);
+    if (p.ncb > kThreads) return false;
+    const long used_cols = static_cast<long>(4 * p.ncb - 1) * g.down_w + span_w + 1;
+    if (used_cols > (1 << 16)) return false;
+    layout_columns(p.st, static_cast<int>(used_cols));
+    auto rows_for = [&](int units) { return static_cast<long>(units * BH - 1) * g.down_h + span_h + 1; };
+    auto bytes = [&](int units) { return rows_for(units) * p.st.pitch * 4; };
+    const int row_units = ceil_div(g.out_h, BH);
+    int units = std::max(1, std::min(row_units, kThreads / p.ncb));
+    while (units > 1 && bytes(units) > dwconv::kLdsBudget) --units;
+    if (bytes(units) > dwconv::kLdsBudget) return false;
+    units = ceil_div(row_units, ceil_div(row_units, units));  // even out the bands
+    p.planes_per_tile = 1;
+    p.groups = g.channel;
+    p.rows_per_tile = units * BH;
+    p.row_tiles = ceil_div(row_units, units);
+    if (!layout_rows(p.st, static_cast<int>(rows_for(units)), 1)) return false;
+    p.items_per_plane = units * p.ncb;
+    p.ncb_magic = magic_u16(p.ncb);
+    p.ipp_magic = magic_u16(p.items_per_plane);
+    const long tiles = static_cast<long>(g.batch) * p.row_tiles;
+    if (tiles > 0x7fffffffL) return false;
+    p.tiles_per_group = static_cast<int>(tiles);
+    int chunks = ceil_div(env_int("DWCONV_WGRAD_WGS", 3072), g.channel);
+    if (chunks > p.tiles_per_group) chunks = p.tiles_per_group;
+    if (chunks < 1) chunks = 1;
+    p.chunks = chunks;
+    p.tiles_per_chunk = ceil_div(p.tiles_per_group, chunks);
+    p.strided = 1;
+    if (static_cast<long>(g.channel) * chunks > 0x7fffffffL) return false;
+    return true;
+}
+
 template <int K, int S, int BH>
 bool make_plan(WgradPlan &p, const WgradGeometry &g, bool fused)
 {
@@ -572,6 +744,49 @@ int try_launch_wgrad_tiled(const IO *in, const IO *gy, IO *gw, void *ws, size_t 
     return l.rc;
 }
 
+size_t wgrad_any_workspace(const WgradGeometry &g, int dil_h, int dil_w)
+{
+    if (!env_int("DWCONV_FIR_ANY", 1)) return 0;
+    WgradPlan p{};
+    AnyTaps a{};
+    if (!make_any_plan(p, a, g, dil_h, dil_w)) return 0;
+    return static_cast<size_t>(g.channel) * p.chunks * g.kernel_h * g.kernel_w * sizeof(float);
+}
+
+template <typename IO>
+int try_launch_wgrad_any(const IO *in, const IO *gy, IO *gw, void *ws, size_t ws_bytes, const WgradGeometry &g, int dil_h,
+                         int dil_w, hipStream_t stream)
+{
+    if (!env_int("DWCONV_FIR_ANY", 1)) return -1;
+    constexpr int BH = 4;
+    WgradPlan p{};
+    AnyTaps a{};
+    if (!make_any_plan(p, a, g, dil_h, dil_w)) return -1;
+    const int KK = g.kernel_h * g.kernel_w;
+    const size_t need = static_cast<size_t>(g.channel) * p.chunks * KK * sizeof(float);
+    if (ws == nullptr || ws_bytes < need)
+        return fail(DWCONV_ERR_WORKSPACE, "grad-weight needs a workspace of %zu bytes, got %zu", need, ws_bytes);
+    p.x = in;
+    p.gy = gy;
+    p.partial = static_cast<float *>(ws);
+    p.st.vec_in = row_vector_mode(g.in_w, in);
+    p.vec_gy = row_vector_mode(g.out_w, gy);
+    const int in_view = stage_vector_mode(p.st, 1, sizeof(IO)), gy_view = vector_mode(1, p.out_plane, sizeof(IO));
+    p.st.vec_in = p.st.vec_in == 1 ? in_view : (p.st.vec_in == 3 && in_view == 2 ? 3 : 0);
+    p.vec_gy = p.vec_gy == 1 ? gy_view : (p.vec_gy == 3 && gy_view == 2 ? 3 : 0);
+    const size_t image = static_cast<size_t>(p.st.plane_pitch) * 4, red = static_cast<size_t>(kThreads / 64) * kAnyTaps * 4;
+    const size_t shmem = image > red ? image : red;
+    const dim3 grid(static_cast<unsigned>(g.channel * p.chunks), static_cast<unsigned>(ceil_div(KK, kAnyTaps))), block(kThreads);
+    if (a.sw == 1) hipLaunchKernelGGL((wgrad_any_kernel<IO, BH, 1>), grid, block, shmem, stream, p, a);
+    else if (a.sw == 2) hipLaunchKernelGGL((wgrad_any_kernel<IO, BH, 2>), grid, block, shmem, stream, p, a);
+    else hipLaunchKernelGGL((wgrad_any_kernel<IO, BH, 0>), grid, block, shmem, stream, p, a);
+    const int rc = check_launch("wgrad_any_kernel");
+    if (rc != DWCONV_OK) return rc;
+    note_variant("wgrad_any%s<k%dx%d,s%dx%d,d%dx%d> rows%d chunks%d passes%d vin%d vgy%d", sizeof(IO) == 2 ? "16" : "", a.kh, a.kw, a.sh,
+                 a.sw, a.dh, a.dw, p.rows_per_tile, p.chunks, ceil_div(KK, kAnyTaps), p.st.vec_in, p.vec_gy);
+    return launch_wgrad_final(static_cast<const float *>(ws), gw, g.channel, KK, p.chunks, stream);
+}
+
 template <typename IO>
 int try_launch_bwd_tiled(const IO *in, const IO *gy, const IO *taps, IO *gx, IO *gw, void *ws, size_t ws_bytes,
                          const WgradGeometry &g, hipStream_t stream)
@@ -589,6 +804,8 @@ int try_launch_bwd_tiled(const IO *in, const IO *gy, const IO *taps, IO *gx, IO 
 
 #define DWCONV_INSTANTIATE(IO)                                                                                        \
     template int launch_wgrad_final<IO>(const float *, IO *, int, int, int, hipStream_t);                             \
+    template int try_launch_wgrad_any<IO>(const IO *, const IO *, IO *, void *, size_t, const WgradGeometry &, int,   \
+                                          int, hipStream_t);                                                          \
     template int try_launch_wgrad_tiled<IO>(const IO *, const IO *, IO *, void *, size_t, const WgradGeometry &,      \
                                             hipStream_t);                                                             \
     template int try_launch_bwd_tiled<IO>(const IO *, const IO *, const IO *, IO *, IO *, void *, size_t,             \

@@ -91,8 +91,8 @@ int dwconv2d_f64(const double *input, const double *kernel, double *out,
  * dwconv2d_small_op, torch_dwconv/dwconv_kernel.cu:734-771): stride-1
  * convolution whose output has the input's extent; `pad_h`,`pad_w` zeros lead
  * each axis and kernel-1-pad trail it.  up_* and down_* must be 1 and the plane
- * at most 32x32 (DWCONV_ERR_UNSUPPORTED otherwise); unlike the reference the
- * kernel may be any size up to 15x15. */
+ * at most 32x32 (DWCONV_ERR_UNSUPPORTED otherwise); the kernel may be any
+ * size. */
 int dwconv2d_small_f32(const float *input, const float *kernel, float *out,
                        int batch, int channel, int in_h, int in_w,
                        int kernel_h, int kernel_w, int up_h, int up_w,

@@ -783,6 +783,62 @@ def test_large_filters_full_size(dw, gpu, shape):
     check_full_size(dw, gpu, shape, seed=83, expect=("tile_stack<k%d" % k, "bwd_stack<k%d" % k))
 
 
+# (N, C, H, W, KH, KW, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w): what only the any-geometry tiled kernels serve
+ANY_GEOMETRY = [
+    (2, 3, 40, 48, 1, 7, 1, 1, 0, 3, 1, 1), (2, 3, 40, 48, 7, 1, 1, 1, 3, 0, 1, 1), (1, 2, 33, 57, 1, 21, 1, 1, 0, 10, 1, 1),
+    (1, 2, 57, 33, 21, 1, 1, 1, 10, 0, 1, 1), (2, 2, 30, 30, 4, 4, 1, 1, 1, 2, 1, 1), (2, 3, 21, 26, 2, 2, 2, 2, 0, 0, 1, 1),
+    (2, 2, 50, 61, 3, 5, 1, 2, 1, 2, 1, 1), (1, 3, 64, 64, 3, 3, 3, 3, 1, 1, 1, 1), (1, 2, 45, 47, 5, 5, 4, 4, 2, 2, 1, 1),
+    (1, 2, 40, 44, 10, 10, 1, 1, 4, 5, 1, 1), (1, 1, 36, 40, 15, 15, 1, 1, 7, 7, 1, 1),
+    (2, 2, 33, 33, 3, 3, 1, 1, 6, 6, 6, 6), (1, 2, 65, 65, 3, 3, 1, 1, 18, 18, 18, 18), (2, 2, 40, 52, 3, 3, 1, 1, 3, 3, 3, 3),
+    (1, 3, 50, 38, 5, 3, 2, 1, 4, 2, 2, 3), (2, 2, 12, 70, 1, 1, 1, 1, 0, 0, 1, 1),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["f32", "f16", "bf16"])
+@pytest.mark.parametrize("case", ANY_GEOMETRY, ids=lambda c: "N%d_C%d_%dx%d_k%dx%d_s%dx%d_p%dx%d_d%dx%d" % c)
+def test_any_geometry_tiled_kernels(dw, gpu, case, dtype):
+    """Rectangular, even-sized and strip filters, strides above 2 and dilations above 2: forward, grad-input (the
+    correlation with the rotated taps where the stride is 1) and grad-weight through the tiled kernels that loop over
+    their taps at run time, against fp64 autograd on the rounded inputs; bit-identical grad-weight."""
+    from torch_dwconv import _C
+    from torch_dwconv.dwconv import depthwise_conv2d_general
+
+    n, c, h, w, kh, kw, sh, sw, ph, pw, dh, dw_ = case
+    step = {torch.float32: 0.0, torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[dtype]
+    g = torch.Generator("cpu").manual_seed(91)
+    x = torch.randn(n, c, h, w, generator=g).to(dtype)
+    wt = (torch.randn(c, 1, kh, kw, generator=g) / (kh * kw) ** 0.5).to(dtype)
+    xr, wr = x.double().requires_grad_(True), wt.double().requires_grad_(True)
+    y_ref = torch.nn.functional.conv2d(xr, wr, stride=(sh, sw), padding=(ph, pw), dilation=(dh, dw_), groups=c)
+    gy = torch.randn(y_ref.shape, generator=g).to(dtype)
+    gx_ref, gw_ref = torch.autograd.grad(y_ref, (xr, wr), gy.double())
+    xg, wg = x.to(gpu).requires_grad_(True), wt.to(gpu).requires_grad_(True)
+    if (dh, dw_) == (1, 1):
+        y = dw.depthwise_conv2d(xg, wg, stride=(sh, sw), padding=(ph, pw))
+    else:
+        y = depthwise_conv2d_general(xg, wg, stride=(sh, sw), padding=(ph, pw), dilation=(dh, dw_))
+    v_fwd = _C.last_variant()
+    _announce(case, str(dtype), v_fwd)
+    sfx = "" if dtype == torch.float32 else "16"
+    assert v_fwd.startswith("tile_any%s<k%dx%d,s%dx%d,d%dx%d,fwd>" % (sfx, kh, kw, sh, sw, dh, dw_)), v_fwd
+    gx, gw = torch.autograd.grad(y, (xg, wg), gy.to(gpu))
+    # (the variant note is per thread and autograd runs the backward on its own: the same calls again from here)
+    if (dh, dw_) == (1, 1):
+        _, gw2 = _C.dwconv2d_backward(xg.detach(), gy.to(gpu), wg.detach(), sh, sw, ph, pw)
+    else:
+        _, gw2 = _C.dwconv2d_general_backward(xg.detach(), gy.to(gpu), wg.detach(), sh, sw, ph, pw, dh, dw_)
+    v_bwd = _C.last_variant()
+    assert "wgrad_any%s<k%dx%d" % (sfx, kh, kw) in v_bwd, v_bwd
+    assert ("tile_any%s<" % sfx in v_bwd and ",rot>" in v_bwd) == ((sh, sw) == (1, 1)), v_bwd
+    assert ("passes%d " % ((kh * kw + 63) // 64)) in v_bwd, v_bwd
+    assert torch.equal(gw, gw2)
+    tol = 1e-5 + step
+    np.testing.assert_allclose(_np(y.detach().double()), y_ref.detach().numpy(), rtol=tol, atol=tol)
+    np.testing.assert_allclose(_np(gx.double()), gx_ref.numpy(), rtol=tol, atol=tol)
+    gtol = 1e-4 + step
+    np.testing.assert_allclose(_np(gw.double()), gw_ref.numpy(), rtol=gtol, atol=gtol * float(gw_ref.abs().max()))
+
+
 def test_tuning_overrides_need_the_master_switch(dw, gpu, monkeypatch):
     """DWCONV_* overrides of the planners are ignored unless DWCONV_TUNING=1 is set too, and ill-formed values always."""
     from torch_dwconv import _C
