@@ -561,7 +561,10 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
 // few taps bound by HBM.  Replaces the generic instantiation of torch_dwconv/dwconv_kernel.cu:69-181 (kernel sizes of
 // -1) for these shapes.
 // SW: the column stride when it is 1 or 2 (the four inputs of a row then sit at immediate offsets), 0 = any.
-template <typename IO, int BH, int SW>
+// KHM x KWM (0: none): at stride 1 and dilation 1, filters of at most that extent walk a register window as the
+// kernels above do (a window row of 3 + kw inputs is read once and used by every tap and output row that meets it),
+// with the loops unrolled to the maxima under uniform bounds: 3 + kw LDS reads for 4 * kw multiply-adds.
+template <typename IO, int BH, int SW, int KHM = 0, int KWM = 0>
 __global__ __launch_bounds__(kThreads) void fir_any_kernel(const TilePlan p)
 {
     extern __shared__ float4 lds_raw[];
@@ -597,15 +600,48 @@ __global__ __launch_bounds__(kThreads) void fir_any_kernel(const TilePlan p)
             for (int o = 0; o < 4; ++o) acc[b][o] = 0.f;
         const float *base = lds + __mul24(pl, p.st.plane_pitch) + __mul24(rb * BH, row_step) + kSlack + 4 * cb * sw;
         const float *tp = lds + p.tap_base + pl * KK;
-        for (int ty = 0; ty < p.kh; ++ty) {
-            const float *trow = base + __mul24(ty * p.dh, p.st.pitch);
-            for (int tx = 0; tx < p.kw; ++tx) {
-                const float t = tp[ty * p.kw + tx];
-                const float *r = trow + tx * p.dw;
+        if constexpr (KHM > 0) {
+            static_assert(SW == 1, "the register window is the stride-1 case");
+            float tapr[KHM][KWM];
 #pragma unroll
-                for (int b = 0; b < BH; ++b)
+            for (int ty = 0; ty < KHM; ++ty)
 #pragma unroll
-                    for (int o = 0; o < 4; ++o) acc[b][o] = fmaf(r[b * row_step + o * sw], t, acc[b][o]);
+                for (int tx = 0; tx < KWM; ++tx) tapr[ty][tx] = (ty < p.kh && tx < p.kw) ? tp[ty * p.kw + tx] : 0.f;
+#pragma unroll
+            for (int wr = 0; wr < BH - 1 + KHM; ++wr) {
+                if (wr < BH - 1 + p.kh) {  // (uniform)
+                    const float *r = base + wr * p.st.pitch;
+                    float win[3 + KWM];
+#pragma unroll
+                    for (int i = 0; i < 3 + KWM; ++i) win[i] = i < 3 + p.kw ? r[i] : 0.f;
+#pragma unroll
+                    for (int b = 0; b < BH; ++b) {
+                        const int ty = wr - b;
+                        if (ty < 0 || ty >= KHM) continue;
+                        if (ty < p.kh) {
+#pragma unroll
+                            for (int tx = 0; tx < KWM; ++tx) {
+                                if (tx < p.kw) {
+#pragma unroll
+                                    for (int o = 0; o < 4; ++o) acc[b][o] = fmaf(win[o + tx], tapr[ty][tx], acc[b][o]);
+                                }
+                            }
+                        }
+                    }
+                    pin_registers(acc);
+                }
+            }
+        } else {
+            for (int ty = 0; ty < p.kh; ++ty) {
+                const float *trow = base + __mul24(ty * p.dh, p.st.pitch);
+                for (int tx = 0; tx < p.kw; ++tx) {
+                    const float t = tp[ty * p.kw + tx];
+                    const float *r = trow + tx * p.dw;
+#pragma unroll
+                    for (int b = 0; b < BH; ++b)
+#pragma unroll
+                        for (int o = 0; o < 4; ++o) acc[b][o] = fmaf(r[b * row_step + o * sw], t, acc[b][o]);
+                }
             }
         }
         if (!p.flip && p.epi.enabled()) epilogue_apply_block<1>(acc, p.epi, static_cast<int>((plane0 + pl) % p.channel));
@@ -847,11 +883,32 @@ int try_launch_fir_any(const IO *in, const IO *taps, IO *out, const Geometry &g,
     settle_vector_modes<IO>(p);
     const dim3 grid(p.n_tiles), block(kThreads);
     const size_t shmem = lds_bytes(p, p.kh * p.kw);
-    if (p.sw == 1) hipLaunchKernelGGL((fir_any_kernel<IO, BH, 1>), grid, block, shmem, stream, p);
+    // stride 1, dilation 1, small extents: the register-window instances (the smallest maxima that hold the filter)
+    const bool plain = p.sh == 1 && p.sw == 1 && p.dh == 1 && p.dw == 1 && env_int("DWCONV_ANY_WINDOW", 1);
+    const char *window = "";
+    if (plain && p.kh == 1 && p.kw <= 8) {
+        hipLaunchKernelGGL((fir_any_kernel<IO, BH, 1, 1, 8>), grid, block, shmem, stream, p);
+        window = " win1x8";
+    } else if (plain && p.kh <= 8 && p.kw == 1) {
+        hipLaunchKernelGGL((fir_any_kernel<IO, BH, 1, 8, 1>), grid, block, shmem, stream, p);
+        window = " win8x1";
+    } else if (plain && p.kh <= 4 && p.kw <= 4) {
+        hipLaunchKernelGGL((fir_any_kernel<IO, BH, 1, 4, 4>), grid, block, shmem, stream, p);
+        window = " win4x4";
+    } else if (plain && p.kh == 1 && p.kw <= 24) {
+        hipLaunchKernelGGL((fir_any_kernel<IO, BH, 1, 1, 24>), grid, block, shmem, stream, p);
+        window = " win1x24";
+    } else if (plain && p.kh <= 24 && p.kw == 1) {
+        hipLaunchKernelGGL((fir_any_kernel<IO, BH, 1, 24, 1>), grid, block, shmem, stream, p);
+        window = " win24x1";
+    } else if (plain && p.kh <= 8 && p.kw <= 8) {
+        hipLaunchKernelGGL((fir_any_kernel<IO, BH, 1, 8, 8>), grid, block, shmem, stream, p);
+        window = " win8x8";
+    } else if (p.sw == 1) hipLaunchKernelGGL((fir_any_kernel<IO, BH, 1>), grid, block, shmem, stream, p);
     else if (p.sw == 2) hipLaunchKernelGGL((fir_any_kernel<IO, BH, 2>), grid, block, shmem, stream, p);
     else hipLaunchKernelGGL((fir_any_kernel<IO, BH, 0>), grid, block, shmem, stream, p);
-    note_variant("tile_any%s<k%dx%d,s%dx%d,d%dx%d,%s> P%d rows%d vin%d vout%d", sizeof(IO) == 2 ? "16" : "", p.kh, p.kw, p.sh, p.sw,
-                 p.dh, p.dw, p.flip ? "rot" : "fwd", p.planes_per_tile, p.rows_per_tile, p.st.vec_in, p.vec_out);
+    note_variant("tile_any%s<k%dx%d,s%dx%d,d%dx%d,%s> P%d rows%d vin%d vout%d%s", sizeof(IO) == 2 ? "16" : "", p.kh, p.kw, p.sh, p.sw,
+                 p.dh, p.dw, p.flip ? "rot" : "fwd", p.planes_per_tile, p.rows_per_tile, p.st.vec_in, p.vec_out, window);
     return check_launch("fir_any_kernel");
 }
 

@@ -353,7 +353,10 @@ struct AnyTaps {
     int kh, kw, sh, sw, dh, dw;
 };
 
-template <typename IO, int BH, int SW>
+// KHM x KWM (0: none): at stride 1 and dilation 1, filters of at most that extent (and at most kAnyTaps taps) walk a
+// register window of x rows instead: a row of 3 + kw inputs is read once for every tap and gy row that meets it, the
+// loops unrolled to the maxima under uniform bounds; sum (ty, tx) lives in acc[ty * KWM + tx].
+template <typename IO, int BH, int SW, int KHM = 0, int KWM = 0>
 __global__ __launch_bounds__(kThreads) void wgrad_any_kernel(const WgradPlan p, const AnyTaps a)
 {
     extern __shared__ float4 lds_raw[];
@@ -368,9 +371,10 @@ __global__ __launch_bounds__(kThreads) void wgrad_any_kernel(const WgradPlan p, 
     const int c = blockIdx.x / p.chunks;
     const int chunk = blockIdx.x - c * p.chunks;
 
-    float acc[kAnyTaps];
+    constexpr int kSums = KHM > 0 ? KHM * KWM : kAnyTaps;
+    float acc[kSums];
 #pragma unroll
-    for (int t = 0; t < kAnyTaps; ++t) acc[t] = 0.f;
+    for (int t = 0; t < kSums; ++t) acc[t] = 0.f;
 
     const bool has_item = static_cast<int>(threadIdx.x) < p.items_per_plane;
     const int item = has_item ? threadIdx.x : 0;
@@ -422,6 +426,36 @@ __global__ __launch_bounds__(kThreads) void wgrad_any_kernel(const WgradPlan p, 
         stage_tile(p.st, x, lds, plane0, 1, oy0 * a.sh - p.pad_h);
         __syncthreads();
 
+        if constexpr (KHM > 0) {
+            static_assert(SW == 1 && KHM * KWM <= kAnyTaps, "the register window is the stride-1 case, one pass");
+#pragma unroll
+            for (int wr = 0; wr < BH - 1 + KHM; ++wr) {
+                if (wr < BH - 1 + a.kh) {  // (uniform)
+                    const float *r = base + wr * p.st.pitch;
+                    float win[3 + KWM];
+#pragma unroll
+                    for (int i = 0; i < 3 + KWM; ++i) win[i] = i < 3 + a.kw ? r[i] : 0.f;
+#pragma unroll
+                    for (int b = 0; b < BH; ++b) {
+                        const int wy = wr - b;
+                        if (wy < 0 || wy >= KHM) continue;
+                        if (wy < a.kh) {
+#pragma unroll
+                            for (int wx = 0; wx < KWM; ++wx) {
+                                if (wx < a.kw) {
+                                    float sum = acc[wy * KWM + wx];
+#pragma unroll
+                                    for (int o = 0; o < 4; ++o) sum = fmaf(g[b][o], win[o + wx], sum);
+                                    acc[wy * KWM + wx] = sum;
+                                }
+                            }
+                        }
+                    }
+                    pin_registers(acc);
+                }
+            }
+            continue;
+        }
         int ty = ty_first, tx = tx_first;
 #pragma unroll
         for (int t = 0; t < kAnyTaps; ++t) {
@@ -443,11 +477,23 @@ __global__ __launch_bounds__(kThreads) void wgrad_any_kernel(const WgradPlan p, 
 
     __syncthreads();  // the tile image is dead; its LDS is reused for the reduction
     // every lane worked on the same channel: wavefront sums, then the four wavefronts in order
+    if constexpr (KHM > 0) {
 #pragma unroll
-    for (int t = 0; t < kAnyTaps; ++t) {
-        if (t < nt) {
-            const float sum = wave_sum_to_last_lane(acc[t]);
-            if ((threadIdx.x & 63) == 63) lds[(threadIdx.x >> 6) * kAnyTaps + t] = sum;
+        for (int wy = 0; wy < KHM; ++wy)
+#pragma unroll
+            for (int wx = 0; wx < KWM; ++wx) {
+                if (wy < a.kh && wx < a.kw) {
+                    const float sum = wave_sum_to_last_lane(acc[wy * KWM + wx]);
+                    if ((threadIdx.x & 63) == 63) lds[(threadIdx.x >> 6) * kAnyTaps + wy * a.kw + wx] = sum;
+                }
+            }
+    } else {
+#pragma unroll
+        for (int t = 0; t < kAnyTaps; ++t) {
+            if (t < nt) {
+                const float sum = wave_sum_to_last_lane(acc[t]);
+                if ((threadIdx.x & 63) == 63) lds[(threadIdx.x >> 6) * kAnyTaps + t] = sum;
+            }
         }
     }
     __syncthreads();
@@ -777,13 +823,33 @@ int try_launch_wgrad_any(const IO *in, const IO *gy, IO *gw, void *ws, size_t ws
     const size_t image = static_cast<size_t>(p.st.plane_pitch) * 4, red = static_cast<size_t>(kThreads / 64) * kAnyTaps * 4;
     const size_t shmem = image > red ? image : red;
     const dim3 grid(static_cast<unsigned>(g.channel * p.chunks), static_cast<unsigned>(ceil_div(KK, kAnyTaps))), block(kThreads);
-    if (a.sw == 1) hipLaunchKernelGGL((wgrad_any_kernel<IO, BH, 1>), grid, block, shmem, stream, p, a);
+    const bool plain = a.sh == 1 && a.sw == 1 && a.dh == 1 && a.dw == 1 && env_int("DWCONV_ANY_WINDOW", 1);
+    const char *window = "";
+    if (plain && a.kh == 1 && a.kw <= 8) {
+        hipLaunchKernelGGL((wgrad_any_kernel<IO, BH, 1, 1, 8>), grid, block, shmem, stream, p, a);
+        window = " win1x8";
+    } else if (plain && a.kh <= 8 && a.kw == 1) {
+        hipLaunchKernelGGL((wgrad_any_kernel<IO, BH, 1, 8, 1>), grid, block, shmem, stream, p, a);
+        window = " win8x1";
+    } else if (plain && a.kh <= 4 && a.kw <= 4) {
+        hipLaunchKernelGGL((wgrad_any_kernel<IO, BH, 1, 4, 4>), grid, block, shmem, stream, p, a);
+        window = " win4x4";
+    } else if (plain && a.kh == 1 && a.kw <= 24) {
+        hipLaunchKernelGGL((wgrad_any_kernel<IO, BH, 1, 1, 24>), grid, block, shmem, stream, p, a);
+        window = " win1x24";
+    } else if (plain && a.kh <= 24 && a.kw == 1) {
+        hipLaunchKernelGGL((wgrad_any_kernel<IO, BH, 1, 24, 1>), grid, block, shmem, stream, p, a);
+        window = " win24x1";
+    } else if (plain && a.kh <= 8 && a.kw <= 8) {
+        hipLaunchKernelGGL((wgrad_any_kernel<IO, BH, 1, 8, 8>), grid, block, shmem, stream, p, a);
+        window = " win8x8";
+    } else if (a.sw == 1) hipLaunchKernelGGL((wgrad_any_kernel<IO, BH, 1>), grid, block, shmem, stream, p, a);
     else if (a.sw == 2) hipLaunchKernelGGL((wgrad_any_kernel<IO, BH, 2>), grid, block, shmem, stream, p, a);
     else hipLaunchKernelGGL((wgrad_any_kernel<IO, BH, 0>), grid, block, shmem, stream, p, a);
     const int rc = check_launch("wgrad_any_kernel");
     if (rc != DWCONV_OK) return rc;
-    note_variant("wgrad_any%s<k%dx%d,s%dx%d,d%dx%d> rows%d chunks%d passes%d vin%d vgy%d", sizeof(IO) == 2 ? "16" : "", a.kh, a.kw, a.sh,
-                 a.sw, a.dh, a.dw, p.rows_per_tile, p.chunks, ceil_div(KK, kAnyTaps), p.st.vec_in, p.vec_gy);
+    note_variant("wgrad_any%s<k%dx%d,s%dx%d,d%dx%d> rows%d chunks%d passes%d vin%d vgy%d%s", sizeof(IO) == 2 ? "16" : "", a.kh, a.kw, a.sh,
+                 a.sw, a.dh, a.dw, p.rows_per_tile, p.chunks, ceil_div(KK, kAnyTaps), p.st.vec_in, p.vec_gy, window);
     return launch_wgrad_final(static_cast<const float *>(ws), gw, g.channel, KK, p.chunks, stream);
 }
 
