@@ -67,6 +67,11 @@ WORKLOADS = {
                                  (64, 384, 14, 14, 7, 1, 3), (64, 768, 7, 7, 7, 1, 3)],
     "stress": lambda batch: [(64, 256, 128, 96, 5, 2, 2)],
     # ConvNeXt-T's first three stages with the larger filters of its successors (9x9, 11x11, 13x13)
+    # what only the kernels that loop over their taps serve: an even-sized filter, a 15x15 one, stride 3, and the
+    # atrous 3x3 layers of a segmentation head at rates 6, 12 and 18 (general entry points)
+    "any_geometry": lambda batch: [(16, 64, 128, 128, 4, 1, 2), (16, 64, 128, 128, 15, 1, 7), (16, 64, 128, 128, 3, 3, 1),
+                                   (16, 256, 65, 65, 3, 1, 6, 6, 1), (16, 256, 65, 65, 3, 1, 12, 12, 1),
+                                   (16, 256, 65, 65, 3, 1, 18, 18, 1)],
     "large_filters": lambda batch: [(64, 96, 56, 56, 9, 1, 4), (64, 192, 28, 28, 11, 1, 5), (64, 384, 14, 14, 13, 1, 6)],
 }
 

@@ -15,7 +15,7 @@ namespace dwconv {
 
 namespace {
 thread_local char g_error[512] = "";
-thread_local char g_variant[128] = "";
+thread_local char g_variant[256] = "";
 
 // DWCONV_FORCE_GENERIC=1 routes every call to the generic kernels (used by the
 // tests to cover that path at fp32 as well).
@@ -280,7 +280,7 @@ int backward_any(const T *in, const T *gy, const T *taps, T *gx, T *gw, void *ws
     if (rc == DWCONV_OK) {
         char second[sizeof(g_variant)];
         std::snprintf(second, sizeof(second), "%s", g_variant);
-        note_variant("%.60s + %.60s", first, second);
+        note_variant("%.120s + %.120s", first, second);
     }
     return rc;
 }
@@ -353,7 +353,7 @@ int nhwc_backward_any(const T *in, const T *gy, const T *taps, T *gx, T *gw, voi
         if (gx != nullptr) {
             char second[sizeof(g_variant)];
             std::snprintf(second, sizeof(second), "%s", g_variant);
-            note_variant("%.60s + %.60s", first, second);
+            note_variant("%.120s + %.120s", first, second);
         }
     }
     return DWCONV_OK;
@@ -547,7 +547,7 @@ int general_backward_any(const T *in, const T *gy, const T *taps, T *gx, T *gw, 
                 if (rc != DWCONV_OK) return rc;
                 char second[sizeof(g_variant)];
                 std::snprintf(second, sizeof(second), "%s", g_variant);
-                note_variant("%.60s + %.60s", first, second);
+                note_variant("%.120s + %.120s", first, second);
                 return DWCONV_OK;
             }
             if (multiplier == 1 && in_h > 0 && in_w > 0) {
@@ -573,7 +573,7 @@ int general_backward_any(const T *in, const T *gy, const T *taps, T *gx, T *gw, 
                 if (rc != DWCONV_OK) return rc;
                 char second[sizeof(g_variant)];
                 std::snprintf(second, sizeof(second), "%s", g_variant);
-                note_variant("%.60s + %.60s", first, second);
+                note_variant("%.120s + %.120s", first, second);
                 return DWCONV_OK;
             }
         }

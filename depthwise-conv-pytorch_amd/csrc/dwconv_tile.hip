@@ -22,6 +22,7 @@
 //                    stride-2 layers, computed as four interleaved stride-1
 //                    correlations (one per output parity) without ever
 //                    forming the zero-stuffed intermediate.
+#include <type_traits>
 #include "dwconv_tile_common.hpp"
 
 namespace dwconv {
@@ -564,6 +565,8 @@ __global__ __launch_bounds__(kThreads) void fir_up2_kernel(const TilePlan p)
 // KHM x KWM (0: none): at stride 1 and dilation 1, filters of at most that extent walk a register window as the
 // kernels above do (a window row of 3 + kw inputs is read once and used by every tap and output row that meets it),
 // with the loops unrolled to the maxima under uniform bounds: 3 + kw LDS reads for 4 * kw multiply-adds.
+// KHM < 0: column stride 1 and undilated columns, any extent, row stride and row dilation: filter rows are walked
+// four taps at a time (see there), which is what keeps 15 x 15 and larger filters off the LDS read rate.
 template <typename IO, int BH, int SW, int KHM = 0, int KWM = 0>
 __global__ __launch_bounds__(kThreads) void fir_any_kernel(const TilePlan p)
 {
@@ -611,9 +614,15 @@ __global__ __launch_bounds__(kThreads) void fir_any_kernel(const TilePlan p)
             for (int wr = 0; wr < BH - 1 + KHM; ++wr) {
                 if (wr < BH - 1 + p.kh) {  // (uniform)
                     const float *r = base + wr * p.st.pitch;
-                    float win[3 + KWM];
+                    // (16-byte LDS reads: consecutive lanes then read consecutive banks; the last may reach into the
+                    // slack of the row)
+                    float win[4 * ((3 + KWM + 3) / 4)];
 #pragma unroll
-                    for (int i = 0; i < 3 + KWM; ++i) win[i] = i < 3 + p.kw ? r[i] : 0.f;
+                    for (int v = 0; v < (3 + KWM + 3) / 4; ++v) {
+                        float4 q = make_float4(0.f, 0.f, 0.f, 0.f);
+                        if (4 * v < 3 + p.kw) q = *reinterpret_cast<const float4 *>(r + 4 * v);
+                        win[4 * v] = q.x, win[4 * v + 1] = q.y, win[4 * v + 2] = q.z, win[4 * v + 3] = q.w;
+                    }
 #pragma unroll
                     for (int b = 0; b < BH; ++b) {
                         const int ty = wr - b;
@@ -631,16 +640,79 @@ __global__ __launch_bounds__(kThreads) void fir_any_kernel(const TilePlan p)
                     pin_registers(acc);
                 }
             }
+        } else if constexpr (KHM < 0) {
+            static_assert(SW == 1, "rows are walked four inputs at a time at column stride 1");
+            // undilated columns: a filter row takes four taps at a time from eight inputs per output row (the four
+            // read for the taps before, and the next four), one 16-byte LDS read per sixteen multiply-adds
+            for (int ty = 0; ty < p.kh; ++ty) {
+                const float *trow = base + __mul24(ty * p.dh, p.st.pitch);
+                const float *tr = tp + ty * p.kw;
+                float w[BH][8];
+#pragma unroll
+                for (int b = 0; b < BH; ++b) {
+                    const float4 v = *reinterpret_cast<const float4 *>(trow + b * row_step);
+                    w[b][4] = v.x, w[b][5] = v.y, w[b][6] = v.z, w[b][7] = v.w;
+                }
+                for (int tx0 = 0; tx0 < p.kw; tx0 += 4) {
+#pragma unroll
+                    for (int b = 0; b < BH; ++b) {
+                        const float4 v = *reinterpret_cast<const float4 *>(trow + b * row_step + tx0 + 4);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) w[b][i] = w[b][4 + i];
+                        w[b][4] = v.x, w[b][5] = v.y, w[b][6] = v.z, w[b][7] = v.w;
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if (tx0 + j < p.kw) {  // (uniform)
+                            const float t = tr[tx0 + j];
+#pragma unroll
+                            for (int b = 0; b < BH; ++b)
+#pragma unroll
+                                for (int o = 0; o < 4; ++o) acc[b][o] = fmaf(w[b][j + o], t, acc[b][o]);
+                        }
+                    }
+                }
+            }
         } else {
             for (int ty = 0; ty < p.kh; ++ty) {
                 const float *trow = base + __mul24(ty * p.dh, p.st.pitch);
                 for (int tx = 0; tx < p.kw; ++tx) {
                     const float t = tp[ty * p.kw + tx];
-                    const float *r = trow + tx * p.dw;
+                    if constexpr (SW == 1 || SW == 2) {
+                        // The four inputs of a row sit within twelve floats.  Lanes are four or eight floats apart, so
+                        // reading them one float at a time would meet the same LDS banks four or eight times over:
+                        // 16-byte reads from the 16-byte boundary before the tap's offset on (the last may reach into
+                        // the slack of the row) and a uniform choice among what they hold.
+                        const int off = tx * p.dw;
+                        const float *r = trow + (off & ~3);
+                        auto rows = [&](auto shift) {
+                            constexpr int S = decltype(shift)::value;
 #pragma unroll
-                    for (int b = 0; b < BH; ++b)
+                            for (int b = 0; b < BH; ++b) {
+                                constexpr int NR = (S + 3 * SW + 4) / 4;  // 16-byte reads that hold inputs S, S + SW .. S + 3 SW
+                                float w8[4 * NR];
 #pragma unroll
-                        for (int o = 0; o < 4; ++o) acc[b][o] = fmaf(r[b * row_step + o * sw], t, acc[b][o]);
+                                for (int v = 0; v < NR; ++v) {
+                                    const float4 q = *reinterpret_cast<const float4 *>(r + b * row_step + 4 * v);
+                                    w8[4 * v] = q.x, w8[4 * v + 1] = q.y, w8[4 * v + 2] = q.z, w8[4 * v + 3] = q.w;
+                                }
+#pragma unroll
+                                for (int o = 0; o < 4; ++o) acc[b][o] = fmaf(w8[S + o * SW], t, acc[b][o]);
+                            }
+                        };
+                        switch (off & 3) {
+                        case 0: rows(std::integral_constant<int, 0>{}); break;
+                        case 1: rows(std::integral_constant<int, 1>{}); break;
+                        case 2: rows(std::integral_constant<int, 2>{}); break;
+                        default: rows(std::integral_constant<int, 3>{}); break;
+                        }
+                    } else {
+                        const float *r = trow + tx * p.dw;
+#pragma unroll
+                        for (int b = 0; b < BH; ++b)
+#pragma unroll
+                            for (int o = 0; o < 4; ++o) acc[b][o] = fmaf(r[b * row_step + o * sw], t, acc[b][o]);
+                    }
                 }
             }
         }
@@ -875,7 +947,13 @@ int try_launch_fir_any(const IO *in, const IO *taps, IO *out, const Geometry &g,
     p.dw = g.dil_w;
     p.flip = !g.forward;
     p.ncb = ceil_div(p.out_w, 4);
-    const long used_cols = static_cast<long>(4 * p.ncb - 1) * p.sw + span_w + 1;
+    // stride 1, dilation 1, small extents: the register-window instances (the smallest maxima that hold the filter)
+    const bool plain = p.sh == 1 && p.sw == 1 && p.dh == 1 && p.dw == 1 && env_int("DWCONV_ANY_WINDOW", 1);
+    const bool windowed = plain && ((p.kh == 1 && p.kw <= 24) || (p.kw == 1 && p.kh <= 24) || (p.kh <= 8 && p.kw <= 8));
+    // otherwise rows of three taps and more, next to each other, are walked four taps at a time
+    const bool walk = !windowed && p.sw == 1 && p.dw == 1 && p.kw >= 3 && env_int("DWCONV_ANY_WALK", 1);
+    // (the walk reads whole groups of four inputs past the last tap)
+    const long used_cols = walk ? 4l * p.ncb + round_up(p.kw, 4) : static_cast<long>(4 * p.ncb - 1) * p.sw + span_w + 1;
     if (used_cols > (1 << 16)) return -1;
     const int sh = p.sh, span = static_cast<int>(span_h);
     auto rows_for = [sh, span](int units) { return (units * BH - 1) * sh + span + 1; };
@@ -883,10 +961,11 @@ int try_launch_fir_any(const IO *in, const IO *taps, IO *out, const Geometry &g,
     settle_vector_modes<IO>(p);
     const dim3 grid(p.n_tiles), block(kThreads);
     const size_t shmem = lds_bytes(p, p.kh * p.kw);
-    // stride 1, dilation 1, small extents: the register-window instances (the smallest maxima that hold the filter)
-    const bool plain = p.sh == 1 && p.sw == 1 && p.dh == 1 && p.dw == 1 && env_int("DWCONV_ANY_WINDOW", 1);
     const char *window = "";
-    if (plain && p.kh == 1 && p.kw <= 8) {
+    if (walk) {
+        hipLaunchKernelGGL((fir_any_kernel<IO, BH, 1, -1>), grid, block, shmem, stream, p);
+        window = " walk4";
+    } else if (plain && p.kh == 1 && p.kw <= 8) {
         hipLaunchKernelGGL((fir_any_kernel<IO, BH, 1, 1, 8>), grid, block, shmem, stream, p);
         window = " win1x8";
     } else if (plain && p.kh <= 8 && p.kw == 1) {

@@ -16,6 +16,7 @@
 // Large maps use one channel per workgroup (all 256 lanes reduce into one tap
 // table); small maps put P channels of one image side by side, each lane staying
 // with its channel for the whole chunk.
+#include <type_traits>
 #include "dwconv_tile_common.hpp"
 
 namespace dwconv {
@@ -351,11 +352,17 @@ constexpr int kAnyTaps = 64;
 
 struct AnyTaps {
     int kh, kw, sh, sw, dh, dw;
+    int walk;  // rows of taps walked in groups of four (the KHM < 0 instance)
 };
+
+constexpr int kWalkGroups = kAnyTaps / 4;  // groups of four taps per pass
 
 // KHM x KWM (0: none): at stride 1 and dilation 1, filters of at most that extent (and at most kAnyTaps taps) walk a
 // register window of x rows instead: a row of 3 + kw inputs is read once for every tap and gy row that meets it, the
 // loops unrolled to the maxima under uniform bounds; sum (ty, tx) lives in acc[ty * KWM + tx].
+// KHM < 0: column stride 1, undilated columns, any extent: every filter row is cut into groups of four taps, a pass
+// holds kWalkGroups of them, and a group takes its sums from eight inputs per gy row (two 16-byte LDS reads, the
+// first shared with the group before it in the same row).
 template <typename IO, int BH, int SW, int KHM = 0, int KWM = 0>
 __global__ __launch_bounds__(kThreads) void wgrad_any_kernel(const WgradPlan p, const AnyTaps a)
 {
@@ -432,9 +439,15 @@ __global__ __launch_bounds__(kThreads) void wgrad_any_kernel(const WgradPlan p, 
             for (int wr = 0; wr < BH - 1 + KHM; ++wr) {
                 if (wr < BH - 1 + a.kh) {  // (uniform)
                     const float *r = base + wr * p.st.pitch;
-                    float win[3 + KWM];
+                    // (16-byte LDS reads: consecutive lanes then read consecutive banks; the last may reach into the
+                    // slack of the row)
+                    float win[4 * ((3 + KWM + 3) / 4)];
 #pragma unroll
-                    for (int i = 0; i < 3 + KWM; ++i) win[i] = i < 3 + a.kw ? r[i] : 0.f;
+                    for (int v = 0; v < (3 + KWM + 3) / 4; ++v) {
+                        float4 q = make_float4(0.f, 0.f, 0.f, 0.f);
+                        if (4 * v < 3 + a.kw) q = *reinterpret_cast<const float4 *>(r + 4 * v);
+                        win[4 * v] = q.x, win[4 * v + 1] = q.y, win[4 * v + 2] = q.z, win[4 * v + 3] = q.w;
+                    }
 #pragma unroll
                     for (int b = 0; b < BH; ++b) {
                         const int wy = wr - b;
@@ -456,16 +469,88 @@ __global__ __launch_bounds__(kThreads) void wgrad_any_kernel(const WgradPlan p, 
             }
             continue;
         }
+        if constexpr (KHM < 0) {
+            static_assert(SW == 1, "rows are walked four inputs at a time at column stride 1");
+            const int gpr = (a.kw + 3) >> 2, groups = a.kh * gpr;
+            const int g_first = blockIdx.y * kWalkGroups;
+            int wy = g_first / gpr, wg = g_first - wy * gpr;
+            float w[BH][8];
+#pragma unroll
+            for (int q = 0; q < kWalkGroups; ++q) {
+                if (g_first + q < groups) {  // (uniform)
+                    const float *r = base + __mul24(wy * a.dh, p.st.pitch) + 4 * wg;
+                    if (q == 0 || wg == 0) {
+#pragma unroll
+                        for (int b = 0; b < BH; ++b) {
+                            const float4 v = *reinterpret_cast<const float4 *>(r + b * row_step);
+                            w[b][4] = v.x, w[b][5] = v.y, w[b][6] = v.z, w[b][7] = v.w;
+                        }
+                    }
+#pragma unroll
+                    for (int b = 0; b < BH; ++b) {
+                        const float4 v = *reinterpret_cast<const float4 *>(r + b * row_step + 4);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) w[b][i] = w[b][4 + i];
+                        w[b][4] = v.x, w[b][5] = v.y, w[b][6] = v.z, w[b][7] = v.w;
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if (4 * wg + j < a.kw) {  // (uniform)
+                            float sum = acc[4 * q + j];
+#pragma unroll
+                            for (int b = 0; b < BH; ++b)
+#pragma unroll
+                                for (int o = 0; o < 4; ++o) sum = fmaf(g[b][o], w[b][j + o], sum);
+                            acc[4 * q + j] = sum;
+                        }
+                    }
+                    if (++wg == gpr) {
+                        wg = 0;
+                        ++wy;
+                    }
+                }
+            }
+            continue;
+        }
         int ty = ty_first, tx = tx_first;
 #pragma unroll
         for (int t = 0; t < kAnyTaps; ++t) {
             if (t < nt) {  // (uniform)
-                const float *r = base + __mul24(ty * a.dh, p.st.pitch) + tx * a.dw;
                 float sum = acc[t];
+                if constexpr (SW == 1 || SW == 2) {
+                    // lanes are four or eight floats apart: 16-byte LDS reads from the boundary before the tap's offset
+                    // on (the last may reach into the slack of the row) and a uniform choice among what they hold,
+                    // instead of single floats that would meet the same banks four or eight times over
+                    const int off = tx * a.dw;
+                    const float *r = base + __mul24(ty * a.dh, p.st.pitch) + (off & ~3);
+                    auto rows = [&](auto shift) {
+                        constexpr int S = decltype(shift)::value;
 #pragma unroll
-                for (int b = 0; b < BH; ++b)
+                        for (int b = 0; b < BH; ++b) {
+                            constexpr int NR = (S + 3 * SW + 4) / 4;  // 16-byte reads that hold inputs S, S + SW .. S + 3 SW
+                            float w8[4 * NR];
 #pragma unroll
-                    for (int o = 0; o < 4; ++o) sum = fmaf(g[b][o], r[b * row_step + o * sw], sum);
+                            for (int v = 0; v < NR; ++v) {
+                                const float4 q = *reinterpret_cast<const float4 *>(r + b * row_step + 4 * v);
+                                w8[4 * v] = q.x, w8[4 * v + 1] = q.y, w8[4 * v + 2] = q.z, w8[4 * v + 3] = q.w;
+                            }
+#pragma unroll
+                            for (int o = 0; o < 4; ++o) sum = fmaf(g[b][o], w8[S + o * SW], sum);
+                        }
+                    };
+                    switch (off & 3) {
+                    case 0: rows(std::integral_constant<int, 0>{}); break;
+                    case 1: rows(std::integral_constant<int, 1>{}); break;
+                    case 2: rows(std::integral_constant<int, 2>{}); break;
+                    default: rows(std::integral_constant<int, 3>{}); break;
+                    }
+                } else {
+                    const float *r = base + __mul24(ty * a.dh, p.st.pitch) + tx * a.dw;
+#pragma unroll
+                    for (int b = 0; b < BH; ++b)
+#pragma unroll
+                        for (int o = 0; o < 4; ++o) sum = fmaf(g[b][o], r[b * row_step + o * sw], sum);
+                }
                 acc[t] = sum;
                 if (++tx == a.kw) {
                     tx = 0;
@@ -487,6 +572,26 @@ __global__ __launch_bounds__(kThreads) void wgrad_any_kernel(const WgradPlan p, 
                     if ((threadIdx.x & 63) == 63) lds[(threadIdx.x >> 6) * kAnyTaps + wy * a.kw + wx] = sum;
                 }
             }
+    } else if constexpr (KHM < 0) {
+        const int gpr = (a.kw + 3) >> 2, groups = a.kh * gpr;
+        const int g_first = blockIdx.y * kWalkGroups;
+#pragma unroll
+        for (int t = 0; t < kAnyTaps; ++t) {
+            if (g_first + t / 4 < groups) {
+                const float sum = wave_sum_to_last_lane(acc[t]);
+                if ((threadIdx.x & 63) == 63) lds[(threadIdx.x >> 6) * kAnyTaps + t] = sum;
+            }
+        }
+        __syncthreads();
+        const int grp = g_first + static_cast<int>(threadIdx.x >> 2);
+        const int wy = grp / gpr, wx = 4 * (grp - wy * gpr) + static_cast<int>(threadIdx.x & 3);
+        if (threadIdx.x < kAnyTaps && grp < groups && wx < a.kw) {
+            float sum = lds[threadIdx.x];
+#pragma unroll
+            for (int w = 1; w < kThreads / 64; ++w) sum += lds[w * kAnyTaps + threadIdx.x];
+            p.partial[(static_cast<long>(c) * p.chunks + chunk) * KK + wy * a.kw + wx] = sum;
+        }
+        return;
     } else {
 #pragma unroll
         for (int t = 0; t < kAnyTaps; ++t) {
@@ -516,7 +621,10 @@ bool make_any_plan(WgradPlan &p, AnyTaps &a, const WgradGeometry &g, int dil_h, 
     if (static_cast<long>(g.in_h) * g.in_w >= (1l << 30) || static_cast<long>(g.out_h) * g.out_w >= (1l << 30)) return false;
     const long span_h = static_cast<long>(g.kernel_h - 1) * dil_h, span_w = static_cast<long>(g.kernel_w - 1) * dil_w;
     if (span_h > 4096 || span_w > 4096 || g.down_h > 64 || g.down_w > 64 || g.pad_h > 4096 || g.pad_w > 4096) return false;
-    a = AnyTaps{g.kernel_h, g.kernel_w, g.down_h, g.down_w, dil_h, dil_w};
+    a = AnyTaps{g.kernel_h, g.kernel_w, g.down_h, g.down_w, dil_h, dil_w, 0};
+    const bool plain = a.sh == 1 && a.sw == 1 && a.dh == 1 && a.dw == 1 && env_int("DWCONV_ANY_WINDOW", 1);
+    const bool windowed = plain && ((a.kh == 1 && a.kw <= 24) || (a.kw == 1 && a.kh <= 24) || (a.kh <= 8 && a.kw <= 8));
+    a.walk = !windowed && a.sw == 1 && a.dw == 1 && a.kw >= 3 && env_int("DWCONV_ANY_WALK", 1);
     p.batch = g.batch;
     p.channel = g.channel;
     p.out_h = g.out_h;
@@ -529,7 +637,8 @@ bool make_any_plan(WgradPlan &p, AnyTaps &a, const WgradGeometry &g, int dil_h, 
     p.st.col_shift = g.pad_w;
     p.ncb = ceil_div(g.out_w, 4);
     if (p.ncb > kThreads) return false;
-    const long used_cols = static_cast<long>(4 * p.ncb - 1) * g.down_w + span_w + 1;
+    // (the walk reads whole groups of four inputs past the last tap)
+    const long used_cols = a.walk ? 4l * p.ncb + round_up(a.kw, 4) : static_cast<long>(4 * p.ncb - 1) * g.down_w + span_w + 1;
     if (used_cols > (1 << 16)) return false;
     layout_columns(p.st, static_cast<int>(used_cols));
     auto rows_for = [&](int units) { return static_cast<long>(units * BH - 1) * g.down_h + span_h + 1; };
@@ -822,10 +931,14 @@ int try_launch_wgrad_any(const IO *in, const IO *gy, IO *gw, void *ws, size_t ws
     p.vec_gy = p.vec_gy == 1 ? gy_view : (p.vec_gy == 3 && gy_view == 2 ? 3 : 0);
     const size_t image = static_cast<size_t>(p.st.plane_pitch) * 4, red = static_cast<size_t>(kThreads / 64) * kAnyTaps * 4;
     const size_t shmem = image > red ? image : red;
-    const dim3 grid(static_cast<unsigned>(g.channel * p.chunks), static_cast<unsigned>(ceil_div(KK, kAnyTaps))), block(kThreads);
+    const int passes = a.walk ? ceil_div(a.kh * ceil_div(a.kw, 4), kWalkGroups) : ceil_div(KK, kAnyTaps);
+    const dim3 grid(static_cast<unsigned>(g.channel * p.chunks), static_cast<unsigned>(passes)), block(kThreads);
     const bool plain = a.sh == 1 && a.sw == 1 && a.dh == 1 && a.dw == 1 && env_int("DWCONV_ANY_WINDOW", 1);
     const char *window = "";
-    if (plain && a.kh == 1 && a.kw <= 8) {
+    if (a.walk) {
+        hipLaunchKernelGGL((wgrad_any_kernel<IO, BH, 1, -1>), grid, block, shmem, stream, p, a);
+        window = " walk4";
+    } else if (plain && a.kh == 1 && a.kw <= 8) {
         hipLaunchKernelGGL((wgrad_any_kernel<IO, BH, 1, 1, 8>), grid, block, shmem, stream, p, a);
         window = " win1x8";
     } else if (plain && a.kh <= 8 && a.kw == 1) {
@@ -849,7 +962,7 @@ int try_launch_wgrad_any(const IO *in, const IO *gy, IO *gw, void *ws, size_t ws
     const int rc = check_launch("wgrad_any_kernel");
     if (rc != DWCONV_OK) return rc;
     note_variant("wgrad_any%s<k%dx%d,s%dx%d,d%dx%d> rows%d chunks%d passes%d vin%d vgy%d%s", sizeof(IO) == 2 ? "16" : "", a.kh, a.kw, a.sh,
-                 a.sw, a.dh, a.dw, p.rows_per_tile, p.chunks, ceil_div(KK, kAnyTaps), p.st.vec_in, p.vec_gy, window);
+                 a.sw, a.dh, a.dw, p.rows_per_tile, p.chunks, passes, p.st.vec_in, p.vec_gy, window);
     return launch_wgrad_final(static_cast<const float *>(ws), gw, g.channel, KK, p.chunks, stream);
 }
 

@@ -791,7 +791,21 @@ ANY_GEOMETRY = [
     (1, 2, 40, 44, 10, 10, 1, 1, 4, 5, 1, 1), (1, 1, 36, 40, 15, 15, 1, 1, 7, 7, 1, 1),
     (2, 2, 33, 33, 3, 3, 1, 1, 6, 6, 6, 6), (1, 2, 65, 65, 3, 3, 1, 1, 18, 18, 18, 18), (2, 2, 40, 52, 3, 3, 1, 1, 3, 3, 3, 3),
     (1, 3, 50, 38, 5, 3, 2, 1, 4, 2, 2, 3), (2, 2, 12, 70, 1, 1, 1, 1, 0, 0, 1, 1),
+    # rows of taps walked four at a time (column stride and dilation 1, wider than the register windows)
+    (1, 2, 40, 44, 31, 31, 1, 1, 15, 15, 1, 1), (2, 2, 37, 51, 9, 17, 1, 1, 4, 8, 1, 1), (1, 3, 61, 43, 17, 3, 2, 1, 16, 1, 2, 1),
+    (2, 2, 29, 66, 3, 9, 1, 1, 1, 4, 1, 1), (1, 2, 48, 39, 5, 6, 3, 1, 2, 3, 1, 1),
+    # tap offsets at every position within a 16-byte LDS read, column strides 1 and 2
+    (2, 2, 41, 53, 3, 3, 1, 1, 5, 5, 5, 5), (1, 3, 47, 45, 3, 3, 1, 1, 7, 7, 7, 7), (2, 3, 41, 53, 4, 4, 2, 2, 1, 1, 1, 1),
+    (1, 2, 50, 38, 3, 3, 2, 2, 3, 3, 3, 3), (2, 2, 33, 70, 2, 5, 1, 2, 0, 5, 1, 3),
 ]
+
+
+def any_geometry_walks(kh, kw, sh, sw, dh, dw_):
+    """Whether the any-geometry kernels walk the filter rows four taps at a time: column stride and dilation 1, three
+    taps a row or more, and no register-window instance that holds the filter."""
+    plain = (sh, sw, dh, dw_) == (1, 1, 1, 1)
+    windowed = plain and ((kh == 1 and kw <= 24) or (kw == 1 and kh <= 24) or (kh <= 8 and kw <= 8))
+    return not windowed and sw == 1 and dw_ == 1 and kw >= 3
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=["f32", "f16", "bf16"])
@@ -821,6 +835,8 @@ def test_any_geometry_tiled_kernels(dw, gpu, case, dtype):
     _announce(case, str(dtype), v_fwd)
     sfx = "" if dtype == torch.float32 else "16"
     assert v_fwd.startswith("tile_any%s<k%dx%d,s%dx%d,d%dx%d,fwd>" % (sfx, kh, kw, sh, sw, dh, dw_)), v_fwd
+    walks = any_geometry_walks(kh, kw, sh, sw, dh, dw_)
+    assert v_fwd.endswith(" walk4") == walks, v_fwd
     gx, gw = torch.autograd.grad(y, (xg, wg), gy.to(gpu))
     # (the variant note is per thread and autograd runs the backward on its own: the same calls again from here)
     if (dh, dw_) == (1, 1):
@@ -830,7 +846,10 @@ def test_any_geometry_tiled_kernels(dw, gpu, case, dtype):
     v_bwd = _C.last_variant()
     assert "wgrad_any%s<k%dx%d" % (sfx, kh, kw) in v_bwd, v_bwd
     assert ("tile_any%s<" % sfx in v_bwd and ",rot>" in v_bwd) == ((sh, sw) == (1, 1)), v_bwd
-    assert ("passes%d " % ((kh * kw + 63) // 64)) in v_bwd, v_bwd
+    # sixty-four sums a pass: sixteen groups of four taps of a row where the rows are walked, else sixty-four taps
+    passes = (kh * ((kw + 3) // 4) + 15) // 16 if walks else (kh * kw + 63) // 64
+    assert ("passes%d " % passes) in v_bwd, v_bwd
+    assert v_bwd.endswith(" walk4") == walks, v_bwd
     assert torch.equal(gw, gw2)
     tol = 1e-5 + step
     np.testing.assert_allclose(_np(y.detach().double()), y_ref.detach().numpy(), rtol=tol, atol=tol)
