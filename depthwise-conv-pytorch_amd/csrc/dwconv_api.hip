@@ -103,6 +103,9 @@ int run_fir(const T *in, const T *taps, T *out, const Geometry &g, hipStream_t s
             rc = try_launch_fir_any<T>(in, taps, out, g, stream);
             if (rc >= 0) return rc;
         }
+    } else if (!force_generic()) {
+        const int rc = try_launch_fir_f64(in, taps, out, g, stream);
+        if (rc >= 0) return rc;
     }
     return launch_fir_direct<T>(in, taps, out, g, stream);
 }
@@ -195,6 +198,9 @@ size_t wgrad_workspace(const WgradGeometry &g)
             const size_t t16 = bwd_tiled16_workspace(g);
             if (t16 > need) need = t16;
         }
+    } else {
+        const size_t f64 = wgrad_f64_workspace(g);
+        if (f64 > need) need = f64;
     }
     return need;
 }
@@ -233,6 +239,9 @@ int wgrad_any(const T *in, const T *gy, T *gw, void *ws, size_t ws_bytes, int ba
             const int r = try_launch_wgrad_any<T>(in, gy, gw, ws, ws_bytes, g, 1, 1, stream);
             if (r >= 0) return r;
         }
+    } else if (!force_generic()) {
+        const int r = try_launch_wgrad_f64(in, gy, gw, ws, ws_bytes, g, stream);
+        if (r >= 0) return r;
     }
     return launch_wgrad_direct<T>(in, gy, gw, ws, ws_bytes, g, stream);
 }

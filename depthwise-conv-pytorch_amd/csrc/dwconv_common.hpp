@@ -218,6 +218,12 @@ template <typename T>
 int launch_wgrad_direct(const T *in, const T *gy, T *gw, void *ws, size_t ws_bytes,
                         const WgradGeometry &g, hipStream_t stream);
 
+// ---- LDS-tiled fp64 kernels: dwconv_f64.hip (-1 when the geometry is not covered; workspace 0 likewise) ----
+int try_launch_fir_f64(const double *in, const double *taps, double *out, const Geometry &g, hipStream_t stream);
+size_t wgrad_f64_workspace(const WgradGeometry &g);
+int try_launch_wgrad_f64(const double *in, const double *gy, double *gw, void *ws, size_t ws_bytes, const WgradGeometry &g,
+                         hipStream_t stream);
+
 // ---- LDS-tiled fp32 kernels: dwconv_tile.hip ----
 // Return DWCONV_OK after launching, a negative value (-1) when the geometry is
 // outside what the tiled kernels cover (the caller then uses the generic kernel),

@@ -640,6 +640,66 @@ def test_c_entry_points_directly(dw, gpu):
         _C.dwconv2d(x, torch.randn(3, 1, 3, 3, device=gpu), 1, 1, 1, 1, 1, 1, 1, 1, True)
 
 
+# (n, c, h, w, kh, kw, up_h, up_w, down_h, down_w, (pad_h0, pad_h1, pad_w0, pad_w1), forward)
+F64_OPERATOR = [
+    (2, 3, 9, 11, 3, 3, 1, 1, 1, 1, (1, 1, 1, 1), True), (2, 3, 9, 11, 3, 3, 2, 2, 1, 1, (1, 2, 0, 3), False),
+    (2, 3, 23, 17, 5, 5, 2, 2, 2, 2, (2, 1, 3, 0), True), (1, 4, 19, 30, 4, 3, 3, 2, 2, 1, (0, 0, 1, 1), False),
+    (2, 2, 40, 37, 3, 3, 1, 1, 1, 1, (2, 0, -1, 2), True), (1, 2, 31, 45, 7, 7, 1, 1, 2, 2, (3, 3, 3, 3), True),
+    (3, 5, 7, 7, 5, 5, 1, 1, 1, 1, (2, 2, 2, 2), False), (2, 40, 6, 5, 3, 3, 1, 1, 1, 1, (1, 1, 1, 1), True),
+    (1, 2, 70, 130, 9, 5, 1, 1, 3, 2, (4, 1, -2, 4), True), (1, 1, 150, 260, 13, 13, 1, 1, 1, 1, (6, 6, 6, 6), False),
+    (2, 3, 28, 28, 5, 5, 2, 2, 1, 1, (2, 3, 2, 3), False), (1, 2, 1, 1, 3, 3, 1, 1, 1, 1, (1, 1, 1, 1), True),
+]
+
+
+@pytest.mark.parametrize("case", F64_OPERATOR, ids=lambda c: "N%d_C%d_%dx%d_k%dx%d_u%dx%d_d%dx%d_%s" % (c[:10] + ("fwd" if c[11] else "rot",)))
+def test_fp64_tiled_operator(gpu, case):
+    """The raw operator on double tensors through the LDS-tiled fp64 kernel (up- and down-sampling together, pads that
+    differ per side and crop, rotated taps, several planes per workgroup, several bands per plane) against the C
+    oracle to 1e-12."""
+    from torch_dwconv import _C
+
+    n, c, h, w, kh, kw, uh, uw, dh, dw_, pads, fwd = case
+    g = torch.Generator("cpu").manual_seed(17)
+    x = torch.randn(n, c, h, w, generator=g, dtype=torch.float64)
+    wt = torch.randn(c, 1, kh, kw, generator=g, dtype=torch.float64)
+    got = _C.dwconv2d(x.to(gpu), wt.to(gpu), uh, uw, dh, dw_, *pads, fwd)
+    variant = _C.last_variant()
+    _announce(case, variant)
+    assert variant.startswith("tile_f64<k%dx%d,u%dx%d,s%dx%d,%s>" % (kh, kw, uh, uw, dh, dw_, "fwd" if fwd else "rot")), variant
+    ref = oracle.dwconv2d(_np(x), _np(wt), uh, uw, dh, dw_, *pads, fwd)
+    assert _np(got).shape == ref.shape
+    np.testing.assert_allclose(_np(got), ref, rtol=1e-12, atol=1e-12)
+
+
+F64_GRAD_WEIGHT = [(2, 3, 9, 11, 3, 3, 1, 1, 1, 1), (3, 4, 28, 28, 5, 5, 2, 2, 2, 2), (5, 6, 7, 7, 5, 5, 1, 1, 2, 2),
+                   (2, 2, 57, 83, 7, 7, 1, 1, 3, 3), (1, 2, 40, 44, 9, 4, 3, 2, 4, 0), (9, 3, 14, 14, 3, 3, 1, 1, 1, 1),
+                   (2, 1, 130, 150, 3, 3, 1, 1, 1, 1), (33, 2, 6, 6, 7, 7, 1, 1, 3, 3)]
+
+
+@pytest.mark.parametrize("case", F64_GRAD_WEIGHT, ids=lambda c: "N%d_C%d_%dx%d_k%dx%d_s%dx%d_p%dx%d" % c)
+def test_fp64_tiled_grad_weight(gpu, case):
+    """Grad-weight on double tensors through the LDS-tiled fp64 kernel (one to two passes of 32 taps, several images
+    per tile on small planes, several bands on large ones) against the C oracle to 1e-11 of the largest sum; the same
+    bits on a second run."""
+    from torch_dwconv import _C
+
+    n, c, h, w, kh, kw, sh, sw, ph, pw = case
+    g = torch.Generator("cpu").manual_seed(23)
+    x = torch.randn(n, c, h, w, generator=g, dtype=torch.float64)
+    oh, ow = (h + 2 * ph - kh) // sh + 1, (w + 2 * pw - kw) // sw + 1
+    gy = torch.randn(n, c, oh, ow, generator=g, dtype=torch.float64)
+    wt = torch.empty(c, 1, kh, kw, dtype=torch.float64)
+    got = _C.dwconv2d_backward_kernel(x.to(gpu), gy.to(gpu), wt.to(gpu), 1, 1, sh, sw, ph, pw)
+    variant = _C.last_variant()
+    _announce(case, variant)
+    assert variant.startswith("wgrad_f64<k%dx%d,s%dx%d>" % (kh, kw, sh, sw)), variant
+    assert ("passes%d" % ((kh * kw + 31) // 32)) in variant, variant
+    ref = oracle.backward_kernel(_np(x), _np(gy), (kh, kw), sh, sw, ph, pw)
+    np.testing.assert_allclose(_np(got).reshape(ref.shape), ref, rtol=1e-11, atol=1e-11 * float(np.abs(ref).max()))
+    again = _C.dwconv2d_backward_kernel(x.to(gpu), gy.to(gpu), wt.to(gpu), 1, 1, sh, sw, ph, pw)
+    assert torch.equal(got, again)
+
+
 HALF_SHAPES = [(2, 6, 14, 14, 3, 1, 1), (2, 5, 28, 28, 5, 2, 2), (2, 4, 56, 56, 3, 1, 1), (2, 3, 57, 59, 5, 2, 2),
                (1, 8, 7, 7, 5, 1, 2), (2, 4, 112, 112, 3, 2, 1), (1, 2, 33, 35, 7, 1, 3), (2, 8, 14, 14, 5, 2, 2),
                (3, 4, 28, 28, 7, 1, 3), (2, 8, 7, 7, 7, 1, 3), (2, 3, 64, 64, 5, 2, 2), (2, 3, 40, 44, 7, 2, 3),

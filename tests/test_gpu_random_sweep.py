@@ -132,7 +132,7 @@ def test_randomised_geometry_sweep(dw, gpu, seed):
         np.testing.assert_allclose(_np(gx.double()), _np(gx_ref), err_msg=case, **_bounds(dtype))
         _assert_grad_weight(gw, _np(gw_ref), dtype, case)
     # the sweep is only worth its name if it reaches every forward kernel family
-    assert {"tile_down", "small_down", "nhwc_down", "tile_any", "direct_f64", "nhwc_fwd_direct"} <= families, families
+    assert {"tile_down", "small_down", "nhwc_down", "tile_any", "tile_f64", "nhwc_fwd_direct"} <= families, families
 
 
 # ---- the other entry points ---------------------------------------------------------------------------
