@@ -103,8 +103,9 @@ int run_fir(const T *in, const T *taps, T *out, const Geometry &g, hipStream_t s
             rc = try_launch_fir_any<T>(in, taps, out, g, stream);
             if (rc >= 0) return rc;
         }
-    } else if (!force_generic()) {
-        const int rc = try_launch_fir_f64(in, taps, out, g, stream);
+    }
+    if (!force_generic()) {
+        const int rc = try_launch_fir_lds<T>(in, taps, out, g, stream);
         if (rc >= 0) return rc;
     }
     return launch_fir_direct<T>(in, taps, out, g, stream);

@@ -219,7 +219,10 @@ int launch_wgrad_direct(const T *in, const T *gy, T *gw, void *ws, size_t ws_byt
                         const WgradGeometry &g, hipStream_t stream);
 
 // ---- LDS-tiled fp64 kernels: dwconv_f64.hip (-1 when the geometry is not covered; workspace 0 likewise) ----
-int try_launch_fir_f64(const double *in, const double *taps, double *out, const Geometry &g, hipStream_t stream);
+// The operator kernel takes any up/down factors, filter extent and pads, and every element type (fp32 image and sums for
+// the 32- and 16-bit ones: their last tiled stop before the per-element kernel).
+template <typename T>
+int try_launch_fir_lds(const T *in, const T *taps, T *out, const Geometry &g, hipStream_t stream);
 size_t wgrad_f64_workspace(const WgradGeometry &g);
 int try_launch_wgrad_f64(const double *in, const double *gy, double *gw, void *ws, size_t ws_bytes, const WgradGeometry &g,
                          hipStream_t stream);

@@ -14,6 +14,11 @@
 //     partial sums per (channel, chunk of images) that a second kernel adds front to back: no atomics, and the same
 //     bits on every run.
 // With 8-byte elements these are bound by HBM for the 3x3 and 5x5 filters and by the LDS read per multiply-add above.
+//
+// The operator kernel is a template over the element type and is instantiated for float, fp16 and bf16 as well (LDS
+// image and sums in fp32): there it is the last LDS-tiled stop before the one-lane-per-element kernel, for what the
+// kernels of those types leave out: up-sampling with filters other than 3x3 / 5x5 / 7x7 (grad-input of strip,
+// even-sized and large filters above stride 1), up and down together, pads that crop.
 #include <algorithm>
 #include <cstdlib>
 
@@ -30,10 +35,11 @@ constexpr int kSums = 32;           // grad-weight sums per lane and pass
 
 __host__ __device__ inline int floor_div(int a, int b) { return a >= 0 ? a / b : -((-a + b - 1) / b); }
 
+template <typename T>
 struct FirPlan {
-    const double *in;
-    const double *taps;
-    double *out;
+    const T *in;
+    const T *taps;
+    T *out;
     long planes;
     int channel;
     int in_h, in_w, out_h, out_w;
@@ -50,8 +56,9 @@ struct FirPlan {
 
 // Stages rows [iy_first, iy_first + lds_rows) x columns [ix_first, ix_first + pitch) of `planes` planes from `src`
 // (`plane_stride` elements apart) into lds, zero outside the planes.
-__device__ inline void stage_f64(double *lds, const double *src, int planes, long plane_stride, int in_h, int in_w, int iy_first,
-                                 int ix_first, int lds_rows, int pitch)
+template <typename T>
+__device__ inline void stage_f64(typename Io<T>::acc_t *lds, const T *src, int planes, long plane_stride, int in_h, int in_w,
+                                 int iy_first, int ix_first, int lds_rows, int pitch)
 {
     const int per_plane = lds_rows * pitch;
     const int total = planes * per_plane;
@@ -61,18 +68,20 @@ __device__ inline void stage_f64(double *lds, const double *src, int planes, lon
         const int r = rem / pitch;
         const int col = rem - r * pitch;
         const int iy = iy_first + r, ix = ix_first + col;
-        double v = 0.0;
+        typename Io<T>::acc_t v = 0;
         if (iy >= 0 && iy < in_h && ix >= 0 && ix < in_w)
-            v = src[pl * plane_stride + static_cast<long>(iy) * in_w + ix];
+            v = Io<T>::in(src[pl * plane_stride + static_cast<long>(iy) * in_w + ix]);
         lds[idx] = v;
     }
 }
 
 // UP: the up-sampling factor of both axes when it is 1 or 2, 0 = taken from the plan (any, per axis).
-template <int UP>
-__global__ __launch_bounds__(kThreads) void fir_f64_kernel(const FirPlan p)
+template <typename T, int UP>
+__global__ __launch_bounds__(kThreads) void fir_f64_kernel(const FirPlan<T> p)
 {
-    extern __shared__ double lds_f64[];
+    using A = typename Io<T>::acc_t;
+    extern __shared__ double lds_raw_f64[];
+    A *const lds_f64 = reinterpret_cast<A *>(lds_raw_f64);
     const int KK = p.kh * p.kw;
     const int up_h = UP ? UP : p.up_h, up_w = UP ? UP : p.up_w;
     const int pg = blockIdx.x / p.row_tiles, rt = blockIdx.x - pg * p.row_tiles;
@@ -86,11 +95,11 @@ __global__ __launch_bounds__(kThreads) void fir_f64_kernel(const FirPlan p)
     const int e_h = u0 - iy_first * up_h;               // 0 <= e_h < up_h
     const int e_w = p.first_w - p.ix_first * up_w;      // 0 <= e_w < up_w
 
-    double *ltaps = lds_f64 + p.planes_per_tile * p.lds_rows * p.pitch;
+    A *ltaps = lds_f64 + p.planes_per_tile * p.lds_rows * p.pitch;
     for (int i = threadIdx.x; i < nplanes * KK; i += blockDim.x) {
         const int pl = i / KK, t = i - pl * KK;
         const int c = static_cast<int>((plane0 + pl) % p.channel);
-        ltaps[i] = p.taps[static_cast<long>(c) * KK + (p.flip ? KK - 1 - t : t)];
+        ltaps[i] = Io<T>::in(p.taps[static_cast<long>(c) * KK + (p.flip ? KK - 1 - t : t)]);
     }
     const long in_plane = static_cast<long>(p.in_h) * p.in_w;
     stage_f64(lds_f64, p.in + plane0 * in_plane, nplanes, in_plane, p.in_h, p.in_w, iy_first, p.ix_first, p.lds_rows, p.pitch);
@@ -102,14 +111,14 @@ __global__ __launch_bounds__(kThreads) void fir_f64_kernel(const FirPlan p)
         const int rem = item - pl * p.items_per_plane;
         const int rb = rem / p.out_w;
         const int ox = rem - rb * p.out_w;
-        const double *img = lds_f64 + pl * p.lds_rows * p.pitch;
-        const double *tp = ltaps + pl * KK;
+        const A *img = lds_f64 + pl * p.lds_rows * p.pitch;
+        const A *tp = ltaps + pl * KK;
         // offsets, in up-sampled steps, of tap (0, 0) of this lane's first output from the image's origin
         const int dy0 = e_h + rb * kRows * p.down_h;
         const int dx0 = e_w + ox * p.down_w;
-        double acc[kRows];
+        A acc[kRows];
 #pragma unroll
-        for (int b = 0; b < kRows; ++b) acc[b] = 0.0;
+        for (int b = 0; b < kRows; ++b) acc[b] = 0;
         for (int ty = 0; ty < p.kh; ++ty) {
             int row[kRows];
             bool row_ok[kRows];
@@ -129,7 +138,7 @@ __global__ __launch_bounds__(kThreads) void fir_f64_kernel(const FirPlan p)
                 }
             }
             for (int tx = 0; tx < p.kw; ++tx) {
-                const double t = tp[ty * p.kw + tx];
+                const A t = tp[ty * p.kw + tx];
                 const int dx = dx0 + tx;
                 int col;
                 bool col_ok;
@@ -145,20 +154,20 @@ __global__ __launch_bounds__(kThreads) void fir_f64_kernel(const FirPlan p)
                 }
 #pragma unroll
                 for (int b = 0; b < kRows; ++b) {
-                    const double v = img[row[b] + col];
-                    acc[b] = fma((row_ok[b] && col_ok) ? v : 0.0, t, acc[b]);
+                    const A v = img[row[b] + col];
+                    acc[b] = fma((row_ok[b] && col_ok) ? v : A(0), t, acc[b]);
                 }
             }
         }
         const int c = static_cast<int>((plane0 + pl) % p.channel);
-        double *dst = p.out + (plane0 + pl) * p.out_h * p.out_w + ox;
+        T *dst = p.out + (plane0 + pl) * p.out_h * p.out_w + ox;
 #pragma unroll
         for (int b = 0; b < kRows; ++b) {
             const int oy = oy0 + rb * kRows + b;
             if (oy < p.out_h) {
-                double v = acc[b];
+                A v = acc[b];
                 if (!p.flip && p.epi.enabled()) v = epilogue_apply(v, p.epi, c);
-                dst[static_cast<long>(oy) * p.out_w] = v;
+                dst[static_cast<long>(oy) * p.out_w] = Io<T>::out(v);
             }
         }
     }
@@ -210,7 +219,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_f64_kernel(const WgradPlan64 p
         for (int rt = 0; rt < p.row_tiles; ++rt) {
             const int oy0 = rt * p.rows_per_tile;
             __syncthreads();  // the previous band's reads are done
-            stage_f64(lds_f64, p.x + plane0 * in_plane, images, p.channel * in_plane, p.in_h, p.in_w, oy0 * p.down_h - p.pad_h,
+            stage_f64<double>(lds_f64, p.x + plane0 * in_plane, images, p.channel * in_plane, p.in_h, p.in_w, oy0 * p.down_h - p.pad_h,
                       -p.pad_w, p.lds_rows, p.pitch);
             __syncthreads();
             for (int item = threadIdx.x; item < images * p.items; item += blockDim.x) {
@@ -331,8 +340,10 @@ bool make_wgrad_plan(WgradPlan64 &p, const WgradGeometry &g)
 
 }  // namespace
 
-int try_launch_fir_f64(const double *in, const double *taps, double *out, const Geometry &g, hipStream_t stream)
+template <typename T>
+int try_launch_fir_lds(const T *in, const T *taps, T *out, const Geometry &g, hipStream_t stream)
 {
+    constexpr int kElem = sizeof(typename Io<T>::acc_t);
     if (g.mult != 1 || g.dil_h != 1 || g.dil_w != 1) return -1;
     if (g.kernel_h < 1 || g.kernel_w < 1 || g.up_h < 1 || g.up_w < 1 || g.down_h < 1 || g.down_w < 1) return -1;
     if (g.in_h < 1 || g.in_w < 1 || g.out_h < 1 || g.out_w < 1 || g.planes() < 1) return -1;
@@ -341,7 +352,7 @@ int try_launch_fir_f64(const double *in, const double *taps, double *out, const 
     if (std::abs(g.pad_h0) > 4096 || std::abs(g.pad_w0) > 4096) return -1;
     if (g.out_w > (1 << 20) || g.out_h > (1 << 20) || g.in_w > (1 << 20) || g.in_h > (1 << 20)) return -1;
 
-    FirPlan p{};
+    FirPlan<T> p{};
     p.in = in;
     p.taps = taps;
     p.out = out;
@@ -368,7 +379,7 @@ int try_launch_fir_f64(const double *in, const double *taps, double *out, const 
     // rows of a band of `units` * kRows output rows: the worst case over the band's alignment to the up-sampling grid
     auto rows_for = [&](long units) { return ((units * kRows - 1) * g.down_h + g.kernel_h - 1 + g.up_h - 1) / g.up_h + 1; };
     const long KK = static_cast<long>(g.kernel_h) * g.kernel_w;
-    auto bytes = [&](long units, long planes) { return planes * (rows_for(units) * pitch + KK) * 8; };
+    auto bytes = [&](long units, long planes) { return planes * (rows_for(units) * pitch + KK) * kElem; };
     const int row_units = ceil_div(g.out_h, kRows);
     const long ipp_full = static_cast<long>(row_units) * g.out_w;
     long units, planes_per_tile;
@@ -396,13 +407,18 @@ int try_launch_fir_f64(const double *in, const double *taps, double *out, const 
     p.n_tiles = static_cast<int>(tiles);
     const size_t shmem = static_cast<size_t>(bytes(units, planes_per_tile));
     const dim3 grid(static_cast<unsigned>(p.n_tiles)), block(kThreads);
-    if (g.up_h == 1 && g.up_w == 1) hipLaunchKernelGGL(fir_f64_kernel<1>, grid, block, shmem, stream, p);
-    else if (g.up_h == 2 && g.up_w == 2) hipLaunchKernelGGL(fir_f64_kernel<2>, grid, block, shmem, stream, p);
-    else hipLaunchKernelGGL(fir_f64_kernel<0>, grid, block, shmem, stream, p);
-    note_variant("tile_f64<k%dx%d,u%dx%d,s%dx%d,%s> P%d rows%d", p.kh, p.kw, p.up_h, p.up_w, p.down_h, p.down_w, p.flip ? "rot" : "fwd",
+    if (g.up_h == 1 && g.up_w == 1) hipLaunchKernelGGL((fir_f64_kernel<T, 1>), grid, block, shmem, stream, p);
+    else if (g.up_h == 2 && g.up_w == 2) hipLaunchKernelGGL((fir_f64_kernel<T, 2>), grid, block, shmem, stream, p);
+    else hipLaunchKernelGGL((fir_f64_kernel<T, 0>), grid, block, shmem, stream, p);
+    note_variant("tile_%s<k%dx%d,u%dx%d,s%dx%d,%s> P%d rows%d", sizeof(T) == 8 ? "f64" : (sizeof(T) == 4 ? "gen" : "gen16"), p.kh, p.kw, p.up_h, p.up_w, p.down_h, p.down_w, p.flip ? "rot" : "fwd",
                  p.planes_per_tile, p.rows_per_tile);
     return check_launch("fir_f64_kernel");
 }
+
+template int try_launch_fir_lds<double>(const double *, const double *, double *, const Geometry &, hipStream_t);
+template int try_launch_fir_lds<float>(const float *, const float *, float *, const Geometry &, hipStream_t);
+template int try_launch_fir_lds<half_t>(const half_t *, const half_t *, half_t *, const Geometry &, hipStream_t);
+template int try_launch_fir_lds<bf16_t>(const bf16_t *, const bf16_t *, bf16_t *, const Geometry &, hipStream_t);
 
 size_t wgrad_f64_workspace(const WgradGeometry &g)
 {

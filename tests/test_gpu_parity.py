@@ -905,7 +905,10 @@ def test_any_geometry_tiled_kernels(dw, gpu, case, dtype):
         _, gw2 = _C.dwconv2d_general_backward(xg.detach(), gy.to(gpu), wg.detach(), sh, sw, ph, pw, dh, dw_)
     v_bwd = _C.last_variant()
     assert "wgrad_any%s<k%dx%d" % (sfx, kh, kw) in v_bwd, v_bwd
+    # grad-input: the same kernel with rotated taps at stride 1, above it the up-sampling tiled kernel
+    # (dilated layers above stride 1: the per-element kernel)
     assert ("tile_any%s<" % sfx in v_bwd and ",rot>" in v_bwd) == ((sh, sw) == (1, 1)), v_bwd
+    assert ("tile_gen%s<k%dx%d,u%dx%d,s1x1,rot>" % (sfx, kh, kw, sh, sw) in v_bwd) == ((sh, sw) != (1, 1) and (dh, dw_) == (1, 1)), v_bwd
     # sixty-four sums a pass: sixteen groups of four taps of a row where the rows are walked, else sixty-four taps
     passes = (kh * ((kw + 3) // 4) + 15) // 16 if walks else (kh * kw + 63) // 64
     assert ("passes%d " % passes) in v_bwd, v_bwd
@@ -1363,15 +1366,19 @@ def test_fused_epilogue(dw, gpu, case, activation):
         np.testing.assert_allclose(_np(y).astype(np.float64), ref.numpy(), rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("route", ["direct", "tile_gen"])
 @pytest.mark.parametrize("activation", [None, "relu6", "silu"])
-def test_fused_epilogue_per_element_kernel(dw, gpu, activation, monkeypatch):
-    """The epilogue inside the per-element kernel, which serves what no tiled kernel takes (here: with the any-geometry
-    tiled kernel switched off)."""
+def test_fused_epilogue_per_element_kernel(dw, gpu, activation, route, monkeypatch):
+    """The epilogue inside the per-element kernel and inside the last tiled stop before it (here: forced, and with the
+    any-geometry tiled kernel switched off)."""
     from torch_dwconv import _C
     from torch_dwconv.dwconv import depthwise_conv2d_fused
 
-    monkeypatch.setenv("DWCONV_TUNING", "1")
-    monkeypatch.setenv("DWCONV_FIR_ANY", "0")
+    if route == "direct":
+        monkeypatch.setenv("DWCONV_FORCE_GENERIC", "1")
+    else:
+        monkeypatch.setenv("DWCONV_TUNING", "1")
+        monkeypatch.setenv("DWCONV_FIR_ANY", "0")
     shape = (2, 3, 9, 11, 4, 1, 1)
     n, c, h, w, k, s, p = shape
     x, wt, _ = make_inputs(shape, seed=43)
@@ -1379,7 +1386,7 @@ def test_fused_epilogue_per_element_kernel(dw, gpu, activation, monkeypatch):
     g = torch.Generator("cpu").manual_seed(44)
     scale, shift = torch.randn(c, generator=g) + 1.5, torch.randn(c, generator=g)
     y = depthwise_conv2d_fused(x.to(gpu), wt.to(gpu), bias=shift.to(gpu), scale=scale.to(gpu), activation=activation, stride=s, padding=p)
-    assert _C.last_variant().startswith("direct"), _C.last_variant()
+    assert _C.last_variant().startswith(route), _C.last_variant()
     ref = oracle.torch_reference_fused(x, wt, scale, shift, activation, s, p)
     np.testing.assert_allclose(_np(y).astype(np.float64), ref.numpy(), rtol=1e-5, atol=1e-5)
 
