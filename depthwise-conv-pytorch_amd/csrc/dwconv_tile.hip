@@ -836,9 +836,11 @@ int launch_down(TilePlan &p, hipStream_t stream)
     // (16-bit elements land in an fp32 image, so the same bytes in flight need twice the LDS: 28 KiB measured best
     // on the 112x112 3x3 layer, -12 %.)  With four rows per lane 16 KiB is another 1-3 % better on 3x3 layers 112-128
     // wide (bands of 12 rows instead of 16-20) and changes nothing for 5x5 ones; with seven rows per lane it would halve
-    // the band (150 -> 75: 248 -> 305 us) and 20 KiB stays.
-    constexpr int kBudget = S == 2 ? (sizeof(IO) == 2 ? 28 : (BH == 7 ? 20 : 16)) * 1024 : dwconv::kLdsBudget;
-    if (!plan_tiles(p, ceil_div(p.out_h, BH), BH, used_cols, K * K, rows_for, kBudget)) return -1;
+    // the band (150 -> 75: 248 -> 305 us) and 20 KiB stays.  Those 16 KiB are for 3x3 layers on wide maps: planes of
+    // 36-40 columns fit one to a tile in them, 25 items for 256 lanes, and two with 20 KiB (38x38 3x3: 71 -> 54 us,
+    // 40x40: 58 -> 45, 36x36 5x5: 69 -> 52; a 64x64 5x5 layer takes bands of 32 rows instead of 16: 76 -> 71).
+    const int budget = S == 2 ? (sizeof(IO) == 2 ? 28 : (BH == 7 || K != 3 || p.st.in_w < 96 ? 20 : 16)) * 1024 : dwconv::kLdsBudget;
+    if (!plan_tiles(p, ceil_div(p.out_h, BH), BH, used_cols, K * K, rows_for, budget)) return -1;
     // a depth multiplier is served where a tile is one plane (and, backward, a lane has one item): larger maps
     if (p.mult > 1 && (p.planes_per_tile != 1 || p.items_per_plane > kThreads)) return -1;
     settle_vector_modes<IO>(p);
