@@ -332,9 +332,11 @@ int try_launch_fir_tiled16(const IO *in, const IO *taps, IO *out, const Geometry
     // (the window's place within its LDS slots is a compile-time constant: left padding K/2 only)
     if (g.pad_h0 < 0 || g.pad_h0 > 7 || g.pad_w0 != K / 2) return -1;
     if (g.in_w % 8 != 0 || g.out_w % (S == 1 ? 8 : 4) != 0 || g.in_h < 1) return -1;
-    // Input rows of at least 96 elements: narrower planes have too few 8-wide blocks to occupy the lanes, and the
-    // fp32-image kernel with its 4-wide blocks is as fast there (56 x 56: 57-58 us either way).
-    if (g.in_w < env_int("DWCONV_T16_MIN_W", 96)) return -1;
+    // Input rows of at least 48 elements at stride 2 and 72 at stride 1: measured against the fp32-image and stacked
+    // kernels on 48 ... 88 wide maps (batch 64, C = 144, bf16 and fp16), stride 2 is 3-29 % faster here at every
+    // width, stride 1 6-19 % from 72 on (88 x 88 5x5: equal) and mixed below (56 x 56 3x3 and 7x7: 8-12 % slower;
+    // narrower planes have too few 8-wide blocks to occupy the lanes).
+    if (g.in_w < env_int("DWCONV_T16_MIN_W", S == 2 ? 48 : 72)) return -1;
     if (reinterpret_cast<uintptr_t>(in) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 16 != 0) return -1;
     if (static_cast<long>(g.in_h) * g.in_w >= (1l << 30) || static_cast<long>(g.out_h) * g.out_w >= (1l << 30)) return -1;
 

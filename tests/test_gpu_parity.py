@@ -490,7 +490,7 @@ HALF_FULL_SIZE = {
     0: ("tile_down16_dot2", "bwd_tile16_dot2"),    # 112x112 C32 3x3: 16-bit LDS images, fused backward
     1: ("tile_down16_dot2", "bwd_tile_s216"),      # 112x112 C96 3x3 stride 2
     2: ("tile_down16<", "bwd_stack16<k3"),         # 56x56 C144 3x3: backward one channel per workgroup over its stacked images
-    3: ("tile_down16<", "bwd_tile_s216"),          # 56x56 C144 5x5 stride 2
+    3: ("tile_down16_dot2", "bwd_tile_s216"),      # 56x56 C144 5x5 stride 2 (16-bit LDS image from 48 columns on at stride 2)
     4: ("small_down16", "small_bwd16"),            # 28x28 C240 5x5
     5: ("small_down16", "small_bwd16"),            # 28x28 C240 3x3 stride 2
     8: ("small_down16", "small_bwd16"),            # 14x14 C672 5x5
@@ -712,7 +712,10 @@ HALF_SHAPES = [(2, 6, 14, 14, 3, 1, 1), (2, 5, 28, 28, 5, 2, 2), (2, 4, 56, 56, 
                # rows of at least 96 elements in whole groups of eight: the kernels with 16-bit LDS images and
                # two-element dot products (7-row and 4-row blocks, several planes per workgroup, odd heights)
                (1, 3, 96, 104, 3, 1, 1), (1, 2, 100, 96, 5, 1, 2), (1, 2, 98, 112, 7, 1, 3), (1, 2, 97, 120, 5, 2, 2),
-               (1, 12, 8, 96, 3, 1, 1), (2, 5, 6, 128, 5, 1, 2), (1, 2, 61, 104, 7, 2, 3), (1, 3, 30, 96, 3, 2, 1)]
+               (1, 12, 8, 96, 3, 1, 1), (2, 5, 6, 128, 5, 1, 2), (1, 2, 61, 104, 7, 2, 3), (1, 3, 30, 96, 3, 2, 1),
+               # the same kernels on narrower rows: from 48 columns at stride 2, from 72 at stride 1
+               (2, 5, 30, 48, 3, 2, 1), (3, 4, 56, 56, 5, 2, 2), (2, 3, 33, 72, 7, 1, 3), (2, 6, 20, 88, 3, 1, 1),
+               (1, 7, 41, 64, 7, 2, 3), (5, 3, 9, 80, 5, 1, 2)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
