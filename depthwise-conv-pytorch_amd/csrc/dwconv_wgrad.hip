@@ -352,7 +352,8 @@ constexpr int kAnyTaps = 64;
 
 struct AnyTaps {
     int kh, kw, sh, sw, dh, dw;
-    int walk;  // rows of taps walked in groups of four (the KHM < 0 instance)
+    int walk;    // rows of taps walked in groups of four (the KHM < 0 instance)
+    int passes;  // launches of kAnyTaps sums each (blockIdx.y)
 };
 
 constexpr int kWalkGroups = kAnyTaps / 4;  // groups of four taps per pass
@@ -621,10 +622,11 @@ bool make_any_plan(WgradPlan &p, AnyTaps &a, const WgradGeometry &g, int dil_h, 
     if (static_cast<long>(g.in_h) * g.in_w >= (1l << 30) || static_cast<long>(g.out_h) * g.out_w >= (1l << 30)) return false;
     const long span_h = static_cast<long>(g.kernel_h - 1) * dil_h, span_w = static_cast<long>(g.kernel_w - 1) * dil_w;
     if (span_h > 4096 || span_w > 4096 || g.down_h > 64 || g.down_w > 64 || g.pad_h > 4096 || g.pad_w > 4096) return false;
-    a = AnyTaps{g.kernel_h, g.kernel_w, g.down_h, g.down_w, dil_h, dil_w, 0};
+    a = AnyTaps{g.kernel_h, g.kernel_w, g.down_h, g.down_w, dil_h, dil_w, 0, 1};
     const bool plain = a.sh == 1 && a.sw == 1 && a.dh == 1 && a.dw == 1 && env_int("DWCONV_ANY_WINDOW", 1);
     const bool windowed = plain && ((a.kh == 1 && a.kw <= 24) || (a.kw == 1 && a.kh <= 24) || (a.kh <= 8 && a.kw <= 8));
     a.walk = !windowed && a.sw == 1 && a.dw == 1 && a.kw >= 3 && env_int("DWCONV_ANY_WALK", 1);
+    a.passes = a.walk ? ceil_div(a.kh * ceil_div(a.kw, 4), kWalkGroups) : ceil_div(static_cast<int>(KK), kAnyTaps);
     p.batch = g.batch;
     p.channel = g.channel;
     p.out_h = g.out_h;
@@ -659,7 +661,14 @@ bool make_any_plan(WgradPlan &p, AnyTaps &a, const WgradGeometry &g, int dil_h, 
     const long tiles = static_cast<long>(g.batch) * p.row_tiles;
     if (tiles > 0x7fffffffL) return false;
     p.tiles_per_group = static_cast<int>(tiles);
-    int chunks = ceil_div(env_int("DWCONV_WGRAD_WGS", 3072), g.channel);
+    // Three workgroups fit a CU (the sums take the registers), and the 64-sum reduction at a workgroup's end is its
+    // largest fixed cost: 768 workgroups in all, passes included, every one resident from the start, measured best
+    // (atrous 3x3 on 65x65 C=256: 98 -> 83 us; 8x8 on 128x128: 78 -> 68; 10x10, two passes: 141 -> 110; 15x15, four:
+    // 268 -> 214; 31x31 on 56x56, sixteen: 401 -> 299; 1024 and 1536 leave a second, part-filled round: 10-20 %
+    // slower); channels that fill less than two such rounds on their own get two chunks each.
+    const long lanes = static_cast<long>(g.channel) * a.passes;
+    const long target = env_int("DWCONV_WGRAD_WGS", 768);
+    int chunks = static_cast<int>(std::min<long>(std::max<long>((target + lanes - 1) / lanes, lanes < 1536 ? 2 : 1), 1 << 20));
     if (chunks > p.tiles_per_group) chunks = p.tiles_per_group;
     if (chunks < 1) chunks = 1;
     p.chunks = chunks;
@@ -931,7 +940,7 @@ int try_launch_wgrad_any(const IO *in, const IO *gy, IO *gw, void *ws, size_t ws
     p.vec_gy = p.vec_gy == 1 ? gy_view : (p.vec_gy == 3 && gy_view == 2 ? 3 : 0);
     const size_t image = static_cast<size_t>(p.st.plane_pitch) * 4, red = static_cast<size_t>(kThreads / 64) * kAnyTaps * 4;
     const size_t shmem = image > red ? image : red;
-    const int passes = a.walk ? ceil_div(a.kh * ceil_div(a.kw, 4), kWalkGroups) : ceil_div(KK, kAnyTaps);
+    const int passes = a.passes;
     const dim3 grid(static_cast<unsigned>(g.channel * p.chunks), static_cast<unsigned>(passes)), block(kThreads);
     const bool plain = a.sh == 1 && a.sw == 1 && a.dh == 1 && a.dw == 1 && env_int("DWCONV_ANY_WINDOW", 1);
     const char *window = "";
