@@ -357,6 +357,7 @@ struct AnyTaps {
 };
 
 constexpr int kWalkGroups = kAnyTaps / 4;  // groups of four taps per pass
+constexpr int kRedSums = 32;               // sums that cross LDS at a time where a workgroup carries several channels
 
 // KHM x KWM (0: none): at stride 1 and dilation 1, filters of at most that extent (and at most kAnyTaps taps) walk a
 // register window of x rows instead: a row of 3 + kw inputs is read once for every tap and gy row that meets it, the
@@ -376,21 +377,26 @@ __global__ __launch_bounds__(kThreads) void wgrad_any_kernel(const WgradPlan p, 
     const int t_first = blockIdx.y * kAnyTaps;
     const int nt = min(kAnyTaps, KK - t_first);
 
-    const int c = blockIdx.x / p.chunks;
-    const int chunk = blockIdx.x - c * p.chunks;
+    // a workgroup carries planes_per_tile channels (whole small planes side by side, one block per lane) or one
+    const int grp = blockIdx.x / p.chunks;
+    const int chunk = blockIdx.x - grp * p.chunks;
+    const int c = grp * p.planes_per_tile;
+    const int nplanes = min(p.planes_per_tile, p.channel - c);
 
     constexpr int kSums = KHM > 0 ? KHM * KWM : kAnyTaps;
     float acc[kSums];
 #pragma unroll
     for (int t = 0; t < kSums; ++t) acc[t] = 0.f;
 
-    const bool has_item = static_cast<int>(threadIdx.x) < p.items_per_plane;
+    const bool has_item = static_cast<int>(threadIdx.x) < nplanes * p.items_per_plane;
     const int item = has_item ? threadIdx.x : 0;
-    const int rb = fast_div(item, p.ncb_magic);
-    const int cb = item - rb * p.ncb;
+    const int pl = p.planes_per_tile > 1 ? fast_div(item, p.ipp_magic) : 0;
+    const int rem = item - __mul24(pl, p.items_per_plane);
+    const int rb = fast_div(rem, p.ncb_magic);
+    const int cb = rem - rb * p.ncb;
     const int ox = 4 * cb;
     const int row_step = a.sh * p.st.pitch;
-    const float *base = lds + __mul24(rb * BH, row_step) + kSlack + 4 * cb * sw;
+    const float *base = lds + __mul24(pl, p.st.plane_pitch) + __mul24(rb * BH, row_step) + kSlack + 4 * cb * sw;
     const int ty_first = t_first / a.kw, tx_first = t_first - ty_first * a.kw;
 
     for (int tile = chunk; tile < p.tiles_per_group; tile += p.chunks) {
@@ -400,18 +406,19 @@ __global__ __launch_bounds__(kThreads) void wgrad_any_kernel(const WgradPlan p, 
 
         // this lane's block of gy (zero where it hangs over the edge of the plane, and for lanes without an item)
         float g[BH][4];
-        const IO *gsrc = gy + plane0 * p.out_plane + ox;
+        const IO *gsrc = gy + (plane0 + pl) * p.out_plane + ox;
+        const long gy_bytes = static_cast<long>(nplanes) * p.out_plane * sizeof(IO);
 #pragma unroll
         for (int b = 0; b < BH; ++b) {
             const int oy = oy0 + rb * BH + b;
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
             if (p.vec_gy >= 2) {
-                const unsigned off = (ox + oy * p.out_w) * static_cast<unsigned>(sizeof(IO));
+                const unsigned off = (__mul24(pl, p.out_plane) + ox + oy * p.out_w) * static_cast<unsigned>(sizeof(IO));
                 const bool ok = has_item && oy < p.out_h;
                 if (p.vec_gy == 3 && mixed_row_starts(gy + plane0 * p.out_plane, p.out_w))
-                    v = any_width_load4<IO>(any_width_view(gy + plane0 * p.out_plane, static_cast<long>(p.out_plane) * sizeof(IO)), ok ? off : kOob);
+                    v = any_width_load4<IO>(any_width_view(gy + plane0 * p.out_plane, gy_bytes), ok ? off : kOob);
                 else
-                    v = view_load4<IO>(buffer_view(gy + plane0 * p.out_plane, static_cast<long>(p.out_plane) * sizeof(IO)), ok ? off : kOob);
+                    v = view_load4<IO>(buffer_view(gy + plane0 * p.out_plane, gy_bytes), ok ? off : kOob);
                 if (p.vec_gy == 3) keep_first(v, p.out_w - ox);
             } else if (has_item && oy < p.out_h) {
                 const IO *row = gsrc + static_cast<long>(oy) * p.out_w;
@@ -431,7 +438,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_any_kernel(const WgradPlan p, 
         }
 
         if (tile != chunk) __syncthreads();  // the previous tile's window reads are done
-        stage_tile(p.st, x, lds, plane0, 1, oy0 * a.sh - p.pad_h);
+        stage_tile(p.st, x, lds, plane0, nplanes, oy0 * a.sh - p.pad_h);
         __syncthreads();
 
         if constexpr (KHM > 0) {
@@ -562,6 +569,40 @@ __global__ __launch_bounds__(kThreads) void wgrad_any_kernel(const WgradPlan p, 
     }
 
     __syncthreads();  // the tile image is dead; its LDS is reused for the reduction
+    if (p.planes_per_tile > 1) {
+        // lanes [q * ipp, (q + 1) * ipp) hold channel c + q: the sums cross LDS kRedSums at a time, a column per lane,
+        // then one lane per (channel, sum) adds its run front to back
+#pragma unroll
+        for (int s0 = 0; s0 < kSums; s0 += kRedSums) {
+            if (s0) __syncthreads();
+#pragma unroll
+            for (int t = 0; t < kRedSums; ++t)
+                if (s0 + t < kSums) lds[t * kRedPitch + threadIdx.x] = acc[s0 + t];
+            __syncthreads();
+            for (int e = threadIdx.x; e < nplanes * kRedSums; e += blockDim.x) {
+                const int q = e / kRedSums, t = e - q * kRedSums, slot = s0 + t;
+                int tap = -1;  // the tap that sum `slot` belongs to
+                if constexpr (KHM > 0) {
+                    const int wy = slot / KWM, wx = slot - wy * KWM;
+                    if (slot < kSums && wy < a.kh && wx < a.kw) tap = wy * a.kw + wx;
+                } else if constexpr (KHM < 0) {
+                    const int gpr = (a.kw + 3) >> 2;
+                    const int walk_group = blockIdx.y * kWalkGroups + (slot >> 2);
+                    const int wy = walk_group / gpr, wx = 4 * (walk_group - wy * gpr) + (slot & 3);
+                    if (wy < a.kh && wx < a.kw) tap = wy * a.kw + wx;
+                } else {
+                    if (slot < nt) tap = t_first + slot;
+                }
+                if (tap >= 0) {
+                    const float *col = lds + t * kRedPitch + q * p.items_per_plane;
+                    float sum = 0.f;
+                    for (int i = 0; i < p.items_per_plane; ++i) sum += col[i];
+                    p.partial[(static_cast<long>(c + q) * p.chunks + chunk) * KK + tap] = sum;
+                }
+            }
+        }
+        return;
+    }
     // every lane worked on the same channel: wavefront sums, then the four wavefronts in order
     if constexpr (KHM > 0) {
 #pragma unroll
@@ -650,11 +691,19 @@ bool make_any_plan(WgradPlan &p, AnyTaps &a, const WgradGeometry &g, int dil_h, 
     while (units > 1 && bytes(units) > dwconv::kLdsBudget) --units;
     if (bytes(units) > dwconv::kLdsBudget) return false;
     units = ceil_div(row_units, ceil_div(row_units, units));  // even out the bands
-    p.planes_per_tile = 1;
-    p.groups = g.channel;
+    // small planes: whole planes of several channels side by side, a block per lane (14x14 with 15x15 taps: 16 of 256
+    // lanes would have one otherwise)
+    int planes = 1;
+    const int ipp_full = row_units * p.ncb;
+    if (units == row_units && 2 * ipp_full <= kThreads && g.channel > 1 && env_int("DWCONV_WGRAD_ANY_PLANES", 1)) {
+        planes = std::min(kThreads / ipp_full, g.channel);
+        while (planes > 1 && planes * bytes(units) > dwconv::kLdsBudget) --planes;
+    }
+    p.planes_per_tile = planes;
+    p.groups = ceil_div(g.channel, planes);
     p.rows_per_tile = units * BH;
     p.row_tiles = ceil_div(row_units, units);
-    if (!layout_rows(p.st, static_cast<int>(rows_for(units)), 1)) return false;
+    if (!layout_rows(p.st, static_cast<int>(rows_for(units)), planes)) return false;
     p.items_per_plane = units * p.ncb;
     p.ncb_magic = magic_u16(p.ncb);
     p.ipp_magic = magic_u16(p.items_per_plane);
@@ -666,7 +715,7 @@ bool make_any_plan(WgradPlan &p, AnyTaps &a, const WgradGeometry &g, int dil_h, 
     // (atrous 3x3 on 65x65 C=256: 98 -> 83 us; 8x8 on 128x128: 78 -> 68; 10x10, two passes: 141 -> 110; 15x15, four:
     // 268 -> 214; 31x31 on 56x56, sixteen: 401 -> 299; 1024 and 1536 leave a second, part-filled round: 10-20 %
     // slower); channels that fill less than two such rounds on their own get two chunks each.
-    const long lanes = static_cast<long>(g.channel) * a.passes;
+    const long lanes = static_cast<long>(p.groups) * a.passes;
     const long target = env_int("DWCONV_WGRAD_WGS", 768);
     int chunks = static_cast<int>(std::min<long>(std::max<long>((target + lanes - 1) / lanes, lanes < 1536 ? 2 : 1), 1 << 20));
     if (chunks > p.tiles_per_group) chunks = p.tiles_per_group;
@@ -674,7 +723,7 @@ bool make_any_plan(WgradPlan &p, AnyTaps &a, const WgradGeometry &g, int dil_h, 
     p.chunks = chunks;
     p.tiles_per_chunk = ceil_div(p.tiles_per_group, chunks);
     p.strided = 1;
-    if (static_cast<long>(g.channel) * chunks > 0x7fffffffL) return false;
+    if (static_cast<long>(p.groups) * chunks > 0x7fffffffL) return false;
     return true;
 }
 
@@ -935,13 +984,14 @@ int try_launch_wgrad_any(const IO *in, const IO *gy, IO *gw, void *ws, size_t ws
     p.partial = static_cast<float *>(ws);
     p.st.vec_in = row_vector_mode(g.in_w, in);
     p.vec_gy = row_vector_mode(g.out_w, gy);
-    const int in_view = stage_vector_mode(p.st, 1, sizeof(IO)), gy_view = vector_mode(1, p.out_plane, sizeof(IO));
+    const int in_view = stage_vector_mode(p.st, p.planes_per_tile, sizeof(IO)), gy_view = vector_mode(p.planes_per_tile, p.out_plane, sizeof(IO));
     p.st.vec_in = p.st.vec_in == 1 ? in_view : (p.st.vec_in == 3 && in_view == 2 ? 3 : 0);
     p.vec_gy = p.vec_gy == 1 ? gy_view : (p.vec_gy == 3 && gy_view == 2 ? 3 : 0);
-    const size_t image = static_cast<size_t>(p.st.plane_pitch) * 4, red = static_cast<size_t>(kThreads / 64) * kAnyTaps * 4;
+    const size_t image = static_cast<size_t>(p.planes_per_tile) * p.st.plane_pitch * 4;
+    const size_t red = p.planes_per_tile > 1 ? static_cast<size_t>(kRedSums) * kRedPitch * 4 : static_cast<size_t>(kThreads / 64) * kAnyTaps * 4;
     const size_t shmem = image > red ? image : red;
     const int passes = a.passes;
-    const dim3 grid(static_cast<unsigned>(g.channel * p.chunks), static_cast<unsigned>(passes)), block(kThreads);
+    const dim3 grid(static_cast<unsigned>(p.groups * p.chunks), static_cast<unsigned>(passes)), block(kThreads);
     const bool plain = a.sh == 1 && a.sw == 1 && a.dh == 1 && a.dw == 1 && env_int("DWCONV_ANY_WINDOW", 1);
     const char *window = "";
     if (a.walk) {
@@ -970,8 +1020,8 @@ int try_launch_wgrad_any(const IO *in, const IO *gy, IO *gw, void *ws, size_t ws
     else hipLaunchKernelGGL((wgrad_any_kernel<IO, BH, 0>), grid, block, shmem, stream, p, a);
     const int rc = check_launch("wgrad_any_kernel");
     if (rc != DWCONV_OK) return rc;
-    note_variant("wgrad_any%s<k%dx%d,s%dx%d,d%dx%d> rows%d chunks%d passes%d vin%d vgy%d%s", sizeof(IO) == 2 ? "16" : "", a.kh, a.kw, a.sh,
-                 a.sw, a.dh, a.dw, p.rows_per_tile, p.chunks, passes, p.st.vec_in, p.vec_gy, window);
+    note_variant("wgrad_any%s<k%dx%d,s%dx%d,d%dx%d> P%d rows%d chunks%d passes%d vin%d vgy%d%s", sizeof(IO) == 2 ? "16" : "", a.kh, a.kw,
+                 a.sh, a.sw, a.dh, a.dw, p.planes_per_tile, p.rows_per_tile, p.chunks, passes, p.st.vec_in, p.vec_gy, window);
     return launch_wgrad_final(static_cast<const float *>(ws), gw, g.channel, KK, p.chunks, stream);
 }
 

@@ -860,6 +860,9 @@ ANY_GEOMETRY = [
     # tap offsets at every position within a 16-byte LDS read, column strides 1 and 2
     (2, 2, 41, 53, 3, 3, 1, 1, 5, 5, 5, 5), (1, 3, 47, 45, 3, 3, 1, 1, 7, 7, 7, 7), (2, 3, 41, 53, 4, 4, 2, 2, 1, 1, 1, 1),
     (1, 2, 50, 38, 3, 3, 2, 2, 3, 3, 3, 3), (2, 2, 33, 70, 2, 5, 1, 2, 0, 5, 1, 3),
+    # small planes: grad-weight with several channels to a workgroup (the last group short of channels)
+    (3, 7, 14, 14, 15, 15, 1, 1, 7, 7, 1, 1), (2, 40, 7, 7, 9, 9, 1, 1, 4, 4, 1, 1), (2, 5, 20, 24, 4, 4, 1, 1, 1, 2, 1, 1),
+    (2, 7, 33, 33, 3, 3, 1, 1, 6, 6, 6, 6), (4, 9, 12, 10, 1, 7, 1, 1, 0, 3, 1, 1), (3, 11, 9, 13, 3, 3, 2, 2, 2, 2, 2, 2),
 ]
 
 
