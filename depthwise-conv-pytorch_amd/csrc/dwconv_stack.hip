@@ -433,7 +433,10 @@ bool make_plan(StackPlan &p, int K, int D, int batch, int channel, int h, int w,
     const long total_units = static_cast<long>(batch) * ru;
     if (total_units >= (1l << 30)) return false;
     p.total_units = static_cast<int>(total_units);
-    const int budget = env_int("DWCONV_STACK_LDS", 56 * 1024);
+    // (two workgroups to a CU either way; with the 12 padding rows of a 13x13 filter between stacked 14-row images the
+    // full 64 KiB hold a sixth more units: fused backward on 14x14 C=384, batch 64, 216 -> 185 us; 9x9 and 11x11 and
+    // the 5x5 / 7x7 layers measured 1-2 % slower with it)
+    const int budget = env_int("DWCONV_STACK_LDS", (K >= 13 ? 64 : 56) * 1024);
     int units = kThreads / ncb;
     auto rows_for = [&](int u) { return u * kStackBH + ke - 1 + padw * ((u - 1) / ru + 2); };
     // (and at most eight loads per lane and image: they wait in registers while the workgroup computes)
