@@ -8,8 +8,8 @@
 //     input coordinates, with the zero padding materialised, so that the tap loop carries no bounds checks;
 //   * a lane owns one output column and four output rows; consecutive lanes read consecutive doubles from LDS and
 //     store consecutive doubles, 512 bytes per wavefront and row;
-//   * up-sampling (grad-input of strided layers) keeps the image in input coordinates and skips the taps that meet a
-//     stuffed zero (a parity test at up = 2, a division otherwise);
+//   * up-sampling (grad-input of strided layers) keeps the image in input coordinates, and a lane walks only the taps
+//     that meet a real input: every up-th row and column from a first one that depends on the output's position;
 //   * grad-weight keeps 32 sums per lane in registers, cuts larger filters into passes of 32 taps, and leaves
 //     partial sums per (channel, chunk of images) that a second kernel adds front to back: no atomics, and the same
 //     bits on every run.
@@ -119,43 +119,33 @@ __global__ __launch_bounds__(kThreads) void fir_f64_kernel(const FirPlan<T> p)
         A acc[kRows];
 #pragma unroll
         for (int b = 0; b < kRows; ++b) acc[b] = 0;
-        for (int ty = 0; ty < p.kh; ++ty) {
-            int row[kRows];
-            bool row_ok[kRows];
+        if constexpr (UP == 1) {
+            for (int ty = 0; ty < p.kh; ++ty) {
+                int row[kRows];
 #pragma unroll
-            for (int b = 0; b < kRows; ++b) {
-                const int dy = dy0 + b * p.down_h + ty;
-                if constexpr (UP == 1) {
-                    row[b] = dy * p.pitch;
-                    row_ok[b] = true;
-                } else if constexpr (UP == 2) {
-                    row[b] = (dy >> 1) * p.pitch;
-                    row_ok[b] = (dy & 1) == 0;
-                } else {
-                    const int q = dy / up_h;
-                    row[b] = q * p.pitch;
-                    row_ok[b] = q * up_h == dy;
+                for (int b = 0; b < kRows; ++b) row[b] = (dy0 + b * p.down_h + ty) * p.pitch;
+                for (int tx = 0; tx < p.kw; ++tx) {
+                    const A t = tp[ty * p.kw + tx];
+                    const int col = dx0 + tx;
+#pragma unroll
+                    for (int b = 0; b < kRows; ++b) acc[b] = fma(img[row[b] + col], t, acc[b]);
                 }
             }
-            for (int tx = 0; tx < p.kw; ++tx) {
-                const A t = tp[ty * p.kw + tx];
-                const int dx = dx0 + tx;
-                int col;
-                bool col_ok;
-                if constexpr (UP == 1) {
-                    col = dx;
-                    col_ok = true;
-                } else if constexpr (UP == 2) {
-                    col = dx >> 1;
-                    col_ok = (dx & 1) == 0;
-                } else {
-                    col = dx / up_w;
-                    col_ok = col * up_w == dx;
-                }
+        } else {
+            // Up-sampling: of the taps of an output only every up-th row and column meets a real input, the others
+            // a stuffed zero.  The lane walks the ones that count: from the first tap row and column whose
+            // up-sampled coordinate is a multiple of up, in steps of up, which are steps of one in the image.
+            const int tx0 = (up_w - dx0 % up_w) % up_w;
+            const int col0 = (dx0 + tx0) / up_w;
 #pragma unroll
-                for (int b = 0; b < kRows; ++b) {
-                    const A v = img[row[b] + col];
-                    acc[b] = fma((row_ok[b] && col_ok) ? v : A(0), t, acc[b]);
+            for (int b = 0; b < kRows; ++b) {
+                const int dyb = dy0 + b * p.down_h;
+                const int ty0 = (up_h - dyb % up_h) % up_h;
+                const A *r = img + ((dyb + ty0) / up_h) * p.pitch + col0;
+                for (int ty = ty0; ty < p.kh; ty += up_h, r += p.pitch) {
+                    const A *t = tp + ty * p.kw;
+                    int col = 0;
+                    for (int tx = tx0; tx < p.kw; tx += up_w, ++col) acc[b] = fma(r[col], t[tx], acc[b]);
                 }
             }
         }
