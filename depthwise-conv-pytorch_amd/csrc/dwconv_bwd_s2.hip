@@ -332,9 +332,11 @@ bool plan_bwd_s2(BwdS2Plan &p, const WgradGeometry &g, int kBq, size_t esize)
     if (p.prefetch) {
         chunks = env_int("DWCONV_WGRAD_WGS", kCus * (K == 7 ? 3 : 4) * 3) / g.channel;
     } else {
-        // (5x5 fp32: 6144 against 12288 measured 3-8 % faster on 48- to 64-wide maps, the same at 75 and 128 x 96)
-        const int wgs = K >= 5 && esize == 4 ? 6144 : 3072;
-        chunks = ceil_div(env_int("DWCONV_WGRAD_WGS", wgs), g.channel);
+        // (5x5 fp32: 6144 against 12288 measured 3-8 % faster on 48- to 64-wide maps, the same at 75 and 128 x 96;
+        // 3x3 fp32: on maps 96 wide and more three workgroups per CU, all resident from the start, against 3072: 2-7 %
+        // faster on 96-, 112- and 120-wide layers; 38 x 38 likes twice as many, 129 -> 121 us)
+        const int wgs = K >= 5 && esize == 4 ? 6144 : (K == 3 && esize == 4 ? (g.in_w >= 96 ? 768 : (g.in_w < 48 ? 6144 : 3072)) : 3072);
+        chunks = ceil_div(env_int(K == 3 ? "DWCONV_S2_WGS_K3" : "DWCONV_WGRAD_WGS", wgs), g.channel);
     }
     if (chunks > p.tiles_per_group) chunks = p.tiles_per_group;
     if (chunks < 1) chunks = 1;

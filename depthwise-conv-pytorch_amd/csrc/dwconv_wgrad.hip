@@ -735,7 +735,7 @@ bool make_plan(WgradPlan &p, const WgradGeometry &g, bool fused)
     // Workgroups in all: the 3x3 kernels gain 2-3 % from four times as many, shorter chunks; the 5x5 ones, whose
     // per-workgroup reduction of K*K sums weighs more, lose 6-7 %; with 49 sums per lane the 7x7 ones want half as
     // many again (56x56 fused backward: 124 -> 114 us).
-    const int target_wgs = env_int("DWCONV_WGRAD_WGS", K == 3 ? 12288 : (K == 5 ? 3072 : 1536));
+    const int target_wgs = env_int(K == 3 ? "DWCONV_WGRAD_WGS_K3" : "DWCONV_WGRAD_WGS", K == 3 ? 12288 : (K == 5 ? 3072 : 1536));
     p.batch = g.batch;
     p.channel = g.channel;
     p.out_h = g.out_h;
