@@ -467,6 +467,15 @@ int general_forward_any(const T *in, const T *taps, T *out, int batch, int chann
             }
         }
     }
+    if (!force_generic() && out_elems > 0 && multiplier == 1) {
+        // the one-column-per-lane tiled kernel: double tensors, and what the kernels above left of the other types
+        Geometry gg{batch, channel, in_h, in_w, kernel_h, kernel_w, 1, 1, stride_h, stride_w,
+                    pad_h, pad_h, pad_w, pad_w, g.out_h, g.out_w, 1};
+        gg.dil_h = dil_h;
+        gg.dil_w = dil_w;
+        const int r = try_launch_fir_lds<T>(in, taps, out, gg, static_cast<hipStream_t>(stream));
+        if (r >= 0) return r;
+    }
     return general_forward<T>(in, taps, out, g, static_cast<hipStream_t>(stream));
 }
 
@@ -496,6 +505,11 @@ size_t general_workspace_any(const GeneralGeometry &g)
             const size_t mt = wgrad_tiled_workspace(multiplied_wgrad_geometry(g));
             if (mt > need) need = mt;
         }
+    } else if (g.multiplier == 1) {
+        const WgradGeometry wg{g.batch, g.channel, g.in_h, g.in_w, g.out_h, g.out_w, g.kernel_h, g.kernel_w,
+                               g.stride_h, g.stride_w, g.pad_h, g.pad_w};
+        const size_t f64 = wgrad_f64_workspace(wg, g.dil_h, g.dil_w);
+        if (f64 > need) need = f64;
     }
     return need;
 }
@@ -586,6 +600,33 @@ int general_backward_any(const T *in, const T *gy, const T *taps, T *gx, T *gw, 
                 note_variant("%.120s + %.120s", first, second);
                 return DWCONV_OK;
             }
+        }
+    }
+    if constexpr (std::is_same<T, double>::value) {
+        if (has_out && !force_generic() && multiplier == 1 && in_h > 0 && in_w > 0) {
+            // double tensors: grad-input of a stride-1 layer as the correlation with the rotated, dilated taps, and
+            // grad-weight, through the fp64 tiled kernels; either falls back to the per-element kernels
+            rc = -1;
+            if (stride_h == 1 && stride_w == 1) {
+                Geometry gi{batch, channel, g.out_h, g.out_w, kernel_h, kernel_w, 1, 1, 1, 1,
+                            dil_h * (kernel_h - 1) - pad_h, in_h - g.out_h + pad_h, dil_w * (kernel_w - 1) - pad_w,
+                            in_w - g.out_w + pad_w, in_h, in_w, 0};
+                gi.dil_h = dil_h;
+                gi.dil_w = dil_w;
+                rc = try_launch_fir_lds<T>(gy, taps, gx, gi, stream);
+            }
+            if (rc < 0) rc = general_grad_input<T>(gy, taps, gx, g, stream);
+            if (rc != DWCONV_OK) return rc;
+            char first[sizeof(g_variant)];
+            std::snprintf(first, sizeof(first), "%s", g_variant);
+            const WgradGeometry wg{batch, channel, in_h, in_w, g.out_h, g.out_w, kernel_h, kernel_w, stride_h, stride_w, pad_h, pad_w};
+            rc = try_launch_wgrad_f64(in, gy, gw, ws, ws_bytes, wg, stream, dil_h, dil_w);
+            if (rc < 0) rc = general_grad_weight<T>(in, gy, gw, ws, ws_bytes, g, stream);
+            if (rc != DWCONV_OK) return rc;
+            char second[sizeof(g_variant)];
+            std::snprintf(second, sizeof(second), "%s", g_variant);
+            note_variant("%.120s + %.120s", first, second);
+            return DWCONV_OK;
         }
     }
     rc = general_grad_input<T>(gy, taps, gx, g, stream);

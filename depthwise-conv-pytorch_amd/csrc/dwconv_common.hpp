@@ -223,9 +223,9 @@ int launch_wgrad_direct(const T *in, const T *gy, T *gw, void *ws, size_t ws_byt
 // the 32- and 16-bit ones: their last tiled stop before the per-element kernel).
 template <typename T>
 int try_launch_fir_lds(const T *in, const T *taps, T *out, const Geometry &g, hipStream_t stream);
-size_t wgrad_f64_workspace(const WgradGeometry &g);
+size_t wgrad_f64_workspace(const WgradGeometry &g, int dil_h = 1, int dil_w = 1);
 int try_launch_wgrad_f64(const double *in, const double *gy, double *gw, void *ws, size_t ws_bytes, const WgradGeometry &g,
-                         hipStream_t stream);
+                         hipStream_t stream, int dil_h = 1, int dil_w = 1);
 
 // ---- LDS-tiled fp32 kernels: dwconv_tile.hip ----
 // Return DWCONV_OK after launching, a negative value (-1) when the geometry is

@@ -44,6 +44,7 @@ struct FirPlan {
     int channel;
     int in_h, in_w, out_h, out_w;
     int kh, kw, up_h, up_w, down_h, down_w;
+    int dil_h, dil_w;  // dilation of the taps (up = 1 only)
     int flip;
     Epilogue epi;
     int planes_per_tile, rows_per_tile, row_tiles;
@@ -123,10 +124,10 @@ __global__ __launch_bounds__(kThreads) void fir_f64_kernel(const FirPlan<T> p)
             for (int ty = 0; ty < p.kh; ++ty) {
                 int row[kRows];
 #pragma unroll
-                for (int b = 0; b < kRows; ++b) row[b] = (dy0 + b * p.down_h + ty) * p.pitch;
+                for (int b = 0; b < kRows; ++b) row[b] = (dy0 + b * p.down_h + ty * p.dil_h) * p.pitch;
                 for (int tx = 0; tx < p.kw; ++tx) {
                     const A t = tp[ty * p.kw + tx];
-                    const int col = dx0 + tx;
+                    const int col = dx0 + tx * p.dil_w;
 #pragma unroll
                     for (int b = 0; b < kRows; ++b) acc[b] = fma(img[row[b] + col], t, acc[b]);
                 }
@@ -169,7 +170,7 @@ struct WgradPlan64 {
     double *partial;
     int batch, channel;
     int in_h, in_w, out_h, out_w;
-    int kh, kw, down_h, down_w, pad_h, pad_w;
+    int kh, kw, down_h, down_w, pad_h, pad_w, dil_h, dil_w;
     int rows_per_tile, row_tiles;
     int lds_rows, pitch;
     int items;  // (rows_per_tile / kRows) * out_w
@@ -230,7 +231,7 @@ __global__ __launch_bounds__(kThreads) void wgrad_f64_kernel(const WgradPlan64 p
 #pragma unroll
                 for (int t = 0; t < kSums; ++t) {
                     if (t < nt) {  // (uniform)
-                        const double *r = base + ty * p.pitch + tx;
+                        const double *r = base + ty * p.dil_h * p.pitch + tx * p.dil_w;
                         double sum = acc[t];
 #pragma unroll
                         for (int b = 0; b < kRows; ++b) sum = fma(g[b], r[b * row_step], sum);
@@ -283,9 +284,11 @@ int f64_chunks(const WgradGeometry &g)
     return ceil_div(g.batch, per);
 }
 
-bool make_wgrad_plan(WgradPlan64 &p, const WgradGeometry &g)
+bool make_wgrad_plan(WgradPlan64 &p, const WgradGeometry &g, int dil_h, int dil_w)
 {
-    if (g.mult != 1 || g.dil != 1) return false;
+    if (g.mult != 1 || g.dil != 1 || dil_h < 1 || dil_w < 1) return false;
+    const long span_h = static_cast<long>(g.kernel_h - 1) * dil_h, span_w = static_cast<long>(g.kernel_w - 1) * dil_w;
+    if (span_h > 4096 || span_w > 4096) return false;
     if (g.kernel_h < 1 || g.kernel_w < 1 || g.down_h < 1 || g.down_w < 1 || g.pad_h < 0 || g.pad_w < 0) return false;
     if (g.batch < 1 || g.channel < 1 || g.in_h < 1 || g.in_w < 1 || g.out_h < 1 || g.out_w < 1) return false;
     if (g.channel > 65535 * 32 || static_cast<long>(g.kernel_h) * g.kernel_w > 4096) return false;
@@ -303,8 +306,10 @@ bool make_wgrad_plan(WgradPlan64 &p, const WgradGeometry &g)
     p.down_w = g.down_w;
     p.pad_h = g.pad_h;
     p.pad_w = g.pad_w;
-    const long pitch = static_cast<long>(g.out_w - 1) * g.down_w + g.kernel_w;
-    auto rows_for = [&](long units) { return (units * kRows - 1) * g.down_h + g.kernel_h; };
+    p.dil_h = dil_h;
+    p.dil_w = dil_w;
+    const long pitch = static_cast<long>(g.out_w - 1) * g.down_w + span_w + 1;
+    auto rows_for = [&](long units) { return (units * kRows - 1) * g.down_h + span_h + 1; };
     const int row_units = ceil_div(g.out_h, kRows);
     long units = std::max(1, std::min(row_units, ceil_div(2 * kThreads, g.out_w)));
     while (units > 1 && rows_for(units) * pitch * 8 > kLdsBytes) --units;
@@ -334,11 +339,14 @@ template <typename T>
 int try_launch_fir_lds(const T *in, const T *taps, T *out, const Geometry &g, hipStream_t stream)
 {
     constexpr int kElem = sizeof(typename Io<T>::acc_t);
-    if (g.mult != 1 || g.dil_h != 1 || g.dil_w != 1) return -1;
+    if (g.mult != 1 || g.dil_h < 1 || g.dil_w < 1) return -1;
+    if ((g.dil_h != 1 || g.dil_w != 1) && (g.up_h != 1 || g.up_w != 1)) return -1;  // dilated taps: without up-sampling
     if (g.kernel_h < 1 || g.kernel_w < 1 || g.up_h < 1 || g.up_w < 1 || g.down_h < 1 || g.down_w < 1) return -1;
     if (g.in_h < 1 || g.in_w < 1 || g.out_h < 1 || g.out_w < 1 || g.planes() < 1) return -1;
     if (static_cast<long>(g.kernel_h) * g.kernel_w > 4096 || g.kernel_h > 4096 || g.kernel_w > 4096) return -1;
     if (g.up_h > 64 || g.up_w > 64 || g.down_h > 64 || g.down_w > 64) return -1;
+    const long span_h = static_cast<long>(g.kernel_h - 1) * g.dil_h, span_w = static_cast<long>(g.kernel_w - 1) * g.dil_w;
+    if (span_h > 4096 || span_w > 4096) return -1;
     if (std::abs(g.pad_h0) > 4096 || std::abs(g.pad_w0) > 4096) return -1;
     if (g.out_w > (1 << 20) || g.out_h > (1 << 20) || g.in_w > (1 << 20) || g.in_h > (1 << 20)) return -1;
 
@@ -358,16 +366,18 @@ int try_launch_fir_lds(const T *in, const T *taps, T *out, const Geometry &g, hi
     p.up_w = g.up_w;
     p.down_h = g.down_h;
     p.down_w = g.down_w;
+    p.dil_h = g.dil_h;
+    p.dil_w = g.dil_w;
     p.flip = !g.forward;
     p.epi = g.epi;
     p.first_h = -g.pad_h0;
     p.first_w = -g.pad_w0;
     // columns: up-sampled coordinates -pad_w0 .. (out_w - 1) * down_w - pad_w0 + kw - 1
     p.ix_first = floor_div(-g.pad_w0, g.up_w);
-    const long u_last_w = static_cast<long>(g.out_w - 1) * g.down_w - g.pad_w0 + g.kernel_w - 1;
+    const long u_last_w = static_cast<long>(g.out_w - 1) * g.down_w - g.pad_w0 + span_w;
     const long pitch = floor_div(static_cast<int>(u_last_w), g.up_w) - p.ix_first + 1;
     // rows of a band of `units` * kRows output rows: the worst case over the band's alignment to the up-sampling grid
-    auto rows_for = [&](long units) { return ((units * kRows - 1) * g.down_h + g.kernel_h - 1 + g.up_h - 1) / g.up_h + 1; };
+    auto rows_for = [&](long units) { return ((units * kRows - 1) * g.down_h + span_h + g.up_h - 1) / g.up_h + 1; };
     const long KK = static_cast<long>(g.kernel_h) * g.kernel_w;
     auto bytes = [&](long units, long planes) { return planes * (rows_for(units) * pitch + KK) * kElem; };
     const int row_units = ceil_div(g.out_h, kRows);
@@ -400,8 +410,10 @@ int try_launch_fir_lds(const T *in, const T *taps, T *out, const Geometry &g, hi
     if (g.up_h == 1 && g.up_w == 1) hipLaunchKernelGGL((fir_f64_kernel<T, 1>), grid, block, shmem, stream, p);
     else if (g.up_h == 2 && g.up_w == 2) hipLaunchKernelGGL((fir_f64_kernel<T, 2>), grid, block, shmem, stream, p);
     else hipLaunchKernelGGL((fir_f64_kernel<T, 0>), grid, block, shmem, stream, p);
-    note_variant("tile_%s<k%dx%d,u%dx%d,s%dx%d,%s> P%d rows%d", sizeof(T) == 8 ? "f64" : (sizeof(T) == 4 ? "gen" : "gen16"), p.kh, p.kw, p.up_h, p.up_w, p.down_h, p.down_w, p.flip ? "rot" : "fwd",
-                 p.planes_per_tile, p.rows_per_tile);
+    char dil[24] = "";
+    if (p.dil_h != 1 || p.dil_w != 1) std::snprintf(dil, sizeof(dil), " d%dx%d", p.dil_h, p.dil_w);
+    note_variant("tile_%s<k%dx%d,u%dx%d,s%dx%d,%s> P%d rows%d%s", sizeof(T) == 8 ? "f64" : (sizeof(T) == 4 ? "gen" : "gen16"), p.kh, p.kw, p.up_h,
+                 p.up_w, p.down_h, p.down_w, p.flip ? "rot" : "fwd", p.planes_per_tile, p.rows_per_tile, dil);
     return check_launch("fir_f64_kernel");
 }
 
@@ -410,18 +422,18 @@ template int try_launch_fir_lds<float>(const float *, const float *, float *, co
 template int try_launch_fir_lds<half_t>(const half_t *, const half_t *, half_t *, const Geometry &, hipStream_t);
 template int try_launch_fir_lds<bf16_t>(const bf16_t *, const bf16_t *, bf16_t *, const Geometry &, hipStream_t);
 
-size_t wgrad_f64_workspace(const WgradGeometry &g)
+size_t wgrad_f64_workspace(const WgradGeometry &g, int dil_h, int dil_w)
 {
     WgradPlan64 p{};
-    if (!make_wgrad_plan(p, g)) return 0;
+    if (!make_wgrad_plan(p, g, dil_h, dil_w)) return 0;
     return static_cast<size_t>(g.channel) * p.chunks * g.kernel_h * g.kernel_w * sizeof(double);
 }
 
 int try_launch_wgrad_f64(const double *in, const double *gy, double *gw, void *ws, size_t ws_bytes, const WgradGeometry &g,
-                         hipStream_t stream)
+                         hipStream_t stream, int dil_h, int dil_w)
 {
     WgradPlan64 p{};
-    if (!make_wgrad_plan(p, g)) return -1;
+    if (!make_wgrad_plan(p, g, dil_h, dil_w)) return -1;
     const int KK = g.kernel_h * g.kernel_w;
     const size_t need = static_cast<size_t>(g.channel) * p.chunks * KK * sizeof(double);
     if (ws == nullptr || ws_bytes < need)
@@ -438,8 +450,10 @@ int try_launch_wgrad_f64(const double *in, const double *gy, double *gw, void *w
     if (rc != DWCONV_OK) return rc;
     const int total = g.channel * KK;
     hipLaunchKernelGGL(wgrad_f64_final_kernel, dim3(ceil_div(total, 256)), dim3(256), 0, stream, p.partial, gw, total, KK, p.chunks);
-    note_variant("wgrad_f64<k%dx%d,s%dx%d> P%d rows%d chunks%d passes%d", p.kh, p.kw, p.down_h, p.down_w, p.images_per_tile, p.rows_per_tile,
-                 p.chunks, passes);
+    char dil[24] = "";
+    if (dil_h != 1 || dil_w != 1) std::snprintf(dil, sizeof(dil), " d%dx%d", dil_h, dil_w);
+    note_variant("wgrad_f64<k%dx%d,s%dx%d> P%d rows%d chunks%d passes%d%s", p.kh, p.kw, p.down_h, p.down_w, p.images_per_tile,
+                 p.rows_per_tile, p.chunks, passes, dil);
     return check_launch("wgrad_f64_final_kernel");
 }
 

@@ -1773,6 +1773,14 @@ def test_dilation_and_depth_multiplier(dw, gpu, case, dtype):
         assert not v_fwd.startswith("general_fwd"), v_fwd  # the plain case runs the tuned kernels
     elif m == 1 and dtype != torch.float64:
         assert v_fwd.startswith("tile_any<k%dx%d,s%dx%d,d%dx%d" % (kh, kw, s, s, d, d)), v_fwd  # any other dilation / stride
+    elif m == 1:
+        # double tensors: the fp64 tiled kernels, with dilated taps; backward as two passes (grad-input of a stride-1
+        # layer through the same kernel with rotated taps)
+        assert v_fwd.startswith("tile_f64<k%dx%d,u1x1,s%dx%d,fwd>" % (kh, kw, s, s)) and v_fwd.endswith(" d%dx%d" % (d, d)), v_fwd
+        _C.dwconv2d_general_backward(xg.detach(), gy.to(gpu), wg.detach(), s, s, p, p, d, d)
+        v_bwd = _C.last_variant()
+        assert ("tile_f64<" in v_bwd and ",rot>" in v_bwd) == (s == 1), v_bwd
+        assert "wgrad_f64<k%dx%d,s%dx%d>" % (kh, kw, s, s) in v_bwd and v_bwd.endswith(" d%dx%d" % (d, d)), v_bwd
     else:
         assert v_fwd.startswith("general_fwd"), v_fwd
     y_ref, gx_ref, gw_ref = oracle.torch_reference_general(x, wt, gy, s, p, d)
